@@ -1,0 +1,193 @@
+"""Headline benchmark: CSR SpMM, fp32, on the GCN-style power-law graph
+(1,048,576 nodes, N = 128 features) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+A step is one C = A @ B through the C ABI of libscorch_hip.so with A, B
+resident in HBM (the output buffer comes from torch's caching allocator).
+Prints ONE JSON line: whole-job GFLOP/s (2 * nnz * N flops per step, the
+reference's convention, tools/benchmark_spmm_variants.py:127-129), the memory
+roofline of the dominant kernel and the CPU baseline timed on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
+WORKLOAD = "gcn_powerlaw_spmm_fp32"
+
+# HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE from
+# rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured
+# for the kernel as it stands.  Summary: profiles/.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def algorithmic_bytes(M, K, N, nnz):
+    """Every array touched once: col_idx + vals, row_ptr, B, C (fp32 / int32)."""
+    return 8 * nnz + 4 * (M + 1) + 4 * K * N + 4 * M * N
+
+
+def gather_bytes(M, N, nnz):
+    """No-reuse model: a B row re-read for every nonzero."""
+    return 8 * nnz + 4 * (M + 1) + 4 * nnz * N + 4 * M * N
+
+
+def cpu_baseline(w, repeats=5):
+    """The reference's spmm_csr_float_v2 (oracle/_ref, compiled from the
+    reference's sources) or, where that module is absent, this repository's C
+    restatement of it, timed on the host cores on the same inputs.  The timed
+    region is the whole native call, as the reference's own eval_time is: it
+    includes allocating and zero-filling C."""
+    from oracle import oracle as O
+    M, N, nnz = w["M"], w["N"], int(w["col_idx"].size)
+    flops = 2.0 * nnz * N
+    kind, times = "port", []
+    if O.have_ref():
+        try:
+            import torch
+            mod = O.ref_module()
+            pos, crd = torch.from_numpy(w["row_ptr"]), torch.from_numpy(w["col_idx"])
+            val, Bf = torch.from_numpy(w["vals"]), torch.from_numpy(w["B"]).reshape(-1)
+            args = ([M, N], [M, w["K"]], [[], [pos, crd]], val, [w["K"], N], [[], []], Bf)
+            for i in range(repeats + 1):
+                t0 = time.perf_counter()
+                out = mod.spmm_csr_float_v2(*args)
+                dt = time.perf_counter() - t0
+                del out
+                if i:
+                    times.append(dt)
+            kind = "reference"
+        except Exception as exc:  # module built for another host
+            print(f"[bench] reference module unusable here ({exc}); timing the C restatement",
+                  file=sys.stderr)
+            times = []
+    if not times:
+        import numpy as np
+        out = np.empty((M, N), dtype=np.float32)
+        for i in range(repeats + 1):
+            t0 = time.perf_counter()
+            O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"], out=out)
+            dt = time.perf_counter() - t0
+            if i:
+                times.append(dt)
+    med = statistics.median(times)
+    return {"value": round(flops / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
+            "kind": kind, "ms_per_step": round(med * 1e3, 3),
+            "sample": f"full workload (M={M}, nnz={nnz}, N={N}), median of {repeats} calls after 1 "
+                      "warm-up, whole native call incl. allocating and zeroing C"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--rows", type=int, default=1 << 20, help="nodes of the graph (default: the headline size)")
+    ap.add_argument("--features", type=int, default=128)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (the kernel shards by rows "
+              "of A with no reduction; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    from scorch_amd import native, workloads
+    from scorch_amd import scorch_ops_hip as H
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 1
+    if not os.path.exists(native.library_path()):
+        print("libscorch_hip.so is not built (python __graft_entry__.py)", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    t0 = time.time()
+    w = workloads.gcn_powerlaw(M=args.rows, N=args.features)
+    M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
+    print(f"[bench] generated {WORKLOAD}: M={M} nnz={nnz} N={N} in {time.time() - t0:.1f}s", file=sys.stderr)
+
+    pos = torch.from_numpy(w["row_ptr"]).to(dev)
+    crd = torch.from_numpy(w["col_idx"]).to(dev)
+    val = torch.from_numpy(w["vals"]).to(dev)
+    B = torch.from_numpy(w["B"]).to(dev).reshape(-1)
+    call = ([M, N], [M, K], [[], [pos, crd]], val, [K, N], [[], []], B)
+
+    for _ in range(args.warmup):
+        out = H.spmm_csr_float_v2(*call)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_begin = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        out = H.spmm_csr_float_v2(*call)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_begin
+    ms_per_step = wall * 1e3 / args.steps
+    event_ms_per_step = start.elapsed_time(stop) / args.steps
+
+    # per-kernel durations: events around each kernel, on the launch stream
+    L = native.lib()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ws_bytes = L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, 4)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    C = out.storage.value
+    kernel_ms = (ctypes.c_float * 2)()
+    merge_ms, fixup_ms = [], []
+    for _ in range(args.steps):
+        native.check(L.scorch_hip_spmm_csr_f32_timed(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                     val.data_ptr(), B.data_ptr(), C.data_ptr(),
+                                                     ws.data_ptr(), ws.numel(), stream, kernel_ms))
+        merge_ms.append(kernel_ms[0])
+        fixup_ms.append(kernel_ms[1])
+    merge_avg = sum(merge_ms) / len(merge_ms)
+    fixup_avg = sum(fixup_ms) / len(fixup_ms)
+
+    flops = 2.0 * nnz * N
+    algo = algorithmic_bytes(M, K, N, nnz)
+    achieved = algo / (merge_avg * 1e-3) / 1e9
+    result = {
+        "metric": "CSR SpMM GFLOP/s + HBM GB/s (% peak), power-law 1M rows, N=128 fp32",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
+        "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": WORKLOAD, "rows": M, "cols": K, "nnz": nnz, "features": N,
+                   "degree": "zipf(2.1) scaled to mean 16, cap 50000, + self-loops",
+                   "values": "D^-1/2 (A+I) D^-1/2", "seed": workloads.SEEDS["gcn_powerlaw"]},
+        "hbm_gbps_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
+        "hbm_frac_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "event_ms_per_step": round(event_ms_per_step, 4),
+        "roofline": {
+            "bound": "hbm", "kernel": "spmm_merge_kernel<float,2,0>",
+            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES,
+            "algorithmic_bytes": algo, "gather_model_bytes": gather_bytes(M, N, nnz),
+            "gather_model_gbps": round(gather_bytes(M, N, nnz) / (merge_avg * 1e-3) / 1e9, 1),
+            "kernel_ms_avg": round(merge_avg, 4), "fixup_kernel_ms_avg": round(fixup_avg, 4),
+        },
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,196 @@
+/*
+ * scorch_hip.h -- C ABI of libscorch_hip.so: Scorch's prebuilt CSR
+ * sparse x dense kernels (SpMM, SDDMM and their neighbours) for AMD MI355X
+ * (gfx950).
+ *
+ * The library replaces, for device-resident operands only, the reference's
+ * pybind11 module `scorch_ops` (csrc/ops.cpp, csrc/spmm.h, csrc/kernels.h).
+ * Where the reference passes (shape, mode_indices, values) triples of torch
+ * tensors, this ABI passes the arrays underneath them:
+ *
+ *   CSR  "d,s":  row_ptr  int32[M + 1]   (mode_indices[1][0], "pos")
+ *                col_idx  int32[nnz]     (mode_indices[1][1], "crd")
+ *                vals     T[nnz]
+ *   COO  "o,o":  row_idx  int32[nnz]     (mode_indices[0][0])
+ *                col_idx  int32[nnz]     (mode_indices[1][0])
+ *   dense "d,d": flat row-major T[rows * cols]
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer on the current HIP device unless it
+ *     says "host".  The caller owns all memory, outputs included (the
+ *     reference mallocs its outputs; here the caller's allocator does).
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL is
+ *     the default stream) and the call returns without waiting for it.
+ *   - Return value: SCORCH_HIP_OK (0), or one of the positive error codes below; the
+ *     message for the calling thread's last failure is in
+ *     scorch_hip_last_error().  Arguments are validated on the host before
+ *     anything is launched; index CONTENTS are not (as in the reference, an
+ *     out-of-range column index is undefined behaviour).
+ *   - row_ptr must be non-decreasing with row_ptr[0] == 0 and
+ *     row_ptr[M] == nnz.  Column indices within a row may be in any order
+ *     and may repeat.
+ *   - No global mutable state: calls from several host threads on different
+ *     streams do not interfere, provided their workspaces are distinct.
+ *   - Integer kernels wrap on overflow, like the reference's.
+ */
+#ifndef SCORCH_HIP_H_
+#define SCORCH_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SCORCH_HIP_ABI_VERSION 1
+
+/* Every function below is exported from libscorch_hip.so. */
+#if defined(__GNUC__)
+#define SCORCH_HIP_API __attribute__((visibility("default")))
+#else
+#define SCORCH_HIP_API
+#endif
+
+enum scorch_hip_status {
+  SCORCH_HIP_OK = 0,
+  SCORCH_HIP_EINVAL = 1,       /* bad argument (null pointer, negative size, misaligned...) */
+  SCORCH_HIP_EWORKSPACE = 2,   /* workspace missing or too small */
+  SCORCH_HIP_ERUNTIME = 3,     /* a HIP runtime call failed */
+  SCORCH_HIP_EUNSUPPORTED = 4  /* shape outside what the kernels handle */
+};
+
+/* Epilogue selector of scorch_hip_spmm_csr_bias_act_f32. */
+enum scorch_hip_act { SCORCH_HIP_ACT_NONE = 0, SCORCH_HIP_ACT_RELU = 1 };
+
+/* ABI version of the loaded library (SCORCH_HIP_ABI_VERSION at build time). */
+SCORCH_HIP_API int scorch_hip_abi_version(void);
+
+/* Message of the calling thread's most recent failed call ("" if none). */
+SCORCH_HIP_API const char *scorch_hip_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * SpMM: C[M,N] = A_csr[M,K] * B[K,N], all of one dtype.
+ *
+ * Replaces spmm_csr_float_v2 (csrc/spmm.h:2007-2089; the fp32 symbol
+ * scorch.matmul resolves first, src/scorch/prebuilt_kernels.py:45) and
+ * spmm_csr_typed<T> (csrc/spmm.h:91-150), bound as
+ * prebuilt_spmm_csr_{f32,f64,i32,i64} (csrc/ops.cpp:30-39,92-98).  The
+ * reference's tile_size argument has no counterpart.
+ *
+ * Every element of C is written (rows without entries become zero); C need
+ * not be initialised.  `workspace` holds partial sums of rows that are split
+ * between wavefronts; it must be at least
+ * scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, sizeof(T)) bytes, 256-byte
+ * aligned, and must not be shared by calls that may run concurrently.
+ * Results are bit-reproducible from run to run for a given shape.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API size_t scorch_hip_spmm_csr_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem_size);
+
+SCORCH_HIP_API int scorch_hip_spmm_csr_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                            const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                            const float *B, float *C,
+                            void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_f64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                            const int32_t *row_ptr, const int32_t *col_idx, const double *vals,
+                            const double *B, double *C,
+                            void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_i32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                            const int32_t *row_ptr, const int32_t *col_idx, const int32_t *vals,
+                            const int32_t *B, int32_t *C,
+                            void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_i64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                            const int32_t *row_ptr, const int32_t *col_idx, const int64_t *vals,
+                            const int64_t *B, int64_t *C,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
+/* Benchmarking aid: scorch_hip_spmm_csr_f32 with each of its two kernels
+ * bracketed by HIP events on `stream`.  Waits for the work to finish and
+ * reports the durations in milliseconds: kernel_ms[0] the merge-path SpMM
+ * kernel, kernel_ms[1] the carry fix-up kernel (host array of two floats).
+ * Same results as scorch_hip_spmm_csr_f32.  It synchronises, so it is not
+ * meant for production loops.  No counterpart in the reference, whose only
+ * timing is wall-clock around the whole call
+ * (src/scorch/prebuilt_kernels.py:217-222). */
+SCORCH_HIP_API int scorch_hip_spmm_csr_f32_timed(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                  const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                  const float *B, float *C,
+                                  void *workspace, size_t workspace_bytes, void *stream,
+                                  float *kernel_ms /* host, [2] */);
+
+/* Fused C = act(A * B + bias), bias is T[N] broadcast over rows.
+ * Replaces spmm_csr_bias_act<float, relu> (csrc/spmm.h:28-89), bound as
+ * spmm_csr_bias_float and spmm_csr_bias_relu_float (csrc/ops.cpp:167-208).
+ * `act` is a scorch_hip_act.  Workspace as for scorch_hip_spmm_csr_f32. */
+SCORCH_HIP_API int scorch_hip_spmm_csr_bias_act_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                     const int32_t *row_ptr, const int32_t *col_idx,
+                                     const float *vals, const float *B, const float *bias,
+                                     int act, float *C,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * SDDMM: out_vals[p] = mask_vals[p] * <A[i_p, 0:K], B[j_p, 0:K]> for every
+ * stored entry p = (i_p, j_p) of the mask.  A is [M, K], B is [n_cols, K]:
+ * B is indexed [j, k], i.e. the dense product is A * B^T.
+ *
+ * _coo replaces sddmm_coo_float_prebuilt (csrc/kernels.h:508-570, bound at
+ * csrc/ops.cpp:210-217): the result's index arrays are the mask's own, so
+ * only values are produced; entries may be in any order.
+ *
+ * _csr covers the "d,s" mask of einsum("ij,ik,jk->ij"), which the reference
+ * serves with generated code whose result is a coordinate tensor with one
+ * entry per mask entry, in mask order, explicit zeros kept
+ * (src/scorch/ops.py:638-666, src/scorch/compiler/cin_lowerer.py:2286-2326).
+ * out_row_idx, when not NULL, receives the row of every entry (the result's
+ * mode_indices[0][0]); its mode_indices[1][0] is col_idx itself.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_sddmm_coo_f32(int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                             const int32_t *row_idx, const int32_t *col_idx,
+                             const float *mask_vals, const float *A, const float *B,
+                             float *out_vals, void *stream);
+SCORCH_HIP_API int scorch_hip_sddmm_csr_f32(int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                             const int32_t *row_ptr, const int32_t *col_idx,
+                             const float *mask_vals, const float *A, const float *B,
+                             float *out_vals, int32_t *out_row_idx, void *stream);
+
+/* ------------------------------------------------------------------------
+ * SpMV: y[M] = A_csr[M,K] * x[K].
+ * Replaces spmv_csr<T> (csrc/kernels.h:13-49), bound as
+ * prebuilt_spmv_csr_{f32,f64,i32,i64} (csrc/ops.cpp:52-61,100-101).
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_spmv_csr_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+                            const int32_t *col_idx, const float *vals, const float *x,
+                            float *y, void *stream);
+SCORCH_HIP_API int scorch_hip_spmv_csr_f64(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+                            const int32_t *col_idx, const double *vals, const double *x,
+                            double *y, void *stream);
+SCORCH_HIP_API int scorch_hip_spmv_csr_i32(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+                            const int32_t *col_idx, const int32_t *vals, const int32_t *x,
+                            int32_t *y, void *stream);
+SCORCH_HIP_API int scorch_hip_spmv_csr_i64(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+                            const int32_t *col_idx, const int64_t *vals, const int64_t *x,
+                            int64_t *y, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Row softmax over the stored values of a CSR matrix:
+ * out[p] = exp(scale * v[p] - m_i) / sum_q exp(scale * v[q] - m_i), q over
+ * row i, m_i the row maximum of scale * v.  out may alias vals.
+ * The reference composes this step from torch scatter ops in its attention
+ * benchmark (_sparse_softmax_csr_vectorized,
+ * bench/bench_sparse_transformer.py:277-297, applied to scores * scale at
+ * :362-368); it has no native kernel for it.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr,
+                               const float *vals, float scale, float *out, void *stream);
+
+/* Rows of a CSR matrix's entries: row_idx[p] = i for row_ptr[i] <= p < row_ptr[i+1].
+ * The device-side counterpart of the "d,s" -> "o,o" index conversion the
+ * reference performs on the host (STensor.from_coo / to_sparse,
+ * src/scorch/stensor.py:318-365). */
+SCORCH_HIP_API int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr,
+                               int32_t *row_idx, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCORCH_HIP_H_ */

@@ -1,0 +1,23 @@
+"""scorch_amd: Scorch's prebuilt CSR sparse x dense kernels (SpMM, SDDMM and
+their neighbours) as hand-written HIP for AMD MI355X, behind Scorch's own
+``matmul`` / ``einsum`` / ``STensor`` interface.
+
+    import scorch_amd as scorch
+    A = scorch.from_csr(torch_csr).to("cuda")
+    C = scorch.matmul(A, B_cuda)                       # CSR x dense -> dense
+    S = scorch.einsum("ij,ik,jk->ij", mask, Q, K)      # SDDMM
+"""
+from .format import LevelFormat, LevelType, TensorFormat, parse_format
+from .stensor import STensor
+from .storage import TensorIndex, TensorStorage
+from .ops import einsum, matmul, spmm_bias_act
+
+from_torch = STensor.from_torch
+from_coo = STensor.from_coo
+from_csr = STensor.from_csr
+
+__version__ = "0.1.0"
+
+__all__ = ["STensor", "TensorFormat", "TensorIndex", "TensorStorage", "LevelFormat", "LevelType",
+           "parse_format", "einsum", "matmul", "spmm_bias_act", "from_torch", "from_coo", "from_csr",
+           "__version__"]

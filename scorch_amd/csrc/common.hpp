@@ -1,0 +1,106 @@
+// Shared host/device helpers of libscorch_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <type_traits>
+
+#include "../../include/scorch_hip.h"
+
+namespace scorch {
+
+constexpr int kWaveSize = 64;       // CDNA wavefront
+constexpr int kBlockThreads = 256;  // 4 wavefronts per workgroup
+constexpr int kWavesPerBlock = kBlockThreads / kWaveSize;
+
+// ---- error reporting --------------------------------------------------------
+// One message buffer per host thread; scorch_hip_last_error() returns it.
+char *error_buffer();
+constexpr size_t kErrorBufferBytes = 512;
+
+inline int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), kErrorBufferBytes, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define SCORCH_REQUIRE(cond, ...)                                   \
+  do {                                                              \
+    if (!(cond)) return ::scorch::fail(SCORCH_HIP_EINVAL, __VA_ARGS__); \
+  } while (0)
+
+#define SCORCH_HIP_CHECK(expr)                                                       \
+  do {                                                                               \
+    hipError_t err__ = (expr);                                                       \
+    if (err__ != hipSuccess)                                                         \
+      return ::scorch::fail(SCORCH_HIP_ERUNTIME, "%s failed: %s", #expr,             \
+                            hipGetErrorString(err__));                               \
+  } while (0)
+
+inline bool aligned_to(const void *p, size_t bytes) {
+  return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+}
+
+// Validation shared by every entry point that takes a CSR operand.
+inline int check_csr_args(const char *fn, int64_t M, int64_t K, int64_t nnz, const void *row_ptr,
+                          const void *col_idx, const void *vals) {
+  if (M < 0 || K < 0 || nnz < 0)
+    return fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld K=%lld nnz=%lld)", fn,
+                (long long)M, (long long)K, (long long)nnz);
+  if (M >= INT32_MAX || K > INT32_MAX || nnz > INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED,
+                "%s: M, K and nnz must fit the int32 index arrays (M=%lld K=%lld nnz=%lld)", fn,
+                (long long)M, (long long)K, (long long)nnz);
+  if (!row_ptr) return fail(SCORCH_HIP_EINVAL, "%s: row_ptr is NULL", fn);
+  if (nnz > 0 && (!col_idx || !vals))
+    return fail(SCORCH_HIP_EINVAL, "%s: col_idx/vals is NULL with nnz=%lld", fn, (long long)nnz);
+  if (nnz > 0 && (M == 0 || K == 0))
+    return fail(SCORCH_HIP_EINVAL, "%s: nnz=%lld in an empty matrix", fn, (long long)nnz);
+  if (!aligned_to(row_ptr, 4) || !aligned_to(col_idx, 4))
+    return fail(SCORCH_HIP_EINVAL, "%s: index arrays must be 4-byte aligned", fn);
+  return SCORCH_HIP_OK;
+}
+
+// ---- arithmetic traits --------------------------------------------------------
+// Integer kernels accumulate in the unsigned type of the same width so that
+// overflow wraps (the reference's signed overflow wraps in practice).
+template <typename T> struct Acc { using type = T; };
+template <> struct Acc<int32_t> { using type = uint32_t; };
+template <> struct Acc<int64_t> { using type = uint64_t; };
+
+// ---- device helpers ---------------------------------------------------------
+template <typename T, int V> struct alignas(sizeof(T) * V) Vec { T v[V]; };
+
+__device__ __forceinline__ int wave_lane() { return threadIdx.x & (kWaveSize - 1); }
+
+// Value of lane 0's copy in a scalar register: tells the compiler a value is
+// wave-uniform so that addresses built from it use scalar arithmetic.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Wave-cooperative search: number of i in [0, n) with key(i) < bound, for a
+// strictly increasing key.  Each step probes 64 evenly spaced positions, so a
+// million-entry array takes four dependent loads instead of twenty.
+template <typename KeyFn>
+__device__ __forceinline__ int wave_count_below(int n, int64_t bound, KeyFn key) {
+  const int lane = wave_lane();
+  int lo = 0, hi = n;
+  while (lo < hi) {
+    const int span = hi - lo;
+    const int step = (span + kWaveSize - 1) / kWaveSize;
+    const int64_t idx = (int64_t)lo + (int64_t)(lane + 1) * step - 1;
+    bool below = false;
+    if (idx < hi) below = key((int)idx) < bound;
+    const int cnt = __popcll(__ballot(below));
+    const int64_t nhi = (int64_t)lo + (int64_t)(cnt + 1) * step - 1;
+    lo = lo + cnt * step;
+    hi = nhi < hi ? (int)nhi : hi;
+  }
+  return uniform(lo);
+}
+
+}  // namespace scorch

@@ -1,0 +1,181 @@
+// Smaller kernels around the SpMM/SDDMM path: SpMV, CSR row softmax, the
+// CSR -> coordinate row expansion, and the library's error/version calls.
+#include "common.hpp"
+
+namespace scorch {
+
+char *error_buffer() {
+  static thread_local char buf[kErrorBufferBytes] = {0};
+  return buf;
+}
+
+// ---- SpMV -------------------------------------------------------------------
+// One group of G lanes per row (G a power of two chosen from the mean row
+// length): the lanes stride over the row's entries and a butterfly reduction
+// adds their partial sums, so the summation order depends only on G.
+template <typename T, int G>
+__global__ __launch_bounds__(kBlockThreads) void spmv_kernel(int M, const int *__restrict__ row_ptr,
+                                                             const int *__restrict__ col_idx,
+                                                             const T *__restrict__ vals,
+                                                             const T *__restrict__ x,
+                                                             T *__restrict__ y) {
+  using A = typename Acc<T>::type;
+  const int64_t group = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
+  const int t = threadIdx.x % G;
+  const bool live = group < M;
+  A acc = (A)0;
+  if (live) {
+    const int lo = row_ptr[group], hi = row_ptr[group + 1];
+    for (int p = lo + t; p < hi; p += G) acc += (A)vals[p] * (A)x[col_idx[p]];
+  }
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) acc += (A)__shfl_xor((T)acc, off);
+  if (live && t == 0) y[group] = (T)acc;
+}
+
+inline int group_width(int64_t M, int64_t nnz) {
+  const int64_t mean = M > 0 ? (nnz + M - 1) / M : 0;
+  int g = 2;
+  while (g < kWaveSize && g < mean) g *= 2;
+  return g;
+}
+
+template <typename T>
+int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+               const int32_t *col_idx, const T *vals, const T *x, T *y, void *stream) {
+  if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
+  if (M == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(y != nullptr, "%s: y is NULL", fn);
+  SCORCH_REQUIRE(K == 0 || x != nullptr, "%s: x is NULL", fn);
+  SCORCH_REQUIRE(aligned_to(x, sizeof(T)) && aligned_to(y, sizeof(T)) && aligned_to(vals, sizeof(T)),
+                 "%s: value arrays must be aligned to their element size", fn);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int g = group_width(M, nnz);
+  const int64_t threads = M * g;
+  const dim3 grid((unsigned)((threads + kBlockThreads - 1) / kBlockThreads));
+  switch (g) {
+    case 2: spmv_kernel<T, 2><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+    case 4: spmv_kernel<T, 4><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+    case 8: spmv_kernel<T, 8><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+    case 16: spmv_kernel<T, 16><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+    case 32: spmv_kernel<T, 32><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+    default: spmv_kernel<T, 64><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
+  }
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+// ---- CSR row softmax ----------------------------------------------------------
+// One group of G lanes per row; three sweeps over the row (maximum, sum of
+// exponentials, normalised write).  The row is re-read from cache, not kept in
+// registers, so any row length works.
+template <int G>
+__global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
+                                                                    const int *__restrict__ row_ptr,
+                                                                    const float *vals, float scale,
+                                                                    float *out) {
+  const int64_t group = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
+  const int t = threadIdx.x % G;
+  const bool live = group < M;
+  int lo = 0, hi = 0;
+  if (live) {
+    lo = row_ptr[group];
+    hi = row_ptr[group + 1];
+  }
+  float mx = -3.402823466e38f;
+  for (int p = lo + t; p < hi; p += G) mx = fmaxf(mx, vals[p] * scale);
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+  float sum = 0.0f;
+  for (int p = lo + t; p < hi; p += G) sum += expf(vals[p] * scale - mx);
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  for (int p = lo + t; p < hi; p += G) out[p] = expf(vals[p] * scale - mx) / sum;
+}
+
+// ---- CSR -> coordinate rows ---------------------------------------------------
+__global__ __launch_bounds__(kBlockThreads) void csr_row_indices_kernel(
+    int M, int64_t nnz, const int *__restrict__ row_ptr, int *__restrict__ row_idx) {
+  const int lane = wave_lane();
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  const int64_t first = wave * kWaveSize;
+  if (first >= nnz) return;
+  const int64_t last = first + kWaveSize < nnz ? first + kWaveSize : nnz;
+  auto end_key = [&](int i) { return (int64_t)row_ptr[i + 1]; };
+  int lo = wave_count_below(M, first + 1, end_key);  // row of the first entry
+  int hi = wave_count_below(M, last, end_key);       // row of the last entry
+  const int64_t p = first + lane;
+  if (p >= last) return;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)row_ptr[mid + 1] <= p) lo = mid + 1; else hi = mid;
+  }
+  row_idx[p] = lo;
+}
+
+}  // namespace scorch
+
+extern "C" {
+
+int scorch_hip_abi_version(void) { return SCORCH_HIP_ABI_VERSION; }
+
+const char *scorch_hip_last_error(void) { return scorch::error_buffer(); }
+
+#define SCORCH_DEFINE_SPMV(SUFFIX, T)                                                           \
+  int scorch_hip_spmv_csr_##SUFFIX(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,   \
+                                   const int32_t *col_idx, const T *vals, const T *x, T *y,     \
+                                   void *stream) {                                              \
+    return scorch::spmv_entry<T>("scorch_hip_spmv_csr_" #SUFFIX, M, K, nnz, row_ptr, col_idx,   \
+                                 vals, x, y, stream);                                           \
+  }
+
+SCORCH_DEFINE_SPMV(f32, float)
+SCORCH_DEFINE_SPMV(f64, double)
+SCORCH_DEFINE_SPMV(i32, int32_t)
+SCORCH_DEFINE_SPMV(i64, int64_t)
+
+int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, const float *vals,
+                               float scale, float *out, void *stream) {
+  const char *fn = "scorch_hip_softmax_csr_f32";
+  if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
+  if (M >= INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
+  if (M == 0 || nnz == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int g = scorch::group_width(M, nnz);
+  const int64_t threads = M * g;
+  const dim3 grid((unsigned)((threads + scorch::kBlockThreads - 1) / scorch::kBlockThreads));
+  const int m = (int)M;
+  switch (g) {
+    case 2: scorch::softmax_csr_kernel<2><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    case 4: scorch::softmax_csr_kernel<4><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    case 8: scorch::softmax_csr_kernel<8><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    case 16: scorch::softmax_csr_kernel<16><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    case 32: scorch::softmax_csr_kernel<32><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    default: scorch::softmax_csr_kernel<64><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+  }
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr, int32_t *row_idx,
+                               void *stream) {
+  const char *fn = "scorch_hip_csr_row_indices";
+  if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
+  if (M >= INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
+  if (nnz == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(M > 0, "%s: nnz=%lld with no rows", fn, (long long)nnz);
+  SCORCH_REQUIRE(row_idx != nullptr, "%s: row_idx is NULL", fn);
+  const int64_t waves = (nnz + scorch::kWaveSize - 1) / scorch::kWaveSize;
+  const dim3 grid((unsigned)((waves + scorch::kWavesPerBlock - 1) / scorch::kWavesPerBlock));
+  scorch::csr_row_indices_kernel<<<grid, scorch::kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
+      (int)M, nnz, row_ptr, row_idx);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,383 @@
+// CSR x dense SpMM for gfx950: merge-path work split, one wavefront per chunk.
+//
+// Work model.  The rows of A and its nonzeros are merged into one sequence of
+// M + nnz items: nonzero p of row i sits at position p + i, the "end of row i"
+// marker at row_ptr[i+1] + i.  The sequence is cut into chunks of
+// kItemsPerWave items; wavefront c owns chunk c.  A wavefront therefore does a
+// bounded amount of work whatever the row-length distribution: a 50 000-entry
+// row is spread over ~200 wavefronts, 250 one-entry rows share one.
+//
+// Within a chunk the wavefront walks its nonzeros in order.  All 64 lanes work
+// on the SAME nonzero: lane l holds VEC consecutive output columns, so one B
+// row is read with a single coalesced wave-wide load (64 * VEC elements) and
+// the column index / value are wave-uniform (scalar registers, scalar address
+// arithmetic).  When the walk reaches an end-of-row marker the accumulator is
+// stored to C and cleared.  Every row's marker belongs to exactly one chunk,
+// so every row of C is stored exactly once (empty rows store zeros) and C
+// needs no prior zero fill.
+//
+// Rows cut by a chunk boundary.  A chunk that ends inside a row has no marker
+// for it; it writes its partial sum to carry_val[chunk] and the row number to
+// carry_row[chunk].  The chunk holding the marker stores only its own part.
+// spmm_fixup_kernel then adds, in chunk order, the carries of each such row
+// to C: a fixed summation order, so results are bit-reproducible, and no
+// atomics.  A fused bias/ReLU epilogue is applied at the store when the row
+// lies wholly inside the chunk, and by the fix-up otherwise.
+//
+// Columns beyond 64 * VEC are covered by blockIdx.y (each column tile walks
+// the same chunk again; A's indices are small next to the B rows gathered).
+#include "common.hpp"
+
+namespace scorch {
+
+constexpr int kItemsPerWave = 256;  // merge items (row ends + nonzeros) per wavefront
+constexpr int kGather = 8;          // B-row loads in flight per wavefront
+
+enum Epilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasRelu = 2 };
+
+template <typename T, int EPI>
+__device__ __forceinline__ T apply_epilogue(typename Acc<T>::type acc, T bias) {
+  T r = (T)acc;
+  if (EPI != kEpiNone) r = r + bias;
+  if (EPI == kEpiBiasRelu) r = r > (T)0 ? r : (T)0;
+  return r;
+}
+
+template <typename T, int VEC, int EPI>
+__global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
+    int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
+    const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
+    const T *__restrict__ bias, int64_t total_items, int *__restrict__ carry_row,
+    T *__restrict__ carry_val) {
+  using A = typename Acc<T>::type;
+  using VecT = Vec<T, VEC>;
+
+  __shared__ int s_col[kWavesPerBlock][kItemsPerWave];
+  __shared__ T s_val[kWavesPerBlock][kItemsPerWave];
+  __shared__ int s_rp[kWavesPerBlock][kItemsPerWave + 2];
+
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  const int64_t chunk = (int64_t)blockIdx.x * kWavesPerBlock + w;
+  const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
+  const bool active = col0 < N;
+
+  // Chunk [d0, d1) of the merged sequence; chunks past the end are empty.
+  int64_t d0 = chunk * kItemsPerWave;
+  d0 = d0 < total_items ? d0 : total_items;
+  int64_t d1 = d0 + kItemsPerWave;
+  d1 = d1 < total_items ? d1 : total_items;
+
+  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
+  const int x0 = wave_count_below(M, d0, row_end_key);  // rows finished before the chunk
+  const int x1 = wave_count_below(M, d1, row_end_key);  // rows finished by its end
+  const int y0 = uniform((int)(d0 - x0));               // first nonzero of the chunk
+  const int y1 = uniform((int)(d1 - x1));
+  const int n_nz = y1 - y0;
+  const int n_rows = x1 - x0;
+
+  // Stage the chunk's slice of A in LDS: coalesced loads now, broadcast reads later.
+  for (int k = lane; k < n_nz; k += kWaveSize) {
+    s_col[w][k] = col_idx[y0 + k];
+    s_val[w][k] = vals[y0 + k];
+  }
+  // s_rp[k] = row_ptr[x0 + k] for k = 0 .. n_rows + 1 (clamped at M).
+  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
+    const int r = x0 + k < M ? x0 + k : M;
+    s_rp[w][k] = row_ptr[r];
+  }
+  __syncthreads();
+
+  T bias_v[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) bias_v[v] = (EPI != kEpiNone && active) ? bias[col0 + v] : (T)0;
+
+  A acc[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+
+  // Row x0 began in an earlier chunk iff its first nonzero precedes y0: then
+  // its store is a partial sum and its epilogue is left to the fix-up.
+  const bool carry_in = uniform(s_rp[w][0]) < y0;
+
+  int x = x0;
+  int next_end = uniform(s_rp[w][1]);
+
+  auto flush_row = [&]() {
+    if (active) {
+      const bool partial = carry_in && x == x0;
+      VecT o;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v)
+        o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
+      *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+    ++x;
+    next_end = uniform(s_rp[w][x - x0 + 1]);
+  };
+
+  auto gather = [&](int k) -> VecT {
+    const int j = uniform(s_col[w][k]);
+    VecT b;
+    if (active) {
+      b = *reinterpret_cast<const VecT *>(B + (size_t)j * (size_t)N + col0);
+    } else {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) b.v[v] = (T)0;
+    }
+    return b;
+  };
+
+  auto consume = [&](int k, const VecT &b) {
+    while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
+    const A a = (A)s_val[w][k];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
+  };
+
+  int k = 0;
+  for (; k + kGather <= n_nz; k += kGather) {
+    VecT b[kGather];
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) b[u] = gather(k + u);
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) consume(k + u, b[u]);
+  }
+  for (; k < n_nz; ++k) consume(k, gather(k));
+  while (x < x1) flush_row();  // markers after the chunk's last nonzero
+
+  // Whatever is left belongs to row x1, whose marker lies in a later chunk.
+  if (chunk * kItemsPerWave < total_items) {
+    const int row_start = uniform(s_rp[w][n_rows]);
+    const int tail = y1 - (row_start > y0 ? row_start : y0);
+    if (blockIdx.y == 0 && lane == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
+    if (tail > 0 && active) {
+      VecT o;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];
+      *reinterpret_cast<VecT *>(carry_val + (size_t)chunk * (size_t)N + col0) = o;
+    }
+  }
+}
+
+// One wavefront per (chunk, column tile).  The first chunk of each run of
+// equal carry_row values sums the run in chunk order and folds it into C.
+template <typename T, int VEC, int EPI>
+__global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
+    int N, int64_t num_chunks, const int *__restrict__ carry_row,
+    const T *__restrict__ carry_val, T *__restrict__ C, const T *__restrict__ bias) {
+  using A = typename Acc<T>::type;
+  using VecT = Vec<T, VEC>;
+  const int lane = wave_lane();
+  const int64_t chunk = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  if (chunk >= num_chunks) return;
+  const int row = uniform(carry_row[chunk]);
+  if (row < 0) return;
+  if (chunk > 0 && uniform(carry_row[chunk - 1]) == row) return;  // not the head of its run
+  const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
+  if (col0 >= N) return;
+
+  int64_t end = chunk + 1;
+  while (end < num_chunks && uniform(carry_row[end]) == row) ++end;
+
+  A sum[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) sum[v] = (A)0;
+  int64_t c = chunk;
+  constexpr int kBatch = 8;
+  for (; c + kBatch <= end; c += kBatch) {
+    VecT part[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      part[u] = *reinterpret_cast<const VecT *>(carry_val + (size_t)(c + u) * (size_t)N + col0);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) sum[v] += (A)part[u].v[v];
+  }
+  for (; c < end; ++c) {
+    const VecT part = *reinterpret_cast<const VecT *>(carry_val + (size_t)c * (size_t)N + col0);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) sum[v] += (A)part.v[v];
+  }
+
+  VecT *dst = reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0);
+  VecT o = *dst;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    const T b = EPI != kEpiNone ? bias[col0 + v] : (T)0;
+    o.v[v] = apply_epilogue<T, EPI>(sum[v] + (A)o.v[v], b);
+  }
+  *dst = o;
+}
+
+// ---- host side ----------------------------------------------------------------
+
+inline int64_t spmm_num_chunks(int64_t M, int64_t nnz) {
+  return (M + nnz + kItemsPerWave - 1) / kItemsPerWave;
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Workspace layout: carry_row int32[num_chunks] padded to 256 bytes, then
+// carry_val T[num_chunks * N].
+inline size_t spmm_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
+  const size_t chunks = (size_t)spmm_num_chunks(M, nnz);
+  return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256);
+}
+
+// Optional per-kernel timing: events recorded on the launch stream around each
+// of the two kernels.
+struct KernelTimer {
+  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+  int init() {
+    for (auto &e : ev) SCORCH_HIP_CHECK(hipEventCreate(&e));
+    return SCORCH_HIP_OK;
+  }
+  ~KernelTimer() {
+    for (auto &e : ev)
+      if (e) (void)hipEventDestroy(e);
+  }
+};
+
+template <typename T, int VEC, int EPI>
+int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
+                const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
+                KernelTimer *timer) {
+  const int64_t chunks = spmm_num_chunks(M, nnz);
+  int *carry_row = static_cast<int *>(workspace);
+  T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
+                                       align_up((size_t)chunks * sizeof(int), 256));
+  const int tile = kWaveSize * VEC;
+  const dim3 grid((unsigned)((chunks + kWavesPerBlock - 1) / kWavesPerBlock),
+                  (unsigned)((N + tile - 1) / tile));
+  if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
+  spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
+      M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, carry_row, carry_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
+  spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(N, chunks, carry_row,
+                                                                    carry_val, C, bias);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
+  return SCORCH_HIP_OK;
+}
+
+// Elements per lane.  Preferred: the widest vector (at most 16 bytes) that
+// divides N, is aligned and still keeps all 64 lanes busy (64 * VEC <= N).
+// Narrow N: the narrowest vector that covers N with one column tile.
+template <typename T>
+int pick_vec(int64_t N, const void *B, const void *C, const void *ws) {
+  constexpr int kMaxVec = (int)(16 / sizeof(T));
+  auto usable = [&](int vec) {
+    const size_t bytes = sizeof(T) * vec;
+    return N % vec == 0 && aligned_to(B, bytes) && aligned_to(C, bytes) && aligned_to(ws, bytes);
+  };
+  for (int vec = kMaxVec; vec > 1; vec /= 2)
+    if (usable(vec) && (int64_t)kWaveSize * vec <= N) return vec;
+  for (int vec = 2; vec <= kMaxVec; vec *= 2)
+    if (usable(vec) && (int64_t)kWaveSize * vec >= N && (int64_t)kWaveSize * (vec / 2) < N) return vec;
+  return 1;
+}
+
+template <typename T, int EPI>
+int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
+               const int32_t *col_idx, const T *vals, const T *B, const T *bias, T *C,
+               void *workspace, size_t workspace_bytes, void *stream,
+               KernelTimer *timer = nullptr) {
+  if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
+  SCORCH_REQUIRE(N >= 0, "%s: negative N=%lld", fn, (long long)N);
+  if (N > INT32_MAX - kWaveSize * 4)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: N=%lld is too large", fn, (long long)N);
+  if (M == 0 || N == 0) return SCORCH_HIP_OK;  // nothing to write
+  SCORCH_REQUIRE(C != nullptr, "%s: C is NULL", fn);
+  SCORCH_REQUIRE(K == 0 || B != nullptr, "%s: B is NULL", fn);
+  SCORCH_REQUIRE(EPI == kEpiNone || bias != nullptr, "%s: bias is NULL", fn);
+  SCORCH_REQUIRE(aligned_to(B, sizeof(T)) && aligned_to(C, sizeof(T)) && aligned_to(vals, sizeof(T)),
+                 "%s: value arrays must be aligned to their element size", fn);
+  const size_t need = spmm_workspace_bytes(M, nnz, N, sizeof(T));
+  if (!workspace || workspace_bytes < need)
+    return fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
+                workspace ? workspace_bytes : (size_t)0);
+  SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
+  const int64_t chunks = spmm_num_chunks(M, nnz);
+  if ((chunks + kWavesPerBlock - 1) / kWavesPerBlock > INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: too many work chunks", fn);
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int vec = pick_vec<T>(N, B, C, workspace);
+  const int m = (int)M, n = (int)N;
+  if constexpr (sizeof(T) == 4) {
+    if (vec == 4)
+      return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
+  }
+  if (vec == 2)
+    return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
+  return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
+}
+
+}  // namespace scorch
+
+extern "C" {
+
+size_t scorch_hip_spmm_csr_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem_size) {
+  if (M < 0 || nnz < 0 || N < 0 || elem_size == 0) return 0;
+  return scorch::spmm_workspace_bytes(M, nnz, N, elem_size);
+}
+
+#define SCORCH_DEFINE_SPMM(SUFFIX, T)                                                            \
+  int scorch_hip_spmm_csr_##SUFFIX(int64_t M, int64_t K, int64_t N, int64_t nnz,                 \
+                                   const int32_t *row_ptr, const int32_t *col_idx, const T *vals, \
+                                   const T *B, T *C, void *workspace, size_t workspace_bytes,    \
+                                   void *stream) {                                               \
+    return scorch::spmm_entry<T, scorch::kEpiNone>("scorch_hip_spmm_csr_" #SUFFIX, M, K, N, nnz, \
+                                                   row_ptr, col_idx, vals, B, nullptr, C,        \
+                                                   workspace, workspace_bytes, stream);          \
+  }
+
+SCORCH_DEFINE_SPMM(f32, float)
+SCORCH_DEFINE_SPMM(f64, double)
+SCORCH_DEFINE_SPMM(i32, int32_t)
+SCORCH_DEFINE_SPMM(i64, int64_t)
+
+int scorch_hip_spmm_csr_f32_timed(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                  const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                  const float *B, float *C, void *workspace,
+                                  size_t workspace_bytes, void *stream, float *kernel_ms) {
+  const char *fn = "scorch_hip_spmm_csr_f32_timed";
+  SCORCH_REQUIRE(kernel_ms != nullptr, "%s: kernel_ms is NULL", fn);
+  kernel_ms[0] = kernel_ms[1] = 0.0f;
+  if (M == 0 || N == 0)
+    return scorch::spmm_entry<float, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B,
+                                                       nullptr, C, workspace, workspace_bytes, stream);
+  scorch::KernelTimer timer;
+  if (int rc = timer.init()) return rc;
+  if (int rc = scorch::spmm_entry<float, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals,
+                                                           B, nullptr, C, workspace,
+                                                           workspace_bytes, stream, &timer))
+    return rc;
+  SCORCH_HIP_CHECK(hipEventSynchronize(timer.ev[2]));
+  SCORCH_HIP_CHECK(hipEventElapsedTime(&kernel_ms[0], timer.ev[0], timer.ev[1]));
+  SCORCH_HIP_CHECK(hipEventElapsedTime(&kernel_ms[1], timer.ev[1], timer.ev[2]));
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_spmm_csr_bias_act_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                     const int32_t *row_ptr, const int32_t *col_idx,
+                                     const float *vals, const float *B, const float *bias, int act,
+                                     float *C, void *workspace, size_t workspace_bytes,
+                                     void *stream) {
+  const char *fn = "scorch_hip_spmm_csr_bias_act_f32";
+  if (act == SCORCH_HIP_ACT_NONE)
+    return scorch::spmm_entry<float, scorch::kEpiBias>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B,
+                                                       bias, C, workspace, workspace_bytes, stream);
+  if (act == SCORCH_HIP_ACT_RELU)
+    return scorch::spmm_entry<float, scorch::kEpiBiasRelu>(fn, M, K, N, nnz, row_ptr, col_idx, vals,
+                                                           B, bias, C, workspace, workspace_bytes,
+                                                           stream);
+  return scorch::fail(SCORCH_HIP_EINVAL, "%s: unknown activation %d", fn, act);
+}
+
+}  // extern "C"

@@ -1,0 +1,88 @@
+"""ctypes binding of libscorch_hip.so (declarations: include/scorch_hip.h).
+
+The library is loaded from this directory.  If it is not there it is built
+once with hipcc (scorch_amd.build); if that is impossible the import of the
+kernels fails with an error -- there is no fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional
+
+from . import build as _build
+
+_i64 = ctypes.c_int64
+_ptr = ctypes.c_void_p
+_size = ctypes.c_size_t
+
+OK, EINVAL, EWORKSPACE, ERUNTIME, EUNSUPPORTED = 0, 1, 2, 3, 4
+
+_SPMM = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
+_SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
+
+# name -> (restype, argtypes); one entry per declaration in include/scorch_hip.h
+SIGNATURES = {
+    "scorch_hip_abi_version": (ctypes.c_int, []),
+    "scorch_hip_last_error": (ctypes.c_char_p, []),
+    "scorch_hip_spmm_csr_workspace_bytes": (_size, [_i64, _i64, _i64, _size]),
+    "scorch_hip_spmm_csr_f32": (ctypes.c_int, _SPMM),
+    "scorch_hip_spmm_csr_f64": (ctypes.c_int, _SPMM),
+    "scorch_hip_spmm_csr_i32": (ctypes.c_int, _SPMM),
+    "scorch_hip_spmm_csr_i64": (ctypes.c_int, _SPMM),
+    "scorch_hip_spmm_csr_f32_timed": (ctypes.c_int, _SPMM + [ctypes.POINTER(ctypes.c_float)]),
+    "scorch_hip_spmm_csr_bias_act_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
+                                                        _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_sddmm_coo_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                                _ptr, _ptr]),
+    "scorch_hip_sddmm_csr_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                                _ptr, _ptr, _ptr]),
+    "scorch_hip_spmv_csr_f32": (ctypes.c_int, _SPMV),
+    "scorch_hip_spmv_csr_f64": (ctypes.c_int, _SPMV),
+    "scorch_hip_spmv_csr_i32": (ctypes.c_int, _SPMV),
+    "scorch_hip_spmv_csr_i64": (ctypes.c_int, _SPMV),
+    "scorch_hip_softmax_csr_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr, _ptr]),
+    "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+_lock = threading.Lock()
+
+
+class ScorchHipError(RuntimeError):
+    """A libscorch_hip call returned a non-zero status."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"libscorch_hip error {code}: {message}")
+        self.code = code
+
+
+def library_path() -> str:
+    return _build.LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library (built first if the file is missing)."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(_build.LIB_PATH):
+                    _build.build_library()
+                handle = ctypes.CDLL(_build.LIB_PATH)
+                for name, (restype, argtypes) in SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype = restype
+                    fn.argtypes = argtypes
+                _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().scorch_hip_last_error().decode("utf-8", "replace")
+
+
+def check(code: int) -> None:
+    if code != OK:
+        raise ScorchHipError(code, last_error())

@@ -1,0 +1,209 @@
+"""matmul / einsum with the reference's call signatures, for device-resident
+operands (reference: src/scorch/ops.py:248-423).
+
+What is routed here: CSR x dense ``matmul`` (and its einsum spelling
+"ij,jk->ik"), CSR x vector ``matmul``, and the SDDMM einsum "ij,ik,jk->ij"
+with a coordinate or CSR mask.  Those are the expressions the reference serves
+with prebuilt native kernels (plus the CSR-mask SDDMM its code generator
+serves); here they run as HIP kernels.  Every other expression belongs to the
+reference's compiler, which this package does not contain: it raises
+``NotImplementedError`` rather than compute anything a different way.
+
+There is no host path: a sparse operand that is not on a HIP device raises
+``RuntimeError``.  (Dense x dense goes to ``torch.matmul`` on whatever device,
+exactly as the reference does at ops.py:256-293.)
+"""
+from __future__ import annotations
+
+import time
+from typing import Any, List, Optional, Tuple, Union
+
+import torch
+
+from . import scorch_ops_hip
+from .format import parse_format
+from .prebuilt_kernels import (_timed, execute_prebuilt_binary_kernel, resolve_prebuilt_fused,
+                               resolve_prebuilt_matmul)
+from .stensor import STensor
+from .storage import TensorIndex
+
+_SPMM_EXPR = "ab,bc->ac"
+_SDDMM_EXPR = "ab,ac,bc->ab"       # "ij,ik,jk->ij": B indexed [j, k]
+_SDDMM_EXPR_KJ = "ab,ac,cb->ab"    # "ij,ik,kj->ij": B indexed [k, j]
+
+
+def _canonical(expression: str) -> str:
+    """Rename subscripts by order of first appearance: "ik,kj->ij" -> "ab,bc->ac"."""
+    names = {}
+    out = []
+    for ch in expression.replace(" ", ""):
+        if ch.isalpha():
+            if ch not in names:
+                names[ch] = chr(ord("a") + len(names))
+            out.append(names[ch])
+        else:
+            out.append(ch)
+    return "".join(out)
+
+
+def _require_device(*tensors: STensor) -> None:
+    for t in tensors:
+        if not t.values.is_cuda:
+            raise RuntimeError(
+                "scorch_amd runs sparse kernels on HIP devices only; this operand is on "
+                f"{t.values.device}. Move it with STensor.to('cuda') (host tensors belong to the "
+                "reference's CPU kernels).")
+
+
+def _wrap(result_cpp, shape, fmt) -> STensor:
+    return STensor(shape=tuple(shape),
+                   index=TensorIndex(mode_indices=result_cpp.storage.index.mode_indices,
+                                     tensor_format=fmt),
+                   value=result_cpp.storage.value)
+
+
+def _not_prebuilt(what: str):
+    return NotImplementedError(
+        f"{what}: no prebuilt device kernel matches; the reference compiles such expressions with "
+        "its code generator, which is outside this package")
+
+
+def _run_prebuilt_matmul(a: STensor, b: STensor, requested_format, time_dict):
+    resolved = resolve_prebuilt_matmul(a, b, output_format=requested_format)
+    if resolved is None:
+        return None
+    _require_device(a, b)
+    result_cpp, result_shape = execute_prebuilt_binary_kernel(resolved.fn, a, b, time_dict=time_dict)
+    return _wrap(result_cpp, result_shape, resolved.output_format)
+
+
+def matmul(a: Union[torch.Tensor, STensor], b: Union[torch.Tensor, STensor],
+           **kwargs: Any) -> Union[torch.Tensor, STensor]:
+    """Matrix product.  Keyword arguments as in the reference: ``format`` /
+    ``output_format``, ``use_cache``, ``time_dict``."""
+    if isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
+        sparse_a = a.layout != torch.strided
+        sparse_b = b.layout != torch.strided
+        if not (sparse_a or sparse_b):
+            return torch.matmul(a, b)
+        if a.layout == torch.sparse_coo and b.layout == torch.sparse_coo:
+            a, b = a.to_sparse_csr(), b.to_sparse_csr()
+    if isinstance(a, torch.Tensor):
+        a = STensor.from_torch(a)
+    if isinstance(b, torch.Tensor):
+        b = STensor.from_torch(b)
+
+    time_dict = kwargs.get("time_dict", None)
+    requested = kwargs.get("format", kwargs.get("output_format", None))
+
+    if a.format.is_dense() and b.format.is_dense():
+        result = _timed(lambda: torch.matmul(a.to_torch(in_place=False), b.to_torch(in_place=False)),
+                        a.values.device, time_dict)
+        if requested is None or parse_format(requested).is_dense():
+            return result
+        return STensor.from_torch(result).to_sparse(parse_format(requested))
+
+    default_order = [0, 1]
+    for operand in (a, b):
+        if operand.dim() == 2 and not operand.format.is_dense() \
+                and operand.index.mode_order != default_order:
+            raise _not_prebuilt("matmul with a non-default mode order")
+
+    if kwargs.get("use_cache", True):
+        result = _run_prebuilt_matmul(a, b, requested, time_dict)
+        if result is None:
+            raise _not_prebuilt(f"matmul({a.format} x {b.format}, {a.values.dtype}, format={requested})")
+    else:
+        # the reference sends use_cache=False through einsum (ops.py:364-367)
+        expr = "ij,jk->ik" if b.dim() == 2 else "ij,j->i"
+        result = einsum(expr, a, b, **kwargs)
+
+    if isinstance(result, STensor) and result.format.is_dense():
+        result = result.to_torch()
+    return result
+
+
+def _sddmm(mask: STensor, A: STensor, B: STensor, time_dict) -> Optional[STensor]:
+    if mask.values.dtype != torch.float32 or A.values.dtype != torch.float32 \
+            or B.values.dtype != torch.float32:
+        return None
+    if str(A.format) != "d,d" or str(B.format) != "d,d":
+        return None
+    mask_fmt = str(mask.format)
+    if mask_fmt == "o,o":
+        fn = scorch_ops_hip.sddmm_coo_float_prebuilt
+    elif mask_fmt == "d,s":
+        fn = scorch_ops_hip.sddmm_csr_float
+    else:
+        return None
+    _require_device(mask, A, B)
+    result_cpp = _timed(lambda: fn(mask.shape, mask.shape, mask.index.mode_indices, mask.values,
+                                   A.shape, A.index.mode_indices, A.values,
+                                   B.shape, B.index.mode_indices, B.values),
+                        mask.values.device, time_dict)
+    # coordinate mask: the result keeps the mask's format and index tensors
+    # (reference ops.py:416-423); CSR mask: all-coordinate result (ops.py:638-666)
+    return _wrap(result_cpp, mask.shape, mask.format if mask_fmt == "o,o" else "oo")
+
+
+def einsum(expression: str, *tensors: Optional[Union[torch.Tensor, STensor]],
+           compile_only: Optional[bool] = False, **kwargs: Any) -> Union[STensor, torch.Tensor]:
+    """Einstein summation for the expressions that have a device kernel."""
+    if compile_only:
+        raise _not_prebuilt("einsum(compile_only=True)")
+    operands = tuple(STensor.from_torch(t) if isinstance(t, torch.Tensor) else t for t in tensors)
+    time_dict = kwargs.get("time_dict", None)
+    requested = kwargs.get("format", kwargs.get("output_format", None))
+    canon = _canonical(expression)
+
+    if canon in (_SDDMM_EXPR, _SDDMM_EXPR_KJ) and len(operands) == 3:
+        mask, A, B = operands
+        if requested is not None and str(parse_format(requested)) != "o,o" \
+                and str(parse_format(requested)) != str(mask.format):
+            raise _not_prebuilt(f"SDDMM with output format {requested}")
+        if canon == _SDDMM_EXPR_KJ:
+            if not B.format.is_dense():
+                raise _not_prebuilt("SDDMM with a sparse right operand")
+            B = STensor.from_torch(B.to_torch().t().contiguous())
+        result = _sddmm(mask, A, B, time_dict)
+        if result is None:
+            raise _not_prebuilt(f"einsum({expression!r}) with formats "
+                                f"{[str(t.format) for t in operands]}")
+        return result
+
+    if canon == _SPMM_EXPR and len(operands) == 2:
+        a, b = operands
+        if a.format.is_dense() and b.format.is_dense():
+            return torch.matmul(a.to_torch(in_place=False), b.to_torch(in_place=False))
+        result = _run_prebuilt_matmul(a, b, requested, time_dict)
+        if result is None:
+            raise _not_prebuilt(f"einsum({expression!r}) with formats {a.format} x {b.format}")
+        return result.to_torch() if result.format.is_dense() else result
+
+    if canon == "ab,b->a" and len(operands) == 2:
+        a, b = operands
+        result = _run_prebuilt_matmul(a, b, requested, time_dict)
+        if result is None:
+            raise _not_prebuilt(f"einsum({expression!r}) with formats {a.format} x {b.format}")
+        return result.to_torch() if result.format.is_dense() else result
+
+    raise _not_prebuilt(f"einsum({expression!r})")
+
+
+def spmm_bias_act(a: STensor, b: Union[torch.Tensor, STensor], bias: torch.Tensor,
+                  relu: bool = False) -> torch.Tensor:
+    """``act(a @ b + bias)`` in one kernel: the call the reference's
+    ``@scorch.compile`` makes when it recognises matmul -> add(bias) [-> relu]
+    (src/scorch/trace.py:232-301).  Returns an (M, N) tensor."""
+    if isinstance(b, torch.Tensor):
+        b = STensor.from_torch(b)
+    kinds = ("add", "relu") if relu else ("add",)
+    resolved = resolve_prebuilt_fused(str(a.format), str(b.format), kinds, a.values.dtype)
+    if resolved is None or b.values.dtype != a.values.dtype:
+        raise _not_prebuilt(f"fused matmul+{'+'.join(kinds)} for {a.format} x {b.format}, "
+                            f"{a.values.dtype}")
+    _require_device(a, b)
+    M, N = a.shape[0], b.shape[1]
+    out = resolved.fn([M, N], list(a.shape), a.index.mode_indices, a.values, list(b.shape),
+                      b.index.mode_indices, b.values, bias)
+    return out.storage.value.view(M, N)

@@ -1,0 +1,271 @@
+"""Device counterpart of the reference's pybind module ``scorch_ops``.
+
+Same function names, same argument lists and the same shape of return value as
+csrc/ops.cpp binds them -- ``fn(result_shape, A_shape, A_mode_indices,
+A_values, B_shape, B_mode_indices, B_values[, ...])`` returning an object with
+``.storage.value`` and ``.storage.index.mode_indices`` -- so the reference's
+dispatch (src/scorch/prebuilt_kernels.py:198-224, src/scorch/ops.py:405-415,
+src/scorch/trace.py:288-299) can call either module.  The tensors must live on
+a HIP device; the work is done by libscorch_hip.so on the current stream of
+the operands' device and the call returns without synchronising.
+
+Only the symbols of the SpMM / SDDMM / SpMV path exist here.  A symbol the
+reference resolves first but this module lacks simply is not found, and the
+reference's resolver moves on (prebuilt_kernels.py:96-101).
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from . import native
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
+
+
+class TensorIndex:
+    def __init__(self, mode_indices=None):
+        self.mode_indices = mode_indices if mode_indices is not None else []
+
+
+class TensorStorage:
+    def __init__(self, value=None, index=None):
+        self.value = value
+        self.index = index if index is not None else TensorIndex()
+
+
+class Tensor:
+    """Result carrier with the fields of the reference's csrc/header.h:4-16."""
+
+    def __init__(self, value=None, mode_indices=None):
+        self.storage = TensorStorage(value, TensorIndex(mode_indices))
+
+
+# ---- helpers -----------------------------------------------------------------
+_workspaces = {}
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    """Scratch buffer for (device, stream), grown on demand.  Kernels on one
+    stream run in order, so they can share it."""
+    key = (device.index, stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _device_of(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError("scorch_ops_hip: operands must be on a HIP device, got " + str(dev))
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError(f"scorch_ops_hip: operands on different devices ({dev} and {t.device})")
+    return dev
+
+
+def _index(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        raise TypeError(f"scorch_ops_hip: {what} must be int32, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _flat(t: torch.Tensor, dtype: torch.dtype, what: str) -> torch.Tensor:
+    if t.dtype != dtype:
+        raise TypeError(f"scorch_ops_hip: {what} must be {dtype}, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _csr_parts(mode_indices, what: str):
+    if len(mode_indices) != 2 or len(mode_indices[1]) != 2:
+        raise ValueError(f"scorch_ops_hip: {what} is not a CSR (\"d,s\") operand")
+    return _index(mode_indices[1][0], what + " pos"), _index(mode_indices[1][1], what + " crd")
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+# ---- SpMM ----------------------------------------------------------------------
+def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values,
+          bias=None, act=0):
+    M, K = int(A_shape[0]), int(A_shape[1])
+    N = int(B_shape[1])
+    if int(B_shape[0]) != K or tuple(int(s) for s in result_shape) != (M, N):
+        raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)} "
+                         f"result{tuple(result_shape)}")
+    pos, crd = _csr_parts(A_mode_indices, "A")
+    a_val = _flat(A_values, dtype, "A values")
+    b_val = _flat(B_values, dtype, "B values")
+    if pos.numel() != M + 1 or b_val.numel() != K * N or crd.numel() != a_val.numel():
+        raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
+    dev = _device_of(pos, crd, a_val, b_val)
+    nnz = a_val.numel()
+    out = torch.empty(M * N, dtype=dtype, device=dev)
+    L = native.lib()
+    with torch.cuda.device(dev):
+        stream = _stream(dev)
+        need = L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, a_val.element_size())
+        ws = _workspace(dev, stream, need)
+        if bias is None:
+            fn = getattr(L, "scorch_hip_spmm_csr_" + _SUFFIX[dtype])
+            rc = fn(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(),
+                    out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        else:
+            bias = _flat(bias, dtype, "bias")
+            if bias.numel() != N or bias.device != dev:
+                raise ValueError("scorch_ops_hip: bias must have N elements on the operands' device")
+            rc = L.scorch_hip_spmm_csr_bias_act_f32(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                    a_val.data_ptr(), b_val.data_ptr(), bias.data_ptr(),
+                                                    act, out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                    stream)
+    native.check(rc)
+    return Tensor(out, [[], []])
+
+
+def _make_spmm(dtype):
+    def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values,
+               tile_size: int = 0):
+        return _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
+                     B_values)
+    return kernel
+
+
+# fp32: the symbol the registry tries first, its typed fallback and the legacy alias
+# (src/scorch/prebuilt_kernels.py:45); one kernel serves all three.
+spmm_csr_float_v2 = _make_spmm(torch.float32)
+prebuilt_spmm_csr_f32 = _make_spmm(torch.float32)
+spmm_csr_float = _make_spmm(torch.float32)
+prebuilt_spmm_csr_f64 = _make_spmm(torch.float64)
+spmm_csr_double = _make_spmm(torch.float64)
+prebuilt_spmm_csr_i32 = _make_spmm(torch.int32)
+prebuilt_spmm_csr_i64 = _make_spmm(torch.int64)
+
+
+def spmm_csr_bias_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
+                        B_values, bias):
+    """C = A @ B + bias (reference: csrc/ops.cpp:179-188)."""
+    return _spmm(torch.float32, result_shape, A_shape, A_mode_indices, A_values, B_shape,
+                 B_mode_indices, B_values, bias=bias, act=0)
+
+
+def spmm_csr_bias_relu_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
+                             B_values, bias):
+    """C = relu(A @ B + bias) (reference: csrc/ops.cpp:168-177)."""
+    return _spmm(torch.float32, result_shape, A_shape, A_mode_indices, A_values, B_shape,
+                 B_mode_indices, B_values, bias=bias, act=1)
+
+
+# ---- SpMV ----------------------------------------------------------------------
+def _make_spmv(dtype):
+    def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+        M, K = int(A_shape[0]), int(A_shape[1])
+        pos, crd = _csr_parts(A_mode_indices, "A")
+        a_val = _flat(A_values, dtype, "A values")
+        x = _flat(B_values, dtype, "x values")
+        if pos.numel() != M + 1 or x.numel() != K or crd.numel() != a_val.numel():
+            raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
+        dev = _device_of(pos, crd, a_val, x)
+        y = torch.empty(M, dtype=dtype, device=dev)
+        with torch.cuda.device(dev):
+            fn = getattr(native.lib(), "scorch_hip_spmv_csr_" + _SUFFIX[dtype])
+            rc = fn(M, K, a_val.numel(), pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), x.data_ptr(),
+                    y.data_ptr(), _stream(dev))
+        native.check(rc)
+        return Tensor(y, [[]])
+    return kernel
+
+
+prebuilt_spmv_csr_f32 = _make_spmv(torch.float32)
+prebuilt_spmv_csr_f64 = _make_spmv(torch.float64)
+prebuilt_spmv_csr_i32 = _make_spmv(torch.int32)
+prebuilt_spmv_csr_i64 = _make_spmv(torch.int64)
+
+
+# ---- SDDMM ---------------------------------------------------------------------
+def _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values):
+    M, n_cols = int(S_shape[0]), int(S_shape[1])
+    K = int(A_shape[1])
+    if int(A_shape[0]) != M or int(B_shape[0]) != n_cols or int(B_shape[1]) != K:
+        raise ValueError(f"scorch_ops_hip: shape mismatch S{tuple(S_shape)} A{tuple(A_shape)} "
+                         f"B{tuple(B_shape)} (B is indexed [j, k])")
+    a = _flat(A_values, torch.float32, "A values")
+    b = _flat(B_values, torch.float32, "B values")
+    if a.numel() != M * K or b.numel() != n_cols * K:
+        raise ValueError("scorch_ops_hip: dense operand length does not match its shape")
+    return M, n_cols, K, a, b
+
+
+def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_mode_indices,
+                             A_values, B_shape, B_mode_indices, B_values):
+    """D = S * (A @ B^T) at S's entries, S in coordinate format
+    (reference: csrc/kernels.h:508-570).  The result shares S's index tensors."""
+    M, n_cols, K, a, b = _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values)
+    if len(S_mode_indices) != 2 or len(S_mode_indices[0]) != 1 or len(S_mode_indices[1]) != 1:
+        raise ValueError("scorch_ops_hip: S is not a coordinate (\"o,o\") operand")
+    row = _index(S_mode_indices[0][0], "S rows")
+    col = _index(S_mode_indices[1][0], "S cols")
+    s_val = _flat(S_values, torch.float32, "S values")
+    if row.numel() != s_val.numel() or col.numel() != s_val.numel():
+        raise ValueError("scorch_ops_hip: S index and value lengths differ")
+    dev = _device_of(row, col, s_val, a, b)
+    out = torch.empty_like(s_val)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(),
+                                                   col.data_ptr(), s_val.data_ptr(), a.data_ptr(),
+                                                   b.data_ptr(), out.data_ptr(), _stream(dev))
+    native.check(rc)
+    return Tensor(out, S_mode_indices)
+
+
+def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_mode_indices, A_values,
+                    B_shape, B_mode_indices, B_values):
+    """SDDMM with a CSR mask.  The result is in coordinate format, one entry per
+    mask entry in mask order: what the reference's generated kernel returns for
+    this case (src/scorch/ops.py:638-666).  mode_indices = [[rows], [S's crd]]."""
+    M, n_cols, K, a, b = _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values)
+    pos, crd = _csr_parts(S_mode_indices, "S")
+    s_val = _flat(S_values, torch.float32, "S values")
+    if pos.numel() != M + 1 or crd.numel() != s_val.numel():
+        raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
+    dev = _device_of(pos, crd, s_val, a, b)
+    out = torch.empty_like(s_val)
+    rows = torch.empty_like(crd)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(),
+                                                   crd.data_ptr(), s_val.data_ptr(), a.data_ptr(),
+                                                   b.data_ptr(), out.data_ptr(), rows.data_ptr(),
+                                                   _stream(dev))
+    native.check(rc)
+    return Tensor(out, [[rows], [crd]])
+
+
+# ---- neighbours of the path ---------------------------------------------------------
+def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Row softmax of ``scale * values`` over a CSR pattern
+    (reference: bench/bench_sparse_transformer.py:277-297)."""
+    pos = _index(row_ptr, "row_ptr")
+    v = _flat(values, torch.float32, "values")
+    dev = _device_of(pos, v)
+    out = torch.empty_like(v)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(),
+                                                     v.data_ptr(), float(scale), out.data_ptr(),
+                                                     _stream(dev))
+    native.check(rc)
+    return out
+
+
+def csr_row_indices(row_ptr: torch.Tensor, nnz: int) -> torch.Tensor:
+    """Row of every stored entry of a CSR pattern (int32[nnz])."""
+    pos = _index(row_ptr, "row_ptr")
+    dev = _device_of(pos)
+    rows = torch.empty(nnz, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_csr_row_indices(pos.numel() - 1, nnz, pos.data_ptr(),
+                                                     rows.data_ptr(), _stream(dev))
+    native.check(rc)
+    return rows

@@ -1,0 +1,231 @@
+"""STensor: a tensor stored in a per-mode format (reference: src/scorch/stensor.py).
+
+This is the part of the reference's tensor model that the prebuilt SpMM/SDDMM
+path touches: construction from torch tensors (dense, CSR, COO), the
+``values`` / ``index.mode_indices`` / ``shape`` / ``format`` accessors the
+kernel dispatch reads, and conversion back to torch.  Unlike the reference,
+whose ``to()`` is a stub (stensor.py:147-150), an STensor here can live on a
+GPU: ``to(device)`` moves the value and index tensors.
+
+Format conversion is done with torch's own sparse routines on whatever device
+the tensor is on; the reference's JIT-compiled converters are not part of this
+package.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Tuple, Union
+
+import torch
+
+from .format import LevelFormat, LevelType, TensorFormat, parse_format
+from .storage import TensorIndex, TensorStorage
+
+_DENSE2 = "dd"
+
+
+class STensor(torch.nn.Module):
+    def __init__(self, name: Optional[str] = None, shape: Optional[Tuple[int, ...]] = None,
+                 storage: Optional[TensorStorage] = None, index: Optional[TensorIndex] = None,
+                 value: Optional[torch.Tensor] = None, requires_grad: Optional[bool] = False) -> None:
+        super().__init__()
+        self._storage = storage if storage is not None else TensorStorage(index=index, value=value,
+                                                                          shape=shape)
+        self._name = name
+        self._shape = tuple(shape) if shape is not None else None
+        if value is not None:
+            self._dtype = value.dtype
+        elif storage is not None and storage._value is not None:
+            self._dtype = storage._value.dtype
+        else:
+            self._dtype = torch.float32
+        self.requires_grad = requires_grad
+
+    # ---- accessors the dispatch reads ------------------------------------------
+    @property
+    def name(self) -> str:
+        assert self._name is not None, "Tensor name is not set."
+        return self._name
+
+    @name.setter
+    def name(self, name: str) -> None:
+        self._name = name
+
+    @property
+    def storage(self) -> TensorStorage:
+        assert self._storage is not None, "Tensor storage is not set."
+        return self._storage
+
+    @property
+    def values(self) -> torch.Tensor:
+        return self.storage.value
+
+    @property
+    def index(self) -> TensorIndex:
+        return self.storage.index
+
+    @property
+    def has_index(self) -> bool:
+        return self.storage.has_index
+
+    @property
+    def format(self) -> TensorFormat:
+        fmt = self.index.format
+        assert fmt is not None, "Tensor format is not set."
+        return fmt
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self._dtype
+
+    @property
+    def shape(self) -> Tuple[int, ...]:
+        return self._shape if self._shape is not None else tuple()
+
+    @property
+    def device(self) -> torch.device:
+        return self.values.device
+
+    @property
+    def is_cuda(self) -> bool:
+        return self.values.is_cuda
+
+    def dim(self) -> int:
+        return len(self.shape)
+
+    def _nnz(self) -> int:
+        return self.values.numel()
+
+    def __repr__(self) -> str:
+        return "Tensor"
+
+    # ---- residency ---------------------------------------------------------------
+    def to(self, device) -> "STensor":
+        """Copy of the tensor with values and indices on ``device``."""
+        return STensor(name=self._name, shape=self.shape, storage=self.storage.to(device))
+
+    def cuda(self) -> "STensor":
+        return self.to(torch.device("cuda", torch.cuda.current_device()))
+
+    def cpu(self) -> "STensor":
+        return self.to(torch.device("cpu"))
+
+    def copy(self) -> "STensor":
+        return STensor(name=self._name, shape=self.shape, storage=self.storage.copy())
+
+    clone = copy
+
+    # ---- construction --------------------------------------------------------------
+    @staticmethod
+    def _csr(shape, crow, col, values, name, mode_order=None) -> "STensor":
+        fmt = TensorFormat([LevelFormat(LevelType.DENSE), LevelFormat(LevelType.COMPRESSED)])
+        return STensor(name=name, shape=tuple(shape), storage=TensorStorage(
+            index=TensorIndex(fmt, [[], [crow, col]], mode_order=mode_order), value=values))
+
+    @staticmethod
+    def _coo(shape, indices, values, name, mode_order=None) -> "STensor":
+        fmt = TensorFormat([LevelFormat(LevelType.COORDINATE) for _ in shape])
+        return STensor(name=name, shape=tuple(shape), storage=TensorStorage(
+            index=TensorIndex(fmt, [[indices[i]] for i in range(len(shape))], mode_order=mode_order),
+            value=values))
+
+    @staticmethod
+    def from_csr(csr_matrix: torch.Tensor, name: Optional[str] = None) -> "STensor":
+        """2-D torch CSR tensor -> "d,s" STensor sharing its arrays
+        (reference: stensor.py:271-315)."""
+        assert csr_matrix.is_sparse_csr, "Input tensor must be a sparse CSR tensor."
+        assert csr_matrix.dim() == 2, "CSR format is only valid for 2D matrices."
+        return STensor._csr(csr_matrix.shape, csr_matrix.crow_indices(), csr_matrix.col_indices(),
+                            csr_matrix.values(), name or "tensor")
+
+    @staticmethod
+    def from_csr_arrays(row_ptr: torch.Tensor, col_idx: torch.Tensor, values: torch.Tensor,
+                        shape: Tuple[int, int], name: Optional[str] = None) -> "STensor":
+        """"d,s" STensor over caller-owned arrays (no torch sparse tensor in between)."""
+        return STensor._csr(shape, row_ptr, col_idx, values, name or "tensor")
+
+    @staticmethod
+    def from_coo(coo_matrix: Optional[torch.Tensor] = None, indices: Optional[torch.Tensor] = None,
+                 values: Optional[torch.Tensor] = None, shape: Optional[Tuple[int, ...]] = None,
+                 name: Optional[str] = None) -> "STensor":
+        """torch COO tensor (coalesced first) or raw (indices, values, shape) ->
+        all-coordinate STensor (reference: stensor.py:318-365)."""
+        if coo_matrix is not None:
+            coo_matrix = coo_matrix.coalesce()
+            indices, values, shape = coo_matrix.indices(), coo_matrix.values(), coo_matrix.shape
+        assert indices is not None and values is not None and shape is not None
+        return STensor._coo(tuple(shape), indices, values, name or "tensor")
+
+    @staticmethod
+    def from_torch(tensor: torch.Tensor, name: Optional[str] = None,
+                   mode_order: Optional[List[int]] = None) -> "STensor":
+        """torch tensor of any layout -> STensor (reference: stensor.py:368-452).
+        Strided tensors become all-dense with ``values = tensor.flatten()``."""
+        name = name or "tensor"
+        if mode_order:
+            tensor = tensor.permute(*mode_order)
+        else:
+            mode_order = list(range(tensor.dim()))
+        if tensor.layout == torch.sparse_coo:
+            tensor = tensor.coalesce()
+            return STensor._coo(tensor.shape, tensor.indices(), tensor.values(), name, mode_order)
+        if tensor.layout == torch.sparse_csr:
+            return STensor._csr(tensor.shape, tensor.crow_indices(), tensor.col_indices(),
+                                tensor.values(), name, mode_order)
+        fmt = TensorFormat([LevelFormat(LevelType.DENSE) for _ in tensor.shape])
+        return STensor(name=name, shape=tuple(tensor.shape), storage=TensorStorage(
+            index=TensorIndex(fmt, [[] for _ in tensor.shape], mode_order=mode_order),
+            value=tensor.flatten()))
+
+    # ---- conversion ------------------------------------------------------------------
+    def _as_torch_sparse(self) -> torch.Tensor:
+        kinds = [t.value for t in self.format.get_level_types()]
+        idx = self.index.mode_indices
+        if kinds == ["d", "s"]:
+            return torch.sparse_csr_tensor(idx[1][0], idx[1][1], self.values, size=self.shape)
+        if all(k == "o" for k in kinds):
+            coords = torch.stack([level[0].to(torch.int64) for level in idx], dim=0)
+            return torch.sparse_coo_tensor(coords, self.values, size=self.shape)
+        raise NotImplementedError(f"no torch layout for format {self.format}")
+
+    def to_dense(self, fmt=None, in_place: bool = False) -> "STensor":
+        if self.format.is_dense():
+            return self
+        return STensor.from_torch(self._as_torch_sparse().to_dense(), self._name)
+
+    def to_sparse(self, fmt: Union[TensorFormat, str, List[str]] = "ds") -> "STensor":
+        """Dense or sparse 2-D STensor -> "d,s" (CSR) or "o,o" (COO)."""
+        fmt = parse_format(fmt)
+        if fmt == self.format:
+            return self
+        if self.dim() != 2:
+            raise NotImplementedError("to_sparse handles matrices only")
+        if self.format.is_dense():
+            dense = self.values.reshape(self.shape)
+        else:
+            dense = self._as_torch_sparse().to_dense()
+        target = str(fmt)
+        if target == "d,s":
+            return STensor.from_csr(dense.to_sparse_csr(), self._name)
+        if target == "o,o":
+            return STensor.from_coo(dense.to_sparse(), name=self._name)
+        if target == "d,d":
+            return STensor.from_torch(dense, self._name)
+        raise NotImplementedError(f"to_sparse: unsupported target format {fmt}")
+
+    def to_torch(self, in_place: bool = True) -> torch.Tensor:
+        """Strided torch tensor of the logical shape (reference: stensor.py:454-475);
+        no copy for a dense STensor in default mode order."""
+        if self.format.is_dense():
+            out = self.values
+        else:
+            out = self._as_torch_sparse().to_dense()
+        if out.dtype != self.dtype:
+            out = out.to(self.dtype)
+        out = out.reshape(self.shape)
+        order = self.index.mode_order
+        if order and list(order) != list(range(self.dim())):
+            inverse = [0] * len(order)
+            for pos, mode in enumerate(order):
+                inverse[mode] = pos
+            out = out.permute(*inverse)
+        return out

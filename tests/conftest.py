@@ -1,0 +1,71 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+GOLDEN_PATH = os.path.join(ROOT, "tests", "golden", "golden_ref.npz")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a HIP device (run on the MI355X box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    """GPU tests skip cleanly where there is no device."""
+    import torch
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no HIP device")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+class Golden:
+    """Cases of tests/golden/golden_ref.npz: golden.case("spmm_rect") -> dict of arrays."""
+
+    def __init__(self, path):
+        self._z = np.load(path, allow_pickle=False)
+        self.names = sorted({k.split("/")[0] for k in self._z.files})
+
+    def case(self, name):
+        prefix = name + "/"
+        out = {k[len(prefix):]: self._z[k] for k in self._z.files if k.startswith(prefix)}
+        if not out:
+            raise KeyError(name)
+        return out
+
+    def cases(self, prefix):
+        return [n for n in self.names if n.startswith(prefix)]
+
+
+@pytest.fixture(scope="session")
+def golden():
+    return Golden(GOLDEN_PATH)
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    from oracle import oracle as O
+    O.lib()
+    return O
+
+
+def random_csr(rng, M, K, density, dtype=np.float32, empty_rows=(), lo=-1.0, hi=1.0):
+    """Random CSR pattern with sorted unique columns; returns (row_ptr, col_idx, vals)."""
+    keep = rng.random((M, K)) < density
+    for r in empty_rows:
+        keep[r, :] = False
+    rows, cols = np.nonzero(keep)
+    row_ptr = np.zeros(M + 1, dtype=np.int32)
+    np.cumsum(np.bincount(rows, minlength=M), out=row_ptr[1:])
+    if np.issubdtype(np.dtype(dtype), np.integer):
+        vals = rng.integers(-1000, 1000, size=rows.size).astype(dtype)
+    else:
+        vals = rng.uniform(lo, hi, size=rows.size).astype(dtype)
+    return row_ptr, cols.astype(np.int32), vals

@@ -1,0 +1,123 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol that
+include/scorch_hip.h declares, and rejects bad arguments on the host before
+launching anything.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from scorch_amd import native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "scorch_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"SCORCH_HIP_API[^;(]*?\b(scorch_hip_\w+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    return native.lib()
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for required in ["scorch_hip_spmm_csr_f32", "scorch_hip_spmm_csr_workspace_bytes",
+                     "scorch_hip_sddmm_csr_f32", "scorch_hip_sddmm_coo_f32",
+                     "scorch_hip_spmm_csr_bias_act_f32", "scorch_hip_last_error"]:
+        assert required in names
+    assert len(names) >= 16
+
+
+def test_library_exports_every_declared_symbol(L):
+    for name in declared_symbols():
+        assert hasattr(L, name), f"{name} is declared in scorch_hip.h but not exported"
+
+
+def test_binding_table_matches_header(L):
+    assert sorted(native.SIGNATURES) == declared_symbols()
+
+
+def test_abi_version(L):
+    m = re.search(r"#define SCORCH_HIP_ABI_VERSION (\d+)", open(HEADER).read())
+    assert L.scorch_hip_abi_version() == int(m.group(1))
+
+
+def test_workspace_bytes_formula(L):
+    f = L.scorch_hip_spmm_csr_workspace_bytes
+    assert f(-1, 0, 4, 4) == 0 and f(4, 4, 4, 0) == 0
+    small = f(10, 100, 128, 4)
+    assert small > 0 and small % 256 == 0
+    # grows with the amount of work and with the row width
+    assert f(1 << 20, 17_000_000, 128, 4) > f(1 << 20, 17_000_000, 64, 4) > small
+    assert f(10, 100, 128, 8) > small
+
+
+NULL = None
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
+
+
+def spmm(L, M=4, K=4, N=4, nnz=4, row_ptr=FAKE, col=FAKE, vals=FAKE, B=FAKE, C=FAKE, ws=FAKE, ws_bytes=1 << 30):
+    return L.scorch_hip_spmm_csr_f32(M, K, N, nnz, row_ptr, col, vals, B, C, ws, ws_bytes, NULL)
+
+
+def test_spmm_rejects_bad_arguments(L):
+    assert spmm(L, M=-1) == native.EINVAL
+    assert b"negative" in L.scorch_hip_last_error()
+    assert spmm(L, row_ptr=NULL) == native.EINVAL
+    assert spmm(L, col=NULL) == native.EINVAL
+    assert spmm(L, C=NULL) == native.EINVAL
+    assert spmm(L, B=NULL) == native.EINVAL
+    assert spmm(L, M=0, K=0, nnz=3) == native.EINVAL
+    assert spmm(L, M=1 << 31) == native.EUNSUPPORTED
+    assert spmm(L, nnz=1 << 31) == native.EUNSUPPORTED
+    assert spmm(L, row_ptr=ctypes.c_void_p(0x1001)) == native.EINVAL  # misaligned
+    assert spmm(L, ws=NULL) == native.EWORKSPACE
+    assert spmm(L, ws_bytes=16) == native.EWORKSPACE
+    assert b"workspace" in L.scorch_hip_last_error()
+    assert spmm(L, ws=ctypes.c_void_p(0x1010)) == native.EINVAL  # not 256-byte aligned
+
+
+def test_spmm_empty_output_is_a_no_op(L):
+    assert spmm(L, M=0, nnz=0, C=NULL, ws=NULL) == native.OK
+    assert spmm(L, N=0, C=NULL, ws=NULL) == native.OK
+
+
+def test_bias_act_rejects_unknown_activation_and_null_bias(L):
+    f = L.scorch_hip_spmm_csr_bias_act_f32
+    assert f(4, 4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, 7, FAKE, FAKE, 1 << 30, NULL) == native.EINVAL
+    assert b"activation" in L.scorch_hip_last_error()
+    assert f(4, 4, 4, 4, FAKE, FAKE, FAKE, FAKE, NULL, 1, FAKE, FAKE, 1 << 30, NULL) == native.EINVAL
+
+
+def test_sddmm_rejects_bad_arguments(L):
+    csr, coo = L.scorch_hip_sddmm_csr_f32, L.scorch_hip_sddmm_coo_f32
+    assert csr(-1, 4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert csr(4, 4, 4, 4, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert csr(4, 4, 4, 4, FAKE, FAKE, FAKE, NULL, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert csr(0, 0, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert coo(4, 4, 4, 4, NULL, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EINVAL
+    assert coo(4, 4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert coo(4, 4, 4, 0, NULL, NULL, NULL, NULL, NULL, NULL, NULL) == native.OK  # nothing to do
+    assert coo(4, 4, 4, 1 << 31, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EUNSUPPORTED
+
+
+def test_spmv_softmax_rows_reject_bad_arguments(L):
+    assert L.scorch_hip_spmv_csr_f64(4, 4, 4, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert L.scorch_hip_spmv_csr_i32(-4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_spmv_csr_i64(0, 4, 0, FAKE, NULL, NULL, NULL, NULL, NULL) == native.OK
+    assert L.scorch_hip_softmax_csr_f32(4, 4, NULL, FAKE, 1.0, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_softmax_csr_f32(4, 4, FAKE, NULL, 1.0, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL
+    assert L.scorch_hip_csr_row_indices(0, 4, FAKE, FAKE, NULL) == native.EINVAL
+
+
+def test_check_raises_with_the_library_message(L):
+    code = spmm(L, M=-3)
+    with pytest.raises(native.ScorchHipError) as info:
+        native.check(code)
+    assert info.value.code == native.EINVAL and "M=-3" in str(info.value)

@@ -1,0 +1,158 @@
+"""SpMV, CSR row softmax and the Python-level matmul / einsum routing on the
+MI355X.  SpMV and softmax tolerances: relative Frobenius error <= 1e-5 against
+fp64; integer SpMV bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import scorch_amd as scorch
+from conftest import random_csr
+from gpu_util import dev, hip_spmv, host
+from scorch_amd import STensor, ops
+from scorch_amd import scorch_ops_hip as H
+from scorch_amd import workloads
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def test_spmv_golden(golden):
+    c = golden.case("spmv_i64_literal")
+    assert hip_spmv(c["row_ptr"], c["col_idx"], c["vals"], c["x"]).tolist() == [7, 22, 0, 29]
+    for name in ("spmv_f32", "spmv_f64", "spmv_i32"):
+        c = golden.case(name)
+        got = hip_spmv(c["row_ptr"], c["col_idx"], c["vals"], c["x"])
+        if name == "spmv_i32":
+            assert np.array_equal(got, c["y"])
+        else:
+            np.testing.assert_allclose(got, c["y"], rtol=1e-5 if name == "spmv_f32" else 1e-13, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("density", [0.002, 0.05, 0.6])   # group widths 2 .. 64
+def test_spmv_against_oracle(oracle, dtype, density):
+    rng = np.random.default_rng(int(density * 1000))
+    rp, ci, v = random_csr(rng, 1500, 400, density, dtype=dtype, empty_rows=(0, 1499))
+    x = (rng.integers(-1000, 1000, 400) if np.issubdtype(dtype, np.integer)
+         else rng.standard_normal(400)).astype(dtype)
+    got = hip_spmv(rp, ci, v, x)
+    want = oracle.spmv_csr_typed(rp, ci, v, x)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(got, want)
+    else:
+        dense64 = oracle.spmm_fp64(rp, ci, v, x.reshape(-1, 1)).reshape(-1)
+        assert oracle.rel_fro(got, dense64) <= (TOL if dtype == np.float32 else 1e-13)
+
+
+def test_softmax_against_oracle(oracle):
+    w = workloads.gcn_powerlaw(M=8000, N=4, seed=12, max_degree=3000)
+    rng = np.random.default_rng(0)
+    vals = rng.standard_normal(w["col_idx"].size).astype(np.float32) * 5
+    got = host(H.softmax_csr_float(dev(w["row_ptr"]), dev(vals), 0.125))
+    assert oracle.rel_fro(got, oracle.softmax_csr_fp64(w["row_ptr"], vals, 0.125)) <= TOL
+    np.testing.assert_allclose(got, oracle.softmax_csr_f32(w["row_ptr"], vals, 0.125), rtol=1e-4, atol=1e-7)
+    sums = np.add.reduceat(got, w["row_ptr"][:-1])
+    np.testing.assert_allclose(sums, 1.0, rtol=1e-5)
+
+
+def test_softmax_with_empty_rows_and_large_values(oracle):
+    rp = np.array([0, 0, 4, 4, 5], np.int32)
+    vals = np.array([1000.0, 1001.0, 999.0, 1000.5, -3.0], np.float32)
+    got = host(H.softmax_csr_float(dev(rp), dev(vals), 1.0))
+    assert np.isfinite(got).all() and got[4] == 1.0
+    np.testing.assert_allclose(got, oracle.softmax_csr_fp64(rp, vals), rtol=1e-5)
+
+
+# ---- the Python interface (reference: tests/test_scorch/test_matmul_dispatch.py) ----------------
+@pytest.mark.parametrize("use_cache", [True, False])
+def test_sparse_stensor_spmm_does_not_call_torch_matmul(use_cache, monkeypatch):
+    torch.manual_seed(0)
+    n = 32
+    a_torch = torch.rand(n, n) * (torch.rand(n, n) < 0.1)
+    b_torch = torch.rand(n, n)
+    expected = torch.matmul(a_torch, b_torch)
+    a = STensor.from_torch(a_torch, "A").to_sparse("ds").to("cuda")
+    b = STensor.from_torch(b_torch, "B").to("cuda")
+
+    def forbidden(*args, **kwargs):
+        raise AssertionError("torch.matmul should not be used for sparse STensor matmul")
+
+    monkeypatch.setattr(ops.torch, "matmul", forbidden)
+    out = scorch.matmul(a, b, format="dd", use_cache=use_cache)
+    assert isinstance(out, torch.Tensor) and out.is_cuda and out.shape == (n, n)
+    assert torch.allclose(out.cpu(), expected, atol=1e-3, rtol=1e-3)
+
+
+def test_matmul_accepts_torch_operands_and_fills_time_dict():
+    torch.manual_seed(1)
+    a = (torch.rand(300, 200) * (torch.rand(300, 200) < 0.05)).cuda()
+    b = torch.rand(200, 128).cuda()
+    td = {}
+    out = scorch.matmul(scorch.from_csr(a.to_sparse_csr()), b, time_dict=td)
+    assert td["eval_time"] > 0
+    assert torch.allclose(out, a @ b, atol=1e-4, rtol=1e-4)
+    out2 = scorch.einsum("ik,kj->ij", a.to_sparse_csr(), b, format="dd")
+    assert torch.equal(out, out2)
+    nc = b.t().contiguous().t()                      # non-contiguous dense operand is flattened first
+    assert torch.equal(scorch.matmul(scorch.from_csr(a.to_sparse_csr()), nc), out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.int32, torch.int64])
+def test_matmul_other_dtypes(dtype):
+    torch.manual_seed(2)
+    a = ((torch.rand(64, 64) * 20).round() * (torch.rand(64, 64) < 0.1)).to(dtype)
+    b = (torch.rand(64, 16) * 20).round().to(dtype)
+    out = scorch.matmul(STensor.from_torch(a).to_sparse("ds").to("cuda"), b.cuda())
+    assert out.dtype == dtype and torch.equal(out.cpu(), a @ b)
+
+
+def test_matmul_vector_operand():
+    torch.manual_seed(3)
+    a = torch.rand(100, 80) * (torch.rand(100, 80) < 0.1)
+    x = torch.rand(80)
+    out = scorch.matmul(STensor.from_torch(a).to_sparse("ds").to("cuda"), x.cuda())
+    assert out.shape == (100,) and torch.allclose(out.cpu(), a @ x, atol=1e-5)
+
+
+@pytest.mark.parametrize("n,d,sparsity", [(16, 8, 0.5), (64, 32, 0.9), (128, 16, 0.95), (256, 64, 0.99)])
+@pytest.mark.parametrize("mask_format", ["ds", "oo"])
+def test_einsum_sddmm(n, d, sparsity, mask_format):
+    """reference: tests/test_scorch/test_kernels_comprehensive.py:376-411"""
+    torch.manual_seed(n + d)
+    mask = torch.rand(n, n) * (torch.rand(n, n) > sparsity)
+    Q, K = torch.rand(n, d), torch.rand(n, d)
+    mask_st = STensor.from_torch(mask).to_sparse(mask_format).to("cuda")
+    result = scorch.einsum("ij,ik,jk->ij", mask_st, Q.cuda(), K.cuda())
+    assert isinstance(result, STensor) and str(result.format) == "o,o"     # all-coordinate output
+    assert result._nnz() == mask_st._nnz()
+    assert torch.allclose(result.to_torch().cpu(), (Q @ K.T) * mask, atol=1e-3, rtol=1e-3)
+    kj = scorch.einsum("ij,ik,kj->ij", mask_st, Q.cuda(), K.t().contiguous().cuda())
+    assert torch.allclose(kj.values, result.values, atol=1e-6)
+
+
+def test_spmm_bias_act_interface():
+    torch.manual_seed(42)
+    a = torch.randn(64, 64) * (torch.rand(64, 64) < 0.1)
+    b, bias = torch.randn(64, 16), torch.randn(16)
+    A = STensor.from_torch(a).to_sparse("ds").to("cuda")
+    plain = scorch.spmm_bias_act(A, b.cuda(), bias.cuda())
+    relu = scorch.spmm_bias_act(A, STensor.from_torch(b.cuda()), bias.cuda(), relu=True)
+    assert torch.allclose(plain.cpu(), a @ b + bias, atol=1e-4)
+    assert torch.allclose(relu.cpu(), torch.relu(a @ b + bias), atol=1e-4)
+
+
+def test_unfused_attention_pipeline_matches_dense(oracle):
+    """SDDMM -> row softmax -> SpMM over a CSR mask, the per-head composition of
+    bench/bench_sparse_transformer.py:354-372, against masked dense attention in fp64."""
+    S, D = 512, 64
+    brp, bci = workloads.blocksparse_pattern(S // 64)
+    rp, ci = workloads.blocks_to_csr(brp, bci, 64)
+    rng = np.random.default_rng(4)
+    q, k, v = (rng.standard_normal((S, D)).astype(np.float32) for _ in range(3))
+    mask = STensor.from_csr_arrays(dev(rp), dev(ci), torch.ones(ci.size, device="cuda"), (S, S))
+    scores = scorch.einsum("ij,ik,jk->ij", mask, dev(q), dev(k))
+    probs = H.softmax_csr_float(dev(rp), scores.values, D ** -0.5)
+    out = scorch.matmul(STensor.from_csr_arrays(dev(rp), dev(ci), probs, (S, S)), dev(v), format="dd")
+    dense_mask = np.zeros((S, S), bool)
+    dense_mask[oracle.rows_of(rp), ci] = True
+    assert oracle.rel_fro(host(out), oracle.attention_dense_fp64(q, k, v, dense_mask, D ** -0.5)) <= TOL

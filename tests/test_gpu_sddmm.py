@@ -1,0 +1,125 @@
+"""SDDMM on the MI355X through the C ABI: coordinate and CSR masks.
+
+Values: relative Frobenius error <= 1e-5 against an fp64 recomputation.
+Structure: the output coordinates are bit-exact -- for a coordinate mask the
+mask's own index tensors come back; for a CSR mask the result is the
+coordinate list (row of each entry, col_idx) in mask order, one entry per mask
+entry, explicit zeros kept.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+from gpu_util import dev, hip_sddmm_coo, hip_sddmm_csr, host
+from scorch_amd import scorch_ops_hip as H
+from scorch_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+SDDMM_CASES = ["sddmm_16_8", "sddmm_64_32", "sddmm_128_16", "sddmm_256_64", "sddmm_40_16", "sddmm_rect_k13"]
+
+
+@pytest.mark.parametrize("name", SDDMM_CASES)
+def test_golden_coo(golden, oracle, name):
+    c = golden.case(name)
+    shape = (c["A"].shape[0], c["B"].shape[0])
+    got = hip_sddmm_coo(c["row_idx"], c["col_idx"], c["vals"], c["A"], c["B"], shape)
+    ref64 = oracle.sddmm_fp64(c["row_idx"], c["col_idx"], c["vals"], c["A"], c["B"])
+    assert oracle.rel_fro(got, ref64) <= TOL
+    np.testing.assert_allclose(got, c["out_val"], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("name", SDDMM_CASES)
+def test_golden_csr(golden, oracle, name):
+    c = golden.case(name)
+    shape = (c["A"].shape[0], c["B"].shape[0])
+    row, col, val = hip_sddmm_csr(c["row_ptr"], c["col_idx"], c["vals"], c["A"], c["B"], shape)
+    assert row.dtype == np.int32 and np.array_equal(row, c["out_row"]) and np.array_equal(col, c["out_col"])
+    assert val.size == c["vals"].size
+    np.testing.assert_allclose(val, c["out_val"], rtol=1e-4, atol=1e-5)
+    assert (val[c["vals"] == 0] == 0).all()
+
+
+# K chosen to hit every group width (4..64 lanes per entry), the scalar path (K % 4 != 0) and K > 256
+@pytest.mark.parametrize("K", [1, 2, 5, 8, 13, 16, 32, 64, 96, 128, 200, 256, 260, 512])
+def test_inner_dimensions(oracle, K):
+    rng = np.random.default_rng(K)
+    rp, ci, s = random_csr(rng, 211, 157, 0.07, empty_rows=(0, 7, 210))
+    rows = oracle.rows_of(rp)
+    A = rng.standard_normal((211, K)).astype(np.float32)
+    B = rng.standard_normal((157, K)).astype(np.float32)
+    ref64 = oracle.sddmm_fp64(rows, ci, s, A, B)
+    coo = hip_sddmm_coo(rows, ci, s, A, B, (211, 157))
+    r, c, csr = hip_sddmm_csr(rp, ci, s, A, B, (211, 157))
+    assert oracle.rel_fro(coo, ref64) <= TOL and oracle.rel_fro(csr, ref64) <= TOL
+    assert np.array_equal(coo, csr)                      # same arithmetic, same order
+    assert np.array_equal(r, rows) and np.array_equal(c, ci)
+    np.testing.assert_allclose(coo, oracle.sddmm_coo_f32(rows, ci, s, A, B), rtol=1e-4, atol=1e-5)
+
+
+def test_coo_entries_in_any_order(oracle):
+    rng = np.random.default_rng(5)
+    rp, ci, s = random_csr(rng, 300, 300, 0.05)
+    rows = oracle.rows_of(rp)
+    A = rng.standard_normal((300, 64)).astype(np.float32)
+    B = rng.standard_normal((300, 64)).astype(np.float32)
+    perm = rng.permutation(s.size)
+    got = hip_sddmm_coo(rows[perm], ci[perm], s[perm], A, B, (300, 300))
+    assert oracle.rel_fro(got, oracle.sddmm_fp64(rows[perm], ci[perm], s[perm], A, B)) <= TOL
+
+
+def test_csr_rows_with_long_empty_stretches(oracle):
+    lens = np.zeros(70000, np.int64)
+    lens[[5, 30000, 30001, 69999]] = [700, 3, 1, 900]
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(6)
+    ci = rng.integers(0, 1000, int(rp[-1])).astype(np.int32)
+    s = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    A = rng.standard_normal((70000, 16)).astype(np.float32)
+    B = rng.standard_normal((1000, 16)).astype(np.float32)
+    r, c, val = hip_sddmm_csr(rp, ci, s, A, B, (70000, 1000))
+    rows = oracle.rows_of(rp)
+    assert np.array_equal(r, rows)
+    assert oracle.rel_fro(val, oracle.sddmm_fp64(rows, ci, s, A, B)) <= TOL
+
+
+def test_closed_forms():
+    n = 64
+    eye = np.eye(n, dtype=np.float32)
+    rows, cols = np.nonzero(np.ones((n, n)))
+    out = hip_sddmm_coo(rows.astype(np.int32), cols.astype(np.int32), np.ones(n * n, np.float32), eye, eye, (n, n))
+    assert np.array_equal(out.reshape(n, n), eye)
+    empty = hip_sddmm_coo(np.zeros(0, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), eye, eye, (n, n))
+    assert empty.size == 0
+
+
+def test_row_indices_kernel_matches_sddmm_rows(oracle):
+    w = workloads.gcn_powerlaw(M=30000, N=4, seed=8, max_degree=4000)
+    rows = H.csr_row_indices(dev(w["row_ptr"]), int(w["col_idx"].size))
+    assert np.array_equal(host(rows), oracle.rows_of(w["row_ptr"]))
+
+
+def test_full_size_workload():
+    """65,536 x 65,536 mask with 64 entries per row, K = 64: values against an
+    fp64 gather-and-dot on the device, coordinates bit-exact."""
+    w = workloads.sddmm_uniform(unit_mask=False)
+    M, n_cols, K = w["M"], w["n_cols"], w["K"]
+    rp, ci, s = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    A, B = dev(w["A"]), dev(w["B"])
+    out = H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [rp, ci]], s, [M, K], [[], []], A.reshape(-1),
+                            [n_cols, K], [[], []], B.reshape(-1))
+    rows_ref = dev(w["row_idx"])
+    assert torch.equal(out.storage.index.mode_indices[0][0], rows_ref)
+    assert out.storage.index.mode_indices[1][0] is ci
+    ref64 = torch.empty(s.numel(), dtype=torch.float64, device="cuda")
+    step = 1 << 20
+    for p0 in range(0, s.numel(), step):
+        sl = slice(p0, p0 + step)
+        ref64[sl] = (A[rows_ref[sl].long()].double() * B[ci[sl].long()].double()).sum(1) * s[sl].double()
+    err = (torch.linalg.norm(out.storage.value.double() - ref64) / torch.linalg.norm(ref64)).item()
+    assert err <= TOL, err
+    coo = H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows_ref], [ci]], s, [M, K], [[], []],
+                                     A.reshape(-1), [n_cols, K], [[], []], B.reshape(-1))
+    assert torch.equal(coo.storage.value, out.storage.value)

@@ -1,0 +1,241 @@
+"""SpMM on the MI355X through the C ABI, against the oracle, the golden
+fixtures, and (at full size) an fp64 recomputation on the device.
+
+Tolerance for fp32 (and fp64) values: relative Frobenius error <= 1e-5 against
+an fp64 recomputation.  Integer results are bit-exact.  The sparsity
+structure of the operands is read-only and C is dense, so "structure bit-exact"
+means here: shape (M, N), every element written, rows without entries zero.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+from gpu_util import dev, hip_spmm, host
+from scorch_amd import scorch_ops_hip as H
+from scorch_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+SPMM_F32_CASES = ["spmm_square95", "spmm_dispatch32", "spmm_rect", "spmm_wide300", "spmm_emptyrows",
+                  "spmm_n1", "spmm_longrow", "spmm_allzero", "spmm_diag_literal"]
+
+
+@pytest.mark.parametrize("name", SPMM_F32_CASES)
+def test_golden_f32(golden, oracle, name):
+    c = golden.case(name)
+    got = hip_spmm(c["row_ptr"], c["col_idx"], c["vals"], c["B"])
+    ref64 = oracle.spmm_fp64(c["row_ptr"], c["col_idx"], c["vals"], c["B"])
+    assert got.shape == c["C_v2"].shape and got.dtype == np.float32
+    assert oracle.rel_fro(got, ref64) <= TOL
+    np.testing.assert_allclose(got, c["C_v2"], rtol=1e-4, atol=1e-5)   # the reference's own output
+    empty = np.diff(c["row_ptr"]) == 0
+    assert not got[empty].any()
+
+
+def test_golden_diag_literal_exact(golden):
+    c = golden.case("spmm_diag_literal")
+    assert np.array_equal(hip_spmm(c["row_ptr"], c["col_idx"], c["vals"], c["B"]), c["C_v2"])
+
+
+def test_golden_f64(golden, oracle):
+    c = golden.case("spmm_f64")
+    got = hip_spmm(c["row_ptr"], c["col_idx"], c["vals"], c["B"])
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got, c["C_typed"], rtol=1e-13, atol=1e-13)
+
+
+@pytest.mark.parametrize("name", ["spmm_i32", "spmm_i64", "spmm_i32_wrap"])
+def test_golden_integer_bit_exact(golden, name):
+    c = golden.case(name)
+    got = hip_spmm(c["row_ptr"], c["col_idx"], c["vals"], c["B"])
+    assert got.dtype == c["C_typed"].dtype and np.array_equal(got, c["C_typed"])
+
+
+@pytest.mark.parametrize("relu", [False, True])
+def test_golden_bias_act(golden, oracle, relu):
+    c = golden.case("spmm_bias")
+    got = hip_spmm(c["row_ptr"], c["col_idx"], c["vals"], c["B"], bias=c["bias"], relu=relu)
+    np.testing.assert_allclose(got, c["C_bias_relu" if relu else "C_bias"], rtol=1e-4, atol=1e-5)
+
+
+# N chosen to hit every vector width and tile count: 1 lane, odd, < 64, = 64,
+# between tiles, 2-wide vectors (128), partial second tile (192), 4-wide (256+), many tiles
+@pytest.mark.parametrize("N", [1, 3, 17, 48, 64, 70, 96, 100, 128, 130, 192, 256, 300, 512, 1028])
+def test_widths_against_oracle(oracle, N):
+    rng = np.random.default_rng(N)
+    rp, ci, v = random_csr(rng, 333, 217, 0.06, empty_rows=(0, 100, 332))
+    B = rng.standard_normal((217, N)).astype(np.float32)
+    got = hip_spmm(rp, ci, v, B)
+    assert oracle.rel_fro(got, oracle.spmm_fp64(rp, ci, v, B)) <= TOL
+    np.testing.assert_allclose(got, oracle.spmm_csr_f32_v2(rp, ci, v, B), rtol=1e-4, atol=1e-5)
+
+
+def row_length_cases():
+    rng = np.random.default_rng(99)
+    cases = {}
+    # one row only, longer than several chunks
+    cases["single_long_row"] = (np.array([0, 3000], np.int32), rng.integers(0, 500, 3000).astype(np.int32))
+    # many empty rows, then entries, then empty rows (chunks made of markers only)
+    lens = np.zeros(5000, np.int64); lens[2500:2510] = 40
+    cases["mostly_empty"] = lens
+    # every row one entry (markers == nonzeros)
+    cases["one_per_row"] = np.ones(3000, np.int64)
+    # rows exactly at chunk size boundaries
+    cases["chunk_aligned"] = np.array([255, 1, 256, 0, 511, 257, 128, 128], np.int64)
+    # power-law in miniature
+    z = np.minimum(rng.zipf(1.7, 2000), 4000); cases["power_law"] = z.astype(np.int64)
+    # last row long, first row long
+    cases["long_ends"] = np.array([1500] + [2] * 300 + [1700], np.int64)
+    out = {}
+    for name, spec in cases.items():
+        if isinstance(spec, tuple):
+            out[name] = spec
+            continue
+        rp = np.concatenate([[0], np.cumsum(spec)]).astype(np.int32)
+        out[name] = (rp, rng.integers(0, 500, int(rp[-1])).astype(np.int32))
+    return out
+
+
+ROW_CASES = row_length_cases()
+
+
+@pytest.mark.parametrize("name", sorted(ROW_CASES))
+@pytest.mark.parametrize("N", [32, 128, 260])
+def test_row_length_distributions(oracle, name, N):
+    rp, ci = ROW_CASES[name]          # columns unsorted and repeating: allowed
+    rng = np.random.default_rng(len(name) + N)
+    v = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    B = rng.standard_normal((500, N)).astype(np.float32)
+    got = hip_spmm(rp, ci, v, B)
+    ref64 = oracle.spmm_fp64(rp, ci, v, B)
+    assert oracle.rel_fro(got, ref64) <= TOL
+    assert not got[np.diff(rp) == 0].any()
+
+
+@pytest.mark.parametrize("name", ["power_law", "long_ends", "mostly_empty"])
+@pytest.mark.parametrize("relu", [False, True])
+def test_bias_act_on_split_rows(oracle, name, relu):
+    rp, ci = ROW_CASES[name]
+    rng = np.random.default_rng(7)
+    v = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    B = rng.standard_normal((500, 128)).astype(np.float32)
+    bias = rng.standard_normal(128).astype(np.float32)
+    got = hip_spmm(rp, ci, v, B, bias=bias, relu=relu)
+    ref = oracle.spmm_fp64(rp, ci, v, B) + bias.astype(np.float64)
+    if relu:
+        ref = np.maximum(ref, 0)
+        assert (got >= 0).all()
+    assert oracle.rel_fro(got, ref) <= TOL
+    np.testing.assert_allclose(got, oracle.spmm_csr_bias_act_f32(rp, ci, v, B, bias, relu), rtol=1e-4,
+                               atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("N", [5, 64, 128, 200])
+def test_other_dtypes_against_oracle(oracle, dtype, N):
+    rp, ci = ROW_CASES["power_law"]
+    rng = np.random.default_rng(N)
+    if np.issubdtype(dtype, np.integer):
+        v = rng.integers(-2 ** 20, 2 ** 20, ci.size).astype(dtype)
+        B = rng.integers(-2 ** 20, 2 ** 20, (500, N)).astype(dtype)
+    else:
+        v = rng.uniform(-1, 1, ci.size).astype(dtype)
+        B = rng.standard_normal((500, N)).astype(dtype)
+    got = hip_spmm(rp, ci, v, B)
+    want = oracle.spmm_csr_typed(rp, ci, v, B)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(got, want)        # wraps identically (int32 products overflow here)
+    else:
+        np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_closed_forms(oracle):
+    rng = np.random.default_rng(1)
+    B = rng.standard_normal((700, 128)).astype(np.float32)
+    ident = hip_spmm(np.arange(701, dtype=np.int32), np.arange(700, dtype=np.int32), np.ones(700, np.float32), B)
+    assert np.array_equal(ident, B)
+    perm = rng.integers(0, 700, 2000).astype(np.int32)
+    gathered = hip_spmm(np.arange(2001, dtype=np.int32), perm, np.ones(2000, np.float32), B)
+    assert np.array_equal(gathered, B[perm])
+    zero = hip_spmm(np.zeros(11, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32), B[:, :6].copy())
+    assert zero.shape == (10, 6) and not zero.any()
+
+
+def test_runs_are_bit_reproducible_and_inputs_untouched():
+    w = workloads.gcn_powerlaw(M=20000, N=128, seed=3, max_degree=5000)
+    rp, ci, v, B = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"]), dev(w["B"]).reshape(-1)
+    args = ([20000, 128], [20000, 20000], [[], [rp, ci]], v, [20000, 128], [[], []], B)
+    first = H.spmm_csr_float_v2(*args).storage.value.clone()
+    for _ in range(3):
+        again = H.spmm_csr_float_v2(*args).storage.value
+        assert torch.equal(first, again)
+    assert np.array_equal(host(rp), w["row_ptr"]) and np.array_equal(host(ci), w["col_idx"])
+    assert np.array_equal(host(v), w["vals"]) and np.array_equal(host(B).reshape(-1, 128), w["B"])
+
+
+def test_output_needs_no_zero_fill():
+    # poison the allocator's recycled block, then check every element was written
+    w = workloads.gcn_powerlaw(M=5000, N=64, seed=4, max_degree=900)
+    junk = torch.full((5000 * 64,), float("nan"), device="cuda")
+    del junk
+    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
+    assert np.isfinite(got).all()
+
+
+def test_uniform_workload_reference_size(oracle):
+    """4096 x 4096 at 1 % density, N = 64: the reference's own CPU-runnable case."""
+    w = workloads.spmm_uniform()
+    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
+    assert oracle.rel_fro(got, oracle.spmm_fp64(w["row_ptr"], w["col_idx"], w["vals"], w["B"])) <= TOL
+    np.testing.assert_allclose(got, oracle.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"]),
+                               rtol=1e-4, atol=1e-5)
+
+
+def test_sae_decoder_workload(oracle):
+    """Sparse-autoencoder decoder shape (32 entries per row, N = 4096) at a quarter of the rows."""
+    w = workloads.sae_decoder(M=1024)
+    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
+    assert oracle.rel_fro(got, oracle.spmm_fp64(w["row_ptr"], w["col_idx"], w["vals"], w["B"])) <= TOL
+
+
+def test_power_law_medium_against_oracle(oracle):
+    w = workloads.gcn_powerlaw(M=1 << 16, N=128, seed=11, max_degree=20000)
+    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
+    assert oracle.rel_fro(got, oracle.spmm_fp64(w["row_ptr"], w["col_idx"], w["vals"], w["B"])) <= TOL
+    np.testing.assert_allclose(got, oracle.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"]),
+                               rtol=1e-4, atol=1e-5)
+
+
+def test_power_law_full_size_properties():
+    """The 1,048,576-row, N = 128 workload.  Size-independent checks on the device:
+    fp64 recomputation with torch's CSR product, linearity in B, and the row sums
+    of A recovered from a column of ones."""
+    w = workloads.gcn_powerlaw()
+    M, N = w["M"], w["N"]
+    rp, ci, v = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    B = dev(w["B"])
+
+    def run(Bmat):
+        return H.spmm_csr_float_v2([M, N], [M, M], [[], [rp, ci]], v, [M, N], [[], []],
+                                   Bmat.reshape(-1)).storage.value.view(M, N)
+
+    C = run(B)
+    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), v.double(), size=(M, M))
+    ref64 = torch.sparse.mm(A64, B.double())
+    err = (torch.linalg.norm(C.double() - ref64) / torch.linalg.norm(ref64)).item()
+    assert err <= TOL, err
+    del ref64
+
+    ones = torch.ones_like(B)
+    row_sums = torch.zeros(M, dtype=torch.float64, device="cuda")
+    rows = torch.repeat_interleave(torch.arange(M, device="cuda"), (rp[1:] - rp[:-1]).long())
+    row_sums.index_add_(0, rows, v.double())
+    Cones = run(ones)
+    assert torch.allclose(Cones[:, 0].double(), row_sums, rtol=1e-5, atol=1e-6)
+    assert torch.equal(Cones[:, 0], Cones[:, N - 1])
+
+    B2 = torch.roll(B, 1, dims=0)
+    lin = run(B + B2) - (C + run(B2))
+    assert (torch.linalg.norm(lin.double()) / torch.linalg.norm(C.double())).item() <= 1e-5

@@ -1,0 +1,219 @@
+"""Host-side logic that mirrors the reference's dispatch: format strings, the
+tensor model, the prebuilt-kernel registry and the routing decisions of
+matmul / einsum.  Mirrors tests/test_scorch/test_prebuilt_kernel_registry.py
+and the format checks of the reference; runs without a GPU."""
+import numpy as np
+import pytest
+import torch
+
+import scorch_amd as scorch
+from scorch_amd import STensor, ops, parse_format, scorch_ops_hip
+from scorch_amd.prebuilt_kernels import (execute_prebuilt_binary_kernel, resolve_prebuilt_fused,
+                                         resolve_prebuilt_matmul)
+
+
+def sparse_dense_pair(n=16, dtype=torch.float32, density=0.2, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.rand(n, n, generator=g, dtype=torch.float64) * (torch.rand(n, n, generator=g) < density)
+    b = torch.rand(n, n, generator=g, dtype=torch.float64)
+    if dtype in (torch.int32, torch.int64):
+        a, b = (a * 10).round(), (b * 10).round()
+    return a.to(dtype), b.to(dtype)
+
+
+# ---- formats ------------------------------------------------------------------------
+@pytest.mark.parametrize("spec,text", [("ds", "d,s"), ("dd", "d,d"), ("oo", "o,o"), ("d", "d"),
+                                       (["dense", "compressed"], "d,s"), (["coord", "coordinate"], "o,o"),
+                                       (["dense", "sparse"], "d,s"), (["d", "c"], "d,s")])
+def test_parse_format_strings(spec, text):
+    assert str(parse_format(spec)) == text
+
+
+def test_parse_format_rejects_unknown_levels():
+    with pytest.raises(ValueError):
+        parse_format("dx")
+    with pytest.raises(ValueError):
+        parse_format(["dense", "singleton"])
+
+
+def test_format_equality_and_density():
+    assert parse_format("dd") == parse_format(["dense", "dense"])
+    assert parse_format("ds") != parse_format("dd")
+    assert parse_format("dd").is_dense() and not parse_format("ds").is_dense()
+    assert parse_format(parse_format("oo")) is not None
+
+
+# ---- tensor model -----------------------------------------------------------------------
+def test_from_torch_dense_flattens_values():
+    t = torch.arange(12, dtype=torch.float32).reshape(3, 4)
+    s = STensor.from_torch(t)
+    assert str(s.format) == "d,d" and s.shape == (3, 4) and s.dim() == 2
+    assert s.index.mode_indices == [[], []]
+    assert s.values.shape == (12,) and torch.equal(s.values, t.flatten())
+    assert torch.equal(s.to_torch(), t)
+
+
+def test_from_csr_shares_arrays_and_coerces_indices_to_int32():
+    a, _ = sparse_dense_pair()
+    csr = a.to_sparse_csr()
+    assert csr.crow_indices().dtype == torch.int64
+    s = STensor.from_csr(csr)
+    pos, crd = s.index.mode_indices[1]
+    assert str(s.format) == "d,s" and s.index.mode_indices[0] == []
+    assert pos.dtype == torch.int32 and crd.dtype == torch.int32
+    assert torch.equal(pos.long(), csr.crow_indices()) and torch.equal(crd.long(), csr.col_indices())
+    assert s.values.data_ptr() == csr.values().data_ptr()
+    assert s._nnz() == csr.values().numel()
+    assert torch.equal(s.to_torch(), a)
+
+
+def test_from_torch_sparse_layouts_and_from_coo():
+    a, _ = sparse_dense_pair(seed=3)
+    s_csr = scorch.from_torch(a.to_sparse_csr())
+    s_coo = scorch.from_torch(a.to_sparse())
+    assert str(s_csr.format) == "d,s" and str(s_coo.format) == "o,o"
+    assert len(s_coo.index.mode_indices) == 2 and s_coo.index.mode_indices[0][0].dtype == torch.int32
+    assert torch.equal(s_coo.to_torch(), a) and torch.equal(s_csr.to_torch(), a)
+    raw = scorch.from_coo(indices=a.to_sparse().indices(), values=a.to_sparse().values(), shape=a.shape)
+    assert torch.equal(raw.to_torch(), a)
+
+
+def test_to_sparse_round_trips():
+    a, _ = sparse_dense_pair(seed=4)
+    d = STensor.from_torch(a)
+    for fmt in ("ds", "oo"):
+        s = d.to_sparse(fmt)
+        assert str(s.format) == str(parse_format(fmt))
+        assert torch.equal(s.to_torch(), a)
+        assert torch.equal(s.to_dense().to_torch(), a)
+    assert str(d.to_sparse("ds").to_sparse("oo").format) == "o,o"
+
+
+def test_copy_is_deep_and_to_cpu_is_a_copy():
+    a, _ = sparse_dense_pair(seed=5)
+    s = STensor.from_torch(a).to_sparse("ds")
+    c = s.copy()
+    c.values.zero_()
+    assert s.values.abs().sum() > 0
+    assert s.to("cpu").index == s.index and not s.is_cuda
+
+
+# ---- registry (reference: tests/test_scorch/test_prebuilt_kernel_registry.py) ---------------
+@pytest.mark.parametrize("dtype,symbol", [(torch.float32, "spmm_csr_float_v2"),
+                                          (torch.float64, "prebuilt_spmm_csr_f64"),
+                                          (torch.int32, "prebuilt_spmm_csr_i32"),
+                                          (torch.int64, "prebuilt_spmm_csr_i64")])
+def test_resolve_prebuilt_spmm_symbol_per_dtype(dtype, symbol):
+    a, b = sparse_dense_pair(dtype=dtype)
+    resolved = resolve_prebuilt_matmul(STensor.from_torch(a).to_sparse("ds"), STensor.from_torch(b))
+    assert resolved is not None and resolved.symbol_name == symbol
+    assert str(resolved.output_format) == "d,d"
+    assert resolved.fn is getattr(scorch_ops_hip, symbol)
+
+
+def test_resolve_prebuilt_spmv_int64_symbol():
+    a = torch.tensor([[1, 0, 2, 0], [0, 3, 0, 4], [0, 0, 0, 0], [5, 0, 0, 6]], dtype=torch.int64)
+    x = torch.tensor([1, 2, 3, 4], dtype=torch.int64)
+    resolved = resolve_prebuilt_matmul(STensor.from_torch(a).to_sparse("ds"), STensor.from_torch(x))
+    assert resolved is not None and resolved.symbol_name == "prebuilt_spmv_csr_i64"
+    assert str(resolved.output_format) == "d"
+
+
+def test_resolve_prebuilt_gates():
+    a, b = sparse_dense_pair()
+    A, B = STensor.from_torch(a).to_sparse("ds"), STensor.from_torch(b)
+    assert resolve_prebuilt_matmul(A, B, output_format="dd") is not None
+    assert resolve_prebuilt_matmul(A, B, output_format="ds") is None          # requested format gate
+    assert resolve_prebuilt_matmul(A, STensor.from_torch(b.double())) is None  # dtype equality gate
+    assert resolve_prebuilt_matmul(B, B) is None                               # dense x dense: no entry
+    assert resolve_prebuilt_matmul(A, STensor.from_torch(b.half())) is None
+    # CSR x CSR is in the table but this package ships no symbol for it
+    assert resolve_prebuilt_matmul(A, A, output_format="dd") is None
+    assert resolve_prebuilt_matmul(A, A) is None
+
+
+def test_resolve_prebuilt_fused():
+    assert resolve_prebuilt_fused("d,s", "d,d", ("add", "relu"), torch.float32).symbol_name == \
+        "spmm_csr_bias_relu_float"
+    assert resolve_prebuilt_fused("d,s", "d,d", ("add",), torch.float32).symbol_name == "spmm_csr_bias_float"
+    assert resolve_prebuilt_fused("d,s", "d,d", ("relu",), torch.float32) is None
+    assert resolve_prebuilt_fused("d,s", "d,d", ("add",), torch.float64) is None
+    assert resolve_prebuilt_fused("o,o", "d,d", ("add",), torch.float32) is None
+
+
+def test_execute_prebuilt_packs_arguments_like_the_reference():
+    a, b = sparse_dense_pair(n=8)
+    A, B = STensor.from_torch(a).to_sparse("ds"), STensor.from_torch(b)
+    seen = {}
+
+    def fake_kernel(*args):
+        seen["args"] = args
+        return "result"
+
+    td = {}
+    result, shape = execute_prebuilt_binary_kernel(fake_kernel, A, B, time_dict=td)
+    assert result == "result" and shape == (8, 8) and td["eval_time"] >= 0
+    args = seen["args"]
+    assert len(args) == 7 and args[0] == (8, 8) and args[1] == (8, 8) and args[4] == (8, 8)
+    assert args[2] is A.index.mode_indices and args[3] is A.values and args[6] is B.values
+    x = STensor.from_torch(b[:, 0].contiguous())
+    _, shape = execute_prebuilt_binary_kernel(fake_kernel, A, x)
+    assert shape == (8,)
+
+
+# ---- routing ---------------------------------------------------------------------------------
+def test_canonical_expression():
+    assert ops._canonical("ik,kj->ij") == "ab,bc->ac" == ops._canonical("ij,jk->ik")
+    assert ops._canonical("ij,ik,jk->ij") == ops._SDDMM_EXPR
+    assert ops._canonical("ij,ik,kj->ij") == ops._SDDMM_EXPR_KJ
+
+
+def test_dense_dense_matmul_uses_torch():
+    _, b = sparse_dense_pair()
+    assert torch.equal(scorch.matmul(b, b), torch.matmul(b, b))
+    assert torch.equal(scorch.matmul(STensor.from_torch(b), STensor.from_torch(b)), torch.matmul(b, b))
+
+
+def test_host_sparse_operands_are_refused_not_computed():
+    a, b = sparse_dense_pair()
+    A = STensor.from_torch(a).to_sparse("ds")
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.matmul(A, b)
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.matmul(A, b, use_cache=False)
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.einsum("ij,ik,jk->ij", A, b, b)
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.einsum("ij,ik,jk->ij", STensor.from_torch(a).to_sparse("oo"), b, b)
+
+
+def test_expressions_outside_the_path_raise_not_implemented():
+    a, b = sparse_dense_pair()
+    A = STensor.from_torch(a).to_sparse("ds")
+    with pytest.raises(NotImplementedError):
+        scorch.matmul(A, A)                      # SpGEMM belongs to the reference's kernels
+    with pytest.raises(NotImplementedError):
+        scorch.einsum("ij,ij->ij", A, A)
+    with pytest.raises(NotImplementedError):
+        scorch.matmul(A, b, format="ds")
+    with pytest.raises(NotImplementedError):
+        scorch.einsum("ij,jk->ik", A, b, compile_only=True)
+    with pytest.raises(NotImplementedError):
+        scorch.spmm_bias_act(STensor.from_torch(a.double()).to_sparse("ds"), b.double(), b[0].double())
+
+
+def test_device_module_rejects_host_and_mistyped_tensors():
+    a, b = sparse_dense_pair(n=8)
+    A, B = STensor.from_torch(a).to_sparse("ds"), STensor.from_torch(b)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        scorch_ops_hip.spmm_csr_float_v2((8, 8), A.shape, A.index.mode_indices, A.values, B.shape,
+                                         B.index.mode_indices, B.values)
+    with pytest.raises(TypeError):
+        scorch_ops_hip.spmm_csr_float_v2((8, 8), A.shape, A.index.mode_indices, A.values.double(),
+                                         B.shape, B.index.mode_indices, B.values)
+    with pytest.raises(ValueError, match="shape mismatch"):
+        scorch_ops_hip.spmm_csr_float_v2((8, 9), A.shape, A.index.mode_indices, A.values, B.shape,
+                                         B.index.mode_indices, B.values)
+    with pytest.raises(ValueError, match="not a CSR"):
+        scorch_ops_hip.spmm_csr_float_v2((8, 8), A.shape, [[], []], A.values, B.shape,
+                                         B.index.mode_indices, B.values)
