@@ -95,6 +95,9 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1 << 20, help="nodes of the graph (default: the headline size)")
     ap.add_argument("--features", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
+                         "WRITE_SIZE counters against a kernel of known traffic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (the kernel shards by rows "
@@ -113,6 +116,17 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.probe_copy:
+        n = 1 << 28                                  # 1 GiB of fp32 read, 1 GiB written per copy
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy", "read_bytes_per_launch": 4 * n,
+                          "write_bytes_per_launch": 4 * n, "launches": args.warmup + args.steps}))
+        return 0
 
     t0 = time.time()
     w = workloads.gcn_powerlaw(M=args.rows, N=args.features)
