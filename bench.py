@@ -87,6 +87,66 @@ def cpu_baseline(w, repeats=5):
                       "warm-up, whole native call incl. allocating and zeroing C"}
 
 
+def _time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def side_workload(args, dev) -> int:
+    """Times one of the other workloads (not the headline metric): same JSON
+    shape, HIP-event time per step, algorithmic and gather-model bandwidth."""
+    import torch
+    from scorch_amd import workloads
+    from scorch_amd import scorch_ops_hip as H
+    t = lambda a: torch.from_numpy(a).to(dev)
+    if args.workload == "sddmm_uniform":
+        w = workloads.sddmm_uniform()
+        M, n_cols, K, nnz = w["M"], w["n_cols"], w["K"], int(w["col_idx"].size)
+        pos, crd, val, A, B = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), t(w["A"]), t(w["B"])
+        rows = t(w["row_idx"])
+        csr = lambda: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [pos, crd]], val, [M, K], [[], []],
+                                        A.reshape(-1), [n_cols, K], [[], []], B.reshape(-1))
+        coo = lambda: H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows], [crd]], val, [M, K],
+                                                 [[], []], A.reshape(-1), [n_cols, K], [[], []],
+                                                 B.reshape(-1))
+        ms = _time_steps(csr, args.steps, args.warmup)
+        ms_coo = _time_steps(coo, args.steps, args.warmup)
+        flops = 2.0 * nnz * K + nnz
+        algo = 4 * (M + 1) + 4 * nnz * 3 + 4 * M * K + 4 * n_cols * K + 4 * nnz   # + row output
+        gather = algo - 4 * n_cols * K + 4 * nnz * K
+        out = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
+               "ms_per_step": round(ms, 4), "ms_per_step_coo_mask": round(ms_coo, 4),
+               "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K}}
+    else:
+        w = workloads.spmm_uniform() if args.workload == "spmm_uniform" else workloads.sae_decoder()
+        M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
+        pos, crd, val, B = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), t(w["B"]).reshape(-1)
+        fn = lambda: H.spmm_csr_float_v2([M, N], [M, K], [[], [pos, crd]], val, [K, N], [[], []], B)
+        ms = _time_steps(fn, args.steps, args.warmup)
+        flops = 2.0 * nnz * N
+        algo, gather = algorithmic_bytes(M, K, N, nnz), gather_bytes(M, N, nnz)
+        out = {"metric": "CSR SpMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
+               "ms_per_step": round(ms, 4),
+               "config": {"workload": args.workload + "_fp32", "rows": M, "cols": K, "nnz": nnz,
+                          "features": N}}
+    out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
+                "data": "synthetic", "higher_is_better": True,
+                "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                "gather_model_bytes": gather, "gather_model_gbps": round(gather / ms / 1e6, 1)})
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +155,9 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1 << 20, help="nodes of the graph (default: the headline size)")
     ap.add_argument("--features", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", default="gcn_powerlaw",
+                    choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform"],
+                    help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")
@@ -127,6 +190,9 @@ def main() -> int:
         print(json.dumps({"probe": "copy", "read_bytes_per_launch": 4 * n,
                           "write_bytes_per_launch": 4 * n, "launches": args.warmup + args.steps}))
         return 0
+
+    if args.workload != "gcn_powerlaw":
+        return side_workload(args, dev)
 
     t0 = time.time()
     w = workloads.gcn_powerlaw(M=args.rows, N=args.features)

@@ -30,7 +30,8 @@
 
 namespace scorch {
 
-constexpr int kItemsPerWave = 256;  // merge items (row ends + nonzeros) per wavefront
+constexpr int kItemsPerWave = 256;  // most merge items (row ends + nonzeros) per wavefront
+constexpr int kMinItemsPerWave = 32;
 constexpr int kGather = 8;          // B-row loads in flight per wavefront
 
 enum Epilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasRelu = 2 };
@@ -47,8 +48,8 @@ template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
-    const T *__restrict__ bias, int64_t total_items, int *__restrict__ carry_row,
-    T *__restrict__ carry_val) {
+    const T *__restrict__ bias, int64_t total_items, int items_per_wave,
+    int *__restrict__ carry_row, T *__restrict__ carry_val) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
 
@@ -63,9 +64,9 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
   const bool active = col0 < N;
 
   // Chunk [d0, d1) of the merged sequence; chunks past the end are empty.
-  int64_t d0 = chunk * kItemsPerWave;
+  int64_t d0 = chunk * items_per_wave;
   d0 = d0 < total_items ? d0 : total_items;
-  int64_t d1 = d0 + kItemsPerWave;
+  int64_t d1 = d0 + items_per_wave;
   d1 = d1 < total_items ? d1 : total_items;
 
   auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
   while (x < x1) flush_row();  // markers after the chunk's last nonzero
 
   // Whatever is left belongs to row x1, whose marker lies in a later chunk.
-  if (chunk * kItemsPerWave < total_items) {
+  if (chunk * items_per_wave < total_items) {
     const int row_start = uniform(s_rp[w][n_rows]);
     const int tail = y1 - (row_start > y0 ? row_start : y0);
     if (blockIdx.y == 0 && lane == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
@@ -176,17 +177,24 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
   const int row = uniform(carry_row[chunk]);
   if (row < 0) return;
   if (chunk > 0 && uniform(carry_row[chunk - 1]) == row) return;  // not the head of its run
+  // End of the run: 64 entries of carry_row are compared per step.
+  int64_t end = chunk + 1;
+  for (;;) {
+    const int64_t probe = end + lane;
+    const bool same = probe < num_chunks && carry_row[probe] == row;
+    const unsigned long long differs = ~__ballot(same);
+    const int matched = differs ? __ffsll(differs) - 1 : kWaveSize;
+    end += matched;
+    if (matched < kWaveSize) break;
+  }
   const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
   if (col0 >= N) return;
-
-  int64_t end = chunk + 1;
-  while (end < num_chunks && uniform(carry_row[end]) == row) ++end;
 
   A sum[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) sum[v] = (A)0;
   int64_t c = chunk;
-  constexpr int kBatch = 8;
+  constexpr int kBatch = 32;  // loads in flight: a long row spans hundreds of chunks
   for (; c + kBatch <= end; c += kBatch) {
     VecT part[kBatch];
 #pragma unroll
@@ -215,8 +223,19 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
 
 // ---- host side ----------------------------------------------------------------
 
+// Items per wavefront: the full 256 when that still yields enough wavefronts to
+// fill the chip (256 CUs x 32 wavefronts), otherwise a smaller power of two so
+// that a small problem is spread over more, shorter wavefronts.
+inline int spmm_items_per_wave(int64_t M, int64_t nnz) {
+  const int64_t per_wave = (M + nnz) / 8192;
+  int ipw = kMinItemsPerWave;
+  while (ipw < kItemsPerWave && ipw * 2 <= per_wave) ipw *= 2;
+  return ipw;
+}
+
 inline int64_t spmm_num_chunks(int64_t M, int64_t nnz) {
-  return (M + nnz + kItemsPerWave - 1) / kItemsPerWave;
+  const int ipw = spmm_items_per_wave(M, nnz);
+  return (M + nnz + ipw - 1) / ipw;
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -255,7 +274,8 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
                   (unsigned)((N + tile - 1) / tile));
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
-      M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, carry_row, carry_val);
+      M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, spmm_items_per_wave(M, nnz),
+      carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
   spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(N, chunks, carry_row,
