@@ -108,6 +108,26 @@ def side_workload(args, dev) -> int:
     from scorch_amd import workloads
     from scorch_amd import scorch_ops_hip as H
     t = lambda a: torch.from_numpy(a).to(dev)
+    if args.workload == "attention_blocksparse":
+        w = workloads.attention_blocksparse()
+        Hh, S, D = w["H"], w["S"], w["D"]
+        q, k, v = (t(w[n]).to(torch.bfloat16) for n in ("q", "k", "v"))
+        brp, bci = t(w["block_row_ptr"]), t(w["block_col_idx"])
+        nnz = int(w["block_col_idx"].size) * w["block"] ** 2
+        fn = lambda: H.attn_blocksparse_bf16(q, k, v, brp, bci, float(w["scale"]))
+        ms = _time_steps(fn, args.steps, args.warmup)
+        flops = 4.0 * nnz * D * Hh
+        algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
+        print(json.dumps({"metric": "fused block-sparse attention TFLOP/s", "value": round(flops / ms / 1e9, 2),
+                          "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
+                          "higher_is_better": True,
+                          "config": {"workload": "attention_blocksparse_bf16", "S": S, "H": Hh, "D": D,
+                                     "block": w["block"], "active_blocks": int(bci.numel()),
+                                     "nnz_per_head": nnz},
+                          "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
+                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
+        return 0
     if args.workload == "sddmm_uniform":
         w = workloads.sddmm_uniform()
         M, n_cols, K, nnz = w["M"], w["n_cols"], w["K"], int(w["col_idx"].size)
@@ -156,7 +176,8 @@ def main() -> int:
     ap.add_argument("--features", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="gcn_powerlaw",
-                    choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform"],
+                    choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
+                             "attention_blocksparse"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "

@@ -183,6 +183,25 @@ SCORCH_HIP_API int scorch_hip_spmv_csr_i64(int64_t M, int64_t K, int64_t nnz, co
 SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr,
                                const float *vals, float scale, float *out, void *stream);
 
+/* ------------------------------------------------------------------------
+ * Fused block-sparse attention, bf16 in / bf16 out, fp32 accumulation:
+ * O[h] = softmax_rows(scale * Q[h] K[h]^T, restricted to the mask) V[h].
+ * Q, K, V, O are [H, S, D] row-major bf16.  The mask is shared by all heads and
+ * given as a block-CSR pattern over (S / block)^2 blocks of block x block
+ * entries: block_row_ptr int32[S / block + 1], block_col_idx
+ * int32[n_active_blocks]; every entry of an active block is live.  Query rows
+ * whose block row has no active block give zeros.
+ * Built for D = 64 and block = 64 (other values: SCORCH_HIP_EUNSUPPORTED).
+ * One kernel does what the reference's attention benchmark composes per head
+ * from SDDMM, a row softmax and SpMM (bench/bench_sparse_transformer.py:354-372);
+ * the reference has no fused or bf16 counterpart.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D, int64_t block,
+                                     int64_t n_active_blocks,
+                                     const int32_t *block_row_ptr, const int32_t *block_col_idx,
+                                     const void *Q, const void *K, const void *V, float scale,
+                                     void *O, void *stream);
+
 /* Rows of a CSR matrix's entries: row_idx[p] = i for row_ptr[i] <= p < row_ptr[i+1].
  * The device-side counterpart of the "d,s" -> "o,o" index conversion the
  * reference performs on the host (STensor.from_coo / to_sparse,

@@ -310,3 +310,17 @@ if __name__ == "__main__":
     build(force="--force" in sys.argv)
     print("liboracle.so:", os.path.exists(_LIB_PATH), " _ref/scorch_ops.so:", have_ref(),
           " threads:", num_threads())
+
+
+def attention_blocksparse_fp64(q, k, v, block_row_ptr, block_col_idx, block: int, scale: float) -> np.ndarray:
+    """Block-sparse attention for (H, S, D) inputs in float64: per head, the
+    masked dense softmax of attention_dense_fp64 with the mask expanded from its
+    block pattern (every entry of an active block live).  Written for small S."""
+    q, k, v = (np.asarray(t, np.float64) for t in (q, k, v))
+    H, S, _ = q.shape
+    nb = S // block
+    blocks = np.zeros((nb, nb), dtype=bool)
+    rows = rows_of(block_row_ptr)
+    blocks[rows, np.asarray(block_col_idx)] = True
+    mask = np.kron(blocks, np.ones((block, block), dtype=bool))
+    return np.stack([attention_dense_fp64(q[h], k[h], v[h], mask, scale) for h in range(H)])

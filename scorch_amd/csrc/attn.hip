@@ -1,0 +1,220 @@
+// Fused block-sparse attention for gfx950: O = softmax(scale * Q K^T restricted
+// to a block mask) V, bf16 operands, fp32 accumulation, one pass over the mask.
+//
+// It replaces, for a mask made of 64 x 64 blocks, the three-step pipeline
+// SDDMM -> row softmax -> SpMM that the reference runs per head
+// (bench/bench_sparse_transformer.py:354-372): the scores are never written to
+// memory.  The contraction inside a block is dense, so it runs on the matrix
+// cores (v_mfma_f32_16x16x32_bf16).
+//
+// Work split.  One workgroup (4 wavefronts) owns one head and one block row of
+// the mask, i.e. 64 queries; each wavefront owns 16 of them.  The workgroup
+// walks the block row's active key blocks.  For each, the 64 x 64 K tile and
+// the 64 x 64 V tile are staged in LDS once for all four wavefronts (V is
+// stored transposed so that eight consecutive keys of one feature are
+// contiguous); the next tile's global loads are in flight while the current
+// one is consumed (two LDS buffers, one barrier per key block).
+//
+// Per wavefront and key block, everything stays in registers:
+//   S^T = K Q^T        (keys x queries: 4 tiles of 16 keys, contraction over D)
+//   online softmax     (running max / sum per query, base-2 exponent)
+//   O^T += V^T P^T     (features x queries: 4 tiles of 16 features, contraction over keys)
+// Working with the transposes makes the layouts chain without any shuffle: an
+// MFMA result tile holds, in lane (g, n) (g = lane / 16, n = lane % 16), rows
+// 4g .. 4g+3 of column n.  Column n is query n throughout, so each lane owns
+// the softmax state of its query; the 16 probabilities it holds after the
+// first product (4 tiles x 4 keys) are exactly the B operand of the second
+// one, provided the V^T operand is gathered with the same key order.
+#include "common.hpp"
+
+namespace scorch {
+
+constexpr int kAttnBlock = 64;  // mask block edge: queries per workgroup, keys per step
+constexpr int kAttnDim = 64;    // head dimension
+constexpr int kLdsRow = 72;     // LDS row length in bf16 (64 + 8 padding against bank conflicts)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
+    int S, int n_blocks, const int *__restrict__ block_row_ptr,
+    const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
+    const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
+    __bf16 *__restrict__ O) {
+  __shared__ __attribute__((aligned(16))) __bf16 s_k[2][kAttnBlock][kLdsRow];   // [key][feature]
+  __shared__ __attribute__((aligned(16))) __bf16 s_vt[2][kAttnDim][kLdsRow];    // [feature][key]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWaveSize - 1);
+  const int w = tid / kWaveSize;
+  const int g = lane >> 4;  // 16-lane group: which keys / features of a tile this lane holds
+  const int n = lane & 15;  // query within the wavefront's 16
+  const int head = blockIdx.y;
+  const int qb = n_blocks - 1 - (int)blockIdx.x;  // longest block rows first
+  const size_t head_off = (size_t)head * (size_t)S * kAttnDim;
+  const __bf16 *Qh = Q + head_off, *Kh = K + head_off, *Vh = V + head_off;
+
+  // B operand of S^T = K Q^T: this lane's query row, features 8g + 32s .. + 7.
+  const int query = qb * kAttnBlock + w * 16 + n;
+  bf16x8 q_op[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+    q_op[s] = *reinterpret_cast<const bf16x8 *>(Qh + (size_t)query * kAttnDim + 8 * g + 32 * s);
+
+  floatx4 o_acc[4];  // O^T tiles: o_acc[dt][r] = O[query][16 dt + 4g + r]
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) o_acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -3.0e38f;  // running maximum of scale * log2(e) * score, equal in the 4 lanes of a query
+  float l_run = 0.0f;      // this lane's share of the running sum
+
+  const int kb_begin = block_row_ptr[qb];
+  const int kb_end = block_row_ptr[qb + 1];
+
+  // Staging: thread handles two 16-byte pieces of each tile; piece c covers
+  // row c / 8 (a key), features 8 (c % 8) .. + 7.
+  bf16x8 k_stage[2], v_stage[2];
+  auto load_tile = [&](int it) {
+    const int kb = block_col_idx[it];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = tid + u * kBlockThreads;
+      const size_t off = (size_t)(kb * kAttnBlock + (c >> 3)) * kAttnDim + (c & 7) * 8;
+      k_stage[u] = *reinterpret_cast<const bf16x8 *>(Kh + off);
+      v_stage[u] = *reinterpret_cast<const bf16x8 *>(Vh + off);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = tid + u * kBlockThreads;
+      const int key = c >> 3, f0 = (c & 7) * 8;
+      *reinterpret_cast<bf16x8 *>(&s_k[buf][key][f0]) = k_stage[u];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s_vt[buf][f0 + e][key] = v_stage[u][e];
+    }
+  };
+
+  if (kb_begin < kb_end) {
+    load_tile(kb_begin);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int it = kb_begin; it < kb_end; ++it) {
+    const int buf = (it - kb_begin) & 1;
+    const bool more = it + 1 < kb_end;
+    if (more) load_tile(it + 1);
+
+    // S^T tile t: keys 16t .. 16t+15 (rows) x 16 queries (columns).
+    floatx4 st[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const bf16x8 k_op = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g + 32 * s]);
+        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_op, q_op[s], st[t], 0, 0, 0);
+      }
+    }
+
+    // Online softmax for query n, in base 2: this lane holds keys 16t + 4g + r.
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        st[t][r] *= scale_log2e;
+        mx = fmaxf(mx, st[t][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = exp2f(m_run - m_new);
+    m_run = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
+
+    // P^T as the B operand of the second product: slot j of step s is key
+    // 32s + 16 (j / 4) + 4g + (j % 4).
+    bf16x8 p_op[2];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = exp2f(st[t][r] - m_new);
+        l_run += p;
+        p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
+      }
+
+    // O^T tile dt: features 16dt .. 16dt+15 (rows) x 16 queries, contraction over the 64 keys.
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const __bf16 *row = &s_vt[buf][16 * dt + n][32 * s + 4 * g];
+        const bf16x4 lo = *reinterpret_cast<const bf16x4 *>(row);
+        const bf16x4 hi = *reinterpret_cast<const bf16x4 *>(row + 16);
+        const bf16x8 v_op = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
+      }
+
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Normalise and store O[query][16dt + 4g .. + 3] (8 bytes per tile and lane).
+  float l = l_run;
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // block rows without key blocks give zeros
+  __bf16 *out = O + head_off + (size_t)query * kAttnDim;
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) {
+    bf16x4 o;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = (__bf16)(o_acc[dt][r] * inv);
+    *reinterpret_cast<bf16x4 *>(out + 16 * dt + 4 * g) = o;
+  }
+}
+
+}  // namespace scorch
+
+extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D, int64_t block,
+                                                int64_t n_active_blocks,
+                                                const int32_t *block_row_ptr,
+                                                const int32_t *block_col_idx, const void *Q,
+                                                const void *K, const void *V, float scale, void *O,
+                                                void *stream) {
+  using namespace scorch;
+  const char *fn = "scorch_hip_attn_blocksparse_bf16";
+  if (H < 0 || S < 0 || D < 0 || block <= 0 || n_active_blocks < 0)
+    return fail(SCORCH_HIP_EINVAL, "%s: negative size (H=%lld S=%lld D=%lld block=%lld)", fn,
+                (long long)H, (long long)S, (long long)D, (long long)block);
+  if (D != kAttnDim || block != kAttnBlock)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: only head dimension %d and %d x %d mask blocks are built "
+                "(got D=%lld block=%lld)", fn, kAttnDim, kAttnBlock, kAttnBlock, (long long)D,
+                (long long)block);
+  if (S % kAttnBlock != 0)
+    return fail(SCORCH_HIP_EINVAL, "%s: S=%lld is not a multiple of the block size", fn, (long long)S);
+  if (H > 65535 || S / kAttnBlock > INT32_MAX || S * D > INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: H=%lld or S=%lld too large", fn, (long long)H, (long long)S);
+  SCORCH_REQUIRE(block_row_ptr != nullptr, "%s: block_row_ptr is NULL", fn);
+  if (H == 0 || S == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(n_active_blocks == 0 || block_col_idx != nullptr, "%s: block_col_idx is NULL", fn);
+  SCORCH_REQUIRE(Q && K && V && O, "%s: NULL Q/K/V/O", fn);
+  SCORCH_REQUIRE(aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16),
+                 "%s: Q, K, V and O must be 16-byte aligned", fn);
+  const int n_blocks = (int)(S / kAttnBlock);
+  const dim3 grid((unsigned)n_blocks, (unsigned)H);
+  const float scale_log2e = scale * 1.4426950408889634f;
+  attn_blocksparse_kernel<<<grid, kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
+      (int)S, n_blocks, block_row_ptr, block_col_idx, static_cast<const __bf16 *>(Q),
+      static_cast<const __bf16 *>(K), static_cast<const __bf16 *>(V), scale_log2e,
+      static_cast<__bf16 *>(O));
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}

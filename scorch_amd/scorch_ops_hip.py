@@ -269,3 +269,30 @@ def csr_row_indices(row_ptr: torch.Tensor, nnz: int) -> torch.Tensor:
                                                      rows.data_ptr(), _stream(dev))
     native.check(rc)
     return rows
+
+
+def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,
+                          block_col_idx: torch.Tensor, scale: float, block: int = 64) -> torch.Tensor:
+    """softmax(scale * q k^T over a block mask) v for q, k, v of shape (H, S, D),
+    bf16, in one kernel; fp32 accumulation, bf16 result.  The fused form of the
+    per-head SDDMM -> softmax -> SpMM pipeline of
+    bench/bench_sparse_transformer.py:354-372."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dtype != torch.bfloat16 or t.dim() != 3:
+            raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
+    if q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
+    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+    brp, bci = _index(block_row_ptr, "block_row_ptr"), _index(block_col_idx, "block_col_idx")
+    dev = _device_of(q, k, v, brp, bci)
+    H, S, D = q.shape
+    if brp.numel() != S // block + 1:
+        raise ValueError("scorch_ops_hip: block_row_ptr length does not match S / block")
+    out = torch.empty_like(q)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),
+                                                           bci.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                                           v.data_ptr(), float(scale), out.data_ptr(),
+                                                           _stream(dev))
+    native.check(rc)
+    return out

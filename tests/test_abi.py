@@ -121,3 +121,21 @@ def test_check_raises_with_the_library_message(L):
     with pytest.raises(native.ScorchHipError) as info:
         native.check(code)
     assert info.value.code == native.EINVAL and "M=-3" in str(info.value)
+
+
+def test_attention_rejects_unsupported_shapes(L):
+    f = L.scorch_hip_attn_blocksparse_bf16
+    ok_args = dict(H=2, S=128, D=64, block=64, nblk=3)
+
+    def call(H=2, S=128, D=64, block=64, nblk=3, brp=FAKE, bci=FAKE, q=FAKE, k=FAKE, v=FAKE, o=FAKE):
+        return f(H, S, D, block, nblk, brp, bci, q, k, v, 0.125, o, NULL)
+
+    assert call(D=128) == native.EUNSUPPORTED
+    assert b"head dimension" in L.scorch_hip_last_error()
+    assert call(block=32) == native.EUNSUPPORTED
+    assert call(S=100) == native.EINVAL
+    assert call(H=-1) == native.EINVAL
+    assert call(brp=NULL) == native.EINVAL
+    assert call(q=NULL) == native.EINVAL
+    assert call(o=ctypes.c_void_p(0x1008)) == native.EINVAL      # not 16-byte aligned
+    assert call(H=0, q=NULL, k=NULL, v=NULL, o=NULL) == native.OK

@@ -1,0 +1,118 @@
+"""Fused block-sparse attention (bf16 in/out, fp32 accumulation) on the MI355X
+through the C ABI.
+
+Tolerance: relative Frobenius error <= 1e-2 against an fp64 recomputation on
+the same (bf16-representable) inputs -- the bar for the bf16 path.  The
+reference has no bf16 or fused kernel, so nothing of its own pins this path:
+the oracle here is the textbook masked softmax (the reference's "dense" mode,
+bench/bench_sparse_transformer.py:330-335) in float64, and, as a second
+witness, this package's own fp32 SDDMM -> softmax -> SpMM pipeline.
+"""
+import numpy as np
+import pytest
+import torch
+
+import scorch_amd as scorch
+from gpu_util import dev, host
+from scorch_amd import STensor, workloads
+from scorch_amd import scorch_ops_hip as H
+
+pytestmark = pytest.mark.gpu
+TOL_BF16 = 1e-2
+
+
+def bf16_inputs(S, heads, D, seed, window=4, stride=8):
+    w = workloads.attention_blocksparse(S=S, H=heads, D=D, seed=seed, window=window, stride=stride)
+    q, k, v = (torch.from_numpy(w[n]).to(torch.bfloat16) for n in ("q", "k", "v"))
+    return w, q, k, v
+
+
+def run_fused(w, q, k, v):
+    out = H.attn_blocksparse_bf16(q.cuda(), k.cuda(), v.cuda(), dev(w["block_row_ptr"]),
+                                  dev(w["block_col_idx"]), float(w["scale"]))
+    assert out.dtype == torch.bfloat16 and out.shape == q.shape
+    return out
+
+
+@pytest.mark.parametrize("S,heads,seed", [(64, 1, 0), (256, 2, 1), (1024, 3, 2)])
+def test_against_fp64_oracle(oracle, S, heads, seed):
+    w, q, k, v = bf16_inputs(S, heads, 64, seed)
+    out = run_fused(w, q, k, v).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            w["block_row_ptr"], w["block_col_idx"], 64, float(w["scale"]))
+    assert oracle.rel_fro(out, ref) <= TOL_BF16
+    # well inside the bar: bf16 rounding of P and of the output is ~2^-9
+    assert oracle.rel_fro(out, ref) <= 5e-3
+
+
+def test_arbitrary_block_pattern_with_empty_block_rows(oracle):
+    S, nb = 512, 8
+    rng = np.random.default_rng(3)
+    active = rng.random((nb, nb)) < 0.4
+    active[2, :] = False                      # a block row with nothing to attend to
+    active[5, :] = True                       # a full block row
+    r, c = np.nonzero(active)
+    brp = np.concatenate([[0], np.cumsum(np.bincount(r, minlength=nb))]).astype(np.int32)
+    bci = c.astype(np.int32)
+    q, k, v = (torch.from_numpy(rng.standard_normal((2, S, 64)).astype(np.float32)).to(torch.bfloat16)
+               for _ in range(3))
+    out = H.attn_blocksparse_bf16(q.cuda(), k.cuda(), v.cuda(), dev(brp), dev(bci), 0.125)
+    out = out.float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            brp, bci, 64, 0.125)
+    assert not out[:, 128:192].any()          # queries of block row 2
+    assert oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+def test_large_scores_do_not_overflow(oracle):
+    w, q, k, v = bf16_inputs(256, 1, 64, 4)
+    out = H.attn_blocksparse_bf16((q * 8).cuda(), (k * 8).cuda(), v.cuda(), dev(w["block_row_ptr"]),
+                                  dev(w["block_col_idx"]), 1.0).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64((q * 8).float().numpy(), (k * 8).float().numpy(),
+                                            v.float().numpy(), w["block_row_ptr"], w["block_col_idx"],
+                                            64, 1.0)
+    assert np.isfinite(out).all() and oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+def test_matches_unfused_fp32_pipeline():
+    """Same inputs through SDDMM -> CSR softmax -> SpMM in fp32 (one head)."""
+    w, q, k, v = bf16_inputs(1024, 1, 64, 5)
+    fused = run_fused(w, q, k, v).float()[0]
+    rp, ci = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], 64)
+    S = 1024
+    mask = STensor.from_csr_arrays(dev(rp), dev(ci), torch.ones(ci.size, device="cuda"), (S, S))
+    scores = scorch.einsum("ij,ik,jk->ij", mask, q[0].float().cuda(), k[0].float().cuda())
+    probs = H.softmax_csr_float(dev(rp), scores.values, float(w["scale"]))
+    unfused = scorch.matmul(STensor.from_csr_arrays(dev(rp), dev(ci), probs, (S, S)), v[0].float().cuda())
+    err = (torch.linalg.norm(fused - unfused) / torch.linalg.norm(unfused)).item()
+    assert err <= TOL_BF16
+
+
+def test_runs_are_bit_reproducible():
+    w, q, k, v = bf16_inputs(2048, 4, 64, 6)
+    a = run_fused(w, q, k, v)
+    b = run_fused(w, q, k, v)
+    assert torch.equal(a, b)
+
+
+def test_full_size_workload():
+    """S = 8192, 16 heads, D = 64, 64 x 64 blocks (window 4 + every 8th): each
+    head against the masked dense softmax in fp64 on the device."""
+    w, q, k, v = bf16_inputs(8192, 16, 64, workloads.SEEDS["attention_blocksparse"])
+    assert w["block_col_idx"].size == 1466
+    out = run_fused(w, q, k, v)
+    nb = 128
+    blocks = torch.zeros(nb, nb, dtype=torch.bool)
+    rows = np.repeat(np.arange(nb), np.diff(w["block_row_ptr"]))
+    blocks[torch.from_numpy(rows), torch.from_numpy(w["block_col_idx"]).long()] = True
+    mask = blocks.cuda().repeat_interleave(64, 0).repeat_interleave(64, 1)
+    worst = 0.0
+    for h in range(16):
+        q64, k64, v64 = (t[h].cuda().double() for t in (q, k, v))
+        s = (q64 @ k64.T) * float(w["scale"])
+        s.masked_fill_(~mask, float("-inf"))
+        ref = torch.softmax(s, dim=-1) @ v64
+        err = (torch.linalg.norm(out[h].double() - ref) / torch.linalg.norm(ref)).item()
+        worst = max(worst, err)
+        del s, ref
+    assert worst <= TOL_BF16, worst
