@@ -16,6 +16,9 @@ import sys
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libscorch_hip.so")
+# memory-system probes for bench.py --probe; not part of the product library
+PROBES_SRC = os.path.join(SRC_DIR, "probes", "membench.hip")
+PROBES_PATH = os.path.join(PKG_DIR, "libscorch_probes.so")
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
@@ -38,16 +41,12 @@ def _stale() -> bool:
     return any(os.path.getmtime(d) > built for d in deps)
 
 
-def build_library(force: bool = False, verbose: bool = False) -> str:
-    """Build libscorch_hip.so if it is missing or older than its sources
-    (always when ``force``).  Returns the library path."""
-    if not force and not _stale():
-        return LIB_PATH
+def _hipcc(srcs, out, verbose):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
-        raise RuntimeError("hipcc not found: cannot build libscorch_hip.so")
-    tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc] + HIPCC_FLAGS + sources() + ["-o", tmp]
+        raise RuntimeError(f"hipcc not found: cannot build {os.path.basename(out)}")
+    tmp = out + ".tmp"
+    cmd = [hipcc] + HIPCC_FLAGS + list(srcs) + ["-o", tmp]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -57,10 +56,26 @@ def build_library(force: bool = False, verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed:\n" + "\n".join(noise))
     if verbose and noise:
         print("\n".join(noise))
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, out)
+    return out
+
+
+def build_library(force: bool = False, verbose: bool = False) -> str:
+    """Build libscorch_hip.so if it is missing or older than its sources
+    (always when ``force``).  Returns the library path."""
+    if not force and not _stale():
+        return LIB_PATH
+    return _hipcc(sources(), LIB_PATH, verbose)
+
+
+def build_probes(force: bool = False, verbose: bool = False) -> str:
+    """Build libscorch_probes.so (bench.py --probe) if missing, stale or forced."""
+    if not force and os.path.exists(PROBES_PATH) \
+            and os.path.getmtime(PROBES_PATH) >= os.path.getmtime(PROBES_SRC):
+        return PROBES_PATH
+    return _hipcc([PROBES_SRC], PROBES_PATH, verbose)
 
 
 if __name__ == "__main__":
-    path = build_library(force="--force" in sys.argv, verbose=True)
-    print(path)
+    print(build_library(force="--force" in sys.argv, verbose=True))
+    print(build_probes(force="--force" in sys.argv, verbose=True))
