@@ -82,6 +82,17 @@ __device__ __forceinline__ int wave_lane() { return threadIdx.x & (kWaveSize - 1
 // wave-uniform so that addresses built from it use scalar arithmetic.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Orders LDS traffic inside one wavefront: writes by any lane before this point
+// are seen by reads of any lane after it.  Enough when the LDS region is
+// private to the wavefront (the hardware runs one wavefront's LDS instructions
+// in order; this keeps the compiler from moving them), and it does not couple
+// the wavefronts of a workgroup the way __syncthreads() does.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Wave-cooperative search: number of i in [0, n) with key(i) < bound, for a
 // strictly increasing key.  Each step probes 64 evenly spaced positions, so a
 // million-entry array takes four dependent loads instead of twenty.

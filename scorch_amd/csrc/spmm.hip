@@ -48,7 +48,7 @@ template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
-    const T *__restrict__ bias, int64_t total_items, int items_per_wave,
+    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int chunks_per_wave,
     int *__restrict__ carry_row, T *__restrict__ carry_val) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
@@ -59,106 +59,119 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int64_t chunk = (int64_t)blockIdx.x * kWavesPerBlock + w;
+  const int64_t span = (int64_t)blockIdx.x * kWavesPerBlock + w;  // this wavefront's share
   const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
   const bool active = col0 < N;
 
-  // Chunk [d0, d1) of the merged sequence; chunks past the end are empty.
-  int64_t d0 = chunk * items_per_wave;
-  d0 = d0 < total_items ? d0 : total_items;
-  int64_t d1 = d0 + items_per_wave;
-  d1 = d1 < total_items ? d1 : total_items;
+  // The wavefront owns chunks_per_wave consecutive chunks of the merged
+  // sequence, [span_d0, span_d1); spans past the end are empty.
+  const int64_t span_items = (int64_t)items_per_chunk * chunks_per_wave;
+  int64_t span_d0 = span * span_items;
+  span_d0 = span_d0 < total_items ? span_d0 : total_items;
+  int64_t span_d1 = span_d0 + span_items;
+  span_d1 = span_d1 < total_items ? span_d1 : total_items;
 
   auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
-  const int x0 = wave_count_below(M, d0, row_end_key);  // rows finished before the chunk
-  const int x1 = wave_count_below(M, d1, row_end_key);  // rows finished by its end
-  const int y0 = uniform((int)(d0 - x0));               // first nonzero of the chunk
-  const int y1 = uniform((int)(d1 - x1));
-  const int n_nz = y1 - y0;
-  const int n_rows = x1 - x0;
-
-  // Stage the chunk's slice of A in LDS: coalesced loads now, broadcast reads later.
-  for (int k = lane; k < n_nz; k += kWaveSize) {
-    s_col[w][k] = col_idx[y0 + k];
-    s_val[w][k] = vals[y0 + k];
-  }
-  // s_rp[k] = row_ptr[x0 + k] for k = 0 .. n_rows + 1 (clamped at M).
-  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
-    const int r = x0 + k < M ? x0 + k : M;
-    s_rp[w][k] = row_ptr[r];
-  }
-  __syncthreads();
+  const int span_x0 = wave_count_below(M, span_d0, row_end_key);  // rows finished before the span
+  const int span_y0 = uniform((int)(span_d0 - span_x0));          // its first nonzero
+  // Row span_x0 began in an earlier span iff its first nonzero precedes
+  // span_y0: then its store is a partial sum and its epilogue is the fix-up's.
+  const bool carry_in = uniform(row_ptr[span_x0 < M ? span_x0 : M]) < span_y0;
 
   T bias_v[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) bias_v[v] = (EPI != kEpiNone && active) ? bias[col0 + v] : (T)0;
 
-  A acc[VEC];
+  A acc[VEC];  // carried in registers from chunk to chunk
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
 
-  // Row x0 began in an earlier chunk iff its first nonzero precedes y0: then
-  // its store is a partial sum and its epilogue is left to the fix-up.
-  const bool carry_in = uniform(s_rp[w][0]) < y0;
+  int x = span_x0;        // next row to finish
+  int y = span_y0;        // next nonzero to consume
+  int last_row_start = 0; // row_ptr[x] after the last chunk
 
-  int x = x0;
-  int next_end = uniform(s_rp[w][1]);
+  for (int sub = 0; sub < chunks_per_wave; ++sub) {
+    int64_t d1 = span_d0 + (int64_t)(sub + 1) * items_per_chunk;
+    d1 = d1 < span_d1 ? d1 : span_d1;
+    // The chunk starts where the walk stands, (x, y); only its end needs a search.
+    const int x0 = x, y0 = y;
+    const int x1 = wave_count_below(M, d1, row_end_key);  // rows finished by the chunk's end
+    const int y1 = uniform((int)(d1 - x1));
+    const int n_nz = y1 - y0;
+    const int n_rows = x1 - x0;
 
-  auto flush_row = [&]() {
-    if (active) {
-      const bool partial = carry_in && x == x0;
-      VecT o;
-#pragma unroll
-      for (int v = 0; v < VEC; ++v)
-        o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
-      *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
+    // Stage the chunk's slice of A in LDS: coalesced loads now, broadcast reads later.
+    for (int k = lane; k < n_nz; k += kWaveSize) {
+      s_col[w][k] = col_idx[y0 + k];
+      s_val[w][k] = vals[y0 + k];
     }
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
-    ++x;
-    next_end = uniform(s_rp[w][x - x0 + 1]);
-  };
-
-  auto gather = [&](int k) -> VecT {
-    const int j = uniform(s_col[w][k]);
-    VecT b;
-    if (active) {
-      b = *reinterpret_cast<const VecT *>(B + (size_t)j * (size_t)N + col0);
-    } else {
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) b.v[v] = (T)0;
+    // s_rp[k] = row_ptr[x0 + k] for k = 0 .. n_rows + 1 (clamped at M).
+    for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
+      const int r = x0 + k < M ? x0 + k : M;
+      s_rp[w][k] = row_ptr[r];
     }
-    return b;
-  };
+    wave_lds_sync();  // the slices are private to this wavefront
 
-  auto consume = [&](int k, const VecT &b) {
-    while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
-    const A a = (A)s_val[w][k];
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
-  };
+    int next_end = uniform(s_rp[w][1]);
 
-  int k = 0;
-  for (; k + kGather <= n_nz; k += kGather) {
-    VecT b[kGather];
+    auto flush_row = [&]() {
+      if (active) {
+        const bool partial = carry_in && x == span_x0;
+        VecT o;
 #pragma unroll
-    for (int u = 0; u < kGather; ++u) b[u] = gather(k + u);
+        for (int v = 0; v < VEC; ++v)
+          o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
+        *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
+      }
 #pragma unroll
-    for (int u = 0; u < kGather; ++u) consume(k + u, b[u]);
+      for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+      ++x;
+      next_end = uniform(s_rp[w][x - x0 + 1]);
+    };
+
+    auto gather = [&](int k) -> VecT {
+      const int j = uniform(s_col[w][k]);
+      VecT b;
+      if (active) {
+        b = *reinterpret_cast<const VecT *>(B + (size_t)j * (size_t)N + col0);
+      } else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) b.v[v] = (T)0;
+      }
+      return b;
+    };
+
+    auto consume = [&](int k, const VecT &b) {
+      while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
+      const A a = (A)s_val[w][k];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
+    };
+
+    int k = 0;
+    for (; k + kGather <= n_nz; k += kGather) {
+      VecT b[kGather];
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) b[u] = gather(k + u);
+#pragma unroll
+      for (int u = 0; u < kGather; ++u) consume(k + u, b[u]);
+    }
+    for (; k < n_nz; ++k) consume(k, gather(k));
+    while (x < x1) flush_row();  // markers after the chunk's last nonzero
+    y = y1;
+    last_row_start = uniform(s_rp[w][n_rows]);  // row_ptr[x1]
+    wave_lds_sync();  // the LDS slices are rewritten by the next chunk
   }
-  for (; k < n_nz; ++k) consume(k, gather(k));
-  while (x < x1) flush_row();  // markers after the chunk's last nonzero
 
-  // Whatever is left belongs to row x1, whose marker lies in a later chunk.
-  if (chunk * items_per_wave < total_items) {
-    const int row_start = uniform(s_rp[w][n_rows]);
-    const int tail = y1 - (row_start > y0 ? row_start : y0);
-    if (blockIdx.y == 0 && lane == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
+  // Whatever is left belongs to row x, whose marker lies in a later span.
+  if (span * span_items < total_items) {
+    const int tail = y - (last_row_start > span_y0 ? last_row_start : span_y0);
+    if (blockIdx.y == 0 && lane == 0) carry_row[span] = tail > 0 ? x : -1;
     if (tail > 0 && active) {
       VecT o;
 #pragma unroll
       for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];
-      *reinterpret_cast<VecT *>(carry_val + (size_t)chunk * (size_t)N + col0) = o;
+      *reinterpret_cast<VecT *>(carry_val + (size_t)span * (size_t)N + col0) = o;
     }
   }
 }
@@ -174,21 +187,32 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
   const int lane = wave_lane();
   const int64_t chunk = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
   if (chunk >= num_chunks) return;
-  const int row = uniform(carry_row[chunk]);
+  // One coalesced load answers three questions: lane 0 holds the previous
+  // chunk's carry row, lane 1 this chunk's, lanes 2.. the following ones.
+  const int64_t first_probe = chunk - 1 + lane;
+  const int seen = (first_probe >= 0 && first_probe < num_chunks) ? carry_row[first_probe] : -2;
+  const int row = __builtin_amdgcn_readlane(seen, 1);
   if (row < 0) return;
-  if (chunk > 0 && uniform(carry_row[chunk - 1]) == row) return;  // not the head of its run
-  // End of the run: 64 entries of carry_row are compared per step.
-  int64_t end = chunk + 1;
-  for (;;) {
-    const int64_t probe = end + lane;
-    const bool same = probe < num_chunks && carry_row[probe] == row;
-    const unsigned long long differs = ~__ballot(same);
-    const int matched = differs ? __ffsll(differs) - 1 : kWaveSize;
-    end += matched;
-    if (matched < kWaveSize) break;
+  if (__builtin_amdgcn_readlane(seen, 0) == row) return;  // not the head of its run
+  // End of the run: 62 entries are already here, then 64 per step.
+  const unsigned long long differs = ~(__ballot(lane >= 2 && seen == row) | 3ull);
+  const int matched = differs ? __ffsll(differs) - 3 : kWaveSize - 2;
+  int64_t end = chunk + 1 + matched;
+  if (matched == kWaveSize - 2) {
+    for (;;) {
+      const int64_t probe = end + lane;
+      const bool same = probe < num_chunks && carry_row[probe] == row;
+      const unsigned long long differs_here = ~__ballot(same);
+      const int run = differs_here ? __ffsll(differs_here) - 1 : kWaveSize;
+      end += run;
+      if (run < kWaveSize) break;
+    }
   }
   const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
   if (col0 >= N) return;
+
+  VecT *dst = reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0);
+  VecT o = *dst;  // issued before the carries so that both are in flight together
 
   A sum[VEC];
 #pragma unroll
@@ -211,8 +235,6 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
     for (int v = 0; v < VEC; ++v) sum[v] += (A)part.v[v];
   }
 
-  VecT *dst = reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0);
-  VecT o = *dst;
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
     const T b = EPI != kEpiNone ? bias[col0 + v] : (T)0;
@@ -223,20 +245,39 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
 
 // ---- host side ----------------------------------------------------------------
 
-// Items per wavefront: the full 256 when that still yields enough wavefronts to
-// fill the chip (256 CUs x 32 wavefronts), otherwise a smaller power of two so
-// that a small problem is spread over more, shorter wavefronts.
-inline int spmm_items_per_wave(int64_t M, int64_t nnz) {
-  const int64_t per_wave = (M + nnz) / 8192;
-  int ipw = kMinItemsPerWave;
-  while (ipw < kItemsPerWave && ipw * 2 <= per_wave) ipw *= 2;
-  return ipw;
+// Shape of the work split.  A chunk holds up to 256 merge items (what the LDS
+// slices hold); a wavefront walks chunks_per_wave consecutive chunks and leaves
+// one carry.  Small problems use smaller chunks, one per wavefront, so that
+// they are spread over more, shorter wavefronts; large ones use several chunks
+// per wavefront, which divides the number of carries the fix-up must fold.
+struct SpmmSplit {
+  int items_per_chunk;
+  int chunks_per_wave;
+  int64_t spans;  // wavefronts with work = carry records
+};
+
+inline SpmmSplit spmm_split(int64_t M, int64_t nnz) {
+  const int64_t total = M + nnz;
+  SpmmSplit sp;
+  const int64_t per_wave = total / 8192;  // 256 CUs x 32 wavefronts
+  sp.items_per_chunk = kMinItemsPerWave;
+  while (sp.items_per_chunk < kItemsPerWave && sp.items_per_chunk * 2 <= per_wave)
+    sp.items_per_chunk *= 2;
+  sp.chunks_per_wave = 1;
+  if (sp.items_per_chunk == kItemsPerWave) {
+    const int64_t chunks_per_slot = per_wave / kItemsPerWave;  // chunks per resident wavefront
+    // Keep at least four rounds of wavefronts so that the last, partly filled
+    // round stays a small share of the run (measured: 2-3 chunks per wavefront
+    // are as fast as 1 at 18 M items and halve the carries; 8 cost 4 %).
+    const int cpw = (int)(chunks_per_slot / 4);
+    sp.chunks_per_wave = cpw < 1 ? 1 : (cpw > 4 ? 4 : cpw);
+  }
+  const int64_t span_items = (int64_t)sp.items_per_chunk * sp.chunks_per_wave;
+  sp.spans = (total + span_items - 1) / span_items;
+  return sp;
 }
 
-inline int64_t spmm_num_chunks(int64_t M, int64_t nnz) {
-  const int ipw = spmm_items_per_wave(M, nnz);
-  return (M + nnz + ipw - 1) / ipw;
-}
+inline int64_t spmm_num_chunks(int64_t M, int64_t nnz) { return spmm_split(M, nnz).spans; }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -265,7 +306,8 @@ template <typename T, int VEC, int EPI>
 int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
                 const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
                 KernelTimer *timer) {
-  const int64_t chunks = spmm_num_chunks(M, nnz);
+  const SpmmSplit split = spmm_split(M, nnz);
+  const int64_t chunks = split.spans;
   int *carry_row = static_cast<int *>(workspace);
   T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
                                        align_up((size_t)chunks * sizeof(int), 256));
@@ -274,8 +316,8 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
                   (unsigned)((N + tile - 1) / tile));
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
-      M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, spmm_items_per_wave(M, nnz),
-      carry_row, carry_val);
+      M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
+      split.chunks_per_wave, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
   spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(N, chunks, carry_row,
