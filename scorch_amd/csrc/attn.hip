@@ -10,10 +10,12 @@
 // Work split.  One workgroup (4 wavefronts) owns one head and one block row of
 // the mask, i.e. 64 queries; each wavefront owns 16 of them.  The workgroup
 // walks the block row's active key blocks.  For each, the 64 x 64 K tile and
-// the 64 x 64 V tile are staged in LDS once for all four wavefronts (V is
-// stored transposed so that eight consecutive keys of one feature are
-// contiguous); the next tile's global loads are in flight while the current
-// one is consumed (two LDS buffers, one barrier per key block).
+// the 64 x 64 V tile are staged in LDS once for all four wavefronts, both
+// row-major; the next tile's global loads are in flight while the current one
+// is consumed (two LDS buffers, one barrier per key block).  The second
+// product needs V by columns (eight keys of one feature per lane): that
+// operand is read with ds_read_b64_tr_b16, which hands each lane of a 16-lane
+// group one column of a 4 x 16 block whose rows the group's lanes address.
 //
 // Per wavefront and key block, everything stays in registers:
 //   S^T = K Q^T        (keys x queries: 4 tiles of 16 keys, contraction over D)
@@ -36,22 +38,41 @@ constexpr int kLdsRow = 72;     // LDS row length in bf16 (64 + 8 padding agains
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef short4v __attribute__((address_space(3))) lds_short4v;
 
 __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
-    int S, int n_blocks, const int *__restrict__ block_row_ptr,
+    int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
     const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O) {
   __shared__ __attribute__((aligned(16))) __bf16 s_k[2][kAttnBlock][kLdsRow];   // [key][feature]
-  __shared__ __attribute__((aligned(16))) __bf16 s_vt[2][kAttnDim][kLdsRow];    // [feature][key]
+  __shared__ __attribute__((aligned(16))) __bf16 s_v[2][kAttnBlock][kLdsRow];   // [key][feature]
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int w = tid / kWaveSize;
   const int g = lane >> 4;  // 16-lane group: which keys / features of a tile this lane holds
   const int n = lane & 15;  // query within the wavefront's 16
-  const int head = blockIdx.y;
-  const int qb = n_blocks - 1 - (int)blockIdx.x;  // longest block rows first
+  // Workgroup -> (head, block row).  Workgroups are dealt to the 8 XCDs round
+  // robin by their linear id, and every XCD has its own 4 MB L2.  When the head
+  // count allows it, all workgroups of a head are given ids of one residue mod
+  // 8, so that a head's K and V (2 * S * 128 bytes) are fetched into one L2 only
+  // and an XCD works through its heads one after the other.
+  int head, rank;
+  {
+    const int id = blockIdx.x;
+    if (n_heads % 8 == 0) {
+      const int xcd = id & 7, slot = id >> 3;
+      head = xcd + 8 * (slot / n_blocks);
+      rank = slot % n_blocks;
+    } else {
+      head = id / n_blocks;
+      rank = id % n_blocks;
+    }
+  }
+  const int qb = n_blocks - 1 - rank;  // longest block rows first
   const size_t head_off = (size_t)head * (size_t)S * kAttnDim;
   const __bf16 *Qh = Q + head_off, *Kh = K + head_off, *Vh = V + head_off;
 
@@ -90,8 +111,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
       const int c = tid + u * kBlockThreads;
       const int key = c >> 3, f0 = (c & 7) * 8;
       *reinterpret_cast<bf16x8 *>(&s_k[buf][key][f0]) = k_stage[u];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s_vt[buf][f0 + e][key] = v_stage[u][e];
+      *reinterpret_cast<bf16x8 *>(&s_v[buf][key][f0]) = v_stage[u];
     }
   };
 
@@ -130,7 +150,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = exp2f(m_run - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     m_run = m_new;
     l_run *= alpha;
 #pragma unroll
@@ -145,20 +165,28 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = exp2f(st[t][r] - m_new);
+        const float p = __builtin_amdgcn_exp2f(st[t][r] - m_new);
         l_run += p;
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
 
-    // O^T tile dt: features 16dt .. 16dt+15 (rows) x 16 queries, contraction over the 64 keys.
+    // O^T tile dt: features 16dt .. 16dt+15 (rows) x 16 queries, contraction over
+    // the 64 keys.  A operand: lane (g, n) needs V[key][16dt + n] for the eight
+    // keys of its slots.  One transposing read covers four consecutive keys:
+    // lane i of the group addresses row key0 + i / 4, features 16dt + 4 (i % 4) .. + 3,
+    // and receives V[key0 .. key0 + 3][16dt + i].
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const __bf16 *row = &s_vt[buf][16 * dt + n][32 * s + 4 * g];
-        const bf16x4 lo = *reinterpret_cast<const bf16x4 *>(row);
-        const bf16x4 hi = *reinterpret_cast<const bf16x4 *>(row + 16);
-        const bf16x8 v_op = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const int key0 = 32 * s + 4 * g + (n >> 2);
+        const int f0 = 16 * dt + 4 * (n & 3);
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4v *)&s_v[buf][key0][f0]);
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4v *)&s_v[buf][key0 + 16][f0]);
+        const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const bf16x8 v_op = __builtin_bit_cast(bf16x8, packed);
         o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
       }
 
@@ -200,7 +228,7 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
                 (long long)block);
   if (S % kAttnBlock != 0)
     return fail(SCORCH_HIP_EINVAL, "%s: S=%lld is not a multiple of the block size", fn, (long long)S);
-  if (H > 65535 || S / kAttnBlock > INT32_MAX || S * D > INT32_MAX)
+  if (H * (S / kAttnBlock) > INT32_MAX || S * D > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "%s: H=%lld or S=%lld too large", fn, (long long)H, (long long)S);
   SCORCH_REQUIRE(block_row_ptr != nullptr, "%s: block_row_ptr is NULL", fn);
   if (H == 0 || S == 0) return SCORCH_HIP_OK;
@@ -209,10 +237,10 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
   SCORCH_REQUIRE(aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16),
                  "%s: Q, K, V and O must be 16-byte aligned", fn);
   const int n_blocks = (int)(S / kAttnBlock);
-  const dim3 grid((unsigned)n_blocks, (unsigned)H);
+  const dim3 grid((unsigned)(n_blocks * H));
   const float scale_log2e = scale * 1.4426950408889634f;
   attn_blocksparse_kernel<<<grid, kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
-      (int)S, n_blocks, block_row_ptr, block_col_idx, static_cast<const __bf16 *>(Q),
+      (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, static_cast<const __bf16 *>(Q),
       static_cast<const __bf16 *>(K), static_cast<const __bf16 *>(V), scale_log2e,
       static_cast<__bf16 *>(O));
   SCORCH_HIP_CHECK(hipGetLastError());
