@@ -24,8 +24,9 @@
 // atomics.  A fused bias/ReLU epilogue is applied at the store when the row
 // lies wholly inside the chunk, and by the fix-up otherwise.
 //
-// Columns beyond 64 * VEC are covered by blockIdx.y (each column tile walks
-// the same chunk again; A's indices are small next to the B rows gathered).
+// Columns beyond 64 * VEC are covered by column tiles (each tile walks the same
+// chunks again; A's indices are small next to the B rows gathered).  Tiles are
+// placed on XCDs so that a tile's slice of B stays in one L2 (map_workgroup).
 #include "common.hpp"
 
 namespace scorch {
@@ -35,6 +36,31 @@ constexpr int kMinItemsPerWave = 32;
 constexpr int kGather = 8;          // B-row loads in flight per wavefront
 
 enum Epilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasRelu = 2 };
+
+// Workgroup id -> (column tile, block of wavefront spans).  Workgroups are dealt
+// to the 8 XCDs round robin by their linear id, and every XCD has its own L2.
+// With a multiple of 8 column tiles, tile t is given to XCD t % 8 and each XCD
+// works through its tiles one after the other: the B rows a tile gathers
+// (K rows of 64 * VEC elements) are then fetched into one L2 only and stay
+// there while the tile is processed.
+struct TileMap {
+  int tile;
+  int64_t block;
+};
+
+__device__ __forceinline__ TileMap map_workgroup(int64_t id, int n_tiles, int64_t blocks_per_tile) {
+  TileMap m;
+  if (n_tiles > 1 && (n_tiles & 7) == 0) {
+    const int xcd = (int)(id & 7);
+    const int64_t slot = id >> 3;
+    m.tile = xcd + 8 * (int)(slot / blocks_per_tile);
+    m.block = slot % blocks_per_tile;
+  } else {
+    m.tile = (int)(id / blocks_per_tile);
+    m.block = id % blocks_per_tile;
+  }
+  return m;
+}
 
 template <typename T, int EPI>
 __device__ __forceinline__ T apply_epilogue(typename Acc<T>::type acc, T bias) {
@@ -49,7 +75,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int chunks_per_wave,
-    int *__restrict__ carry_row, T *__restrict__ carry_val) {
+    int n_tiles, int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
 
@@ -59,8 +85,9 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int64_t span = (int64_t)blockIdx.x * kWavesPerBlock + w;  // this wavefront's share
-  const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
+  const TileMap where = map_workgroup(blockIdx.x, n_tiles, blocks_per_tile);
+  const int64_t span = where.block * kWavesPerBlock + w;  // this wavefront's share
+  const int col0 = (where.tile * kWaveSize + lane) * VEC;
   const bool active = col0 < N;
 
   // The wavefront owns chunks_per_wave consecutive chunks of the merged
@@ -166,7 +193,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
   // Whatever is left belongs to row x, whose marker lies in a later span.
   if (span * span_items < total_items) {
     const int tail = y - (last_row_start > span_y0 ? last_row_start : span_y0);
-    if (blockIdx.y == 0 && lane == 0) carry_row[span] = tail > 0 ? x : -1;
+    if (where.tile == 0 && lane == 0) carry_row[span] = tail > 0 ? x : -1;
     if (tail > 0 && active) {
       VecT o;
 #pragma unroll
@@ -180,12 +207,14 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 // equal carry_row values sums the run in chunk order and folds it into C.
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
-    int N, int64_t num_chunks, const int *__restrict__ carry_row,
-    const T *__restrict__ carry_val, T *__restrict__ C, const T *__restrict__ bias) {
+    int N, int64_t num_chunks, int n_tiles, int64_t blocks_per_tile,
+    const int *__restrict__ carry_row, const T *__restrict__ carry_val, T *__restrict__ C,
+    const T *__restrict__ bias) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   const int lane = wave_lane();
-  const int64_t chunk = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  const TileMap where = map_workgroup(blockIdx.x, n_tiles, blocks_per_tile);
+  const int64_t chunk = where.block * kWavesPerBlock + threadIdx.x / kWaveSize;
   if (chunk >= num_chunks) return;
   // One coalesced load answers three questions: lane 0 holds the previous
   // chunk's carry row, lane 1 this chunk's, lanes 2.. the following ones.
@@ -208,7 +237,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
       if (run < kWaveSize) break;
     }
   }
-  const int col0 = ((int)blockIdx.y * kWaveSize + lane) * VEC;
+  const int col0 = (where.tile * kWaveSize + lane) * VEC;
   if (col0 >= N) return;
 
   VecT *dst = reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0);
@@ -256,10 +285,12 @@ struct SpmmSplit {
   int64_t spans;  // wavefronts with work = carry records
 };
 
-inline SpmmSplit spmm_split(int64_t M, int64_t nnz) {
+inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   const int64_t total = M + nnz;
   SpmmSplit sp;
-  const int64_t per_wave = total / 8192;  // 256 CUs x 32 wavefronts
+  // every column tile (up to 1 KiB of a row) walks all chunks again
+  const int64_t tiles = (N * (int64_t)elem + 1023) / 1024;
+  const int64_t per_wave = total * (tiles > 0 ? tiles : 1) / 8192;  // 256 CUs x 32 wavefronts
   sp.items_per_chunk = kMinItemsPerWave;
   while (sp.items_per_chunk < kItemsPerWave && sp.items_per_chunk * 2 <= per_wave)
     sp.items_per_chunk *= 2;
@@ -277,14 +308,16 @@ inline SpmmSplit spmm_split(int64_t M, int64_t nnz) {
   return sp;
 }
 
-inline int64_t spmm_num_chunks(int64_t M, int64_t nnz) { return spmm_split(M, nnz).spans; }
+inline int64_t spmm_num_chunks(int64_t M, int64_t nnz, int64_t N, size_t elem) {
+  return spmm_split(M, nnz, N, elem).spans;
+}
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Workspace layout: carry_row int32[num_chunks] padded to 256 bytes, then
 // carry_val T[num_chunks * N].
 inline size_t spmm_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
-  const size_t chunks = (size_t)spmm_num_chunks(M, nnz);
+  const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
   return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256);
 }
 
@@ -306,22 +339,26 @@ template <typename T, int VEC, int EPI>
 int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
                 const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
                 KernelTimer *timer) {
-  const SpmmSplit split = spmm_split(M, nnz);
+  const SpmmSplit split = spmm_split(M, nnz, N, sizeof(T));
   const int64_t chunks = split.spans;
   int *carry_row = static_cast<int *>(workspace);
   T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
                                        align_up((size_t)chunks * sizeof(int), 256));
   const int tile = kWaveSize * VEC;
-  const dim3 grid((unsigned)((chunks + kWavesPerBlock - 1) / kWavesPerBlock),
-                  (unsigned)((N + tile - 1) / tile));
+  const int n_tiles = (N + tile - 1) / tile;
+  const int64_t blocks_per_tile = (chunks + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks_per_tile * n_tiles > INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
+                (long long)(blocks_per_tile * n_tiles));
+  const dim3 grid((unsigned)(blocks_per_tile * n_tiles));
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
-      split.chunks_per_wave, carry_row, carry_val);
+      split.chunks_per_wave, n_tiles, blocks_per_tile, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
-  spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(N, chunks, carry_row,
-                                                                    carry_val, C, bias);
+  spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
+      N, chunks, n_tiles, blocks_per_tile, carry_row, carry_val, C, bias);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
   return SCORCH_HIP_OK;
@@ -364,9 +401,6 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
     return fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
                 workspace ? workspace_bytes : (size_t)0);
   SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
-  const int64_t chunks = spmm_num_chunks(M, nnz);
-  if ((chunks + kWavesPerBlock - 1) / kWavesPerBlock > INT32_MAX)
-    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: too many work chunks", fn);
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int vec = pick_vec<T>(N, B, C, workspace);
