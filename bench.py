@@ -26,10 +26,13 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
 WORKLOAD = "gcn_powerlaw_spmm_fp32"
 
-# HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE from
-# rocprofv3 --pmc, scaled by a copy kernel of known size); None until measured
-# for the kernel as it stands.  Summary: profiles/.
-MEASURED_TRAFFIC_BYTES = None
+# Bytes through the L2-to-fabric boundary per launch of the dominant kernel at
+# the headline size: FETCH_SIZE (4,322,622 KiB x 2.0, the factor a 1 GiB copy
+# kernel gives for this counter) + WRITE_SIZE (541,521 KiB x 1.0) from two
+# rocprofv3 --pmc runs of this script.  It is a measured constant, valid for
+# the default workload only; the summary with the commands is
+# profiles/spmm_merge_kernel_gcn_powerlaw.md.
+MEASURED_TRAFFIC_BYTES = 9_407_247_000
 
 
 def algorithmic_bytes(M, K, N, nnz):
@@ -325,7 +328,7 @@ def main() -> int:
             "bound": "hbm", "kernel": "spmm_merge_kernel<float,2,0>",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "traffic": MEASURED_TRAFFIC_BYTES if (M, N) == (1 << 20, 128) else None,
             "algorithmic_bytes": algo, "gather_model_bytes": gather_bytes(M, N, nnz),
             "gather_model_gbps": round(gather_bytes(M, N, nnz) / (merge_avg * 1e-3) / 1e9, 1),
             "kernel_ms_avg": round(merge_avg, 4), "fixup_kernel_ms_avg": round(fixup_avg, 4),
