@@ -156,3 +156,60 @@ def test_unfused_attention_pipeline_matches_dense(oracle):
     dense_mask = np.zeros((S, S), bool)
     dense_mask[oracle.rows_of(rp), ci] = True
     assert oracle.rel_fro(host(out), oracle.attention_dense_fp64(q, k, v, dense_mask, D ** -0.5)) <= TOL
+
+
+# ---- @compile (reference: tests/test_scorch/test_compile.py:70-127) ----------------------------
+def _csr_and_dense_cuda(n=64, k=16, density=0.1, seed=42):
+    torch.manual_seed(seed)
+    vals = torch.rand(n, n) * (torch.rand(n, n) < density).float()
+    return vals, STensor.from_csr(vals.to_sparse_csr(), "A").to("cuda"), torch.rand(n, k)
+
+
+def test_compile_spmm_bias_relu_csr():
+    dense_a, adj, x = _csr_and_dense_cuda()
+    bias = torch.rand(x.size(1))
+
+    @scorch.compile
+    def fused(adj, x, bias):
+        h = scorch.matmul(adj, x, format="dd")
+        h = h + bias
+        return torch.relu(h)
+
+    result = fused(adj, x.cuda(), bias.cuda())
+    assert isinstance(result, torch.Tensor) and result.is_cuda
+    assert torch.allclose(result.cpu(), torch.relu(dense_a @ x + bias), atol=1e-4)
+    assert list(fused._cache.values())[0].fused_symbol == "spmm_csr_bias_relu_float"
+    # second call reuses the trace and the runner
+    again = fused(adj, x.cuda(), bias.cuda())
+    assert torch.equal(result, again) and len(fused._cache) == 1
+
+
+def test_compile_spmm_bias_csr_and_unfused_chain():
+    dense_a, adj, x = _csr_and_dense_cuda(seed=7)
+    bias = torch.rand(x.size(1))
+
+    @scorch.compile
+    def bias_only(adj, x, bias):
+        return scorch.matmul(adj, x, format="dd") + bias
+
+    @scorch.compile
+    def tanh_chain(adj, x, bias):
+        return torch.tanh(scorch.matmul(adj, x, format="dd") * bias)
+
+    out = bias_only(adj, x.cuda(), bias.cuda())
+    assert torch.allclose(out.cpu(), dense_a @ x + bias, atol=1e-4)
+    chained = tanh_chain(adj, x.cuda(), bias.cuda())
+    assert list(tanh_chain._cache.values())[0].fused_symbol is None      # runs matmul + torch ops
+    assert torch.allclose(chained.cpu(), torch.tanh((dense_a @ x) * bias), atol=1e-4)
+
+
+def test_compile_matches_unfused():
+    _, adj, x = _csr_and_dense_cuda(n=300, k=128, seed=9)
+    bias = torch.rand(128).cuda()
+
+    @scorch.compile
+    def fused(adj, x, bias):
+        return torch.relu(scorch.matmul(adj, x, format="dd") + bias)
+
+    unfused = torch.relu(scorch.matmul(adj, x.cuda(), format="dd") + bias)
+    assert torch.allclose(fused(adj, x.cuda(), bias), unfused, atol=1e-5)
