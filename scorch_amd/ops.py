@@ -103,11 +103,13 @@ def matmul(a: Union[torch.Tensor, STensor], b: Union[torch.Tensor, STensor],
             return result
         return STensor.from_torch(result).to_sparse(parse_format(requested))
 
-    default_order = [0, 1]
-    for operand in (a, b):
-        if operand.dim() == 2 and not operand.format.is_dense() \
-                and operand.index.mode_order != default_order:
-            raise _not_prebuilt("matmul with a non-default mode order")
+    # Sparse matrices stored in a non-default mode order are re-stored in the
+    # default one first, as the reference does (ops.py:299-303,333-346).
+    if a.dim() == 2 and b.dim() in (1, 2) and not (a.format.is_dense() and b.format.is_dense()):
+        if a.index.mode_order != [0, 1]:
+            a = a.copy().change_mode_order([0, 1])
+        if b.dim() == 2 and b.index.mode_order != [0, 1]:
+            b = b.copy().change_mode_order([0, 1])
 
     if kwargs.get("use_cache", True):
         result = _run_prebuilt_matmul(a, b, requested, time_dict)

@@ -20,7 +20,23 @@ import torch
 from .format import LevelFormat, LevelType, TensorFormat, parse_format
 from .storage import TensorIndex, TensorStorage
 
-_DENSE2 = "dd"
+
+
+def _sorted_unique_entries(rows: torch.Tensor, cols: torch.Tensor, values: torch.Tensor, n_cols: int):
+    """Entries sorted by (row, col); values of repeated coordinates are summed."""
+    if rows.numel() == 0:
+        return rows, cols, values
+    key = rows * int(n_cols) + cols
+    key, order = torch.sort(key, stable=True)
+    values = values[order]
+    first = torch.ones_like(key, dtype=torch.bool)
+    first[1:] = key[1:] != key[:-1]
+    if not bool(first.all()):
+        segment = torch.cumsum(first.to(torch.int64), dim=0) - 1
+        summed = torch.zeros(int(segment[-1]) + 1, dtype=values.dtype, device=values.device)
+        summed.index_add_(0, segment, values)
+        key, values = key[first], summed
+    return key // int(n_cols), key % int(n_cols), values
 
 
 class STensor(torch.nn.Module):
@@ -211,6 +227,56 @@ class STensor(torch.nn.Module):
         if target == "d,d":
             return STensor.from_torch(dense, self._name)
         raise NotImplementedError(f"to_sparse: unsupported target format {fmt}")
+
+    def change_mode_order(self, mode_order: List[int]) -> "STensor":
+        """Re-store a matrix so that its physical mode order becomes ``mode_order``
+        (e.g. ``[1, 0]`` stores the transpose), in place; returns ``self``.
+
+        Covers what the reference's 2-D fast path covers (stensor.py:785-896):
+        "d,d", "d,s" and "o,o" matrices, with torch operations on whatever device
+        the tensor is on.  Sparse results are sorted by (row, column) of the new
+        layout and duplicate coordinates are summed.  Other tensors go through
+        the reference's code generator, which is not part of this package."""
+        dim = self.dim()
+        if sorted(mode_order) != list(range(dim)):
+            raise ValueError("mode_order must be a permutation of the modes")
+        current = list(self.index.mode_order) if self.index.mode_order else list(range(dim))
+        if current == list(mode_order):
+            return self
+        layout = str(self.format)
+        if dim != 2 or layout not in ("d,d", "d,s", "o,o"):
+            raise NotImplementedError(f"change_mode_order for a {dim}-D \"{layout}\" tensor")
+        # mode_order[p] is the logical mode stored at physical position p
+        where = {logical: physical for physical, logical in enumerate(current)}
+        perm = [where[logical] for logical in mode_order]      # old physical axis of each new axis
+        new_shape = tuple(self.shape[p] for p in perm)
+
+        if layout == "d,d":
+            values = self.values.reshape(self.shape).permute(*perm).contiguous().reshape(-1)
+            indices = [[], []]
+        else:
+            if layout == "d,s":
+                pos, crd = self.index.mode_indices[1]
+                counts = (pos[1:] - pos[:-1]).to(torch.int64)
+                rows = torch.repeat_interleave(
+                    torch.arange(self.shape[0], dtype=torch.int64, device=crd.device), counts)
+                coords = [rows, crd.to(torch.int64)]
+            else:
+                coords = [self.index.mode_indices[0][0].to(torch.int64),
+                          self.index.mode_indices[1][0].to(torch.int64)]
+            rows, cols, values = _sorted_unique_entries(coords[perm[0]], coords[perm[1]], self.values,
+                                                        new_shape[1])
+            if layout == "d,s":
+                pos = torch.zeros(new_shape[0] + 1, dtype=torch.int64, device=rows.device)
+                if rows.numel():
+                    pos[1:] = torch.cumsum(torch.bincount(rows, minlength=new_shape[0]), dim=0)
+                indices = [[], [pos.to(torch.int32), cols.to(torch.int32)]]
+            else:
+                indices = [[rows.to(torch.int32)], [cols.to(torch.int32)]]
+        self._storage = TensorStorage(index=TensorIndex(self.format, indices, mode_order=list(mode_order)),
+                                      value=values)
+        self._shape = new_shape
+        return self
 
     def to_torch(self, in_place: bool = True) -> torch.Tensor:
         """Strided torch tensor of the logical shape (reference: stensor.py:454-475);

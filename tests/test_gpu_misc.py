@@ -213,3 +213,16 @@ def test_compile_matches_unfused():
 
     unfused = torch.relu(scorch.matmul(adj, x.cuda(), format="dd") + bias)
     assert torch.allclose(fused(adj, x.cuda(), bias), unfused, atol=1e-5)
+
+
+def test_matmul_normalises_a_transposed_csr_operand():
+    """A CSR operand stored in mode order [1, 0] is re-stored before dispatch
+    (reference: src/scorch/ops.py:333-346)."""
+    torch.manual_seed(11)
+    a = torch.rand(50, 70) * (torch.rand(50, 70) < 0.1)
+    b = torch.rand(70, 32)
+    A = STensor.from_torch(a).to_sparse("ds").to("cuda").change_mode_order([1, 0])
+    assert A.shape == (70, 50) and A.index.mode_order == [1, 0]
+    out = scorch.matmul(A, b.cuda())
+    assert torch.allclose(out.cpu(), a @ b, atol=1e-5)
+    assert A.index.mode_order == [1, 0]          # the caller's tensor is left as it was

@@ -217,3 +217,42 @@ def test_device_module_rejects_host_and_mistyped_tensors():
     with pytest.raises(ValueError, match="not a CSR"):
         scorch_ops_hip.spmm_csr_float_v2((8, 8), A.shape, [[], []], A.values, B.shape,
                                          B.index.mode_indices, B.values)
+
+
+# ---- mode order (reference: src/scorch/stensor.py:785-896) -------------------------------------
+@pytest.mark.parametrize("fmt", ["dd", "ds", "oo"])
+def test_change_mode_order_transposes_storage(fmt):
+    a, _ = sparse_dense_pair(n=12, seed=6)
+    a = a[:, :9].contiguous()                                  # rectangular 12 x 9
+    s = STensor.from_torch(a)
+    s = s if fmt == "dd" else s.to_sparse(fmt)
+    t = s.copy().change_mode_order([1, 0])
+    assert t.shape == (9, 12) and t.index.mode_order == [1, 0] and str(t.format) == str(s.format)
+    assert torch.equal(t.to_torch(), a)                         # logical tensor unchanged
+    stored = STensor(shape=t.shape, index=type(t.index)(t.format, t.index.mode_indices), value=t.values)
+    assert torch.equal(stored.to_torch(), a.t())                # physical storage is the transpose
+    if fmt == "ds":
+        pos, crd = t.index.mode_indices[1]
+        assert pos.dtype == torch.int32 and pos[-1] == s._nnz()
+        for r in range(9):
+            seg = crd[pos[r]:pos[r + 1]]
+            assert torch.all(seg[1:] > seg[:-1])                # sorted, unique
+    back = t.change_mode_order([0, 1])
+    assert back.shape == (12, 9) and torch.equal(back.to_torch(), a)
+    assert back.change_mode_order([0, 1]) is back               # no-op when already there
+
+
+def test_change_mode_order_sums_duplicate_coordinates():
+    idx = torch.tensor([[0, 0, 1, 0], [2, 2, 0, 1]])
+    vals = torch.tensor([1.0, 2.0, 5.0, 7.0])
+    s = scorch.from_coo(indices=idx, values=vals, shape=(2, 3))
+    t = s.change_mode_order([1, 0])
+    assert t._nnz() == 3
+    assert torch.equal(t.to_torch(), torch.tensor([[0.0, 7.0, 3.0], [5.0, 0.0, 0.0]]))
+
+
+def test_change_mode_order_rejects_what_it_cannot_do():
+    with pytest.raises(ValueError):
+        STensor.from_torch(torch.rand(3, 3)).change_mode_order([0, 0])
+    with pytest.raises(NotImplementedError):
+        STensor.from_torch(torch.rand(2, 3, 4)).change_mode_order([2, 0, 1])
