@@ -172,6 +172,52 @@ SCORCH_HIP_API int scorch_hip_spmv_csr_i64(int64_t M, int64_t K, int64_t nnz, co
                             int64_t *y, void *stream);
 
 /* ------------------------------------------------------------------------
+ * SpGEMM: C_csr[M,N] = A_csr[M,K] * B_csr[K,N], in two calls.
+ * Replaces spmspm_csr<T> (csrc/kernels.h:52-202), bound as
+ * prebuilt_spmspm_csr_{f32,f64,i32,i64} and spmspm_csr_float
+ * (csrc/ops.cpp:41-50,99,113).  The reference allocates the result inside one
+ * call; here the caller owns it, so the call is split where the size becomes
+ * known:
+ *   1. _symbolic writes c_row_ptr[M + 1] (device).  The caller reads
+ *      c_row_ptr[M] back (that read synchronises) and allocates c_col_idx
+ *      and c_vals of that length.
+ *   2. _numeric_<T> fills c_col_idx and c_vals.
+ * As in the reference, column indices are ascending within each row and every
+ * structurally reachable entry is stored, also when its value sums to zero.
+ * The structure is exact and the same on every run; floating-point sums are
+ * accumulated atomically, so their last bits may vary between runs.
+ * `workspace`: scorch_hip_spgemm_csr_workspace_bytes(M, N, sizeof(T)) bytes,
+ * 256-byte aligned (the symbolic call needs no more than elem_size = 1).
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API size_t scorch_hip_spgemm_csr_workspace_bytes(int64_t M, int64_t N, size_t elem_size);
+
+SCORCH_HIP_API int scorch_hip_spgemm_csr_symbolic(int64_t M, int64_t K, int64_t N,
+                                   const int32_t *a_row_ptr, const int32_t *a_col_idx,
+                                   const int32_t *b_row_ptr, const int32_t *b_col_idx,
+                                   int32_t *c_row_ptr,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spgemm_csr_numeric_f32(int64_t M, int64_t K, int64_t N,
+                                   const int32_t *a_row_ptr, const int32_t *a_col_idx, const float *a_vals,
+                                   const int32_t *b_row_ptr, const int32_t *b_col_idx, const float *b_vals,
+                                   const int32_t *c_row_ptr, int32_t *c_col_idx, float *c_vals,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spgemm_csr_numeric_f64(int64_t M, int64_t K, int64_t N,
+                                   const int32_t *a_row_ptr, const int32_t *a_col_idx, const double *a_vals,
+                                   const int32_t *b_row_ptr, const int32_t *b_col_idx, const double *b_vals,
+                                   const int32_t *c_row_ptr, int32_t *c_col_idx, double *c_vals,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spgemm_csr_numeric_i32(int64_t M, int64_t K, int64_t N,
+                                   const int32_t *a_row_ptr, const int32_t *a_col_idx, const int32_t *a_vals,
+                                   const int32_t *b_row_ptr, const int32_t *b_col_idx, const int32_t *b_vals,
+                                   const int32_t *c_row_ptr, int32_t *c_col_idx, int32_t *c_vals,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spgemm_csr_numeric_i64(int64_t M, int64_t K, int64_t N,
+                                   const int32_t *a_row_ptr, const int32_t *a_col_idx, const int64_t *a_vals,
+                                   const int32_t *b_row_ptr, const int32_t *b_col_idx, const int64_t *b_vals,
+                                   const int32_t *c_row_ptr, int32_t *c_col_idx, int64_t *c_vals,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
  * Row softmax over the stored values of a CSR matrix:
  * out[p] = exp(scale * v[p] - m_i) / sum_q exp(scale * v[q] - m_i), q over
  * row i, m_i the row maximum of scale * v.  out may alias vals.

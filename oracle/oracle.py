@@ -155,6 +155,34 @@ def spmv_csr_typed(row_ptr, col_idx, vals, x) -> np.ndarray:
     return out
 
 
+def spgemm_csr_typed(a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, b_vals, n_cols: int):
+    """C = A @ B with all three in CSR, f32/f64/i32/i64: the three phases of
+    spmspm_csr<T> (csrc/kernels.h:52-202).  Returns (row_ptr, col_idx, vals);
+    columns ascending within a row, structural zeros kept."""
+    a_vals = np.ascontiguousarray(a_vals)
+    suffix = _NP_SUFFIX[a_vals.dtype]
+    a_pos, a_crd = _c(a_row_ptr, np.int32), _c(a_col_idx, np.int32)
+    b_pos, b_crd, b_vals = _c(b_row_ptr, np.int32), _c(b_col_idx, np.int32), _c(b_vals, a_vals.dtype)
+    M = a_pos.size - 1
+    c_pos = np.zeros(M + 1, dtype=np.int32)
+    lib().oracle_spgemm_csr_count(ctypes.c_int(M), ctypes.c_int(n_cols), _ptr(a_pos), _ptr(a_crd),
+                                  _ptr(b_pos), _ptr(b_crd), _ptr(c_pos))
+    nnz = int(c_pos[-1])
+    c_crd = np.zeros(nnz, dtype=np.int32)
+    c_val = np.zeros(nnz, dtype=a_vals.dtype)
+    getattr(lib(), "oracle_spgemm_csr_" + suffix)(ctypes.c_int(M), ctypes.c_int(n_cols), _ptr(a_pos),
+                                                  _ptr(a_crd), _ptr(a_vals), _ptr(b_pos), _ptr(b_crd),
+                                                  _ptr(b_vals), _ptr(c_pos), _ptr(c_crd), _ptr(c_val))
+    return c_pos, c_crd, c_val
+
+
+def spgemm_fp64(a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, b_vals, shape_a, n_cols):
+    """(A @ B) as a dense float64 array (small cases) via scipy."""
+    A = _scipy_csr(a_row_ptr, a_col_idx, a_vals, shape_a)
+    B = _scipy_csr(b_row_ptr, b_col_idx, b_vals, (shape_a[1], n_cols))
+    return np.asarray((A @ B).todense())
+
+
 def softmax_csr_f32(row_ptr, vals, scale: float = 1.0) -> np.ndarray:
     """Row softmax over stored values (bench/bench_sparse_transformer.py:277-297)."""
     row_ptr, vals = _c(row_ptr, np.int32), _c(vals, np.float32)
@@ -290,6 +318,22 @@ def ref_spmm_bias(row_ptr, col_idx, vals, B, bias, relu: bool) -> np.ndarray:
 
 def ref_spmv(symbol: str, row_ptr, col_idx, vals, x) -> np.ndarray:
     return _ref_binary(symbol, row_ptr, col_idx, vals, x)
+
+
+def ref_spgemm(symbol: str, a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, b_vals, shape_a, n_cols):
+    """Call one of the reference's CSR x CSR symbols (e.g. "prebuilt_spmspm_csr_f32");
+    returns (row_ptr, col_idx, vals)."""
+    import torch
+    m = ref_module()
+    M, K = shape_a
+    t = lambda a, dt: torch.from_numpy(_c(a, dt))
+    a_vals = np.ascontiguousarray(a_vals)
+    out = getattr(m, symbol)([M, n_cols], [M, K], [[], [t(a_row_ptr, np.int32), t(a_col_idx, np.int32)]],
+                             torch.from_numpy(a_vals), [K, n_cols],
+                             [[], [t(b_row_ptr, np.int32), t(b_col_idx, np.int32)]],
+                             torch.from_numpy(_c(b_vals, a_vals.dtype)))
+    idx = out.storage.index.mode_indices[1]
+    return idx[0].numpy().copy(), idx[1].numpy().copy(), out.storage.value.numpy().copy()
 
 
 def ref_sddmm_coo(row_idx, col_idx, svals, A, B, shape):

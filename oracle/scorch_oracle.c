@@ -280,3 +280,87 @@ ORACLE_API void oracle_softmax_csr_f32(int M, const int32_t *pos,
     for (int p = lo; p < hi; ++p) out[p] = out[p] / sum;
   }
 }
+
+/* ------------------------------------------------------------------------
+ * SpGEMM: C = A * B, all three CSR, for the four dtypes.
+ * Restates spmspm_csr<T>, csrc/kernels.h:52-202 (bound as
+ * prebuilt_spmspm_csr_{f32,f64,i32,i64}, csrc/ops.cpp:41-50,99, and
+ * spmspm_csr_float, :113):
+ *   phase 1 (73-104)  per row, the number of distinct columns reached through
+ *                     A's entries, with a per-thread "next" array used as a
+ *                     linked list of touched columns;
+ *   phase 2 (107-113) prefix sum -> row pointer;
+ *   phase 3 (119-186) per row, sums[k] += a * b in traversal order, then the
+ *                     touched columns are collected and sorted ascending.
+ * Every structurally reachable column is stored, also when its sum is zero.
+ * Two calls, like any two-phase SpGEMM: `oracle_spgemm_csr_count` fills
+ * c_pos[M + 1]; the typed call fills c_crd / c_val, which the caller sized
+ * from c_pos[M].
+ * ---------------------------------------------------------------------- */
+ORACLE_API void oracle_spgemm_csr_count(int M, int N, const int32_t *a_pos, const int32_t *a_crd,
+                                        const int32_t *b_pos, const int32_t *b_crd, int32_t *c_pos) {
+  c_pos[0] = 0;
+#pragma omp parallel
+  {
+    int *next = (int *)malloc((size_t)(N > 0 ? N : 1) * sizeof(int));
+    for (int k = 0; k < N; ++k) next[k] = -1;
+#pragma omp for schedule(dynamic, 64)
+    for (int i = 0; i < M; ++i) {
+      int head = -2, length = 0;
+      for (int p = a_pos[i]; p < a_pos[i + 1]; ++p) {
+        const int j = a_crd[p];
+        for (int q = b_pos[j]; q < b_pos[j + 1]; ++q) {
+          const int k = b_crd[q];
+          if (next[k] == -1) { next[k] = head; head = k; ++length; }
+        }
+      }
+      c_pos[i + 1] = length;
+      while (head >= 0) { const int t = head; head = next[head]; next[t] = -1; }
+    }
+    free(next);
+  }
+  for (int i = 0; i < M; ++i) c_pos[i + 1] += c_pos[i];
+}
+
+static int cmp_int32(const void *x, const void *y) {
+  const int32_t a = *(const int32_t *)x, b = *(const int32_t *)y;
+  return (a > b) - (a < b);
+}
+
+#define DEFINE_SPGEMM_TYPED(NAME, T, ACC)                                                          \
+  ORACLE_API void NAME(int M, int N, const int32_t *a_pos, const int32_t *a_crd, const T *a_val,   \
+                       const int32_t *b_pos, const int32_t *b_crd, const T *b_val,                 \
+                       const int32_t *c_pos, int32_t *c_crd, T *c_val) {                           \
+    _Pragma("omp parallel")                                                                        \
+    {                                                                                              \
+      int *next = (int *)malloc((size_t)(N > 0 ? N : 1) * sizeof(int));                            \
+      ACC *sums = (ACC *)calloc((size_t)(N > 0 ? N : 1), sizeof(ACC));                             \
+      for (int k = 0; k < N; ++k) next[k] = -1;                                                    \
+      _Pragma("omp for schedule(dynamic, 64)")                                                     \
+      for (int i = 0; i < M; ++i) {                                                                \
+        int head = -2, length = 0;                                                                 \
+        for (int p = a_pos[i]; p < a_pos[i + 1]; ++p) {                                            \
+          const int j = a_crd[p];                                                                  \
+          const ACC v = (ACC)a_val[p];                                                             \
+          for (int q = b_pos[j]; q < b_pos[j + 1]; ++q) {                                          \
+            const int k = b_crd[q];                                                                \
+            sums[k] += v * (ACC)b_val[q];                                                          \
+            if (next[k] == -1) { next[k] = head; head = k; ++length; }                             \
+          }                                                                                        \
+        }                                                                                          \
+        int32_t *crd = c_crd + c_pos[i];                                                           \
+        int n = 0;                                                                                 \
+        while (head >= 0) { crd[n++] = head; const int t = head; head = next[head]; next[t] = -1; } \
+        qsort(crd, (size_t)n, sizeof(int32_t), cmp_int32);                                         \
+        for (int e = 0; e < n; ++e) { c_val[c_pos[i] + e] = (T)sums[crd[e]]; sums[crd[e]] = 0; }   \
+        (void)length;                                                                              \
+      }                                                                                            \
+      free(next);                                                                                  \
+      free(sums);                                                                                  \
+    }                                                                                              \
+  }
+
+DEFINE_SPGEMM_TYPED(oracle_spgemm_csr_f32, float, float)
+DEFINE_SPGEMM_TYPED(oracle_spgemm_csr_f64, double, double)
+DEFINE_SPGEMM_TYPED(oracle_spgemm_csr_i32, int32_t, uint32_t)
+DEFINE_SPGEMM_TYPED(oracle_spgemm_csr_i64, int64_t, uint64_t)

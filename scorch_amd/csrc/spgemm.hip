@@ -1,0 +1,540 @@
+// CSR x CSR -> CSR (SpGEMM) for gfx950, in the usual two phases: a symbolic
+// pass that counts the distinct columns of every output row and turns the
+// counts into the row pointer, and a numeric pass that fills column indices
+// (ascending within a row) and values.  Every structurally reachable column is
+// stored, also when its sum happens to be zero -- the reference's rule.
+//
+// A row of C is the union of the rows of B selected by the row of A.  How a row
+// is processed depends on an upper bound of its size, the number of products
+// it sums (sum over its entries of the length of the B row they select):
+//
+//   up to 256 products   one wavefront, hash table of 512 slots in LDS
+//   up to 4096 products  one workgroup, hash table of 8192 slots in LDS
+//   more                 one workgroup with a bitmap over all N columns (and,
+//                        in the numeric pass, a dense accumulator of N values)
+//                        in global memory; a fixed pool of such workgroups
+//                        walks the list of these rows
+//
+// Hash rows are emitted sorted: the wavefront version ranks every entry by
+// counting smaller keys (at most 256 of them), the workgroup version runs a
+// bitonic sort in LDS.  Bitmap rows come out sorted by construction.
+// Floating-point sums are accumulated with atomics, so their rounding can
+// differ from run to run in the last bits; the structure never does, and
+// integer results are exact.
+#include <climits>
+
+#include "common.hpp"
+
+namespace scorch {
+
+constexpr int kTinyProducts = 256;
+constexpr int kTinySlots = 512;
+constexpr int kMediumProducts = 4096;
+constexpr int kMediumSlots = 8192;
+constexpr int kHugeWorkgroups = 64;
+constexpr int kMediumWorkgroups = 2048;
+
+__device__ __forceinline__ int hash_slot(int key, int mask) {
+  return (int)(((unsigned)key * 2654435761u) >> 12) & mask;
+}
+
+// Slot of `key` in an open-addressing table (empty = -1); inserts it if absent.
+__device__ __forceinline__ int hash_insert(int *keys, int mask, int key) {
+  int s = hash_slot(key, mask);
+  for (;;) {
+    const int prev = atomicCAS(&keys[s], -1, key);
+    if (prev == -1 || prev == key) return s;
+    s = (s + 1) & mask;
+  }
+}
+
+// *addr += v, atomically (LDS or global memory).
+template <typename A>
+__device__ __forceinline__ void atomic_accumulate(A *addr, A v) { atomicAdd(addr, v); }
+template <>
+__device__ __forceinline__ void atomic_accumulate<uint64_t>(uint64_t *addr, uint64_t v) {
+  atomicAdd(reinterpret_cast<unsigned long long *>(addr), (unsigned long long)v);
+}
+
+template <typename A>
+__device__ __forceinline__ A agent_load(const A *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Exclusive prefix sum of one int per thread over the workgroup; `total`
+// receives the sum.  `scratch` holds kWavesPerBlock + 1 ints.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &total) {
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  int incl = v;
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  __syncthreads();  // scratch may still be read from a previous call
+  if (lane == kWaveSize - 1) scratch[w] = incl;
+  __syncthreads();
+  int before = 0;
+#pragma unroll
+  for (int i = 0; i < kWavesPerBlock; ++i) {
+    if (i < w) before += scratch[i];
+  }
+  total = scratch[0] + scratch[1] + scratch[2] + scratch[3];
+  return before + incl - v;
+}
+
+// ---- exclusive prefix sum of n ints, in place (counts -> row pointer) ------------------
+// Three small kernels: per-tile totals, a one-workgroup scan of the totals, and
+// a rescan of every tile from its offset.
+constexpr int kScanPerThread = 16;
+constexpr int kScanTile = kBlockThreads * kScanPerThread;
+
+__global__ __launch_bounds__(kBlockThreads) void scan_tile_totals_kernel(const int *__restrict__ data,
+                                                                         int64_t n,
+                                                                         int *__restrict__ totals) {
+  __shared__ int s_scan[kWavesPerBlock + 1];
+  const int64_t first = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+  int mine = 0;
+  for (int e = 0; e < kScanPerThread; ++e) mine += first + e < n ? data[first + e] : 0;
+  int total = 0;
+  (void)block_exclusive_scan(mine, s_scan, total);
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void scan_spine_kernel(int *__restrict__ totals,
+                                                                   int64_t n_tiles) {
+  __shared__ int s_scan[kWavesPerBlock + 1];
+  int carried = 0;
+  for (int64_t base = 0; base < n_tiles; base += kBlockThreads) {
+    const int64_t i = base + threadIdx.x;
+    const int v = i < n_tiles ? totals[i] : 0;
+    int total = 0;
+    const int before = block_exclusive_scan(v, s_scan, total);
+    if (i < n_tiles) totals[i] = carried + before;
+    carried += total;
+  }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restrict__ data, int64_t n,
+                                                                   const int *__restrict__ totals) {
+  __shared__ int s_scan[kWavesPerBlock + 1];
+  const int64_t first = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
+  int v[kScanPerThread];
+  int mine = 0;
+  for (int e = 0; e < kScanPerThread; ++e) {
+    v[e] = first + e < n ? data[first + e] : 0;
+    mine += v[e];
+  }
+  int total = 0;
+  int running = totals[blockIdx.x] + block_exclusive_scan(mine, s_scan, total);
+  for (int e = 0; e < kScanPerThread; ++e) {
+    if (first + e < n) data[first + e] = running;
+    running += v[e];
+  }
+}
+
+// ---- pass 0: products per row, and the lists of rows too big for a wavefront ----
+__global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
+    int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
+    const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ medium_rows,
+    int *__restrict__ huge_rows, int *__restrict__ counters) {
+  constexpr int G = 8;  // lanes per row
+  const int64_t row = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
+  const int t = threadIdx.x % G;
+  long long sum = 0;
+  if (row < M)
+    for (int p = a_pos[row] + t; p < a_pos[row + 1]; p += G) {
+      const int j = a_crd[p];
+      sum += b_pos[j + 1] - b_pos[j];
+    }
+#pragma unroll
+  for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  if (row < M && t == 0) {
+    const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
+    products[row] = bound;
+    if (bound > kMediumProducts) huge_rows[atomicAdd(&counters[1], 1)] = (int)row;
+    else if (bound > kTinyProducts) medium_rows[atomicAdd(&counters[0], 1)] = (int)row;
+  }
+}
+
+__global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
+  if (threadIdx.x < 4) counters[threadIdx.x] = 0;
+  if (threadIdx.x == 0 && c_pos_last) *c_pos_last = 0;
+}
+
+// ---- rows of at most kTinyProducts products: one wavefront each ---------------------
+template <typename T, bool NUMERIC>
+__global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
+    int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
+    const int *__restrict__ products, int *__restrict__ c_pos, int *__restrict__ c_crd,
+    T *__restrict__ c_val) {
+  using A = typename Acc<T>::type;
+  __shared__ int s_keys[kWavesPerBlock][kTinySlots];
+  __shared__ A s_vals[kWavesPerBlock][NUMERIC ? kTinySlots : 1];
+  __shared__ int s_ck[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
+  __shared__ A s_cv[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
+
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + w;
+  if (row >= M) return;
+  if (products[row] > kTinyProducts) return;  // a workgroup kernel owns this row
+
+  for (int s = lane; s < kTinySlots; s += kWaveSize) {
+    s_keys[w][s] = -1;
+    if (NUMERIC) s_vals[w][s] = (A)0;
+  }
+  wave_lds_sync();
+
+  const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
+  for (int p = a_lo; p < a_hi; ++p) {
+    const int j = uniform(a_crd[p]);
+    const A av = NUMERIC ? (A)a_val[p] : (A)0;
+    for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
+      const int slot = hash_insert(s_keys[w], kTinySlots - 1, b_crd[q]);
+      if (NUMERIC) atomic_accumulate<A>(&s_vals[w][slot], av * (A)b_val[q]);
+    }
+  }
+  wave_lds_sync();
+
+  // Count the occupied slots; in the numeric pass, also compact them.
+  int n = 0;
+  for (int base = 0; base < kTinySlots; base += kWaveSize) {
+    const int key = s_keys[w][base + lane];
+    const unsigned long long occupied = __ballot(key != -1);
+    if (NUMERIC && key != -1) {
+      const int at = n + __popcll(occupied & ((1ull << lane) - 1ull));
+      s_ck[w][at] = key;
+      s_cv[w][at] = s_vals[w][base + lane];
+    }
+    n += __popcll(occupied);
+  }
+  if (!NUMERIC) {
+    if (lane == 0) c_pos[row] = n;
+    return;
+  }
+  wave_lds_sync();
+
+  // Rank = number of smaller keys (keys are distinct): the sorted position.
+  const int out = c_pos[row];
+  for (int e = lane; e < n; e += kWaveSize) {
+    const int key = s_ck[w][e];
+    int rank = 0;
+    for (int x = 0; x < n; ++x) rank += s_ck[w][x] < key ? 1 : 0;
+    c_crd[out + rank] = key;
+    c_val[out + rank] = (T)s_cv[w][e];
+  }
+}
+
+// ---- rows of at most kMediumProducts products: one workgroup each -------------------
+template <typename T, bool NUMERIC>
+__global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
+    const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
+    const int *__restrict__ rows, const int *__restrict__ counters, int *__restrict__ c_pos,
+    int *__restrict__ c_crd, T *__restrict__ c_val) {
+  using A = typename Acc<T>::type;
+  __shared__ int s_keys[kMediumSlots];
+  __shared__ A s_vals[NUMERIC ? kMediumSlots : 1];
+  __shared__ int s_ck[NUMERIC ? kMediumProducts : 1];
+  __shared__ A s_cv[NUMERIC ? kMediumProducts : 1];
+  __shared__ int s_scan[kWavesPerBlock + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = wave_lane();
+  const int w = tid / kWaveSize;
+  const int n_rows = counters[0];
+
+  for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
+    const int row = rows[idx];
+    for (int s = tid; s < kMediumSlots; s += kBlockThreads) {
+      s_keys[s] = -1;
+      if (NUMERIC) s_vals[s] = (A)0;
+    }
+    __syncthreads();
+
+    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
+    for (int p = a_lo + w; p < a_hi; p += kWavesPerBlock) {
+      const int j = uniform(a_crd[p]);
+      const A av = NUMERIC ? (A)a_val[p] : (A)0;
+      for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
+        const int slot = hash_insert(s_keys, kMediumSlots - 1, b_crd[q]);
+        if (NUMERIC) atomic_accumulate<A>(&s_vals[slot], av * (A)b_val[q]);
+      }
+    }
+    __syncthreads();
+
+    // Each thread owns a contiguous run of slots; an exclusive scan of the
+    // per-thread counts places the occupied ones.
+    constexpr int kRun = kMediumSlots / kBlockThreads;
+    int mine = 0;
+    for (int s = 0; s < kRun; ++s) mine += s_keys[tid * kRun + s] != -1 ? 1 : 0;
+    int n = 0;
+    int at = block_exclusive_scan(mine, s_scan, n);
+    if (!NUMERIC) {
+      if (tid == 0) c_pos[row] = n;
+      __syncthreads();
+      continue;
+    }
+    for (int s = 0; s < kRun; ++s) {
+      const int key = s_keys[tid * kRun + s];
+      if (key != -1) {
+        s_ck[at] = key;
+        s_cv[at] = s_vals[tid * kRun + s];
+        ++at;
+      }
+    }
+    int padded = 1;
+    while (padded < n) padded <<= 1;
+    __syncthreads();
+    for (int e = n + tid; e < padded; e += kBlockThreads) s_ck[e] = INT_MAX;
+    __syncthreads();
+
+    // Bitonic sort of (key, value) pairs by key.
+    for (int size = 2; size <= padded; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int e = tid; e < padded / 2; e += kBlockThreads) {
+          const int lo = 2 * e - (e & (stride - 1));
+          const int hi = lo + stride;
+          const bool ascending = (lo & size) == 0;
+          const int klo = s_ck[lo], khi = s_ck[hi];
+          if ((klo > khi) == ascending) {
+            s_ck[lo] = khi;
+            s_ck[hi] = klo;
+            const A v = s_cv[lo];
+            s_cv[lo] = s_cv[hi];
+            s_cv[hi] = v;
+          }
+        }
+        __syncthreads();
+      }
+    }
+    const int out = c_pos[row];
+    for (int e = tid; e < n; e += kBlockThreads) {
+      c_crd[out + e] = s_ck[e];
+      c_val[out + e] = (T)s_cv[e];
+    }
+    __syncthreads();
+  }
+}
+
+// ---- rows beyond that: bitmap (and dense accumulator) over all columns ---------------
+template <typename T, bool NUMERIC>
+__global__ __launch_bounds__(kBlockThreads) void spgemm_huge_kernel(
+    int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
+    const int *__restrict__ rows, const int *__restrict__ counters, unsigned *__restrict__ bitmaps,
+    typename Acc<T>::type *__restrict__ dense, int *__restrict__ c_pos, int *__restrict__ c_crd,
+    T *__restrict__ c_val) {
+  using A = typename Acc<T>::type;
+  __shared__ int s_scan[kWavesPerBlock + 1];
+  const int tid = threadIdx.x;
+  const int lane = wave_lane();
+  const int w = tid / kWaveSize;
+  const int n_rows = counters[1];
+  if ((int)blockIdx.x >= n_rows) return;
+
+  const int words = (N + 31) / 32;
+  unsigned *bitmap = bitmaps + (size_t)blockIdx.x * (size_t)words;
+  A *sums = NUMERIC ? dense + (size_t)blockIdx.x * (size_t)N : nullptr;
+  // This workgroup's slab starts clean and is left clean after every row.
+  for (int i = tid; i < words; i += kBlockThreads) bitmap[i] = 0u;
+  if (NUMERIC)
+    for (int i = tid; i < N; i += kBlockThreads) sums[i] = (A)0;
+  __threadfence();
+  __syncthreads();
+
+  for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
+    const int row = rows[idx];
+    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
+    for (int p = a_lo + w; p < a_hi; p += kWavesPerBlock) {
+      const int j = uniform(a_crd[p]);
+      const A av = NUMERIC ? (A)a_val[p] : (A)0;
+      for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
+        const int k = b_crd[q];
+        atomicOr(&bitmap[k >> 5], 1u << (k & 31));
+        if (NUMERIC) atomic_accumulate<A>(&sums[k], av * (A)b_val[q]);
+      }
+    }
+    __threadfence();
+    __syncthreads();
+
+    // Walk the bitmap in order; the set bits are the row's columns, ascending.
+    int emitted = 0;
+    const int out = NUMERIC ? c_pos[row] : 0;
+    for (int base = 0; base < words; base += kBlockThreads) {
+      const int word = base + tid;
+      unsigned bits = word < words ? agent_load(&bitmap[word]) : 0u;
+      int total = 0;
+      int at = block_exclusive_scan(__popc(bits), s_scan, total);
+      if (bits) {
+        if (NUMERIC) {
+          at += out + emitted;
+          while (bits) {
+            const int bit = __ffs(bits) - 1;
+            bits &= bits - 1;
+            const int col = word * 32 + bit;
+            c_crd[at] = col;
+            c_val[at] = (T)agent_load(&sums[col]);
+            sums[col] = (A)0;
+            ++at;
+          }
+        }
+        bitmap[word] = 0u;
+      }
+      emitted += total;
+    }
+    if (!NUMERIC && tid == 0) c_pos[row] = emitted;
+    __threadfence();
+    __syncthreads();
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------
+struct SpgemmWorkspace {
+  int *products, *medium_rows, *huge_rows, *counters;
+  int *scan_totals;
+  unsigned *bitmaps;
+  void *dense;
+  size_t total;
+};
+
+inline size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+
+inline SpgemmWorkspace spgemm_layout(char *base, int64_t M, int64_t N, size_t elem) {
+  SpgemmWorkspace ws;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { char *p = base ? base + off : nullptr; off += round256(bytes); return p; };
+  ws.products = reinterpret_cast<int *>(take((size_t)M * 4));
+  ws.medium_rows = reinterpret_cast<int *>(take((size_t)M * 4));
+  ws.huge_rows = reinterpret_cast<int *>(take((size_t)M * 4));
+  ws.counters = reinterpret_cast<int *>(take(16));
+  ws.scan_totals = reinterpret_cast<int *>(take(((size_t)(M + 1) / kScanTile + 1) * 4));
+  ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)kHugeWorkgroups * ((size_t)(N + 31) / 32) * 4));
+  ws.dense = take((size_t)kHugeWorkgroups * (size_t)N * elem);
+  ws.total = off;
+  return ws;
+}
+
+inline int spgemm_check(const char *fn, int64_t M, int64_t K, int64_t N, const void *a_pos,
+                        const void *a_crd, const void *b_pos, const void *b_crd, const void *c_pos,
+                        const void *workspace, size_t workspace_bytes, size_t elem) {
+  if (M < 0 || K < 0 || N < 0)
+    return fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld K=%lld N=%lld)", fn, (long long)M,
+                (long long)K, (long long)N);
+  if (M >= INT32_MAX || K >= INT32_MAX || N >= INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  SCORCH_REQUIRE(a_pos && b_pos && c_pos, "%s: NULL row pointer", fn);
+  SCORCH_REQUIRE(aligned_to(a_pos, 4) && aligned_to(a_crd, 4) && aligned_to(b_pos, 4) &&
+                     aligned_to(b_crd, 4) && aligned_to(c_pos, 4),
+                 "%s: index arrays must be 4-byte aligned", fn);
+  const size_t need = spgemm_layout(nullptr, M, N, elem).total;
+  if (!workspace || workspace_bytes < need)
+    return fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
+                workspace ? workspace_bytes : (size_t)0);
+  SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
+  return SCORCH_HIP_OK;
+}
+
+template <typename T, bool NUMERIC>
+int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val, const int *b_pos,
+               const int *b_crd, const T *b_val, int *c_pos, int *c_crd, T *c_val,
+               const SpgemmWorkspace &ws, hipStream_t stream) {
+  using A = typename Acc<T>::type;
+  spgemm_reset_kernel<<<1, 64, 0, stream>>>(ws.counters, NUMERIC ? nullptr : c_pos + M);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  const unsigned row_groups = (unsigned)(((int64_t)M * 8 + kBlockThreads - 1) / kBlockThreads);
+  spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, a_pos, a_crd, b_pos, ws.products,
+                                                                ws.medium_rows, ws.huge_rows,
+                                                                ws.counters);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  const unsigned tiny_blocks = (unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock);
+  spgemm_tiny_kernel<T, NUMERIC><<<tiny_blocks, kBlockThreads, 0, stream>>>(
+      M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  const unsigned medium_blocks = (unsigned)(M < kMediumWorkgroups ? M : kMediumWorkgroups);
+  spgemm_medium_kernel<T, NUMERIC><<<medium_blocks, kBlockThreads, 0, stream>>>(
+      a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  spgemm_huge_kernel<T, NUMERIC><<<kHugeWorkgroups, kBlockThreads, 0, stream>>>(
+      N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
+      static_cast<A *>(ws.dense), c_pos, c_crd, c_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  if (!NUMERIC) {
+    const int64_t n = (int64_t)M + 1;
+    const unsigned tiles = (unsigned)((n + kScanTile - 1) / kScanTile);
+    scan_tile_totals_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    scan_spine_kernel<<<1, kBlockThreads, 0, stream>>>(ws.scan_totals, tiles);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    scan_apply_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals);
+    SCORCH_HIP_CHECK(hipGetLastError());
+  }
+  return SCORCH_HIP_OK;
+}
+
+template <typename T>
+int spgemm_numeric_entry(const char *fn, int64_t M, int64_t K, int64_t N, const int32_t *a_pos,
+                         const int32_t *a_crd, const T *a_val, const int32_t *b_pos,
+                         const int32_t *b_crd, const T *b_val, const int32_t *c_pos, int32_t *c_crd,
+                         T *c_val, void *workspace, size_t workspace_bytes, void *stream) {
+  if (int rc = spgemm_check(fn, M, K, N, a_pos, a_crd, b_pos, b_crd, c_pos, workspace, workspace_bytes,
+                            sizeof(T)))
+    return rc;
+  if (M == 0 || N == 0 || K == 0) return SCORCH_HIP_OK;
+  const SpgemmWorkspace ws = spgemm_layout(static_cast<char *>(workspace), M, N, sizeof(T));
+  return spgemm_run<T, true>((int)M, (int)N, a_pos, a_crd, a_val, b_pos, b_crd, b_val,
+                             const_cast<int32_t *>(c_pos), c_crd, c_val, ws,
+                             static_cast<hipStream_t>(stream));
+}
+
+}  // namespace scorch
+
+extern "C" {
+
+size_t scorch_hip_spgemm_csr_workspace_bytes(int64_t M, int64_t N, size_t elem_size) {
+  if (M < 0 || N < 0 || M >= INT32_MAX || elem_size == 0) return 0;
+  return scorch::spgemm_layout(nullptr, M, N, elem_size).total;
+}
+
+int scorch_hip_spgemm_csr_symbolic(int64_t M, int64_t K, int64_t N, const int32_t *a_row_ptr,
+                                   const int32_t *a_col_idx, const int32_t *b_row_ptr,
+                                   const int32_t *b_col_idx, int32_t *c_row_ptr, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+  using namespace scorch;
+  const char *fn = "scorch_hip_spgemm_csr_symbolic";
+  // the symbolic pass never touches the dense accumulators: size them for 1-byte elements
+  if (int rc = spgemm_check(fn, M, K, N, a_row_ptr, a_col_idx, b_row_ptr, b_col_idx, c_row_ptr,
+                            workspace, workspace_bytes, 1))
+    return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (M == 0) {
+    spgemm_reset_kernel<<<1, 64, 0, s>>>(static_cast<int *>(workspace), c_row_ptr);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    return SCORCH_HIP_OK;
+  }
+  const SpgemmWorkspace ws = spgemm_layout(static_cast<char *>(workspace), M, N, 1);
+  return spgemm_run<float, false>((int)M, (int)N, a_row_ptr, a_col_idx, nullptr, b_row_ptr, b_col_idx,
+                                  nullptr, c_row_ptr, nullptr, nullptr, ws, s);
+}
+
+#define SCORCH_DEFINE_SPGEMM(SUFFIX, T)                                                             \
+  int scorch_hip_spgemm_csr_numeric_##SUFFIX(                                                        \
+      int64_t M, int64_t K, int64_t N, const int32_t *a_row_ptr, const int32_t *a_col_idx,           \
+      const T *a_vals, const int32_t *b_row_ptr, const int32_t *b_col_idx, const T *b_vals,          \
+      const int32_t *c_row_ptr, int32_t *c_col_idx, T *c_vals, void *workspace,                      \
+      size_t workspace_bytes, void *stream) {                                                        \
+    return scorch::spgemm_numeric_entry<T>("scorch_hip_spgemm_csr_numeric_" #SUFFIX, M, K, N,       \
+                                           a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx,      \
+                                           b_vals, c_row_ptr, c_col_idx, c_vals, workspace,         \
+                                           workspace_bytes, stream);                                \
+  }
+
+SCORCH_DEFINE_SPGEMM(f32, float)
+SCORCH_DEFINE_SPGEMM(f64, double)
+SCORCH_DEFINE_SPGEMM(i32, int32_t)
+SCORCH_DEFINE_SPGEMM(i64, int64_t)
+
+}  // extern "C"

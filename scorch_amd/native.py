@@ -20,6 +20,7 @@ _size = ctypes.c_size_t
 OK, EINVAL, EWORKSPACE, ERUNTIME, EUNSUPPORTED = 0, 1, 2, 3, 4
 
 _SPMM = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
+_SPGEMM = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 _SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
 
 # name -> (restype, argtypes); one entry per declaration in include/scorch_hip.h
@@ -34,6 +35,13 @@ SIGNATURES = {
     "scorch_hip_spmm_csr_f32_timed": (ctypes.c_int, _SPMM + [ctypes.POINTER(ctypes.c_float)]),
     "scorch_hip_spmm_csr_bias_act_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_spgemm_csr_workspace_bytes": (_size, [_i64, _i64, _size]),
+    "scorch_hip_spgemm_csr_symbolic": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                                      _size, _ptr]),
+    "scorch_hip_spgemm_csr_numeric_f32": (ctypes.c_int, _SPGEMM),
+    "scorch_hip_spgemm_csr_numeric_f64": (ctypes.c_int, _SPGEMM),
+    "scorch_hip_spgemm_csr_numeric_i32": (ctypes.c_int, _SPGEMM),
+    "scorch_hip_spgemm_csr_numeric_i64": (ctypes.c_int, _SPGEMM),
     "scorch_hip_sddmm_coo_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr,
                                                 _ptr, _ptr]),
     "scorch_hip_sddmm_csr_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr,

@@ -159,6 +159,50 @@ def spmm_csr_bias_relu_float(result_shape, A_shape, A_mode_indices, A_values, B_
                  B_mode_indices, B_values, bias=bias, act=1)
 
 
+# ---- SpGEMM --------------------------------------------------------------------
+def _make_spgemm(dtype):
+    def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+        """C = A @ B, all CSR (reference: csrc/kernels.h:52-202).  Two kernels
+        passes with one host read of the result size in between."""
+        M, K, N = int(A_shape[0]), int(A_shape[1]), int(B_shape[1])
+        if int(B_shape[0]) != K:
+            raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)}")
+        a_pos, a_crd = _csr_parts(A_mode_indices, "A")
+        b_pos, b_crd = _csr_parts(B_mode_indices, "B")
+        a_val = _flat(A_values, dtype, "A values")
+        b_val = _flat(B_values, dtype, "B values")
+        if a_pos.numel() != M + 1 or b_pos.numel() != K + 1 or a_crd.numel() != a_val.numel() \
+                or b_crd.numel() != b_val.numel():
+            raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
+        dev = _device_of(a_pos, a_crd, a_val, b_pos, b_crd, b_val)
+        L = native.lib()
+        with torch.cuda.device(dev):
+            stream = _stream(dev)
+            need = L.scorch_hip_spgemm_csr_workspace_bytes(M, N, a_val.element_size())
+            ws = _workspace(dev, stream, need)
+            c_pos = torch.empty(M + 1, dtype=torch.int32, device=dev)
+            native.check(L.scorch_hip_spgemm_csr_symbolic(M, K, N, a_pos.data_ptr(), a_crd.data_ptr(),
+                                                          b_pos.data_ptr(), b_crd.data_ptr(),
+                                                          c_pos.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                          stream))
+            nnz = int(c_pos[-1].item())
+            c_crd = torch.empty(nnz, dtype=torch.int32, device=dev)
+            c_val = torch.empty(nnz, dtype=dtype, device=dev)
+            fn = getattr(L, "scorch_hip_spgemm_csr_numeric_" + _SUFFIX[dtype])
+            native.check(fn(M, K, N, a_pos.data_ptr(), a_crd.data_ptr(), a_val.data_ptr(),
+                            b_pos.data_ptr(), b_crd.data_ptr(), b_val.data_ptr(), c_pos.data_ptr(),
+                            c_crd.data_ptr(), c_val.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        return Tensor(c_val, [[], [c_pos, c_crd]])
+    return kernel
+
+
+prebuilt_spmspm_csr_f32 = _make_spgemm(torch.float32)
+spmspm_csr_float = _make_spgemm(torch.float32)
+prebuilt_spmspm_csr_f64 = _make_spgemm(torch.float64)
+prebuilt_spmspm_csr_i32 = _make_spgemm(torch.int32)
+prebuilt_spmspm_csr_i64 = _make_spgemm(torch.int64)
+
+
 # ---- SpMV ----------------------------------------------------------------------
 def _make_spmv(dtype):
     def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):

@@ -5,7 +5,7 @@ Run once, in a container that holds the reference sources, after
 ``make -C oracle ref`` has compiled the reference's csrc/ops.cpp into
 oracle/_ref/scorch_ops.so.  The outputs stored here come from that module
 (symbols spmm_csr_float_v2, prebuilt_spmm_csr_{f32,f64,i32,i64},
-spmm_csr_bias[_relu]_float, sddmm_coo_float_prebuilt,
+spmm_csr_bias[_relu]_float, prebuilt_spmspm_csr_{f32,f64,i32,i64}, sddmm_coo_float_prebuilt,
 prebuilt_spmv_csr_{f32,f64,i32,i64}); the inputs come from this script's own
 seeded numpy generators.  The file holds data only.
 
@@ -16,6 +16,7 @@ test_matmul_dispatch.py:9-27 (n=32, 10 % dense), test_kernels.py:1310-1358
 (literal diag(1..5)), test_kernels_comprehensive.py:260-271 (30x50 . 50x20),
 :376-411 (SDDMM n/d/sparsity grid), test_compile.py:70-127 (n=64, k=16 fused
 bias/ReLU), test_prebuilt_kernel_registry.py:21-38 (literal 4x4 int64 SpMV),
+test_matmul_dispatch.py:30-48 (CSR x CSR),
 plus the edge cases the kernels must survive (empty rows, no entries at all,
 more than one 256-wide column tile, a row far longer than the rest).
 
@@ -174,6 +175,23 @@ def main() -> None:
         x = dense(rng, (70,), dtype=dt)
         put(f"spmv_{suffix}", row_ptr=rp, col_idx=ci, vals=v, x=x,
             y=O.ref_spmv(f"prebuilt_spmv_csr_{suffix}", rp, ci, v, x))
+
+    # ---- SpGEMM (CSR x CSR -> CSR) --------------------------------------------------
+    for suffix, dt in (("f32", np.float32), ("f64", np.float64), ("i32", np.int32), ("i64", np.int64)):
+        rng = np.random.default_rng(1200 + ord(suffix[0]) + int(suffix[1:]))
+        arp, aci, av = random_csr(rng, 48, 40, 0.12, dtype=dt, empty_rows=(5,))
+        brp, bci, bv = random_csr(rng, 40, 56, 0.15, dtype=dt, empty_rows=(0, 17))
+        crp, cci, cv = O.ref_spgemm(f"prebuilt_spmspm_csr_{suffix}", arp, aci, av, brp, bci, bv, (48, 40), 56)
+        put(f"spgemm_{suffix}", a_row_ptr=arp, a_col_idx=aci, a_vals=av, b_row_ptr=brp, b_col_idx=bci,
+            b_vals=bv, n_cols=np.int64(56), c_row_ptr=crp, c_col_idx=cci, c_vals=cv)
+    # exact cancellation: the entry is stored although its value is zero
+    arp = np.array([0, 2, 3], np.int32); aci = np.array([0, 1, 1], np.int32)
+    av = np.array([1.0, -1.0, 2.0], np.float32)
+    brp = np.array([0, 2, 4], np.int32); bci = np.array([0, 2, 0, 1], np.int32)
+    bv = np.array([3.0, 5.0, 3.0, 7.0], np.float32)
+    crp, cci, cv = O.ref_spgemm("spmspm_csr_float", arp, aci, av, brp, bci, bv, (2, 2), 3)
+    put("spgemm_cancel", a_row_ptr=arp, a_col_idx=aci, a_vals=av, b_row_ptr=brp, b_col_idx=bci, b_vals=bv,
+        n_cols=np.int64(3), c_row_ptr=crp, c_col_idx=cci, c_vals=cv)
 
     np.savez_compressed(OUT, **data)
     print(f"wrote {OUT}: {len(data)} arrays, {os.path.getsize(OUT) / 1024:.1f} KiB")

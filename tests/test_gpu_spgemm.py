@@ -1,0 +1,136 @@
+"""CSR x CSR -> CSR on the MI355X through the C ABI.
+
+Structure (row_ptr, col_idx) is compared bit for bit with the oracle, which is
+itself bit-identical to the reference's; values to 1e-5 relative Frobenius
+error against fp64 (floating point) or bit for bit (integers).
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+
+import scorch_amd as scorch
+from conftest import random_csr
+from gpu_util import dev, host
+from scorch_amd import STensor
+from scorch_amd import scorch_ops_hip as H
+
+pytestmark = pytest.mark.gpu
+SYMBOL = {np.dtype(np.float32): "prebuilt_spmspm_csr_f32", np.dtype(np.float64): "prebuilt_spmspm_csr_f64",
+          np.dtype(np.int32): "prebuilt_spmspm_csr_i32", np.dtype(np.int64): "prebuilt_spmspm_csr_i64"}
+
+
+def hip_spgemm(arp, aci, av, brp, bci, bv, n_cols):
+    M, K = len(arp) - 1, len(brp) - 1
+    out = getattr(H, SYMBOL[np.dtype(av.dtype)])(
+        [M, n_cols], [M, K], [[], [dev(arp), dev(aci)]], dev(av), [K, n_cols], [[], [dev(brp), dev(bci)]], dev(bv))
+    idx = out.storage.index.mode_indices
+    assert idx[0] == []
+    return host(idx[1][0]), host(idx[1][1]), host(out.storage.value)
+
+
+def check(oracle, arp, aci, av, brp, bci, bv, n_cols):
+    rp, ci, v = hip_spgemm(arp, aci, av, brp, bci, bv, n_cols)
+    wrp, wci, wv = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, n_cols)
+    assert rp.dtype == np.int32 and ci.dtype == np.int32
+    assert np.array_equal(rp, wrp), "row pointer differs"
+    assert np.array_equal(ci, wci), "column indices differ"
+    if np.issubdtype(av.dtype, np.integer):
+        assert np.array_equal(v, wv)
+    else:
+        A = sp.csr_matrix((av.astype(np.float64), aci, arp), shape=(len(arp) - 1, len(brp) - 1))
+        B = sp.csr_matrix((bv.astype(np.float64), bci, brp), shape=(len(brp) - 1, n_cols))
+        dense = np.asarray((A @ B).todense())
+        ref64 = dense[np.repeat(np.arange(len(rp) - 1), np.diff(rp)), ci]
+        assert oracle.rel_fro(v, ref64) <= (1e-5 if av.dtype == np.float32 else 1e-13)
+    return rp, ci, v
+
+
+@pytest.mark.parametrize("name", ["spgemm_f32", "spgemm_f64", "spgemm_i32", "spgemm_i64", "spgemm_cancel"])
+def test_golden(golden, name):
+    c = golden.case(name)
+    rp, ci, v = hip_spgemm(c["a_row_ptr"], c["a_col_idx"], c["a_vals"], c["b_row_ptr"], c["b_col_idx"],
+                           c["b_vals"], int(c["n_cols"]))
+    assert np.array_equal(rp, c["c_row_ptr"]) and np.array_equal(ci, c["c_col_idx"])
+    if np.issubdtype(v.dtype, np.integer):
+        assert np.array_equal(v, c["c_vals"])
+    else:
+        np.testing.assert_allclose(v, c["c_vals"], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_small_rows_one_wavefront_each(oracle, dtype):
+    rng = np.random.default_rng(1)
+    arp, aci, av = random_csr(rng, 700, 500, 0.01, dtype=dtype, empty_rows=(0, 699))
+    brp, bci, bv = random_csr(rng, 500, 900, 0.012, dtype=dtype, empty_rows=(3,))
+    check(oracle, arp, aci, av, brp, bci, bv, 900)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
+def test_medium_rows_one_workgroup_each(oracle, dtype):
+    # ~60 entries per A row x ~40 per B row = ~2400 products: the LDS-hash workgroup path
+    rng = np.random.default_rng(2)
+    arp, aci, av = random_csr(rng, 150, 600, 0.1, dtype=dtype)
+    brp, bci, bv = random_csr(rng, 600, 3000, 0.013, dtype=dtype)
+    rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, 3000)
+    assert np.diff(rp).max() > 256
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_huge_rows_bitmap_path_and_all_three_mixed(oracle, dtype):
+    # a few A rows select hundreds of B rows of ~100 entries (> 4096 products), the rest are small
+    rng = np.random.default_rng(3)
+    lens = rng.integers(0, 6, 400)
+    lens[[7, 123, 399]] = [300, 650, 90]
+    arp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    aci = np.concatenate([np.sort(rng.choice(800, int(n), replace=False)) for n in lens]).astype(np.int32)
+    av = (rng.integers(-9, 9, aci.size) if np.issubdtype(dtype, np.integer)
+          else rng.uniform(-1, 1, aci.size)).astype(dtype)
+    brp, bci, bv = random_csr(rng, 800, 5000, 0.02, dtype=dtype)
+    rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, 5000)
+    assert np.diff(rp).max() > 4096
+
+
+def test_structure_is_the_same_on_every_run_and_inputs_untouched(oracle):
+    rng = np.random.default_rng(4)
+    arp, aci, av = random_csr(rng, 300, 300, 0.05)
+    first = hip_spgemm(arp, aci, av, arp, aci, av, 300)
+    for _ in range(3):
+        again = hip_spgemm(arp, aci, av, arp, aci, av, 300)
+        assert np.array_equal(first[0], again[0]) and np.array_equal(first[1], again[1])
+        np.testing.assert_allclose(first[2], again[2], rtol=1e-5, atol=1e-6)   # atomics: summation order varies
+
+
+def test_empty_operands():
+    z = np.zeros(0, np.int32)
+    rp, ci, v = hip_spgemm(np.zeros(6, np.int32), z, np.zeros(0, np.float32), np.zeros(4, np.int32), z,
+                           np.zeros(0, np.float32), 9)
+    assert rp.tolist() == [0] * 6 and ci.size == 0 and v.size == 0
+
+
+@pytest.mark.parametrize("use_cache", [True, False])
+def test_sparse_stensor_spgemm_does_not_call_torch_matmul(use_cache, monkeypatch):
+    """reference: tests/test_scorch/test_matmul_dispatch.py:30-48 (with the CSR result kept sparse)"""
+    from scorch_amd import ops
+    torch.manual_seed(1)
+    n = 32
+    a_t = torch.rand(n, n) * (torch.rand(n, n) < 0.05)
+    b_t = torch.rand(n, n) * (torch.rand(n, n) < 0.05)
+    expected = torch.matmul(a_t, b_t)
+    a = STensor.from_torch(a_t, "A").to_sparse("ds").to("cuda")
+    b = STensor.from_torch(b_t, "B").to_sparse("ds").to("cuda")
+
+    def forbidden(*args, **kwargs):
+        raise AssertionError("torch.matmul should not be used for sparse STensor matmul")
+
+    monkeypatch.setattr(ops.torch, "matmul", forbidden)
+    out = scorch.matmul(a, b, use_cache=use_cache)
+    assert isinstance(out, STensor) and str(out.format) == "d,s" and out.shape == (n, n)
+    assert torch.allclose(out.to_torch().cpu(), expected, atol=1e-5)
+
+
+def test_graph_squared_power_law(oracle):
+    """A @ A for a power-law graph: rows from one entry to tens of thousands."""
+    from scorch_amd import workloads
+    w = workloads.gcn_powerlaw(M=20000, N=4, seed=21, max_degree=3000)
+    check(oracle, w["row_ptr"], w["col_idx"], w["vals"], w["row_ptr"], w["col_idx"], w["vals"], 20000)

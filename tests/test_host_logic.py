@@ -127,9 +127,15 @@ def test_resolve_prebuilt_gates():
     assert resolve_prebuilt_matmul(A, STensor.from_torch(b.double())) is None  # dtype equality gate
     assert resolve_prebuilt_matmul(B, B) is None                               # dense x dense: no entry
     assert resolve_prebuilt_matmul(A, STensor.from_torch(b.half())) is None
-    # CSR x CSR is in the table but this package ships no symbol for it
+    # CSR x CSR produces CSR: a dense result cannot be requested from the prebuilt kernel
+    # (reference: test_prebuilt_kernel_registry.py:41-51)
     assert resolve_prebuilt_matmul(A, A, output_format="dd") is None
-    assert resolve_prebuilt_matmul(A, A) is None
+    spgemm = resolve_prebuilt_matmul(A, A)
+    assert spgemm.symbol_name == "prebuilt_spmspm_csr_f32" and str(spgemm.output_format) == "d,s"
+    assert resolve_prebuilt_matmul(A, A, output_format="ds").symbol_name == "prebuilt_spmspm_csr_f32"
+    # coordinate-format products are in the table but have no device symbol
+    coo = STensor.from_torch(a).to_sparse("oo")
+    assert resolve_prebuilt_matmul(coo, coo) is None and resolve_prebuilt_matmul(coo, B) is None
 
 
 def test_resolve_prebuilt_fused():
@@ -191,7 +197,9 @@ def test_expressions_outside_the_path_raise_not_implemented():
     a, b = sparse_dense_pair()
     A = STensor.from_torch(a).to_sparse("ds")
     with pytest.raises(NotImplementedError):
-        scorch.matmul(A, A)                      # SpGEMM belongs to the reference's kernels
+        scorch.matmul(A, A, format="dd")         # CSR x CSR -> dense is the code generator's
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.matmul(A, A)                      # CSR x CSR -> CSR has a kernel, on the device
     with pytest.raises(NotImplementedError):
         scorch.einsum("ij,ij->ij", A, A)
     with pytest.raises(NotImplementedError):

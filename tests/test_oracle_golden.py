@@ -121,3 +121,22 @@ def test_spmv_matches_reference_output(golden, oracle, name, exact):
         assert np.array_equal(got, c["y"])
     else:
         np.testing.assert_allclose(got, c["y"], rtol=1e-5 if name.endswith("f32") else 1e-13, atol=1e-6)
+
+
+# ---- SpGEMM ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["spgemm_f32", "spgemm_f64", "spgemm_i32", "spgemm_i64", "spgemm_cancel"])
+def test_spgemm_matches_reference_output(golden, oracle, name):
+    c = golden.case(name)
+    rp, ci, v = oracle.spgemm_csr_typed(c["a_row_ptr"], c["a_col_idx"], c["a_vals"], c["b_row_ptr"],
+                                        c["b_col_idx"], c["b_vals"], int(c["n_cols"]))
+    assert np.array_equal(rp, c["c_row_ptr"]) and np.array_equal(ci, c["c_col_idx"])   # structure: exact
+    if np.issubdtype(v.dtype, np.integer):
+        assert np.array_equal(v, c["c_vals"])
+    else:
+        np.testing.assert_allclose(v, c["c_vals"], rtol=1e-6, atol=1e-7)
+
+
+def test_spgemm_keeps_entries_that_cancel_to_zero(golden):
+    c = golden.case("spgemm_cancel")
+    assert c["c_row_ptr"].tolist() == [0, 3, 5] and c["c_col_idx"].tolist() == [0, 1, 2, 0, 1]
+    assert c["c_vals"][0] == 0.0                      # 1*3 + (-1)*3, stored all the same

@@ -221,3 +221,33 @@ def test_attention_dense_fp64_matches_csr_pipeline(oracle):
     mask[rows, ci] = True
     np.testing.assert_allclose(out, oracle.attention_dense_fp64(q, k, v, mask, D ** -0.5), rtol=1e-10,
                                atol=1e-12)
+
+
+# ---- SpGEMM ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_spgemm_matches_scipy_structure_and_values(oracle, dtype):
+    rng = np.random.default_rng(14)
+    arp, aci, av = random_csr(rng, 37, 29, 0.15, dtype=dtype, empty_rows=(2,), lo=0.5, hi=1.5)
+    brp, bci, bv = random_csr(rng, 29, 41, 0.2, dtype=dtype, empty_rows=(7,), lo=0.5, hi=1.5)
+    if np.issubdtype(dtype, np.integer):
+        av, bv = np.abs(av) + 1, np.abs(bv) + 1            # no cancellation: scipy's pattern == structural
+    rp, ci, v = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, 41)
+    A = sp.csr_matrix((av.astype(np.float64), aci, arp), shape=(37, 29))
+    B = sp.csr_matrix((bv.astype(np.float64), bci, brp), shape=(29, 41))
+    C = (A @ B).tocsr()
+    C.sort_indices()
+    assert np.array_equal(rp, C.indptr) and np.array_equal(ci, C.indices)
+    for i in range(37):
+        assert (np.diff(ci[rp[i]:rp[i + 1]]) > 0).all()     # ascending, unique
+    np.testing.assert_allclose(v.astype(np.float64), C.data, rtol=1e-5 if dtype == np.float32 else 1e-12)
+
+
+def test_spgemm_identity_and_empty_operands(oracle):
+    rng = np.random.default_rng(15)
+    brp, bci, bv = random_csr(rng, 20, 33, 0.2)
+    eye_rp, eye_ci, eye_v = np.arange(21, dtype=np.int32), np.arange(20, dtype=np.int32), np.ones(20, np.float32)
+    rp, ci, v = oracle.spgemm_csr_typed(eye_rp, eye_ci, eye_v, brp, bci, bv, 33)
+    assert np.array_equal(rp, brp) and np.array_equal(ci, bci) and np.array_equal(v, bv)
+    rp, ci, v = oracle.spgemm_csr_typed(np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32),
+                                        brp, bci, bv, 33)
+    assert rp.tolist() == [0] * 6 and ci.size == 0 and v.size == 0

@@ -89,3 +89,18 @@ def test_spmv(ref, suffix, dtype):
         assert np.array_equal(got, expect)
     else:
         np.testing.assert_allclose(got, expect, rtol=1e-5 if dtype == np.float32 else 1e-13, atol=1e-6)
+
+
+@pytest.mark.parametrize("suffix,dtype", [("f32", np.float32), ("f64", np.float64), ("i32", np.int32),
+                                          ("i64", np.int64)])
+def test_spgemm(ref, suffix, dtype):
+    rng = np.random.default_rng(40)
+    arp, aci, av = random_csr(rng, 130, 90, 0.08, dtype=dtype, empty_rows=(0, 129))
+    brp, bci, bv = random_csr(rng, 90, 150, 0.1, dtype=dtype, empty_rows=(4,))
+    got = ref.spgemm_csr_typed(arp, aci, av, brp, bci, bv, 150)
+    want = ref.ref_spgemm("prebuilt_spmspm_csr_" + suffix, arp, aci, av, brp, bci, bv, (130, 90), 150)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(got[2], want[2])
+    else:
+        np.testing.assert_allclose(got[2], want[2], rtol=1e-6 if dtype == np.float32 else 1e-14)
