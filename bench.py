@@ -173,6 +173,29 @@ def side_workload(args, dev) -> int:
                           "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
                           "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
         return 0
+    if args.workload == "spgemm_powerlaw":
+        # A @ A for the power-law graph at 1/8 of the headline size (the square of the
+        # full graph has billions of products)
+        rows = args.rows if args.rows != 1 << 20 else 1 << 17
+        w = workloads.gcn_powerlaw(M=rows, N=4, max_degree=5000)
+        M = w["M"]
+        pos, crd, val = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"])
+        fn = lambda: H.prebuilt_spmspm_csr_f32([M, M], [M, M], [[], [pos, crd]], val, [M, M],
+                                               [[], [pos, crd]], val)
+        out = fn()
+        nnz_c = int(out.storage.value.numel())
+        deg = (pos[1:] - pos[:-1]).long()
+        products = int(deg[crd.long()].sum().item())
+        ms = _time_steps(fn, args.steps, args.warmup)
+        print(json.dumps({"metric": "CSR SpGEMM GFLOP/s (2 flops per product)",
+                          "value": round(2.0 * products / ms / 1e6, 2), "unit": "GFLOP/s",
+                          "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "dtype": "f32", "data": "synthetic",
+                          "higher_is_better": True,
+                          "config": {"workload": "spgemm_powerlaw_fp32", "rows": M, "nnz_a": int(crd.numel()),
+                                     "products": products, "nnz_c": nnz_c},
+                          "note": "symbolic + numeric passes and the host read of nnz(C) between them"}))
+        return 0
     if args.workload == "sddmm_uniform":
         w = workloads.sddmm_uniform()
         M, n_cols, K, nnz = w["M"], w["n_cols"], w["K"], int(w["col_idx"].size)
@@ -222,7 +245,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="gcn_powerlaw",
                     choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
-                             "attention_blocksparse"],
+                             "attention_blocksparse", "spgemm_powerlaw"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "

@@ -9,11 +9,14 @@
 // it sums (sum over its entries of the length of the B row they select):
 //
 //   up to 256 products   one wavefront, hash table of 512 slots in LDS
-//   up to 4096 products  one workgroup, hash table of 8192 slots in LDS
+//   up to 1024 products  one workgroup, hash table of 2048 slots in LDS
+//   up to 4096 products  one workgroup, hash table of 8192 slots in LDS (the
+//                        smaller table of the tier above lets more workgroups
+//                        share a CU)
 //   more                 one workgroup with a bitmap over all N columns (and,
 //                        in the numeric pass, a dense accumulator of N values)
-//                        in global memory; a fixed pool of such workgroups
-//                        walks the list of these rows
+//                        in global memory; a pool of such workgroups, sized to
+//                        about 1 GiB of slabs, walks the list of these rows
 //
 // Hash rows are emitted sorted: the wavefront version ranks every entry by
 // counting smaller keys (at most 256 of them), the workgroup version runs a
@@ -29,10 +32,22 @@ namespace scorch {
 
 constexpr int kTinyProducts = 256;
 constexpr int kTinySlots = 512;
-constexpr int kMediumProducts = 4096;
-constexpr int kMediumSlots = 8192;
-constexpr int kHugeWorkgroups = 64;
+constexpr int kSmallProducts = 1024;   // workgroup tier 1 (2048 slots)
+constexpr int kMediumProducts = 4096;  // workgroup tier 2 (8192 slots)
 constexpr int kMediumWorkgroups = 2048;
+constexpr int kMinHugeWorkgroups = 64;
+constexpr int kMaxHugeWorkgroups = 1024;
+constexpr size_t kHugeSlabBudget = (size_t)1 << 30;
+
+// Number of bitmap workgroups: as many slabs (N bits + N values) as fit the
+// budget.  Priced for 8-byte values whatever the dtype, so that the pool -- and
+// with it the workspace layout up to the slabs -- is the same for both passes.
+inline int huge_workgroups(int64_t N) {
+  const size_t slab = (size_t)(N + 31) / 32 * 4 + (size_t)N * 8 + 1;
+  const size_t fit = kHugeSlabBudget / slab;
+  return (int)(fit < (size_t)kMinHugeWorkgroups ? kMinHugeWorkgroups
+                                                : (fit > (size_t)kMaxHugeWorkgroups ? kMaxHugeWorkgroups : fit));
+}
 
 __device__ __forceinline__ int hash_slot(int key, int mask) {
   return (int)(((unsigned)key * 2654435761u) >> 12) & mask;
@@ -137,8 +152,8 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
 // ---- pass 0: products per row, and the lists of rows too big for a wavefront ----
 __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
-    const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ medium_rows,
-    int *__restrict__ huge_rows, int *__restrict__ counters) {
+    const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ small_rows,
+    int *__restrict__ medium_rows, int *__restrict__ huge_rows, int *__restrict__ counters) {
   constexpr int G = 8;  // lanes per row
   const int64_t row = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
   const int t = threadIdx.x % G;
@@ -154,7 +169,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
     products[row] = bound;
     if (bound > kMediumProducts) huge_rows[atomicAdd(&counters[1], 1)] = (int)row;
-    else if (bound > kTinyProducts) medium_rows[atomicAdd(&counters[0], 1)] = (int)row;
+    else if (bound > kSmallProducts) medium_rows[atomicAdd(&counters[0], 1)] = (int)row;
+    else if (bound > kTinyProducts) small_rows[atomicAdd(&counters[2], 1)] = (int)row;
   }
 }
 
@@ -228,28 +244,29 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
   }
 }
 
-// ---- rows of at most kMediumProducts products: one workgroup each -------------------
-template <typename T, bool NUMERIC>
+// ---- rows of at most PRODUCTS products: one workgroup each, 2 * PRODUCTS hash slots ----
+template <typename T, bool NUMERIC, int PRODUCTS, int COUNTER>
 __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, const int *__restrict__ counters, int *__restrict__ c_pos,
     int *__restrict__ c_crd, T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
-  __shared__ int s_keys[kMediumSlots];
-  __shared__ A s_vals[NUMERIC ? kMediumSlots : 1];
-  __shared__ int s_ck[NUMERIC ? kMediumProducts : 1];
-  __shared__ A s_cv[NUMERIC ? kMediumProducts : 1];
+  constexpr int kSlots = 2 * PRODUCTS;
+  __shared__ int s_keys[kSlots];
+  __shared__ A s_vals[NUMERIC ? kSlots : 1];
+  __shared__ int s_ck[NUMERIC ? PRODUCTS : 1];
+  __shared__ A s_cv[NUMERIC ? PRODUCTS : 1];
   __shared__ int s_scan[kWavesPerBlock + 1];
 
   const int tid = threadIdx.x;
   const int lane = wave_lane();
   const int w = tid / kWaveSize;
-  const int n_rows = counters[0];
+  const int n_rows = counters[COUNTER];
 
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
     const int row = rows[idx];
-    for (int s = tid; s < kMediumSlots; s += kBlockThreads) {
+    for (int s = tid; s < kSlots; s += kBlockThreads) {
       s_keys[s] = -1;
       if (NUMERIC) s_vals[s] = (A)0;
     }
@@ -260,7 +277,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       const int j = uniform(a_crd[p]);
       const A av = NUMERIC ? (A)a_val[p] : (A)0;
       for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
-        const int slot = hash_insert(s_keys, kMediumSlots - 1, b_crd[q]);
+        const int slot = hash_insert(s_keys, kSlots - 1, b_crd[q]);
         if (NUMERIC) atomic_accumulate<A>(&s_vals[slot], av * (A)b_val[q]);
       }
     }
@@ -268,7 +285,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
 
     // Each thread owns a contiguous run of slots; an exclusive scan of the
     // per-thread counts places the occupied ones.
-    constexpr int kRun = kMediumSlots / kBlockThreads;
+    constexpr int kRun = kSlots / kBlockThreads;
     int mine = 0;
     for (int s = 0; s < kRun; ++s) mine += s_keys[tid * kRun + s] != -1 ? 1 : 0;
     int n = 0;
@@ -394,7 +411,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_huge_kernel(
 
 // ---- host side ------------------------------------------------------------------------------
 struct SpgemmWorkspace {
-  int *products, *medium_rows, *huge_rows, *counters;
+  int *products, *small_rows, *medium_rows, *huge_rows, *counters;
+  int huge_pool;
   int *scan_totals;
   unsigned *bitmaps;
   void *dense;
@@ -408,12 +426,14 @@ inline SpgemmWorkspace spgemm_layout(char *base, int64_t M, int64_t N, size_t el
   size_t off = 0;
   auto take = [&](size_t bytes) { char *p = base ? base + off : nullptr; off += round256(bytes); return p; };
   ws.products = reinterpret_cast<int *>(take((size_t)M * 4));
+  ws.small_rows = reinterpret_cast<int *>(take((size_t)M * 4));
   ws.medium_rows = reinterpret_cast<int *>(take((size_t)M * 4));
   ws.huge_rows = reinterpret_cast<int *>(take((size_t)M * 4));
   ws.counters = reinterpret_cast<int *>(take(16));
   ws.scan_totals = reinterpret_cast<int *>(take(((size_t)(M + 1) / kScanTile + 1) * 4));
-  ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)kHugeWorkgroups * ((size_t)(N + 31) / 32) * 4));
-  ws.dense = take((size_t)kHugeWorkgroups * (size_t)N * elem);
+  ws.huge_pool = huge_workgroups(N);
+  ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
+  ws.dense = take((size_t)ws.huge_pool * (size_t)N * elem);
   ws.total = off;
   return ws;
 }
@@ -447,18 +467,21 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned row_groups = (unsigned)(((int64_t)M * 8 + kBlockThreads - 1) / kBlockThreads);
   spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, a_pos, a_crd, b_pos, ws.products,
-                                                                ws.medium_rows, ws.huge_rows,
-                                                                ws.counters);
+                                                                ws.small_rows, ws.medium_rows,
+                                                                ws.huge_rows, ws.counters);
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned tiny_blocks = (unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock);
   spgemm_tiny_kernel<T, NUMERIC><<<tiny_blocks, kBlockThreads, 0, stream>>>(
       M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned medium_blocks = (unsigned)(M < kMediumWorkgroups ? M : kMediumWorkgroups);
-  spgemm_medium_kernel<T, NUMERIC><<<medium_blocks, kBlockThreads, 0, stream>>>(
+  spgemm_medium_kernel<T, NUMERIC, kSmallProducts, 2><<<medium_blocks, kBlockThreads, 0, stream>>>(
+      a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.small_rows, ws.counters, c_pos, c_crd, c_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
       a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  spgemm_huge_kernel<T, NUMERIC><<<kHugeWorkgroups, kBlockThreads, 0, stream>>>(
+  spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kBlockThreads, 0, stream>>>(
       N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
       static_cast<A *>(ws.dense), c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
