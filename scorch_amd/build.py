@@ -24,6 +24,9 @@ HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
     # packed fp32 instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results stay in ordinary vector registers: the attention kernel feeds them
+    # straight to vector instructions, and accumulator registers would cost copies
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
 ]
 

@@ -42,6 +42,7 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 typedef short4v __attribute__((address_space(3))) lds_short4v;
 
+template <bool NEGATIVE_SCALE>
 __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
     const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
@@ -130,33 +131,34 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     floatx4 st[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const bf16x8 k_op = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g + 32 * s]);
-        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_op, q_op[s], st[t], 0, 0, 0);
-      }
+      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g]);
+      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g + 32]);
+      st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_lo, q_op[0], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_hi, q_op[1], st[t], 0, 0, 0);
     }
 
     // Online softmax for query n, in base 2: this lane holds keys 16t + 4g + r.
-    float mx = -3.0e38f;
+    // With scale > 0 the maximum of the scaled scores is the scaled maximum.
+    float mx = st[0][0];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        st[t][r] *= scale_log2e;
-        mx = fmaxf(mx, st[t][r]);
-      }
+      for (int r = 0; r < 4; ++r) mx = NEGATIVE_SCALE ? fminf(mx, st[t][r]) : fmaxf(mx, st[t][r]);
+    mx *= scale_log2e;
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    // Rescale what has been accumulated only when some query's maximum moved
+    // (after the first few key blocks it rarely does).
+    if (__any(m_new > m_run)) {
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
+    }
     m_run = m_new;
-    l_run *= alpha;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
 
     // P^T as the B operand of the second product: slot j of step s is key
     // 32s + 16 (j / 4) + 4g + (j % 4).
@@ -165,7 +167,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(st[t][r] - m_new);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_new));
         l_run += p;
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
@@ -239,10 +241,17 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
   const int n_blocks = (int)(S / kAttnBlock);
   const dim3 grid((unsigned)(n_blocks * H));
   const float scale_log2e = scale * 1.4426950408889634f;
-  attn_blocksparse_kernel<<<grid, kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
-      (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, static_cast<const __bf16 *>(Q),
-      static_cast<const __bf16 *>(K), static_cast<const __bf16 *>(V), scale_log2e,
-      static_cast<__bf16 *>(O));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const __bf16 *q = static_cast<const __bf16 *>(Q), *k = static_cast<const __bf16 *>(K),
+               *v = static_cast<const __bf16 *>(V);
+  if (scale < 0.0f)
+    attn_blocksparse_kernel<true><<<grid, kBlockThreads, 0, s>>>(
+        (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
+        static_cast<__bf16 *>(O));
+  else
+    attn_blocksparse_kernel<false><<<grid, kBlockThreads, 0, s>>>(
+        (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
+        static_cast<__bf16 *>(O));
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }
