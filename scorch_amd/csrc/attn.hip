@@ -93,39 +93,48 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   const int kb_begin = block_row_ptr[qb];
   const int kb_end = block_row_ptr[qb + 1];
 
-  // Staging: thread handles two 16-byte pieces of each tile; piece c covers
-  // row c / 8 (a key), features 8 (c % 8) .. + 7.
-  bf16x8 k_stage[2], v_stage[2];
-  auto load_tile = [&](int it) {
+  // Staging: a thread handles two 16-byte pieces of each tile; piece c covers
+  // row c / 8 (a key), features 8 (c % 8) .. + 7.  Tiles alternate between two
+  // register sets and two LDS buffers by parity: while tile `it` is consumed
+  // from LDS, tile it + 1 waits in registers and tile it + 2 is being fetched,
+  // so a fetch has a whole key block of work to hide behind.
+  bf16x8 k_stage[2][2], v_stage[2][2];
+  auto load_tile = [&](auto set_tag, int it) {
+    constexpr int kSet = decltype(set_tag)::value;
     const int kb = block_col_idx[it];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c = tid + u * kBlockThreads;
       const size_t off = (size_t)(kb * kAttnBlock + (c >> 3)) * kAttnDim + (c & 7) * 8;
-      k_stage[u] = *reinterpret_cast<const bf16x8 *>(Kh + off);
-      v_stage[u] = *reinterpret_cast<const bf16x8 *>(Vh + off);
+      k_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(Kh + off);
+      v_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(Vh + off);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](auto set_tag) {  // register set p -> LDS buffer p
+    constexpr int kSet = decltype(set_tag)::value;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int c = tid + u * kBlockThreads;
       const int key = c >> 3, f0 = (c & 7) * 8;
-      *reinterpret_cast<bf16x8 *>(&s_k[buf][key][f0]) = k_stage[u];
-      *reinterpret_cast<bf16x8 *>(&s_v[buf][key][f0]) = v_stage[u];
+      *reinterpret_cast<bf16x8 *>(&s_k[kSet][key][f0]) = k_stage[kSet][u];
+      *reinterpret_cast<bf16x8 *>(&s_v[kSet][key][f0]) = v_stage[kSet][u];
     }
   };
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
 
   if (kb_begin < kb_end) {
-    load_tile(kb_begin);
-    store_tile(0);
+    load_tile(Even{}, kb_begin);
+    store_tile(Even{});
+    if (kb_begin + 1 < kb_end) load_tile(Odd{}, kb_begin + 1);
   }
   __syncthreads();
 
-  for (int it = kb_begin; it < kb_end; ++it) {
-    const int buf = (it - kb_begin) & 1;
-    const bool more = it + 1 < kb_end;
-    if (more) load_tile(it + 1);
+  // One key block: tile `it` has parity P = decltype(tag)::value.
+  auto key_block = [&](auto tag, int it) {
+    constexpr int buf = decltype(tag)::value;
+    using Other = std::integral_constant<int, buf ^ 1>;
+    if (it + 2 < kb_end) load_tile(tag, it + 2);  // this parity's registers are free again
 
     // S^T tile t: keys 16t .. 16t+15 (rows) x 16 queries (columns).
     floatx4 st[4];
@@ -192,8 +201,13 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
         o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
       }
 
-    if (more) store_tile(buf ^ 1);
+    if (it + 1 < kb_end) store_tile(Other{});
     __syncthreads();
+  };
+
+  for (int it = kb_begin; it < kb_end; it += 2) {
+    key_block(Even{}, it);
+    if (it + 1 < kb_end) key_block(Odd{}, it + 1);
   }
 
   // Normalise and store O[query][16dt + 4g .. + 3] (8 bytes per tile and lane).

@@ -116,3 +116,28 @@ def test_full_size_workload():
         worst = max(worst, err)
         del s, ref
     assert worst <= TOL_BF16, worst
+
+
+def test_negative_scale(oracle):
+    w, q, k, v = bf16_inputs(256, 2, 64, 7)
+    out = H.attn_blocksparse_bf16(q.cuda(), k.cuda(), v.cuda(), dev(w["block_row_ptr"]),
+                                  dev(w["block_col_idx"]), -0.25).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            w["block_row_ptr"], w["block_col_idx"], 64, -0.25)
+    assert oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+@pytest.mark.parametrize("blocks_per_row", [1, 2, 3, 5])
+def test_short_and_odd_block_rows(oracle, blocks_per_row):
+    """Every block row has the same small number of key blocks (the tile pipeline's start-up cases)."""
+    S, nb = 512, 8
+    rng = np.random.default_rng(blocks_per_row)
+    cols = np.stack([np.sort(rng.choice(nb, blocks_per_row, replace=False)) for _ in range(nb)])
+    brp = (np.arange(nb + 1) * blocks_per_row).astype(np.int32)
+    bci = cols.reshape(-1).astype(np.int32)
+    q, k, v = (torch.from_numpy(rng.standard_normal((8, S, 64)).astype(np.float32)).to(torch.bfloat16)
+               for _ in range(3))
+    out = H.attn_blocksparse_bf16(q.cuda(), k.cuda(), v.cuda(), dev(brp), dev(bci), 0.125).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            brp, bci, 64, 0.125)
+    assert oracle.rel_fro(out, ref) <= TOL_BF16
