@@ -173,6 +173,25 @@ def side_workload(args, dev) -> int:
                           "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
                           "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
         return 0
+    if args.workload in ("spmv_powerlaw", "softmax_powerlaw"):
+        w = workloads.gcn_powerlaw(M=args.rows, N=1)
+        M, nnz = w["M"], int(w["col_idx"].size)
+        pos, crd, val = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"])
+        x = t(w["B"]).reshape(-1)
+        if args.workload == "spmv_powerlaw":
+            fn = lambda: H.prebuilt_spmv_csr_f32([M], [M, M], [[], [pos, crd]], val, [M], [[]], x)
+            algo, flops, name = 8 * nnz + 4 * (M + 1) + 8 * M, 2.0 * nnz, "CSR SpMV GFLOP/s"
+        else:
+            fn = lambda: H.softmax_csr_float(pos, val, 1.0)
+            algo, flops, name = 8 * nnz + 4 * (M + 1), 4.0 * nnz, "CSR row softmax GFLOP/s (4 flops per entry)"
+        ms = _time_steps(fn, args.steps, args.warmup)
+        print(json.dumps({"metric": name, "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
+                          "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                          "dtype": "f32", "data": "synthetic", "higher_is_better": True,
+                          "config": {"workload": args.workload + "_fp32", "rows": M, "nnz": nnz},
+                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                          "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}))
+        return 0
     if args.workload == "spgemm_powerlaw":
         # A @ A for the power-law graph at 1/8 of the headline size (the square of the
         # full graph has billions of products)
@@ -245,7 +264,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="gcn_powerlaw",
                     choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
-                             "attention_blocksparse", "spgemm_powerlaw"],
+                             "attention_blocksparse", "spgemm_powerlaw", "spmv_powerlaw",
+                             "softmax_powerlaw"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "

@@ -157,19 +157,24 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_f32(int64_t M, int64_t n_cols, int64_t K
  * SpMV: y[M] = A_csr[M,K] * x[K].
  * Replaces spmv_csr<T> (csrc/kernels.h:13-49), bound as
  * prebuilt_spmv_csr_{f32,f64,i32,i64} (csrc/ops.cpp:52-61,100-101).
+ * Every element of y is written.  `workspace` (partial sums of rows split
+ * between wavefronts): scorch_hip_spmv_csr_workspace_bytes(M, nnz, sizeof(T))
+ * bytes, 256-byte aligned.  Results are bit-reproducible from run to run.
  * ---------------------------------------------------------------------- */
+SCORCH_HIP_API size_t scorch_hip_spmv_csr_workspace_bytes(int64_t M, int64_t nnz, size_t elem_size);
+
 SCORCH_HIP_API int scorch_hip_spmv_csr_f32(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
                             const int32_t *col_idx, const float *vals, const float *x,
-                            float *y, void *stream);
+                            float *y, void *workspace, size_t workspace_bytes, void *stream);
 SCORCH_HIP_API int scorch_hip_spmv_csr_f64(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
                             const int32_t *col_idx, const double *vals, const double *x,
-                            double *y, void *stream);
+                            double *y, void *workspace, size_t workspace_bytes, void *stream);
 SCORCH_HIP_API int scorch_hip_spmv_csr_i32(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
                             const int32_t *col_idx, const int32_t *vals, const int32_t *x,
-                            int32_t *y, void *stream);
+                            int32_t *y, void *workspace, size_t workspace_bytes, void *stream);
 SCORCH_HIP_API int scorch_hip_spmv_csr_i64(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
                             const int32_t *col_idx, const int64_t *vals, const int64_t *x,
-                            int64_t *y, void *stream);
+                            int64_t *y, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * SpGEMM: C_csr[M,N] = A_csr[M,K] * B_csr[K,N], in two calls.

@@ -1,4 +1,4 @@
-// Smaller kernels around the SpMM/SDDMM path: SpMV, CSR row softmax, the
+// Smaller kernels around the SpMM/SDDMM path: CSR row softmax, the
 // CSR -> coordinate row expansion, and the library's error/version calls.
 #include "common.hpp"
 
@@ -9,60 +9,13 @@ char *error_buffer() {
   return buf;
 }
 
-// ---- SpMV -------------------------------------------------------------------
-// One group of G lanes per row (G a power of two chosen from the mean row
-// length): the lanes stride over the row's entries and a butterfly reduction
-// adds their partial sums, so the summation order depends only on G.
-template <typename T, int G>
-__global__ __launch_bounds__(kBlockThreads) void spmv_kernel(int M, const int *__restrict__ row_ptr,
-                                                             const int *__restrict__ col_idx,
-                                                             const T *__restrict__ vals,
-                                                             const T *__restrict__ x,
-                                                             T *__restrict__ y) {
-  using A = typename Acc<T>::type;
-  const int64_t group = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
-  const int t = threadIdx.x % G;
-  const bool live = group < M;
-  A acc = (A)0;
-  if (live) {
-    const int lo = row_ptr[group], hi = row_ptr[group + 1];
-    for (int p = lo + t; p < hi; p += G) acc += (A)vals[p] * (A)x[col_idx[p]];
-  }
-#pragma unroll
-  for (int off = G / 2; off > 0; off >>= 1) acc += (A)__shfl_xor((T)acc, off);
-  if (live && t == 0) y[group] = (T)acc;
-}
-
+// Lanes per row for the group-per-row kernels: the power of two nearest above
+// the mean row length, between 2 and 64.
 inline int group_width(int64_t M, int64_t nnz) {
   const int64_t mean = M > 0 ? (nnz + M - 1) / M : 0;
   int g = 2;
   while (g < kWaveSize && g < mean) g *= 2;
   return g;
-}
-
-template <typename T>
-int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
-               const int32_t *col_idx, const T *vals, const T *x, T *y, void *stream) {
-  if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
-  if (M == 0) return SCORCH_HIP_OK;
-  SCORCH_REQUIRE(y != nullptr, "%s: y is NULL", fn);
-  SCORCH_REQUIRE(K == 0 || x != nullptr, "%s: x is NULL", fn);
-  SCORCH_REQUIRE(aligned_to(x, sizeof(T)) && aligned_to(y, sizeof(T)) && aligned_to(vals, sizeof(T)),
-                 "%s: value arrays must be aligned to their element size", fn);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int g = group_width(M, nnz);
-  const int64_t threads = M * g;
-  const dim3 grid((unsigned)((threads + kBlockThreads - 1) / kBlockThreads));
-  switch (g) {
-    case 2: spmv_kernel<T, 2><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-    case 4: spmv_kernel<T, 4><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-    case 8: spmv_kernel<T, 8><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-    case 16: spmv_kernel<T, 16><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-    case 32: spmv_kernel<T, 32><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-    default: spmv_kernel<T, 64><<<grid, kBlockThreads, 0, s>>>((int)M, row_ptr, col_idx, vals, x, y); break;
-  }
-  SCORCH_HIP_CHECK(hipGetLastError());
-  return SCORCH_HIP_OK;
 }
 
 // ---- CSR row softmax ----------------------------------------------------------
@@ -120,19 +73,6 @@ extern "C" {
 int scorch_hip_abi_version(void) { return SCORCH_HIP_ABI_VERSION; }
 
 const char *scorch_hip_last_error(void) { return scorch::error_buffer(); }
-
-#define SCORCH_DEFINE_SPMV(SUFFIX, T)                                                           \
-  int scorch_hip_spmv_csr_##SUFFIX(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,   \
-                                   const int32_t *col_idx, const T *vals, const T *x, T *y,     \
-                                   void *stream) {                                              \
-    return scorch::spmv_entry<T>("scorch_hip_spmv_csr_" #SUFFIX, M, K, nnz, row_ptr, col_idx,   \
-                                 vals, x, y, stream);                                           \
-  }
-
-SCORCH_DEFINE_SPMV(f32, float)
-SCORCH_DEFINE_SPMV(f64, double)
-SCORCH_DEFINE_SPMV(i32, int32_t)
-SCORCH_DEFINE_SPMV(i64, int64_t)
 
 int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, const float *vals,
                                float scale, float *out, void *stream) {

@@ -414,6 +414,129 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
   return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
 }
 
+
+// ---- SpMV: the same merge-path split with one output column ------------------------------
+// A wavefront owns kSpmvItems consecutive items of the merged (row ends + nonzeros)
+// sequence.  Its lanes first form all products val * x[col] in parallel (coalesced
+// reads of col_idx / vals, gathered reads of x) and park them in LDS; then lane r
+// sums the products of the r-th row the chunk touches.  A row with many entries
+// in the chunk is summed by the whole wavefront instead (strided partial sums,
+// butterfly reduction).  The part of the last row that continues in the next
+// chunk becomes a carry, folded into y by spmm_fixup_kernel exactly as for SpMM,
+// so the summation order is fixed and results are bit-reproducible.
+constexpr int kSpmvItems = 512;
+constexpr int kSpmvLaneRowMax = 32;  // longer in-chunk rows are summed by the whole wavefront
+
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void spmv_merge_kernel(
+    int M, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
+    const T *__restrict__ vals, const T *__restrict__ x, T *__restrict__ y, int64_t total_items,
+    int *__restrict__ carry_row, T *__restrict__ carry_val) {
+  using A = typename Acc<T>::type;
+  __shared__ A s_prod[kWavesPerBlock][kSpmvItems];
+  __shared__ int s_rp[kWavesPerBlock][kSpmvItems + 2];
+
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  const int64_t span = (int64_t)blockIdx.x * kWavesPerBlock + w;
+  int64_t d0 = span * kSpmvItems;
+  if (d0 >= total_items) return;  // nothing here uses workgroup barriers
+  int64_t d1 = d0 + kSpmvItems;
+  d1 = d1 < total_items ? d1 : total_items;
+
+  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
+  const int x0 = wave_count_below(M, d0, row_end_key);
+  const int x1 = wave_count_below(M, d1, row_end_key);
+  const int y0 = uniform((int)(d0 - x0));
+  const int y1 = uniform((int)(d1 - x1));
+  const int n_nz = y1 - y0;
+  const int n_rows = x1 - x0;
+
+  for (int k = lane; k < n_nz; k += kWaveSize)
+    s_prod[w][k] = (A)vals[y0 + k] * (A)x[col_idx[y0 + k]];
+  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
+    const int r = x0 + k < M ? x0 + k : M;
+    s_rp[w][k] = row_ptr[r];
+  }
+  wave_lds_sync();
+
+  // Row slot r is row x0 + r; slot n_rows is the row that continues past the chunk.
+  for (int base = 0; base <= n_rows; base += kWaveSize) {
+    const int r = base + lane;
+    const bool live = r <= n_rows;
+    int lo = 0, hi = 0;
+    if (live) {
+      const int begin = s_rp[w][r], end = s_rp[w][r + 1];
+      lo = (begin > y0 ? begin : y0) - y0;
+      hi = (end < y1 ? end : y1) - y0;
+      if (hi < lo) hi = lo;
+    }
+    const int len = hi - lo;
+    A sum = (A)0;
+    if (len <= kSpmvLaneRowMax)
+      for (int k = lo; k < hi; ++k) sum += s_prod[w][k];
+    // rows with many entries in the chunk: one at a time, all lanes
+    unsigned long long pending = __ballot(len > kSpmvLaneRowMax);
+    while (pending) {
+      const int owner = __ffsll(pending) - 1;
+      pending &= pending - 1;
+      const int olo = __shfl(lo, owner), ohi = __shfl(hi, owner);
+      A part = (A)0;
+      for (int k = olo + lane; k < ohi; k += kWaveSize) part += s_prod[w][k];
+#pragma unroll
+      for (int off = kWaveSize / 2; off > 0; off >>= 1) part += (A)__shfl_xor((T)part, off);
+      if (lane == owner) sum = part;
+    }
+    if (live) {
+      if (r < n_rows) {
+        y[x0 + r] = (T)sum;
+      } else {
+        carry_row[span] = len > 0 ? x1 : -1;
+        if (len > 0) carry_val[span] = (T)sum;
+      }
+    }
+  }
+}
+
+inline int64_t spmv_num_spans(int64_t M, int64_t nnz) {
+  return (M + nnz + kSpmvItems - 1) / kSpmvItems;
+}
+
+inline size_t spmv_workspace_bytes(int64_t M, int64_t nnz, size_t elem) {
+  const size_t spans = (size_t)spmv_num_spans(M, nnz);
+  return align_up(spans * sizeof(int), 256) + align_up(spans * elem, 256);
+}
+
+template <typename T>
+int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+               const int32_t *col_idx, const T *vals, const T *x, T *y, void *workspace,
+               size_t workspace_bytes, void *stream) {
+  if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
+  if (M == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(y != nullptr, "%s: y is NULL", fn);
+  SCORCH_REQUIRE(K == 0 || x != nullptr, "%s: x is NULL", fn);
+  SCORCH_REQUIRE(aligned_to(x, sizeof(T)) && aligned_to(y, sizeof(T)) && aligned_to(vals, sizeof(T)),
+                 "%s: value arrays must be aligned to their element size", fn);
+  const size_t need = spmv_workspace_bytes(M, nnz, sizeof(T));
+  if (!workspace || workspace_bytes < need)
+    return fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
+                workspace ? workspace_bytes : (size_t)0);
+  SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t spans = spmv_num_spans(M, nnz);
+  int *carry_row = static_cast<int *>(workspace);
+  T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
+                                       align_up((size_t)spans * sizeof(int), 256));
+  const int64_t blocks = (spans + kWavesPerBlock - 1) / kWavesPerBlock;
+  spmv_merge_kernel<T><<<dim3((unsigned)blocks), kBlockThreads, 0, s>>>(
+      (int)M, row_ptr, col_idx, vals, x, y, M + nnz, carry_row, carry_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  spmm_fixup_kernel<T, 1, kEpiNone><<<dim3((unsigned)blocks), kBlockThreads, 0, s>>>(
+      1, spans, 1, blocks, carry_row, carry_val, y, nullptr);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
 }  // namespace scorch
 
 extern "C" {
@@ -437,6 +560,24 @@ SCORCH_DEFINE_SPMM(f32, float)
 SCORCH_DEFINE_SPMM(f64, double)
 SCORCH_DEFINE_SPMM(i32, int32_t)
 SCORCH_DEFINE_SPMM(i64, int64_t)
+
+size_t scorch_hip_spmv_csr_workspace_bytes(int64_t M, int64_t nnz, size_t elem_size) {
+  if (M < 0 || nnz < 0 || elem_size == 0) return 0;
+  return scorch::spmv_workspace_bytes(M, nnz, elem_size);
+}
+
+#define SCORCH_DEFINE_SPMV(SUFFIX, T)                                                           \
+  int scorch_hip_spmv_csr_##SUFFIX(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,   \
+                                   const int32_t *col_idx, const T *vals, const T *x, T *y,     \
+                                   void *workspace, size_t workspace_bytes, void *stream) {     \
+    return scorch::spmv_entry<T>("scorch_hip_spmv_csr_" #SUFFIX, M, K, nnz, row_ptr, col_idx,   \
+                                 vals, x, y, workspace, workspace_bytes, stream);               \
+  }
+
+SCORCH_DEFINE_SPMV(f32, float)
+SCORCH_DEFINE_SPMV(f64, double)
+SCORCH_DEFINE_SPMV(i32, int32_t)
+SCORCH_DEFINE_SPMV(i64, int64_t)
 
 int scorch_hip_spmm_csr_f32_timed(int64_t M, int64_t K, int64_t N, int64_t nnz,
                                   const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

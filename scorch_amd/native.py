@@ -21,7 +21,7 @@ OK, EINVAL, EWORKSPACE, ERUNTIME, EUNSUPPORTED = 0, 1, 2, 3, 4
 
 _SPMM = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 _SPGEMM = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
-_SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
+_SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 
 # name -> (restype, argtypes); one entry per declaration in include/scorch_hip.h
 SIGNATURES = {
@@ -46,6 +46,7 @@ SIGNATURES = {
                                                 _ptr, _ptr]),
     "scorch_hip_sddmm_csr_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr,
                                                 _ptr, _ptr, _ptr]),
+    "scorch_hip_spmv_csr_workspace_bytes": (_size, [_i64, _i64, _size]),
     "scorch_hip_spmv_csr_f32": (ctypes.c_int, _SPMV),
     "scorch_hip_spmv_csr_f64": (ctypes.c_int, _SPMV),
     "scorch_hip_spmv_csr_i32": (ctypes.c_int, _SPMV),

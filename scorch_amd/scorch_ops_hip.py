@@ -214,10 +214,14 @@ def _make_spmv(dtype):
             raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
         dev = _device_of(pos, crd, a_val, x)
         y = torch.empty(M, dtype=dtype, device=dev)
+        L = native.lib()
         with torch.cuda.device(dev):
-            fn = getattr(native.lib(), "scorch_hip_spmv_csr_" + _SUFFIX[dtype])
+            stream = _stream(dev)
+            ws = _workspace(dev, stream, L.scorch_hip_spmv_csr_workspace_bytes(M, a_val.numel(),
+                                                                              a_val.element_size()))
+            fn = getattr(L, "scorch_hip_spmv_csr_" + _SUFFIX[dtype])
             rc = fn(M, K, a_val.numel(), pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), x.data_ptr(),
-                    y.data_ptr(), _stream(dev))
+                    y.data_ptr(), ws.data_ptr(), ws.numel(), stream)
         native.check(rc)
         return Tensor(y, [[]])
     return kernel

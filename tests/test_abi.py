@@ -107,9 +107,11 @@ def test_sddmm_rejects_bad_arguments(L):
 
 
 def test_spmv_softmax_rows_reject_bad_arguments(L):
-    assert L.scorch_hip_spmv_csr_f64(4, 4, 4, FAKE, FAKE, FAKE, FAKE, NULL, NULL) == native.EINVAL
-    assert L.scorch_hip_spmv_csr_i32(-4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EINVAL
-    assert L.scorch_hip_spmv_csr_i64(0, 4, 0, FAKE, NULL, NULL, NULL, NULL, NULL) == native.OK
+    assert L.scorch_hip_spmv_csr_f64(4, 4, 4, FAKE, FAKE, FAKE, FAKE, NULL, FAKE, 1 << 20, NULL) == native.EINVAL
+    assert L.scorch_hip_spmv_csr_i32(-4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1 << 20, NULL) == native.EINVAL
+    assert L.scorch_hip_spmv_csr_i64(0, 4, 0, FAKE, NULL, NULL, NULL, NULL, NULL, 0, NULL) == native.OK
+    assert L.scorch_hip_spmv_csr_f32(4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, 0, NULL) == native.EWORKSPACE
+    assert L.scorch_hip_spmv_csr_workspace_bytes(1000, 5000, 4) % 256 == 0
     assert L.scorch_hip_softmax_csr_f32(4, 4, NULL, FAKE, 1.0, FAKE, NULL) == native.EINVAL
     assert L.scorch_hip_softmax_csr_f32(4, 4, FAKE, NULL, 1.0, FAKE, NULL) == native.EINVAL
     assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL

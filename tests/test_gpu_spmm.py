@@ -239,3 +239,37 @@ def test_power_law_full_size_properties():
     B2 = torch.roll(B, 1, dims=0)
     lin = run(B + B2) - (C + run(B2))
     assert (torch.linalg.norm(lin.double()) / torch.linalg.norm(C.double())).item() <= 1e-5
+
+
+# ---- SpMV shares the merge-path split -----------------------------------------------------------
+@pytest.mark.parametrize("name", sorted(ROW_CASES))
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
+def test_spmv_row_length_distributions(oracle, name, dtype):
+    from gpu_util import hip_spmv
+    rp, ci = ROW_CASES[name]
+    rng = np.random.default_rng(len(name))
+    if np.issubdtype(dtype, np.integer):
+        v = rng.integers(-1000, 1000, ci.size).astype(dtype)
+        x = rng.integers(-1000, 1000, 500).astype(dtype)
+    else:
+        v = rng.uniform(-1, 1, ci.size).astype(dtype)
+        x = rng.standard_normal(500).astype(dtype)
+    got = hip_spmv(rp, ci, v, x)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(got, oracle.spmv_csr_typed(rp, ci, v, x))
+    else:
+        ref64 = oracle.spmm_fp64(rp, ci, v, x.reshape(-1, 1)).reshape(-1)
+        assert oracle.rel_fro(got, ref64) <= (TOL if dtype == np.float32 else 1e-13)
+    assert not got[np.diff(rp) == 0].any()
+
+
+def test_spmv_full_size_and_reproducible():
+    w = workloads.gcn_powerlaw(N=1)
+    M = w["M"]
+    rp, ci, v, x = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"]), dev(w["B"]).reshape(-1)
+    call = lambda: H.prebuilt_spmv_csr_f32([M], [M, M], [[], [rp, ci]], v, [M], [[]], x).storage.value
+    y = call()
+    assert torch.equal(y, call())
+    A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), v.double(), size=(M, M))
+    ref = torch.mv(A64, x.double())
+    assert (torch.linalg.norm(y.double() - ref) / torch.linalg.norm(ref)).item() <= TOL
