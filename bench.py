@@ -276,7 +276,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (the kernel shards by rows "
-              "of A with no reduction; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "of A, every GPU writing its own rows of C, with no reduction). Run with --gpus 1.", file=sys.stderr)
         return 2
 
     import torch
