@@ -19,9 +19,12 @@ inline int group_width(int64_t M, int64_t nnz) {
 }
 
 // ---- CSR row softmax ----------------------------------------------------------
-// One group of G lanes per row; three sweeps over the row (maximum, sum of
-// exponentials, normalised write).  The row is re-read from cache, not kept in
+// One group of G lanes per row (rows of up to kSoftmaxLongRow entries); three
+// sweeps over the row (maximum, sum of exponentials, normalised write).  The row is re-read from cache, not kept in
 // registers, so any row length works.
+constexpr int kSoftmaxLongRow = 256;   // longer rows get a whole workgroup
+constexpr int kSoftmaxLongWorkgroups = 2048;
+
 template <int G>
 __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                                     const int *__restrict__ row_ptr,
@@ -34,6 +37,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   if (live) {
     lo = row_ptr[group];
     hi = row_ptr[group + 1];
+    if (hi - lo > kSoftmaxLongRow) hi = lo;  // softmax_csr_long_kernel owns this row
   }
   float mx = -3.402823466e38f;
   for (int p = lo + t; p < hi; p += G) mx = fmaxf(mx, vals[p] * scale);
@@ -44,6 +48,44 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
 #pragma unroll
   for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   for (int p = lo + t; p < hi; p += G) out[p] = expf(vals[p] * scale - mx) / sum;
+}
+
+// Rows longer than kSoftmaxLongRow: one workgroup per row, the same three sweeps
+// with workgroup-wide reductions (fixed order: lanes, then wavefronts).  A fixed
+// pool of workgroups scans the row pointer for such rows.
+__device__ __forceinline__ float block_reduce(float v, float *scratch, bool take_max) {
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off);
+    v = take_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads();
+  if (lane == 0) scratch[w] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < kWavesPerBlock; ++i) r = take_max ? fmaxf(r, scratch[i]) : r + scratch[i];
+  return r;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void softmax_csr_long_kernel(int M,
+                                                                         const int *__restrict__ row_ptr,
+                                                                         const float *vals, float scale,
+                                                                         float *out) {
+  __shared__ float s_red[kWavesPerBlock];
+  for (int row = blockIdx.x; row < M; row += gridDim.x) {
+    const int lo = row_ptr[row], hi = row_ptr[row + 1];
+    if (hi - lo <= kSoftmaxLongRow) continue;  // uniform across the workgroup
+    float mx = -3.402823466e38f;
+    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) mx = fmaxf(mx, vals[p] * scale);
+    mx = block_reduce(mx, s_red, true);
+    float sum = 0.0f;
+    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) sum += expf(vals[p] * scale - mx);
+    sum = block_reduce(sum, s_red, false);
+    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) out[p] = expf(vals[p] * scale - mx) / sum;
+  }
 }
 
 // ---- CSR -> coordinate rows ---------------------------------------------------
@@ -96,6 +138,9 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
     case 32: scorch::softmax_csr_kernel<32><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
     default: scorch::softmax_csr_kernel<64><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
   }
+  SCORCH_HIP_CHECK(hipGetLastError());
+  const unsigned pool = (unsigned)(M < scorch::kSoftmaxLongWorkgroups ? M : scorch::kSoftmaxLongWorkgroups);
+  scorch::softmax_csr_long_kernel<<<pool, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out);
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }
