@@ -203,6 +203,151 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
   }
 }
 
+// ---- narrow column tiles: one lane group per row --------------------------------------------
+// When a column tile is narrower than a wavefront's 64 lanes can cover with
+// full vectors, the wavefront is divided into G = 64 / LPR groups of LPR lanes
+// and every group works on a different row of the chunk: group g takes the
+// chunk's row slots g, g + G, ... and walks each one's nonzeros itself (up to
+// four B-row loads in flight per group, so 4 G per wavefront).  No reduction
+// between groups is needed, since a row is summed by one group.  A row with many
+// nonzeros in the chunk would leave the other groups idle: such rows are summed
+// by all groups together (strided over its nonzeros, then combined with
+// shuffles in a fixed order).  Used for small N, and for large N when narrow
+// tiles let the B rows a tile gathers stay in one L2 (see use_narrow_tiles).
+constexpr int kGroupRowMax = 24;  // longer in-chunk rows are shared by all groups
+
+template <typename T, int VEC, int LPR, int EPI>
+__global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
+    int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
+    const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
+    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int n_tiles,
+    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
+  using A = typename Acc<T>::type;
+  using VecT = Vec<T, VEC>;
+  constexpr int G = kWaveSize / LPR;
+
+  __shared__ int s_col[kWavesPerBlock][kItemsPerWave];
+  __shared__ T s_val[kWavesPerBlock][kItemsPerWave];
+  __shared__ int s_rp[kWavesPerBlock][kItemsPerWave + 2];
+
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  const int g = lane / LPR;
+  const int t = lane % LPR;
+  const TileMap where = map_workgroup(blockIdx.x, n_tiles, blocks_per_tile);
+  const int64_t span = where.block * kWavesPerBlock + w;
+  const int col0 = (where.tile * LPR + t) * VEC;
+  const bool active = col0 < N;
+
+  int64_t d0 = span * items_per_chunk;
+  if (d0 >= total_items) return;  // only wave-level synchronisation below
+  int64_t d1 = d0 + items_per_chunk;
+  d1 = d1 < total_items ? d1 : total_items;
+
+  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
+  const int x0 = wave_count_below(M, d0, row_end_key);
+  const int x1 = wave_count_below(M, d1, row_end_key);
+  const int y0 = uniform((int)(d0 - x0));
+  const int y1 = uniform((int)(d1 - x1));
+  const int n_nz = y1 - y0;
+  const int n_rows = x1 - x0;
+
+  for (int k = lane; k < n_nz; k += kWaveSize) {
+    s_col[w][k] = col_idx[y0 + k];
+    s_val[w][k] = vals[y0 + k];
+  }
+  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
+    const int r = x0 + k < M ? x0 + k : M;
+    s_rp[w][k] = row_ptr[r];
+  }
+  wave_lds_sync();
+
+  const bool carry_in = uniform(s_rp[w][0]) < y0;  // row x0 began in an earlier chunk
+  T bias_v[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) bias_v[v] = (EPI != kEpiNone && active) ? bias[col0 + v] : (T)0;
+
+  auto add_entry = [&](A (&acc)[VEC], int k) {
+    const A a = (A)s_val[w][k];
+    const VecT b = *reinterpret_cast<const VecT *>(B + (size_t)s_col[w][k] * (size_t)N + col0);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
+  };
+
+  // Row slot r is row x0 + r; slot n_rows is the row that continues past the chunk.
+  for (int base = 0; base <= n_rows; base += G) {
+    const int slot = base + g;
+    const bool live = slot <= n_rows;
+    int lo = 0, hi = 0;
+    if (live) {
+      const int begin = s_rp[w][slot], end = s_rp[w][slot + 1];
+      lo = (begin > y0 ? begin : y0) - y0;
+      hi = (end < y1 ? end : y1) - y0;
+      if (hi < lo) hi = lo;
+    }
+    const int len = hi - lo;
+    A acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+
+    if (active && len <= kGroupRowMax) {
+      int k = lo;
+      for (; k + 4 <= hi; k += 4) {
+        VecT b[4];
+        A a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          a[u] = (A)s_val[w][k + u];
+          b[u] = *reinterpret_cast<const VecT *>(B + (size_t)s_col[w][k + u] * (size_t)N + col0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) acc[v] += a[u] * (A)b[u].v[v];
+      }
+      for (; k < hi; ++k) add_entry(acc, k);
+    }
+
+    // Rows with many nonzeros in the chunk: one at a time, all groups.
+    unsigned long long pending = __ballot(len > kGroupRowMax && t == 0);
+    while (pending) {
+      const int owner_lane = __ffsll(pending) - 1;  // lane 0 of the owning group
+      pending &= pending - 1;
+      const int olo = __shfl(lo, owner_lane), ohi = __shfl(hi, owner_lane);
+      A part[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) part[v] = (A)0;
+      if (active)
+        for (int k = olo + g; k < ohi; k += G) add_entry(part, k);
+#pragma unroll
+      for (int off = LPR; off < kWaveSize; off <<= 1)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) part[v] += (A)__shfl_xor((T)part[v], off);
+      if (g == owner_lane / LPR) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = part[v];
+      }
+    }
+
+    if (live && active) {
+      VecT o;
+      if (slot < n_rows) {
+        const bool partial = carry_in && slot == 0;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+          o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
+        *reinterpret_cast<VecT *>(C + (size_t)(x0 + slot) * (size_t)N + col0) = o;
+      } else if (len > 0) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];
+        *reinterpret_cast<VecT *>(carry_val + (size_t)span * (size_t)N + col0) = o;
+      }
+    }
+    if (live && slot == n_rows && where.tile == 0 && t == 0) carry_row[span] = len > 0 ? x1 : -1;
+  }
+}
+
+
 // One wavefront per (chunk, column tile).  The first chunk of each run of
 // equal carry_row values sums the run in chunk order and folds it into C.
 template <typename T, int VEC, int EPI>
@@ -308,8 +453,11 @@ inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   return sp;
 }
 
+// Carry records the workspace must hold: the most any kernel variant produces
+// for this shape (one record per chunk of the wide-tile split).
 inline int64_t spmm_num_chunks(int64_t M, int64_t nnz, int64_t N, size_t elem) {
-  return spmm_split(M, nnz, N, elem).spans;
+  const SpmmSplit sp = spmm_split(M, nnz, N, elem);
+  return (M + nnz + sp.items_per_chunk - 1) / sp.items_per_chunk;
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -342,8 +490,9 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
   const SpmmSplit split = spmm_split(M, nnz, N, sizeof(T));
   const int64_t chunks = split.spans;
   int *carry_row = static_cast<int *>(workspace);
-  T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
-                                       align_up((size_t)chunks * sizeof(int), 256));
+  T *carry_val = reinterpret_cast<T *>(
+      static_cast<char *>(workspace) +
+      align_up((size_t)spmm_num_chunks(M, nnz, N, sizeof(T)) * sizeof(int), 256));
   const int tile = kWaveSize * VEC;
   const int n_tiles = (N + tile - 1) / tile;
   const int64_t blocks_per_tile = (chunks + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -362,6 +511,53 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
   return SCORCH_HIP_OK;
+}
+
+// Narrow-tile variant: lane groups of LPR lanes, tiles of LPR * VEC columns, one
+// chunk per wavefront.  The fix-up does not care how the main kernel tiled the
+// columns; it runs with scalar lanes over ceil(N / 64) tiles.
+template <typename T, int VEC, int LPR, int EPI>
+int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx,
+                        const T *vals, const T *B, const T *bias, T *C, void *workspace,
+                        hipStream_t stream) {
+  const int64_t total = (int64_t)M + nnz;
+  const int tile = LPR * VEC;
+  const int n_tiles = (N + tile - 1) / tile;
+  // as in spmm_split, with the real tile count: fill 8192 wavefront slots, at most 256 items each
+  const int64_t per_wave = total * n_tiles / 8192;
+  int ipc = kMinItemsPerWave;
+  while (ipc < kItemsPerWave && ipc * 2 <= per_wave) ipc *= 2;
+  const int wide_ipc = spmm_split(M, nnz, N, sizeof(T)).items_per_chunk;
+  if (ipc < wide_ipc) ipc = wide_ipc;  // never more carry records than the workspace holds
+  const int64_t spans = (total + ipc - 1) / ipc;
+  int *carry_row = static_cast<int *>(workspace);
+  T *carry_val = reinterpret_cast<T *>(
+      static_cast<char *>(workspace) +
+      align_up((size_t)spmm_num_chunks(M, nnz, N, sizeof(T)) * sizeof(int), 256));
+  const int64_t blocks_per_tile = (spans + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks_per_tile * n_tiles > INT32_MAX)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
+                (long long)(blocks_per_tile * n_tiles));
+  spmm_grouped_kernel<T, VEC, LPR, EPI><<<dim3((unsigned)(blocks_per_tile * n_tiles)), kBlockThreads, 0, stream>>>(
+      M, N, row_ptr, col_idx, vals, B, C, bias, total, ipc, n_tiles, blocks_per_tile, carry_row,
+      carry_val);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  const int fix_tiles = (N + kWaveSize - 1) / kWaveSize;
+  spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)(blocks_per_tile * fix_tiles)), kBlockThreads, 0, stream>>>(
+      N, spans, fix_tiles, blocks_per_tile, carry_row, carry_val, C, bias);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+// Narrow tiles pay off when N is small: a row of B is under 256 bytes, so
+// full-width tiles would leave most lanes idle.  Returns the tile width in
+// bytes, or 0 for wide tiles.  (Tiling a wide B by columns so that K narrow rows
+// stay in one XCD's L2 was measured and lost: the workgroups resident on an XCD
+// span several tiles at once and evict each other's slices.)
+inline int narrow_tile_bytes(int64_t K, int64_t N, int64_t nnz, size_t elem) {
+  (void)K; (void)nnz;
+  const int64_t row_bytes = N * (int64_t)elem;
+  return row_bytes < 256 ? (int)row_bytes : 0;
 }
 
 // Elements per lane.  Preferred: the widest vector (at most 16 bytes) that
@@ -403,8 +599,33 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
   SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
 
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int vec = pick_vec<T>(N, B, C, workspace);
   const int m = (int)M, n = (int)N;
+  if (const int tile_bytes = timer ? 0 : narrow_tile_bytes(K, N, nnz, sizeof(T))) {
+    // widest vector (at most 16 bytes) that divides N and is aligned; lanes to cover the tile
+    constexpr int kMaxVec = (int)(16 / sizeof(T));
+    int vec = kMaxVec;
+    while (vec > 1 && !(N % vec == 0 && aligned_to(B, sizeof(T) * vec) && aligned_to(C, sizeof(T) * vec)))
+      vec /= 2;
+    const int64_t tile_elems = tile_bytes / (int)sizeof(T) < N ? tile_bytes / (int)sizeof(T) : N;
+    const int64_t lanes = (tile_elems + vec - 1) / vec;
+#define SCORCH_GROUPED(VEC, LPR) \
+  return launch_spmm_grouped<T, VEC, LPR, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s)
+#define SCORCH_GROUPED_LANES(VEC)                      \
+  do {                                                 \
+    if (lanes <= 8) SCORCH_GROUPED(VEC, 8);            \
+    if (lanes <= 16) SCORCH_GROUPED(VEC, 16);          \
+    if (lanes <= 32) SCORCH_GROUPED(VEC, 32);          \
+  } while (0)
+    if constexpr (sizeof(T) == 4) {
+      if (vec == 4) SCORCH_GROUPED_LANES(4);
+    }
+    if (vec == 2) SCORCH_GROUPED_LANES(2);
+    if (vec == 1) SCORCH_GROUPED_LANES(1);
+#undef SCORCH_GROUPED_LANES
+#undef SCORCH_GROUPED
+    // more than 32 lanes needed (odd N with scalar lanes): the wide kernel handles it
+  }
+  const int vec = pick_vec<T>(N, B, C, workspace);
   if constexpr (sizeof(T) == 4) {
     if (vec == 4)
       return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
