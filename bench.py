@@ -104,6 +104,20 @@ def _time_steps(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def vendor_spmm(pos, crd, val, B2d, steps, warmup):
+    """torch.sparse.mm on the same CSR operands (torch routes it to the ROCm
+    sparse library): a second GPU implementation timed beside ours.  Returns a
+    JSON-ready dict; never part of `value`."""
+    import torch
+    M = pos.numel() - 1
+    A = torch.sparse_csr_tensor(pos, crd, val, size=(M, B2d.shape[0]))
+    try:
+        ms = _time_steps(lambda: torch.sparse.mm(A, B2d), steps, warmup)
+    except RuntimeError as err:                       # e.g. unsupported size
+        return {"call": "torch.sparse.mm(csr, dense)", "error": str(err).splitlines()[0]}
+    return {"call": "torch.sparse.mm(csr, dense)", "ms_per_step": round(ms, 4)}
+
+
 def probe_memory(args, dev) -> int:
     """Streaming-read and random-row-gather rates of this GPU, from
     libscorch_probes.so (scorch_amd/csrc/probes/membench.hip).  One JSON line."""
@@ -245,6 +259,8 @@ def side_workload(args, dev) -> int:
                "ms_per_step": round(ms, 4),
                "config": {"workload": args.workload + "_fp32", "rows": M, "cols": K, "nnz": nnz,
                           "features": N}}
+        if args.vendor:
+            out["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
     out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
                 "data": "synthetic", "higher_is_better": True,
                 "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
@@ -267,6 +283,8 @@ def main() -> int:
                              "attention_blocksparse", "spgemm_powerlaw", "spmv_powerlaw",
                              "softmax_powerlaw"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
+    ap.add_argument("--vendor", action="store_true",
+                    help="also time torch.sparse.mm on the same operands (SpMM workloads only)")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")
@@ -368,7 +386,7 @@ def main() -> int:
         "hbm_frac_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "event_ms_per_step": round(event_ms_per_step, 4),
         "roofline": {
-            "bound": "hbm", "kernel": "spmm_merge_kernel<float,2,0>",
+            "bound": "hbm", "kernel": "spmm_merge_kernel<float,2,0>" if N == 128 else "spmm_merge_kernel",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES if (M, N) == (1 << 20, 128) else None,
@@ -377,6 +395,8 @@ def main() -> int:
             "kernel_ms_avg": round(merge_avg, 4), "fixup_kernel_ms_avg": round(fixup_avg, 4),
         },
     }
+    if args.vendor:
+        result["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result))

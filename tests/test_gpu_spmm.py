@@ -184,6 +184,41 @@ def test_output_needs_no_zero_fill():
     assert np.isfinite(got).all()
 
 
+def test_output_beyond_two_to_the_31_elements():
+    """M * N = 2^31 + 3072 elements of C: the reference keeps this count in an int
+    (csrc/spmm.h:113); here every offset is 64-bit.  One unit entry per row makes
+    C a row gather of B, checked bit for bit on the device."""
+    M, K, N = (1 << 21) + 3, 512, 1024
+    g = torch.Generator(device="cuda").manual_seed(5)
+    B = torch.randn(K, N, device="cuda", generator=g)
+    col = torch.randint(0, K, (M,), device="cuda", generator=g, dtype=torch.int32)
+    rp = torch.arange(M + 1, device="cuda", dtype=torch.int32)
+    out = H.spmm_csr_float_v2([M, N], [M, K], [[], [rp, col]], torch.ones(M, device="cuda"), [K, N],
+                              [[], []], B.reshape(-1)).storage.value.reshape(M, N)
+    for r0 in range(0, M, 1 << 19):  # compare in slabs to bound the extra memory
+        r1 = min(M, r0 + (1 << 19))
+        assert torch.equal(out[r0:r1], B[col[r0:r1].long()])
+    assert torch.equal(out[M - 1], B[col[M - 1].long()])
+
+
+def test_dense_operand_beyond_two_to_the_31_elements():
+    """K * N > 2^31: rows of B past the 8 GiB mark are gathered with 64-bit offsets."""
+    M, K, N = 4096, (1 << 21) + 5, 1024
+    g = torch.Generator(device="cuda").manual_seed(6)
+    B = torch.empty(K, N, device="cuda")
+    B[:, :] = torch.arange(K, device="cuda", dtype=torch.float32)[:, None]  # row k holds k
+    B[K - 4096:, :] += torch.randn(4096, N, device="cuda", generator=g)
+    col = torch.randint(K - 4096, K, (M, 2), device="cuda", generator=g, dtype=torch.int32)
+    col[:, 0] = torch.randint(0, 4096, (M,), device="cuda", generator=g, dtype=torch.int32)
+    col, _ = torch.sort(col, dim=1)
+    rp = torch.arange(0, 2 * M + 1, 2, device="cuda", dtype=torch.int32)
+    vals = torch.ones(2 * M, device="cuda")
+    out = H.spmm_csr_float_v2([M, N], [M, K], [[], [rp, col.reshape(-1).contiguous()]], vals, [K, N],
+                              [[], []], B.reshape(-1)).storage.value.reshape(M, N)
+    want = B[col[:, 0].long()] + B[col[:, 1].long()]
+    assert torch.equal(out, want)
+
+
 def test_uniform_workload_reference_size(oracle):
     """4096 x 4096 at 1 % density, N = 64: the reference's own CPU-runnable case."""
     w = workloads.spmm_uniform()
