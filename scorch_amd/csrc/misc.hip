@@ -9,82 +9,198 @@ char *error_buffer() {
   return buf;
 }
 
-// Lanes per row for the group-per-row kernels: the power of two nearest above
-// the mean row length, between 2 and 64.
-inline int group_width(int64_t M, int64_t nnz) {
+// ---- CSR row softmax ----------------------------------------------------------
+// p = exp(s - max_row) / sum_row over the stored entries of each row, in three
+// phases (maximum, sum of exponentials, normalised write) like the five torch
+// passes it replaces.  One kernel; a workgroup owns 256 / G consecutive rows and
+// serves them in tiers by length, so that a long row never stalls the lanes
+// beside it:
+//   up to kSoftmaxRegs * G entries   one group of G lanes per row, all at once;
+//   up to kSoftmaxRegs * 16 entries  quarter wavefronts, sixteen rows at a time
+//                                    (only when G < 16);
+//   up to kSoftmaxRegs * 64 entries  one wavefront per row, the workgroup's four
+//                                    wavefronts sharing those rows out;
+//   up to 2048 entries               the whole workgroup, one row after the other.
+// In all of these a row sits in registers between the phases and is read from
+// memory once.  Rows beyond 2048 entries are left to softmax_csr_giant_kernel:
+// workgroups of 1024 threads that look through 1024 row lengths each and sweep
+// the giant rows among them, the first 8192 entries in registers and the rest
+// re-read from cache.
+constexpr int kSoftmaxRegs = 4;
+constexpr int kSoftmaxBlockRegs = 8;
+constexpr int kSoftmaxQuarter = kWaveSize / 4;
+constexpr int kSoftmaxQuarterRowMax = kSoftmaxRegs * kSoftmaxQuarter;
+constexpr int kSoftmaxWaveRowMax = kSoftmaxRegs * kWaveSize;
+constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
+constexpr int kSoftmaxGiantThreads = 1024;
+constexpr float kSoftmaxLowest = -3.402823466e38f;
+
+// Lanes per row: the smallest power of two, between 2 and 64, whose groups hold
+// a row of mean length in registers.
+inline int softmax_group_width(int64_t M, int64_t nnz) {
   const int64_t mean = M > 0 ? (nnz + M - 1) / M : 0;
   int g = 2;
-  while (g < kWaveSize && g < mean) g *= 2;
+  while (g < kWaveSize && (int64_t)g * kSoftmaxRegs < mean) g *= 2;
   return g;
 }
 
-// ---- CSR row softmax ----------------------------------------------------------
-// One group of G lanes per row (rows of up to kSoftmaxLongRow entries); three
-// sweeps over the row (maximum, sum of exponentials, normalised write).  The row is re-read from cache, not kept in
-// registers, so any row length works.
-constexpr int kSoftmaxLongRow = 256;   // longer rows get a whole workgroup
-constexpr int kSoftmaxLongWorkgroups = 2048;
+// The three phases for entries [lo, hi) by a team of TEAM threads (this one is
+// number t); `reduce(value, take_max)` combines a value over the team.
+template <int TEAM, int REGS, bool TAIL, typename Reduce>
+__device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *vals, float scale,
+                                            float *out, Reduce reduce) {
+  float v[REGS];
+  float mx = kSoftmaxLowest;
+#pragma unroll
+  for (int u = 0; u < REGS; ++u) {
+    const int p = lo + t + u * TEAM;
+    v[u] = p < hi ? vals[p] * scale : kSoftmaxLowest;
+    mx = fmaxf(mx, v[u]);
+  }
+  const int rest = lo + REGS * TEAM + t;  // this thread's first entry beyond the registers
+  if (TAIL) {
+#pragma unroll 8
+    for (int p = rest; p < hi; p += TEAM) mx = fmaxf(mx, vals[p] * scale);
+  }
+  mx = reduce(mx, true);
+  float sum = 0.0f;
+#pragma unroll
+  for (int u = 0; u < REGS; ++u) {
+    v[u] = lo + t + u * TEAM < hi ? expf(v[u] - mx) : 0.0f;
+    sum += v[u];
+  }
+  if (TAIL) {
+#pragma unroll 8
+    for (int p = rest; p < hi; p += TEAM) sum += expf(vals[p] * scale - mx);
+  }
+  sum = reduce(sum, false);
+#pragma unroll
+  for (int u = 0; u < REGS; ++u) {
+    const int p = lo + t + u * TEAM;
+    if (p < hi) out[p] = v[u] / sum;
+  }
+  if (TAIL) {
+#pragma unroll 8
+    for (int p = rest; p < hi; p += TEAM) out[p] = expf(vals[p] * scale - mx) / sum;
+  }
+}
+
+template <int WIDTH>
+__device__ __forceinline__ float softmax_shuffle_reduce(float v, bool take_max) {
+#pragma unroll
+  for (int off = WIDTH / 2; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off);
+    v = take_max ? fmaxf(v, o) : v + o;
+  }
+  return v;
+}
 
 template <int G>
 __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                                     const int *__restrict__ row_ptr,
                                                                     const float *vals, float scale,
                                                                     float *out) {
-  const int64_t group = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
+  constexpr int kRows = kBlockThreads / G;  // rows per workgroup
+  __shared__ float s_red[kWavesPerBlock];
+  __shared__ int s_lo[kRows], s_hi[kRows];
+  // row slots left to the quarter wavefronts [0], the wavefronts [1] and the workgroup [2]
+  __shared__ int s_list[3][kRows];
+  __shared__ int s_count[3];
+  if (threadIdx.x < 3) s_count[threadIdx.x] = 0;
+  __syncthreads();
+  const int slot = threadIdx.x / G;
   const int t = threadIdx.x % G;
-  const bool live = group < M;
+  const int64_t row = (int64_t)blockIdx.x * kRows + slot;
   int lo = 0, hi = 0;
-  if (live) {
-    lo = row_ptr[group];
-    hi = row_ptr[group + 1];
-    if (hi - lo > kSoftmaxLongRow) hi = lo;  // softmax_csr_long_kernel owns this row
+  if (row < M) {
+    lo = row_ptr[row];
+    hi = row_ptr[row + 1];
   }
-  float mx = -3.402823466e38f;
-  for (int p = lo + t; p < hi; p += G) mx = fmaxf(mx, vals[p] * scale);
-#pragma unroll
-  for (int off = G / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-  float sum = 0.0f;
-  for (int p = lo + t; p < hi; p += G) sum += expf(vals[p] * scale - mx);
-#pragma unroll
-  for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  for (int p = lo + t; p < hi; p += G) out[p] = expf(vals[p] * scale - mx) / sum;
-}
-
-// Rows longer than kSoftmaxLongRow: one workgroup per row, the same three sweeps
-// with workgroup-wide reductions (fixed order: lanes, then wavefronts).  A fixed
-// pool of workgroups scans the row pointer for such rows.
-__device__ __forceinline__ float block_reduce(float v, float *scratch, bool take_max) {
+  const int len = hi - lo;
+  if (len > G * kSoftmaxRegs) {
+    if (t == 0 && len <= kSoftmaxBlockRowMax) {
+      const int tier = len > kSoftmaxWaveRowMax ? 2 : (len > kSoftmaxQuarterRowMax || G >= kSoftmaxQuarter);
+      s_lo[slot] = lo;
+      s_hi[slot] = hi;
+      s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
+    }
+    hi = lo;
+  }
+  softmax_row<G, kSoftmaxRegs, false>(lo, hi, t, vals, scale, out, softmax_shuffle_reduce<G>);
+  __syncthreads();
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-#pragma unroll
-  for (int off = kWaveSize / 2; off > 0; off >>= 1) {
-    const float o = __shfl_xor(v, off);
-    v = take_max ? fmaxf(v, o) : v + o;
+  const int n_quarter = s_count[0], n_wave = s_count[1], n_block = s_count[2];
+  if (G < kSoftmaxQuarter) {
+    constexpr int kTeams = kBlockThreads / kSoftmaxQuarter;
+    for (int base = 0; base < n_quarter; base += kTeams) {  // uniform over the workgroup
+      const int i = base + (int)threadIdx.x / kSoftmaxQuarter;
+      int l = 0, h = 0;
+      if (i < n_quarter) {
+        const int k = s_list[0][i];
+        l = s_lo[k];
+        h = s_hi[k];
+      }
+      softmax_row<kSoftmaxQuarter, kSoftmaxRegs, false>(l, h, lane % kSoftmaxQuarter, vals, scale, out,
+                                                        softmax_shuffle_reduce<kSoftmaxQuarter>);
+    }
   }
-  __syncthreads();
-  if (lane == 0) scratch[w] = v;
-  __syncthreads();
-  float r = scratch[0];
+  if (G < kWaveSize) {
+    for (int i = w; i < n_wave; i += kWavesPerBlock) {
+      const int k = s_list[1][i];
+      softmax_row<kWaveSize, kSoftmaxRegs, false>(s_lo[k], s_hi[k], lane, vals, scale, out,
+                                                  softmax_shuffle_reduce<kWaveSize>);
+    }
+  }
+  for (int i = 0; i < n_block; ++i) {  // uniform over the workgroup
+    const int k = s_list[2][i];
+    softmax_row<kBlockThreads, kSoftmaxBlockRegs, false>(
+        s_lo[k], s_hi[k], (int)threadIdx.x, vals, scale, out, [&](float v, bool take_max) {
+          v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
+          __syncthreads();
+          if (lane == 0) s_red[w] = v;
+          __syncthreads();
+          float r = s_red[0];
 #pragma unroll
-  for (int i = 1; i < kWavesPerBlock; ++i) r = take_max ? fmaxf(r, scratch[i]) : r + scratch[i];
-  return r;
+          for (int j = 1; j < kWavesPerBlock; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
+          return r;
+        });
+  }
 }
 
-__global__ __launch_bounds__(kBlockThreads) void softmax_csr_long_kernel(int M,
-                                                                         const int *__restrict__ row_ptr,
-                                                                         const float *vals, float scale,
-                                                                         float *out) {
-  __shared__ float s_red[kWavesPerBlock];
-  for (int row = blockIdx.x; row < M; row += gridDim.x) {
+__global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel(
+    int M, const int *__restrict__ row_ptr, const float *vals, float scale, float *out) {
+  constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
+  __shared__ float s_red[kWaves];
+  __shared__ int s_lo[kSoftmaxGiantThreads], s_hi[kSoftmaxGiantThreads];
+  __shared__ int s_count;
+  if (threadIdx.x == 0) s_count = 0;
+  __syncthreads();
+  const int64_t row = (int64_t)blockIdx.x * kSoftmaxGiantThreads + threadIdx.x;
+  if (row < M) {
     const int lo = row_ptr[row], hi = row_ptr[row + 1];
-    if (hi - lo <= kSoftmaxLongRow) continue;  // uniform across the workgroup
-    float mx = -3.402823466e38f;
-    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) mx = fmaxf(mx, vals[p] * scale);
-    mx = block_reduce(mx, s_red, true);
-    float sum = 0.0f;
-    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) sum += expf(vals[p] * scale - mx);
-    sum = block_reduce(sum, s_red, false);
-    for (int p = lo + threadIdx.x; p < hi; p += kBlockThreads) out[p] = expf(vals[p] * scale - mx) / sum;
+    if (hi - lo > kSoftmaxBlockRowMax) {
+      const int k = atomicAdd(&s_count, 1);  // rows are independent: their order is free
+      s_lo[k] = lo;
+      s_hi[k] = hi;
+    }
+  }
+  __syncthreads();
+  const int n = s_count;
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  for (int i = 0; i < n; ++i) {  // uniform over the workgroup
+    softmax_row<kSoftmaxGiantThreads, kSoftmaxBlockRegs, true>(
+        s_lo[i], s_hi[i], (int)threadIdx.x, vals, scale, out, [&](float v, bool take_max) {
+          v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
+          __syncthreads();
+          if (lane == 0) s_red[w] = v;
+          __syncthreads();
+          float r = s_red[0];
+#pragma unroll
+          for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
+          return r;
+        });
   }
 }
 
@@ -126,9 +242,9 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
   if (M == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int g = scorch::group_width(M, nnz);
-  const int64_t threads = M * g;
-  const dim3 grid((unsigned)((threads + scorch::kBlockThreads - 1) / scorch::kBlockThreads));
+  const int g = scorch::softmax_group_width(M, nnz);
+  const int64_t rows_per_block = scorch::kBlockThreads / g;
+  const dim3 grid((unsigned)((M + rows_per_block - 1) / rows_per_block));
   const int m = (int)M;
   switch (g) {
     case 2: scorch::softmax_csr_kernel<2><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
@@ -139,9 +255,11 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
     default: scorch::softmax_csr_kernel<64><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
   }
   SCORCH_HIP_CHECK(hipGetLastError());
-  const unsigned pool = (unsigned)(M < scorch::kSoftmaxLongWorkgroups ? M : scorch::kSoftmaxLongWorkgroups);
-  scorch::softmax_csr_long_kernel<<<pool, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out);
-  SCORCH_HIP_CHECK(hipGetLastError());
+  if (nnz > scorch::kSoftmaxBlockRowMax) {  // else no row can be that long
+    const dim3 giant_grid((unsigned)((M + scorch::kSoftmaxGiantThreads - 1) / scorch::kSoftmaxGiantThreads));
+    scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(m, row_ptr, vals, scale, out);
+    SCORCH_HIP_CHECK(hipGetLastError());
+  }
   return SCORCH_HIP_OK;
 }
 

@@ -55,6 +55,23 @@ def test_softmax_against_oracle(oracle):
     np.testing.assert_allclose(sums, 1.0, rtol=1e-5)
 
 
+def test_softmax_every_row_length_tier(oracle):
+    """Row lengths chosen around each hand-over of the kernel: lane groups, quarter
+    wavefronts, wavefronts, the workgroup (up to 2048 entries) and the giant-row
+    kernel (first 8192 entries in registers, the rest re-read)."""
+    lens = np.array([0, 1, 7, 8, 9, 16, 17, 63, 64, 65, 255, 256, 257, 0, 2047, 2048, 2049, 3,
+                     8191, 8192, 8193, 20000, 5, 0], np.int64)
+    rng = np.random.default_rng(3)
+    for mean_pad in (0, 400):  # few short rows -> narrow groups; many -> group width follows the mean
+        all_lens = np.concatenate([lens, np.full(mean_pad, 2, np.int64)])
+        rp = np.concatenate([[0], np.cumsum(all_lens)]).astype(np.int32)
+        vals = (rng.standard_normal(int(rp[-1])) * 4).astype(np.float32)
+        got = host(H.softmax_csr_float(dev(rp), dev(vals), 0.5))
+        want = oracle.softmax_csr_fp64(rp, vals, 0.5)
+        assert oracle.rel_fro(got, want) <= TOL
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-12)
+
+
 def test_softmax_with_empty_rows_and_large_values(oracle):
     rp = np.array([0, 0, 4, 4, 5], np.int32)
     vals = np.array([1000.0, 1001.0, 999.0, 1000.5, -3.0], np.float32)
