@@ -667,19 +667,46 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_merge_kernel(
 
   auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
   const int x0 = wave_count_below(M, d0, row_end_key);
-  const int x1 = wave_count_below(M, d1, row_end_key);
   const int y0 = uniform((int)(d0 - x0));
-  const int y1 = uniform((int)(d1 - x1));
-  const int n_nz = y1 - y0;
-  const int n_rows = x1 - x0;
 
-  for (int k = lane; k < n_nz; k += kWaveSize)
-    s_prod[w][k] = (A)vals[y0 + k] * (A)x[col_idx[y0 + k]];
-  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
-    const int r = x0 + k < M ? x0 + k : M;
-    s_rp[w][k] = row_ptr[r];
+  // Everything the chunk can touch is known from its start alone: at most
+  // kSpmvItems nonzeros from y0 and kSpmvItems + 1 row pointers from x0.  All
+  // of it is requested at once (one round trip for indices, values and row
+  // pointers, one for the gathered x), and the chunk's end is then found in LDS.
+  constexpr int kNzLoads = kSpmvItems / kWaveSize;
+  constexpr int kRpLoads = (kSpmvItems + 2 + kWaveSize - 1) / kWaveSize;
+  const int64_t nnz = total_items - M;
+  int col[kNzLoads];
+  T val[kNzLoads];
+#pragma unroll
+  for (int u = 0; u < kNzLoads; ++u) {
+    const int64_t p = (int64_t)y0 + lane + u * kWaveSize;
+    const bool ok = p < nnz;
+    col[u] = ok ? col_idx[p] : -1;
+    val[u] = ok ? vals[p] : (T)0;
   }
+  int rp[kRpLoads];
+#pragma unroll
+  for (int u = 0; u < kRpLoads; ++u) {
+    const int64_t r = (int64_t)x0 + lane + u * kWaveSize;
+    rp[u] = row_ptr[r < M ? r : M];
+  }
+#pragma unroll
+  for (int u = 0; u < kNzLoads; ++u) {
+    const A xv = col[u] >= 0 ? (A)x[col[u]] : (A)0;
+    s_prod[w][lane + u * kWaveSize] = (A)val[u] * xv;
+  }
+#pragma unroll
+  for (int u = 0; u < kRpLoads; ++u)
+    if (lane + u * kWaveSize < kSpmvItems + 2) s_rp[w][lane + u * kWaveSize] = rp[u];
   wave_lds_sync();
+
+  // rows ending inside the chunk: row x0 + j ends at merged position s_rp[j + 1] + x0 + j,
+  // and no row from x0 + kSpmvItems on can end before d1
+  const int reach = M - x0 < kSpmvItems ? M - x0 : kSpmvItems;
+  const int n_rows = wave_count_below(reach, d1, [&](int j) { return (int64_t)s_rp[w][j + 1] + x0 + j; });
+  const int x1 = x0 + n_rows;
+  const int y1 = uniform((int)(d1 - x1));
 
   // Row slot r is row x0 + r; slot n_rows is the row that continues past the chunk.
   for (int base = 0; base <= n_rows; base += kWaveSize) {
