@@ -104,6 +104,14 @@ def _time_steps(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def _vendor_time(call_name, fn, steps, warmup):
+    """Times a torch routine on the same operands; an error becomes a field."""
+    try:
+        return {"call": call_name, "ms_per_step": round(_time_steps(fn, steps, warmup), 4)}
+    except RuntimeError as err:
+        return {"call": call_name, "error": str(err).splitlines()[0]}
+
+
 def vendor_spmm(pos, crd, val, B2d, steps, warmup):
     """torch.sparse.mm on the same CSR operands (torch routes it to the ROCm
     sparse library): a second GPU implementation timed beside ours.  Returns a
@@ -199,7 +207,12 @@ def side_workload(args, dev) -> int:
             fn = lambda: H.softmax_csr_float(pos, val, 1.0)
             algo, flops, name = 8 * nnz + 4 * (M + 1), 4.0 * nnz, "CSR row softmax GFLOP/s (4 flops per entry)"
         ms = _time_steps(fn, args.steps, args.warmup)
-        print(json.dumps({"metric": name, "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
+        vendor = None
+        if args.vendor and args.workload == "spmv_powerlaw":
+            A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, M))
+            vendor = _vendor_time("torch.mv(csr, x)", lambda: torch.mv(A_t, x), args.steps, args.warmup)
+        print(json.dumps({**({"vendor_library": vendor} if vendor else {}),
+                          "metric": name, "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
                           "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
                           "dtype": "f32", "data": "synthetic", "higher_is_better": True,
                           "config": {"workload": args.workload + "_fp32", "rows": M, "nnz": nnz},
@@ -220,6 +233,11 @@ def side_workload(args, dev) -> int:
         deg = (pos[1:] - pos[:-1]).long()
         products = int(deg[crd.long()].sum().item())
         ms = _time_steps(fn, args.steps, args.warmup)
+        vendor = None
+        if args.vendor:
+            A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, M))
+            vendor = _vendor_time("torch.sparse.mm(csr, csr)", lambda: torch.sparse.mm(A_t, A_t),
+                                  max(2, args.steps // 4), 1)
         print(json.dumps({"metric": "CSR SpGEMM GFLOP/s (2 flops per product)",
                           "value": round(2.0 * products / ms / 1e6, 2), "unit": "GFLOP/s",
                           "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
@@ -227,7 +245,8 @@ def side_workload(args, dev) -> int:
                           "higher_is_better": True,
                           "config": {"workload": "spgemm_powerlaw_fp32", "rows": M, "nnz_a": int(crd.numel()),
                                      "products": products, "nnz_c": nnz_c},
-                          "note": "symbolic + numeric passes and the host read of nnz(C) between them"}))
+                          "note": "symbolic + numeric passes and the host read of nnz(C) between them",
+                          **({"vendor_library": vendor} if vendor else {})}))
         return 0
     if args.workload == "sddmm_uniform":
         w = workloads.sddmm_uniform()
@@ -247,6 +266,12 @@ def side_workload(args, dev) -> int:
         out = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
                "ms_per_step": round(ms, 4), "ms_per_step_coo_mask": round(ms_coo, 4),
                "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K}}
+        if args.vendor:
+            mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
+            Bt = B.t().contiguous()
+            out["vendor_library"] = _vendor_time(
+                "torch.sparse.sampled_addmm(mask, A, B^T, beta=0)",
+                lambda: torch.sparse.sampled_addmm(mask, A, Bt, beta=0.0), args.steps, args.warmup)
     else:
         w = workloads.spmm_uniform() if args.workload == "spmm_uniform" else workloads.sae_decoder()
         M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
@@ -284,7 +309,7 @@ def main() -> int:
                              "softmax_powerlaw"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--vendor", action="store_true",
-                    help="also time torch.sparse.mm on the same operands (SpMM workloads only)")
+                    help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")
