@@ -27,6 +27,9 @@ HIPCC_FLAGS = [
     # MFMA results stay in ordinary vector registers: the attention kernel feeds them
     # straight to vector instructions, and accumulator registers would cost copies
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # floating-point atomic adds (SpGEMM accumulators) as the hardware's add instructions, not
+    # compare-and-swap loops; their targets are LDS and ordinary device memory
+    "-munsafe-fp-atomics",
     "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
 ]
 

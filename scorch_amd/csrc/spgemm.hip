@@ -63,22 +63,39 @@ __device__ __forceinline__ int hash_insert(int *keys, int mask, int key) {
   }
 }
 
-// *addr += v, atomically (LDS or global memory).
+// *addr += v, atomically (LDS or global memory).  Floating-point sums use the
+// hardware's add instructions (global_atomic_add_f32 / _f64, ds_add_f32 / _f64)
+// rather than a compare-and-swap loop; they are exact for ordinary device
+// memory, which is what the workspace must be.
 template <typename A>
 __device__ __forceinline__ void atomic_accumulate(A *addr, A v) { atomicAdd(addr, v); }
+template <>
+__device__ __forceinline__ void atomic_accumulate<float>(float *addr, float v) { unsafeAtomicAdd(addr, v); }
+template <>
+__device__ __forceinline__ void atomic_accumulate<double>(double *addr, double v) { unsafeAtomicAdd(addr, v); }
 template <>
 __device__ __forceinline__ void atomic_accumulate<uint64_t>(uint64_t *addr, uint64_t v) {
   atomicAdd(reinterpret_cast<unsigned long long *>(addr), (unsigned long long)v);
 }
 
+// A workgroup's slab in global memory is private to it: its wavefronts share one
+// CU and one L2, so workgroup scope is all the ordering it needs.  (A
+// device-scope fence would make the L2 write its dirty lines back, once per
+// row and workgroup.)  Read after the atomics of other wavefronts of the
+// workgroup, behind a __syncthreads().
 template <typename A>
-__device__ __forceinline__ A agent_load(const A *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ A workgroup_load(const A *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+template <typename A>
+__device__ __forceinline__ void workgroup_store(A *p, A v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// Exclusive prefix sum of one int per thread over the workgroup; `total`
-// receives the sum.  `scratch` holds kWavesPerBlock + 1 ints.
-__device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &total) {
+// Exclusive prefix sum of one int per thread over a workgroup of WAVES
+// wavefronts; `total` receives the sum.  `scratch` holds WAVES ints.
+template <int WAVES>
+__device__ __forceinline__ int block_exclusive_scan_n(int v, int *scratch, int &total) {
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
   int incl = v;
@@ -90,13 +107,91 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &to
   __syncthreads();  // scratch may still be read from a previous call
   if (lane == kWaveSize - 1) scratch[w] = incl;
   __syncthreads();
-  int before = 0;
+  int before = 0, all = 0;
 #pragma unroll
-  for (int i = 0; i < kWavesPerBlock; ++i) {
-    if (i < w) before += scratch[i];
+  for (int i = 0; i < WAVES; ++i) {
+    const int part = scratch[i];
+    if (i < w) before += part;
+    all += part;
   }
-  total = scratch[0] + scratch[1] + scratch[2] + scratch[3];
+  total = all;
   return before + incl - v;
+}
+
+__device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &total) {
+  return block_exclusive_scan_n<kWavesPerBlock>(v, scratch, total);
+}
+
+// ---- walking the products of one row of C ------------------------------------------------
+// The products of a row are the entries of the B rows its A entries select.  B
+// rows are often much shorter than a wavefront, so handing one B row to a team
+// at a time wastes most lanes and chains three dependent loads per A entry.
+// Instead the team (TEAM = 64: one wavefront, TEAM = 256: the workgroup) takes
+// TEAM entries of A at once -- thread t reads entry t, its B row's start and
+// length -- turns the lengths into offsets with a prefix sum, and then walks the
+// batch's products flat: product x belongs to the entry e with off[e] <= x <
+// off[e + 1], found by bisection in LDS.  All lanes stay busy and consecutive
+// lanes read consecutive entries of a B row.
+template <int TEAM, typename A>
+struct ProductBatch {
+  int off[TEAM];  // first product of each entry within the batch
+  int b_lo[TEAM];
+  A a_val[TEAM];
+};
+
+template <int TEAM>
+__device__ __forceinline__ void team_sync() {
+  if (TEAM == kWaveSize) wave_lds_sync(); else __syncthreads();
+}
+
+template <int TEAM>
+__device__ __forceinline__ int team_exclusive_scan(int v, int *scratch, int &total) {
+  if (TEAM != kWaveSize) return block_exclusive_scan_n<TEAM / kWaveSize>(v, scratch, total);
+  const int lane = wave_lane();
+  int incl = v;
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+  total = __shfl(incl, kWaveSize - 1);
+  return incl - v;
+}
+
+// fn(column, product) for every product of A entries [a_lo, a_hi); `t` is the
+// thread's number in the team.  Uniform over the team.
+template <int TEAM, bool NUMERIC, typename T, typename A, typename Fn>
+__device__ __forceinline__ void for_each_product(int a_lo, int a_hi, int t, const int *__restrict__ a_crd,
+                                                 const T *__restrict__ a_val, const int *__restrict__ b_pos,
+                                                 const int *__restrict__ b_crd, const T *__restrict__ b_val,
+                                                 ProductBatch<TEAM, A> &batch, int *scan_scratch, Fn fn) {
+  for (int base = a_lo; base < a_hi; base += TEAM) {
+    const int p = base + t;
+    int lo = 0, len = 0;
+    A av = (A)0;
+    if (p < a_hi) {
+      const int j = a_crd[p];
+      lo = b_pos[j];
+      len = b_pos[j + 1] - lo;
+      if (NUMERIC) av = (A)a_val[p];
+    }
+    int total = 0;
+    const int first = team_exclusive_scan<TEAM>(len, scan_scratch, total);
+    team_sync<TEAM>();  // the previous batch has been read by everyone
+    batch.off[t] = first;
+    batch.b_lo[t] = lo;
+    if (NUMERIC) batch.a_val[t] = av;
+    team_sync<TEAM>();
+#pragma unroll 8
+    for (int x = t; x < total; x += TEAM) {
+      int e = 0;  // the last entry whose offset is <= x (entries without products share an offset)
+#pragma unroll
+      for (int step = TEAM / 2; step > 0; step >>= 1)
+        if (batch.off[e + step] <= x) e += step;
+      const int q = batch.b_lo[e] + (x - batch.off[e]);
+      fn(b_crd[q], NUMERIC ? batch.a_val[e] * (A)b_val[q] : (A)0);
+    }
+  }
 }
 
 // ---- exclusive prefix sum of n ints, in place (counts -> row pointer) ------------------
@@ -191,6 +286,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
   __shared__ A s_vals[kWavesPerBlock][NUMERIC ? kTinySlots : 1];
   __shared__ int s_ck[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
   __shared__ A s_cv[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
+  __shared__ ProductBatch<kWaveSize, A> s_batch[kWavesPerBlock];
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
@@ -204,15 +300,12 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
   }
   wave_lds_sync();
 
-  const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
-  for (int p = a_lo; p < a_hi; ++p) {
-    const int j = uniform(a_crd[p]);
-    const A av = NUMERIC ? (A)a_val[p] : (A)0;
-    for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
-      const int slot = hash_insert(s_keys[w], kTinySlots - 1, b_crd[q]);
-      if (NUMERIC) atomic_accumulate<A>(&s_vals[w][slot], av * (A)b_val[q]);
-    }
-  }
+  for_each_product<kWaveSize, NUMERIC, T, A>(
+      a_pos[row], a_pos[row + 1], lane, a_crd, a_val, b_pos, b_crd, b_val, s_batch[w], nullptr,
+      [&](int col, A product) {
+        const int slot = hash_insert(s_keys[w], kTinySlots - 1, col);
+        if (NUMERIC) atomic_accumulate<A>(&s_vals[w][slot], product);
+      });
   wave_lds_sync();
 
   // Count the occupied slots; in the numeric pass, also compact them.
@@ -258,10 +351,9 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   __shared__ int s_ck[NUMERIC ? PRODUCTS : 1];
   __shared__ A s_cv[NUMERIC ? PRODUCTS : 1];
   __shared__ int s_scan[kWavesPerBlock + 1];
+  __shared__ ProductBatch<kBlockThreads, A> s_batch;
 
   const int tid = threadIdx.x;
-  const int lane = wave_lane();
-  const int w = tid / kWaveSize;
   const int n_rows = counters[COUNTER];
 
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
@@ -272,15 +364,12 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     }
     __syncthreads();
 
-    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
-    for (int p = a_lo + w; p < a_hi; p += kWavesPerBlock) {
-      const int j = uniform(a_crd[p]);
-      const A av = NUMERIC ? (A)a_val[p] : (A)0;
-      for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
-        const int slot = hash_insert(s_keys, kSlots - 1, b_crd[q]);
-        if (NUMERIC) atomic_accumulate<A>(&s_vals[slot], av * (A)b_val[q]);
-      }
-    }
+    for_each_product<kBlockThreads, NUMERIC, T, A>(
+        a_pos[row], a_pos[row + 1], tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
+        [&](int col, A product) {
+          const int slot = hash_insert(s_keys, kSlots - 1, col);
+          if (NUMERIC) atomic_accumulate<A>(&s_vals[slot], product);
+        });
     __syncthreads();
 
     // Each thread owns a contiguous run of slots; an exclusive scan of the
@@ -338,18 +427,24 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
 }
 
 // ---- rows beyond that: bitmap (and dense accumulator) over all columns ---------------
+// Workgroups of 1024 threads: such a row has tens of thousands of products and
+// is one workgroup's alone, so its width is the row's parallelism.
+constexpr int kHugeThreads = 1024;
+constexpr int kHugeWaves = kHugeThreads / kWaveSize;
+constexpr int kHugeEmitWords = 256;  // bitmap words emitted per step (at most 8192 columns)
+
 template <typename T, bool NUMERIC>
-__global__ __launch_bounds__(kBlockThreads) void spgemm_huge_kernel(
+__global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
     int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, const int *__restrict__ counters, unsigned *__restrict__ bitmaps,
     typename Acc<T>::type *__restrict__ dense, int *__restrict__ c_pos, int *__restrict__ c_crd,
     T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
-  __shared__ int s_scan[kWavesPerBlock + 1];
+  __shared__ int s_scan[kHugeWaves];
+  __shared__ ProductBatch<kHugeThreads, A> s_batch;
+  __shared__ int s_cols[NUMERIC ? kHugeEmitWords * 32 : 1];
   const int tid = threadIdx.x;
-  const int lane = wave_lane();
-  const int w = tid / kWaveSize;
   const int n_rows = counters[1];
   if ((int)blockIdx.x >= n_rows) return;
 
@@ -357,55 +452,66 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_huge_kernel(
   unsigned *bitmap = bitmaps + (size_t)blockIdx.x * (size_t)words;
   A *sums = NUMERIC ? dense + (size_t)blockIdx.x * (size_t)N : nullptr;
   // This workgroup's slab starts clean and is left clean after every row.
-  for (int i = tid; i < words; i += kBlockThreads) bitmap[i] = 0u;
+  for (int i = tid; i < words; i += kHugeThreads) workgroup_store(&bitmap[i], 0u);
   if (NUMERIC)
-    for (int i = tid; i < N; i += kBlockThreads) sums[i] = (A)0;
-  __threadfence();
+    for (int i = tid; i < N; i += kHugeThreads) workgroup_store(&sums[i], (A)0);
   __syncthreads();
 
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
     const int row = rows[idx];
-    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
-    for (int p = a_lo + w; p < a_hi; p += kWavesPerBlock) {
-      const int j = uniform(a_crd[p]);
-      const A av = NUMERIC ? (A)a_val[p] : (A)0;
-      for (int q = b_pos[j] + lane; q < b_pos[j + 1]; q += kWaveSize) {
-        const int k = b_crd[q];
-        atomicOr(&bitmap[k >> 5], 1u << (k & 31));
-        if (NUMERIC) atomic_accumulate<A>(&sums[k], av * (A)b_val[q]);
-      }
-    }
-    __threadfence();
-    __syncthreads();
+    for_each_product<kHugeThreads, NUMERIC, T, A>(
+        a_pos[row], a_pos[row + 1], tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
+        [&](int k, A product) {
+          __hip_atomic_fetch_or(&bitmap[k >> 5], 1u << (k & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (NUMERIC) __hip_atomic_fetch_add(&sums[k], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        });
+      __syncthreads();
 
-    // Walk the bitmap in order; the set bits are the row's columns, ascending.
-    int emitted = 0;
-    const int out = NUMERIC ? c_pos[row] : 0;
-    for (int base = 0; base < words; base += kBlockThreads) {
-      const int word = base + tid;
-      unsigned bits = word < words ? agent_load(&bitmap[word]) : 0u;
-      int total = 0;
-      int at = block_exclusive_scan(__popc(bits), s_scan, total);
-      if (bits) {
-        if (NUMERIC) {
-          at += out + emitted;
-          while (bits) {
-            const int bit = __ffs(bits) - 1;
-            bits &= bits - 1;
-            const int col = word * 32 + bit;
-            c_crd[at] = col;
-            c_val[at] = (T)agent_load(&sums[col]);
-            sums[col] = (A)0;
-            ++at;
-          }
+    if (!NUMERIC) {
+      // count the set bits and clear them
+      int mine = 0;
+      for (int word = tid; word < words; word += kHugeThreads) {
+        const unsigned bits = workgroup_load(&bitmap[word]);
+        if (bits) {
+          mine += __popc(bits);
+          workgroup_store(&bitmap[word], 0u);
         }
-        bitmap[word] = 0u;
       }
-      emitted += total;
+      int total = 0;
+      block_exclusive_scan_n<kHugeWaves>(mine, s_scan, total);
+      if (tid == 0) c_pos[row] = total;
+    } else {
+      // Walk the bitmap in order, kHugeEmitWords words at a time: the set bits of
+      // a step are listed in LDS (ascending), then all threads fetch the sums of
+      // the listed columns side by side and write the step's entries coalesced.
+      int emitted = c_pos[row];
+      for (int base = 0; base < words; base += kHugeEmitWords) {
+        const int word = base + tid;
+        unsigned bits = 0u;
+        if (tid < kHugeEmitWords && word < words) {
+          bits = workgroup_load(&bitmap[word]);
+          if (bits) workgroup_store(&bitmap[word], 0u);
+        }
+        int total = 0;
+        int at = block_exclusive_scan_n<kHugeWaves>(__popc(bits), s_scan, total);
+        while (bits) {
+          const int bit = __ffs(bits) - 1;
+          bits &= bits - 1;
+          s_cols[at++] = word * 32 + bit;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int e = tid; e < total; e += kHugeThreads) {
+          const int col = s_cols[e];
+          c_crd[emitted + e] = col;
+          c_val[emitted + e] = (T)workgroup_load(&sums[col]);
+          workgroup_store(&sums[col], (A)0);
+        }
+        emitted += total;
+        // the next step's scan starts with a barrier, which also protects s_cols
+      }
     }
-    if (!NUMERIC && tid == 0) c_pos[row] = emitted;
-    __threadfence();
-    __syncthreads();
+      __syncthreads();
   }
 }
 
@@ -481,7 +587,7 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
       a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kBlockThreads, 0, stream>>>(
+  spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kHugeThreads, 0, stream>>>(
       N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
       static_cast<A *>(ws.dense), c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
