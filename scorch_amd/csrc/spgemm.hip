@@ -19,8 +19,9 @@
 //                        about 1 GiB of slabs, walks the list of these rows
 //
 // Hash rows are emitted sorted: the wavefront version ranks every entry by
-// counting smaller keys (at most 256 of them), the workgroup version runs a
-// bitonic sort in LDS.  Bitmap rows come out sorted by construction.
+// counting smaller keys (at most 256 of them), the workgroup version sorts in
+// LDS by buckets over the row's column range (a bitonic sort when the columns
+// cluster).  Bitmap rows come out sorted by construction.
 // Floating-point sums are accumulated with atomics, so their rounding can
 // differ from run to run in the last bits; the structure never does, and
 // integer results are exact.
@@ -116,6 +117,23 @@ __device__ __forceinline__ int block_exclusive_scan_n(int v, int *scratch, int &
   }
   total = all;
   return before + incl - v;
+}
+
+// Maximum (or minimum) of one int per thread over a 256-thread workgroup.
+template <bool MAX>
+__device__ __forceinline__ int block_reduce_int(int v, int *scratch) {
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+    const int o = __shfl_xor(v, off);
+    v = MAX ? (o > v ? o : v) : (o < v ? o : v);
+  }
+  __syncthreads();  // scratch may still be read from a previous call
+  if (wave_lane() == 0) scratch[threadIdx.x / kWaveSize] = v;
+  __syncthreads();
+  int r = scratch[0];
+#pragma unroll
+  for (int i = 1; i < kWavesPerBlock; ++i) r = MAX ? (scratch[i] > r ? scratch[i] : r) : (scratch[i] < r ? scratch[i] : r);
+  return r;
 }
 
 __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &total) {
@@ -245,28 +263,88 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
 }
 
 // ---- pass 0: products per row, and the lists of rows too big for a wavefront ----
+// A workgroup takes kBoundsRows consecutive rows, eight lanes per row; rows of A
+// with more than kBoundsLongRow entries are queued in LDS and summed by the whole
+// workgroup afterwards, so that a hub row does not leave its neighbours' lanes
+// waiting on a long dependent chain.  The three row lists are gathered in LDS
+// first and appended to the global lists with one atomic per list and
+// workgroup: thousands of atomics on one counter would serialise in the L2.
+constexpr int kBoundsLongRow = 64;
+constexpr int kBoundsRows = 256;
+
 __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
     const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ small_rows,
     int *__restrict__ medium_rows, int *__restrict__ huge_rows, int *__restrict__ counters) {
   constexpr int G = 8;  // lanes per row
-  const int64_t row = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) / G;
+  constexpr int kStep = kBlockThreads / G;
+  __shared__ int s_long[kBoundsRows];
+  __shared__ int s_list[3][kBoundsRows];  // counters' order: medium, huge, small
+  __shared__ int s_n[4];                  // [3]: long rows queued
+  __shared__ int s_base[3];
+  __shared__ long long s_part[kWavesPerBlock];
+  if (threadIdx.x < 4) s_n[threadIdx.x] = 0;
+  __syncthreads();
+  auto file_row = [&](int row, long long sum) {
+    const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
+    products[row] = bound;
+    const int list = bound > kMediumProducts ? 1 : bound > kSmallProducts ? 0 : bound > kTinyProducts ? 2 : -1;
+    if (list >= 0) s_list[list][atomicAdd(&s_n[list], 1)] = row;
+  };
+
   const int t = threadIdx.x % G;
-  long long sum = 0;
-  if (row < M)
-    for (int p = a_pos[row] + t; p < a_pos[row + 1]; p += G) {
+  const int64_t first = (int64_t)blockIdx.x * kBoundsRows;
+  for (int it = 0; it < kBoundsRows / kStep; ++it) {
+    const int64_t row = first + it * kStep + threadIdx.x / G;
+    int lo = 0, hi = 0;
+    if (row < M) {
+      lo = a_pos[row];
+      hi = a_pos[row + 1];
+    }
+    const bool is_long = hi - lo > kBoundsLongRow;
+    if (is_long) {
+      if (t == 0) s_long[atomicAdd(&s_n[3], 1)] = (int)row;
+      hi = lo;
+    }
+    long long sum = 0;
+    for (int p = lo + t; p < hi; p += G) {
       const int j = a_crd[p];
       sum += b_pos[j + 1] - b_pos[j];
     }
 #pragma unroll
-  for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  if (row < M && t == 0) {
-    const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
-    products[row] = bound;
-    if (bound > kMediumProducts) huge_rows[atomicAdd(&counters[1], 1)] = (int)row;
-    else if (bound > kSmallProducts) medium_rows[atomicAdd(&counters[0], 1)] = (int)row;
-    else if (bound > kTinyProducts) small_rows[atomicAdd(&counters[2], 1)] = (int)row;
+    for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (row < M && t == 0 && !is_long) file_row((int)row, sum);
   }
+  __syncthreads();
+
+  const int n_long = s_n[3];
+  for (int i = 0; i < n_long; ++i) {  // uniform over the workgroup
+    const int r = s_long[i];
+    long long part = 0;
+#pragma unroll 4
+    for (int p = a_pos[r] + (int)threadIdx.x; p < a_pos[r + 1]; p += kBlockThreads) {
+      const int j = a_crd[p];
+      part += b_pos[j + 1] - b_pos[j];
+    }
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) part += __shfl_xor(part, off);
+    __syncthreads();
+    if (wave_lane() == 0) s_part[threadIdx.x / kWaveSize] = part;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      long long total = 0;
+      for (int w = 0; w < kWavesPerBlock; ++w) total += s_part[w];
+      file_row(r, total);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 3 && s_n[threadIdx.x] > 0)
+    s_base[threadIdx.x] = atomicAdd(&counters[threadIdx.x], s_n[threadIdx.x]);
+  __syncthreads();
+  int *const lists[3] = {medium_rows, huge_rows, small_rows};
+#pragma unroll
+  for (int l = 0; l < 3; ++l)
+    for (int i = threadIdx.x; i < s_n[l]; i += kBlockThreads) lists[l][s_base[l] + i] = s_list[l][i];
 }
 
 __global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
@@ -346,11 +424,15 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     int *__restrict__ c_crd, T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
   constexpr int kSlots = 2 * PRODUCTS;
+  constexpr int kBuckets = PRODUCTS / 2;
+  constexpr int kBucketCrowd = 32;  // a fuller bucket sends the row to the bitonic sort
   __shared__ int s_keys[kSlots];
   __shared__ A s_vals[NUMERIC ? kSlots : 1];
   __shared__ int s_ck[NUMERIC ? PRODUCTS : 1];
   __shared__ A s_cv[NUMERIC ? PRODUCTS : 1];
   __shared__ int s_scan[kWavesPerBlock + 1];
+  __shared__ int s_red[kWavesPerBlock];
+  __shared__ int s_cnt[NUMERIC ? kBuckets : 1];
   __shared__ ProductBatch<kBlockThreads, A> s_batch;
 
   const int tid = threadIdx.x;
@@ -375,8 +457,15 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     // Each thread owns a contiguous run of slots; an exclusive scan of the
     // per-thread counts places the occupied ones.
     constexpr int kRun = kSlots / kBlockThreads;
-    int mine = 0;
-    for (int s = 0; s < kRun; ++s) mine += s_keys[tid * kRun + s] != -1 ? 1 : 0;
+    int mine = 0, key_min = INT_MAX, key_max = -1;
+    for (int s = 0; s < kRun; ++s) {
+      const int key = s_keys[tid * kRun + s];
+      if (key != -1) {
+        ++mine;
+        key_min = key < key_min ? key : key_min;
+        key_max = key > key_max ? key : key_max;
+      }
+    }
     int n = 0;
     int at = block_exclusive_scan(mine, s_scan, n);
     if (!NUMERIC) {
@@ -384,37 +473,96 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       __syncthreads();
       continue;
     }
+
+    // Sorting the row's (column, value) pairs.  First choice: buckets.  The
+    // columns' range [min, max] is cut into kBuckets equal power-of-two intervals
+    // (about two entries each when the columns are spread evenly), a prefix sum of
+    // the bucket counts places the buckets, and a thread sorts each bucket by
+    // insertion.  If some bucket is crowded (clustered columns), a bitonic sort
+    // of the whole row takes over.
+    key_min = block_reduce_int<false>(key_min, s_red);
+    key_max = block_reduce_int<true>(key_max, s_red);
+    int shift = 0;
+    while (((key_max - key_min) >> shift) >= kBuckets) ++shift;  // n > 0 here: the row has products
+    for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) s_cnt[bkt] = 0;
+    __syncthreads();
     for (int s = 0; s < kRun; ++s) {
       const int key = s_keys[tid * kRun + s];
-      if (key != -1) {
-        s_ck[at] = key;
-        s_cv[at] = s_vals[tid * kRun + s];
-        ++at;
-      }
+      if (key != -1) atomicAdd(&s_cnt[(key - key_min) >> shift], 1);
     }
-    int padded = 1;
-    while (padded < n) padded <<= 1;
     __syncthreads();
-    for (int e = n + tid; e < padded; e += kBlockThreads) s_ck[e] = INT_MAX;
-    __syncthreads();
-
-    // Bitonic sort of (key, value) pairs by key.
-    for (int size = 2; size <= padded; size <<= 1) {
-      for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int e = tid; e < padded / 2; e += kBlockThreads) {
-          const int lo = 2 * e - (e & (stride - 1));
-          const int hi = lo + stride;
-          const bool ascending = (lo & size) == 0;
-          const int klo = s_ck[lo], khi = s_ck[hi];
-          if ((klo > khi) == ascending) {
-            s_ck[lo] = khi;
-            s_ck[hi] = klo;
-            const A v = s_cv[lo];
-            s_cv[lo] = s_cv[hi];
-            s_cv[hi] = v;
-          }
+    constexpr int kBucketRun = kBuckets / kBlockThreads;
+    int run_total = 0, crowd = 0;
+    for (int i = 0; i < kBucketRun; ++i) {
+      const int c = s_cnt[tid * kBucketRun + i];
+      run_total += c;
+      crowd = c > crowd ? c : crowd;
+    }
+    int unused = 0;
+    int start = block_exclusive_scan(run_total, s_scan, unused);
+    crowd = block_reduce_int<true>(crowd, s_red);
+    if (crowd <= kBucketCrowd) {
+      for (int i = 0; i < kBucketRun; ++i) {  // counts -> first positions
+        const int c = s_cnt[tid * kBucketRun + i];
+        s_cnt[tid * kBucketRun + i] = start;
+        start += c;
+      }
+      __syncthreads();
+      for (int s = 0; s < kRun; ++s) {
+        const int key = s_keys[tid * kRun + s];
+        if (key != -1) {
+          const int pos = atomicAdd(&s_cnt[(key - key_min) >> shift], 1);  // ends as the bucket's end
+          s_ck[pos] = key;
+          s_cv[pos] = s_vals[tid * kRun + s];
         }
-        __syncthreads();
+      }
+      __syncthreads();
+      for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) {
+        const int lo = bkt ? s_cnt[bkt - 1] : 0, hi = s_cnt[bkt];
+        for (int i = lo + 1; i < hi; ++i) {
+          const int key = s_ck[i];
+          const A val = s_cv[i];
+          int j = i;
+          for (; j > lo && s_ck[j - 1] > key; --j) {
+            s_ck[j] = s_ck[j - 1];
+            s_cv[j] = s_cv[j - 1];
+          }
+          s_ck[j] = key;
+          s_cv[j] = val;
+        }
+      }
+      __syncthreads();
+    } else {
+      for (int s = 0; s < kRun; ++s) {
+        const int key = s_keys[tid * kRun + s];
+        if (key != -1) {
+          s_ck[at] = key;
+          s_cv[at] = s_vals[tid * kRun + s];
+          ++at;
+        }
+      }
+      int padded = 1;
+      while (padded < n) padded <<= 1;
+      __syncthreads();
+      for (int e = n + tid; e < padded; e += kBlockThreads) s_ck[e] = INT_MAX;
+      __syncthreads();
+      for (int size = 2; size <= padded; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+          for (int e = tid; e < padded / 2; e += kBlockThreads) {
+            const int lo = 2 * e - (e & (stride - 1));
+            const int hi = lo + stride;
+            const bool ascending = (lo & size) == 0;
+            const int klo = s_ck[lo], khi = s_ck[hi];
+            if ((klo > khi) == ascending) {
+              s_ck[lo] = khi;
+              s_ck[hi] = klo;
+              const A v = s_cv[lo];
+              s_cv[lo] = s_cv[hi];
+              s_cv[hi] = v;
+            }
+          }
+          __syncthreads();
+        }
       }
     }
     const int out = c_pos[row];
@@ -571,7 +719,7 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   using A = typename Acc<T>::type;
   spgemm_reset_kernel<<<1, 64, 0, stream>>>(ws.counters, NUMERIC ? nullptr : c_pos + M);
   SCORCH_HIP_CHECK(hipGetLastError());
-  const unsigned row_groups = (unsigned)(((int64_t)M * 8 + kBlockThreads - 1) / kBlockThreads);
+  const unsigned row_groups = (unsigned)(((int64_t)M + kBoundsRows - 1) / kBoundsRows);
   spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, a_pos, a_crd, b_pos, ws.products,
                                                                 ws.small_rows, ws.medium_rows,
                                                                 ws.huge_rows, ws.counters);

@@ -91,6 +91,31 @@ def test_huge_rows_bitmap_path_and_all_three_mixed(oracle, dtype):
     assert np.diff(rp).max() > 4096
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
+def test_clustered_columns_fall_back_to_the_whole_row_sort(oracle, dtype):
+    """Rows whose columns crowd a few sorting buckets: a dense run of columns plus
+    one far outlier stretches the bucket width, so the run lands in a handful of
+    buckets and the kernel has to sort the whole row instead.  One row for each
+    workgroup tier (about 600 and about 2400 products), each column hit twice."""
+    n_cols = 1 << 20
+    rng = np.random.default_rng(21)
+    b_rows, b_cols = [], []
+    for r, (lo, hi) in enumerate([(5000, 5300), (5150, 5450), (70000, 71200), (70600, 71800)]):
+        cols = np.arange(lo, hi)
+        if r % 2:
+            cols = np.append(cols, n_cols - 1 - r)  # the outlier
+        b_rows.append(np.full(cols.size, r))
+        b_cols.append(cols)
+    b_rows, b_cols = np.concatenate(b_rows), np.concatenate(b_cols)
+    B = sp.csr_matrix((rng.integers(1, 5, b_cols.size).astype(dtype), (b_rows, b_cols)), shape=(4, n_cols))
+    A = sp.csr_matrix((np.array([2, 3, 1, 2, 1], dtype), (np.array([0, 0, 1, 1, 2]), np.array([0, 1, 2, 3, 0]))),
+                      shape=(3, 4))
+    A.sort_indices(), B.sort_indices()
+    rp, ci, _ = check(oracle, A.indptr.astype(np.int32), A.indices.astype(np.int32), A.data,
+                      B.indptr.astype(np.int32), B.indices.astype(np.int32), B.data, n_cols)
+    assert list(np.diff(rp)) == [451, 1801, 300]
+
+
 def test_structure_is_the_same_on_every_run_and_inputs_untouched(oracle):
     rng = np.random.default_rng(4)
     arp, aci, av = random_csr(rng, 300, 300, 0.05)
