@@ -89,3 +89,55 @@ def test_spgemm_random(oracle, seed):
     else:
         np.testing.assert_allclose(v, wv, rtol=1e-4 if dtype == np.float32 else 1e-12,
                                    atol=1e-3 if dtype == np.float32 else 1e-10)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_softmax_random(oracle, seed):
+    """Row lengths from a heavy-tailed draw (so that every tier of the kernel and
+    the giant-row kernel meet rows), empty rows included, scale of either sign."""
+    from gpu_util import dev, host
+    from scorch_amd import scorch_ops_hip as H
+    rng = np.random.default_rng(5000 + seed)
+    M = int(rng.integers(1, 3000))
+    lens = np.minimum(rng.zipf(1.6, size=M) - 1, int(rng.choice([40, 300, 3000, 12000]))).astype(np.int64)
+    lens[rng.random(M) < 0.1] = 0
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    vals = (rng.standard_normal(int(rp[-1])) * float(rng.choice([0.1, 3.0, 30.0]))).astype(np.float32)
+    scale = float(rng.choice([1.0, 0.125, -0.5]))
+    got = host(H.softmax_csr_float(dev(rp), dev(vals), scale))
+    want = oracle.softmax_csr_fp64(rp, vals, scale)
+    assert got.shape == want.shape
+    if want.size:
+        np.testing.assert_allclose(got, want, rtol=3e-5, atol=1e-10)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_attention_random_block_patterns(oracle, seed):
+    """Random block masks (some block rows empty, some full), head counts that are
+    and are not multiples of eight, sequence lengths from one block up."""
+    import torch
+    from gpu_util import dev
+    from scorch_amd import scorch_ops_hip as H
+    rng = np.random.default_rng(6000 + seed)
+    nb = int(rng.choice([1, 2, 5, 9, 16]))
+    heads = int(rng.choice([1, 3, 8, 16]))
+    S = 64 * nb
+    active = rng.random((nb, nb)) < float(rng.choice([0.15, 0.5, 1.0]))
+    if nb > 2:
+        active[int(rng.integers(nb)), :] = False
+        active[int(rng.integers(nb)), :] = True
+    r, c = np.nonzero(active)
+    brp = np.concatenate([[0], np.cumsum(np.bincount(r, minlength=nb))]).astype(np.int32)
+    bci = c.astype(np.int32)
+    q, k, v = (torch.from_numpy((rng.standard_normal((heads, S, 64)) * float(rng.choice([0.3, 1.0, 3.0])))
+                                .astype(np.float32)).to(torch.bfloat16) for _ in range(3))
+    scale = float(rng.choice([0.125, 0.05, -0.125]))
+    out = H.attn_blocksparse_bf16(q.cuda(), k.cuda(), v.cuda(), dev(brp), dev(bci), scale).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            brp, bci, 64, scale)
+    assert np.isfinite(out).all()
+    empty_rows = np.nonzero(np.diff(brp) == 0)[0]
+    for b in empty_rows:
+        assert not out[:, 64 * b:64 * (b + 1)].any()
+    if np.linalg.norm(ref) > 0:
+        assert oracle.rel_fro(out, ref) <= 1e-2
