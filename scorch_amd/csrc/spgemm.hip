@@ -13,10 +13,11 @@
 //   up to 4096 products  one workgroup, hash table of 8192 slots in LDS (the
 //                        smaller table of the tier above lets more workgroups
 //                        share a CU)
-//   more                 one workgroup with a bitmap over all N columns (and,
-//                        in the numeric pass, a dense accumulator of N values)
-//                        in global memory; a pool of such workgroups, sized to
-//                        about 1 GiB of slabs, walks the list of these rows
+//   more                 one workgroup of 1024 threads with a bitmap over all N
+//                        columns in global memory (plus, in the numeric pass,
+//                        one rank per bitmap word, so that a column's place in
+//                        the row follows from its bit); a pool of such
+//                        workgroups walks the list of these rows
 //
 // Hash rows are emitted sorted: the wavefront version ranks every entry by
 // counting smaller keys (at most 256 of them), the workgroup version sorts in
@@ -40,11 +41,10 @@ constexpr int kMinHugeWorkgroups = 64;
 constexpr int kMaxHugeWorkgroups = 1024;
 constexpr size_t kHugeSlabBudget = (size_t)1 << 30;
 
-// Number of bitmap workgroups: as many slabs (N bits + N values) as fit the
-// budget.  Priced for 8-byte values whatever the dtype, so that the pool -- and
-// with it the workspace layout up to the slabs -- is the same for both passes.
+// Number of bitmap workgroups: as many slabs (N bits and N / 32 ranks) as fit
+// the budget, within [kMinHugeWorkgroups, kMaxHugeWorkgroups].
 inline int huge_workgroups(int64_t N) {
-  const size_t slab = (size_t)(N + 31) / 32 * 4 + (size_t)N * 8 + 1;
+  const size_t slab = (size_t)(N + 31) / 32 * 8 + 1;
   const size_t fit = kHugeSlabBudget / slab;
   return (int)(fit < (size_t)kMinHugeWorkgroups ? kMinHugeWorkgroups
                                                 : (fit > (size_t)kMaxHugeWorkgroups ? kMaxHugeWorkgroups : fit));
@@ -574,9 +574,16 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   }
 }
 
-// ---- rows beyond that: bitmap (and dense accumulator) over all columns ---------------
+// ---- rows beyond that: a bitmap over all columns -------------------------------------------
 // Workgroups of 1024 threads: such a row has tens of thousands of products and
-// is one workgroup's alone, so its width is the row's parallelism.
+// is one workgroup's alone, so its width is the row's parallelism.  The
+// symbolic pass sets a bit per product and counts the bits.  The numeric pass
+// walks the products twice: first for the bits again, from which it writes the
+// row's column indices (ascending by construction), zeroes the row's values and
+// notes the rank of every bitmap word's first column; then for the values, each
+// product adding itself to the row's output at rank(word) + (bits below its own)
+// -- no accumulator over all N columns, whose lines would go through the L2 once
+// per product.
 constexpr int kHugeThreads = 1024;
 constexpr int kHugeWaves = kHugeThreads / kWaveSize;
 constexpr int kHugeEmitWords = 256;  // bitmap words emitted per step (at most 8192 columns)
@@ -586,8 +593,7 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
     int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, const int *__restrict__ counters, unsigned *__restrict__ bitmaps,
-    typename Acc<T>::type *__restrict__ dense, int *__restrict__ c_pos, int *__restrict__ c_crd,
-    T *__restrict__ c_val) {
+    int *__restrict__ ranks, int *__restrict__ c_pos, int *__restrict__ c_crd, T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
   __shared__ int s_scan[kHugeWaves];
   __shared__ ProductBatch<kHugeThreads, A> s_batch;
@@ -598,22 +604,20 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
 
   const int words = (N + 31) / 32;
   unsigned *bitmap = bitmaps + (size_t)blockIdx.x * (size_t)words;
-  A *sums = NUMERIC ? dense + (size_t)blockIdx.x * (size_t)N : nullptr;
-  // This workgroup's slab starts clean and is left clean after every row.
+  int *rank = NUMERIC ? ranks + (size_t)blockIdx.x * (size_t)words : nullptr;
+  A *acc = reinterpret_cast<A *>(c_val);  // sums wrap (integers) or round (floating point) as T's do
+  // This workgroup's bitmap starts clean and is left clean after every row.
   for (int i = tid; i < words; i += kHugeThreads) workgroup_store(&bitmap[i], 0u);
-  if (NUMERIC)
-    for (int i = tid; i < N; i += kHugeThreads) workgroup_store(&sums[i], (A)0);
   __syncthreads();
 
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
     const int row = rows[idx];
-    for_each_product<kHugeThreads, NUMERIC, T, A>(
-        a_pos[row], a_pos[row + 1], tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
-        [&](int k, A product) {
+    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
+    for_each_product<kHugeThreads, false, T, A>(
+        a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A) {
           __hip_atomic_fetch_or(&bitmap[k >> 5], 1u << (k & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          if (NUMERIC) __hip_atomic_fetch_add(&sums[k], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         });
-      __syncthreads();
+    __syncthreads();
 
     if (!NUMERIC) {
       // count the set bits and clear them
@@ -629,37 +633,140 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
       block_exclusive_scan_n<kHugeWaves>(mine, s_scan, total);
       if (tid == 0) c_pos[row] = total;
     } else {
-      // Walk the bitmap in order, kHugeEmitWords words at a time: the set bits of
-      // a step are listed in LDS (ascending), then all threads fetch the sums of
-      // the listed columns side by side and write the step's entries coalesced.
-      int emitted = c_pos[row];
+      // The bitmap in order, kHugeEmitWords words at a time: the set bits of a step
+      // are listed in LDS, then written as column indices, coalesced.
+      const int out = c_pos[row];
+      int emitted = 0;
       for (int base = 0; base < words; base += kHugeEmitWords) {
         const int word = base + tid;
-        unsigned bits = 0u;
-        if (tid < kHugeEmitWords && word < words) {
-          bits = workgroup_load(&bitmap[word]);
-          if (bits) workgroup_store(&bitmap[word], 0u);
-        }
+        const bool mine = tid < kHugeEmitWords && word < words;
+        unsigned bits = mine ? workgroup_load(&bitmap[word]) : 0u;
         int total = 0;
         int at = block_exclusive_scan_n<kHugeWaves>(__popc(bits), s_scan, total);
+        if (mine) workgroup_store(&rank[word], emitted + at);
         while (bits) {
           const int bit = __ffs(bits) - 1;
           bits &= bits - 1;
           s_cols[at++] = word * 32 + bit;
         }
         __syncthreads();
-#pragma unroll 8
         for (int e = tid; e < total; e += kHugeThreads) {
-          const int col = s_cols[e];
-          c_crd[emitted + e] = col;
-          c_val[emitted + e] = (T)workgroup_load(&sums[col]);
-          workgroup_store(&sums[col], (A)0);
+          c_crd[out + emitted + e] = s_cols[e];
+          workgroup_store(&acc[out + emitted + e], (A)0);
         }
         emitted += total;
         // the next step's scan starts with a barrier, which also protects s_cols
       }
-    }
       __syncthreads();
+      for_each_product<kHugeThreads, true, T, A>(
+          a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
+            const unsigned bits = workgroup_load(&bitmap[k >> 5]);
+            const int at = out + workgroup_load(&rank[k >> 5]) + __popc(bits & ((1u << (k & 31)) - 1u));
+            __hip_atomic_fetch_add(&acc[at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          });
+      __syncthreads();
+      for (int word = tid; word < words; word += kHugeThreads)
+        if (workgroup_load(&bitmap[word])) workgroup_store(&bitmap[word], 0u);
+    }
+    __syncthreads();
+  }
+}
+
+// ---- the same tier when the bitmap fits LDS ---------------------------------------------------
+// Atomics on a bitmap in global memory all land on a few hundred cache lines and
+// queue up in the L2's atomic units (the 13.7 M products of a power-law square
+// spend 0.4 ms there per walk).  For N up to 32 * WORDS columns the bitmap lives
+// in LDS instead, with one rank per four bitmap words, and so do the row's sums
+// when the row has at most kAccEntries distinct columns (else they are added
+// into the output with global atomics as above).  Rows are handed out through a
+// counter, one at a time, so the workgroups stay evenly loaded.
+constexpr int kLdsBudget = 160 * 1024 - 1024;
+
+template <typename T, bool NUMERIC, int WORDS>
+__global__ __launch_bounds__(kHugeThreads) void spgemm_lds_bitmap_kernel(
+    int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
+    const int *__restrict__ rows, int *__restrict__ counters, int *__restrict__ c_pos,
+    int *__restrict__ c_crd, T *__restrict__ c_val) {
+  using A = typename Acc<T>::type;
+  constexpr int kGroups = WORDS / 4;
+  constexpr int kFixed = WORDS * 4 + (NUMERIC ? kGroups * 4 : 0) + (int)sizeof(ProductBatch<kHugeThreads, A>) + 512;
+  constexpr int kAccEntries = NUMERIC ? (kLdsBudget - kFixed) / (int)sizeof(A) : 1;
+  __shared__ unsigned s_bits[WORDS];
+  __shared__ int s_rank[NUMERIC ? kGroups : 1];  // rank of the first column of every group of four words
+  __shared__ A s_acc[kAccEntries];
+  __shared__ ProductBatch<kHugeThreads, A> s_batch;
+  __shared__ int s_scan[kHugeWaves];
+  __shared__ int s_next;
+  const int tid = threadIdx.x;
+  const int n_rows = counters[1];
+  const int words = (N + 31) / 32;
+  const int groups = (words + 3) / 4;
+  A *acc = reinterpret_cast<A *>(c_val);
+
+  for (;;) {
+    __syncthreads();  // everyone is done with the previous row (and with s_next)
+    if (tid == 0) s_next = atomicAdd(&counters[3], 1);
+    for (int i = tid; i < 4 * groups; i += kHugeThreads) s_bits[i] = 0u;
+    __syncthreads();
+    const int idx = s_next;
+    if (idx >= n_rows) return;  // the same for every thread
+    const int row = rows[idx];
+    const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
+    for_each_product<kHugeThreads, false, T, A>(
+        a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
+        [&](int k, A) { atomicOr(&s_bits[k >> 5], 1u << (k & 31)); });
+    __syncthreads();
+
+    // distinct columns, and the rank of each group's first one
+    int n = 0;
+    for (int base = 0; base < groups; base += kHugeThreads) {
+      const int g = base + tid;
+      int cnt = 0;
+      if (g < groups)
+        cnt = __popc(s_bits[4 * g]) + __popc(s_bits[4 * g + 1]) + __popc(s_bits[4 * g + 2]) + __popc(s_bits[4 * g + 3]);
+      int total = 0;
+      const int at = block_exclusive_scan_n<kHugeWaves>(cnt, s_scan, total);
+      if (NUMERIC && g < groups) s_rank[g] = n + at;
+      n += total;
+    }
+    if (!NUMERIC) {
+      if (tid == 0) c_pos[row] = n;
+      continue;
+    }
+
+    const int out = c_pos[row];
+    const bool sums_in_lds = n <= kAccEntries;  // uniform
+    __syncthreads();                            // s_rank is complete
+    for (int g = tid; g < groups; g += kHugeThreads) {
+      int at = out + s_rank[g];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        unsigned bits = s_bits[4 * g + i];
+        while (bits) {
+          const int bit = __ffs(bits) - 1;
+          bits &= bits - 1;
+          c_crd[at++] = (4 * g + i) * 32 + bit;
+        }
+      }
+    }
+    if (sums_in_lds) {
+      for (int e = tid; e < n; e += kHugeThreads) s_acc[e] = (A)0;
+    } else {
+      for (int e = tid; e < n; e += kHugeThreads) workgroup_store(&acc[out + e], (A)0);
+    }
+    __syncthreads();
+    for_each_product<kHugeThreads, true, T, A>(
+        a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
+          const int w = k >> 5;
+          int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (k & 31)) - 1u));
+          for (int i = w & ~3; i < w; ++i) at += __popc(s_bits[i]);
+          if (sums_in_lds) atomic_accumulate<A>(&s_acc[at], product);
+          else __hip_atomic_fetch_add(&acc[out + at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        });
+    __syncthreads();
+    if (sums_in_lds)
+      for (int e = tid; e < n; e += kHugeThreads) c_val[out + e] = (T)s_acc[e];
   }
 }
 
@@ -669,7 +776,7 @@ struct SpgemmWorkspace {
   int huge_pool;
   int *scan_totals;
   unsigned *bitmaps;
-  void *dense;
+  int *ranks;
   size_t total;
 };
 
@@ -687,7 +794,8 @@ inline SpgemmWorkspace spgemm_layout(char *base, int64_t M, int64_t N, size_t el
   ws.scan_totals = reinterpret_cast<int *>(take(((size_t)(M + 1) / kScanTile + 1) * 4));
   ws.huge_pool = huge_workgroups(N);
   ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
-  ws.dense = take((size_t)ws.huge_pool * (size_t)N * elem);
+  ws.ranks = reinterpret_cast<int *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
+  (void)elem;  // no part of the workspace depends on the value type
   ws.total = off;
   return ws;
 }
@@ -716,7 +824,6 @@ template <typename T, bool NUMERIC>
 int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val, const int *b_pos,
                const int *b_crd, const T *b_val, int *c_pos, int *c_crd, T *c_val,
                const SpgemmWorkspace &ws, hipStream_t stream) {
-  using A = typename Acc<T>::type;
   spgemm_reset_kernel<<<1, 64, 0, stream>>>(ws.counters, NUMERIC ? nullptr : c_pos + M);
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned row_groups = (unsigned)(((int64_t)M + kBoundsRows - 1) / kBoundsRows);
@@ -735,9 +842,18 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
       a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kHugeThreads, 0, stream>>>(
-      N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
-      static_cast<A *>(ws.dense), c_pos, c_crd, c_val);
+  // one workgroup per CU's worth of LDS; more only queue up behind them
+  const unsigned lds_pool = (unsigned)(M < 512 ? M : 512);
+  if (N <= 32 * 4096)
+    spgemm_lds_bitmap_kernel<T, NUMERIC, 4096><<<lds_pool, kHugeThreads, 0, stream>>>(
+        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
+  else if (N <= 32 * 16384)
+    spgemm_lds_bitmap_kernel<T, NUMERIC, 16384><<<lds_pool, kHugeThreads, 0, stream>>>(
+        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
+  else
+    spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kHugeThreads, 0, stream>>>(
+        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
+        ws.ranks, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (!NUMERIC) {
     const int64_t n = (int64_t)M + 1;
@@ -782,7 +898,6 @@ int scorch_hip_spgemm_csr_symbolic(int64_t M, int64_t K, int64_t N, const int32_
                                    size_t workspace_bytes, void *stream) {
   using namespace scorch;
   const char *fn = "scorch_hip_spgemm_csr_symbolic";
-  // the symbolic pass never touches the dense accumulators: size them for 1-byte elements
   if (int rc = spgemm_check(fn, M, K, N, a_row_ptr, a_col_idx, b_row_ptr, b_col_idx, c_row_ptr,
                             workspace, workspace_bytes, 1))
     return rc;

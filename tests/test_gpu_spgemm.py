@@ -38,10 +38,9 @@ def check(oracle, arp, aci, av, brp, bci, bv, n_cols):
     if np.issubdtype(av.dtype, np.integer):
         assert np.array_equal(v, wv)
     else:
-        A = sp.csr_matrix((av.astype(np.float64), aci, arp), shape=(len(arp) - 1, len(brp) - 1))
-        B = sp.csr_matrix((bv.astype(np.float64), bci, brp), shape=(len(brp) - 1, n_cols))
-        dense = np.asarray((A @ B).todense())
-        ref64 = dense[np.repeat(np.arange(len(rp) - 1), np.diff(rp)), ci]
+        # fp64 values on the same structure (the oracle's structure is the reference's, checked above)
+        _, _, ref64 = oracle.spgemm_csr_typed(arp, aci, av.astype(np.float64), brp, bci, bv.astype(np.float64),
+                                              n_cols)
         assert oracle.rel_fro(v, ref64) <= (1e-5 if av.dtype == np.float32 else 1e-13)
     return rp, ci, v
 
@@ -89,6 +88,29 @@ def test_huge_rows_bitmap_path_and_all_three_mixed(oracle, dtype):
     brp, bci, bv = random_csr(rng, 800, 5000, 0.02, dtype=dtype)
     rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, 5000)
     assert np.diff(rp).max() > 4096
+
+
+@pytest.mark.parametrize("n_cols,dtype", [(100_000, np.float32), (100_000, np.float64), (300_000, np.float32),
+                                          (300_000, np.int64), (600_000, np.float32), (600_000, np.float64),
+                                          (600_000, np.int32)])
+def test_bitmap_tier_by_width(oracle, n_cols, dtype):
+    """Rows beyond 4096 products at three widths of B: bitmap in LDS (4096 and
+    16384 words) and in global memory.  One row has ~39,000 distinct columns,
+    more than the LDS accumulators hold; the others fit."""
+    rng = np.random.default_rng(7)
+    lens = rng.integers(0, 4, 60)
+    lens[[5, 31, 59]] = [500, 120, 60]
+    arp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    aci = np.concatenate([np.sort(rng.choice(900, int(n), replace=False)) for n in lens]).astype(np.int32)
+    av = (rng.integers(-9, 9, aci.size) if np.issubdtype(dtype, np.integer)
+          else rng.uniform(-1, 1, aci.size)).astype(dtype)
+    b_lens = np.full(900, 100)
+    brp = np.concatenate([[0], np.cumsum(b_lens)]).astype(np.int32)
+    bci = np.concatenate([np.sort(rng.choice(n_cols, 100, replace=False)) for _ in range(900)]).astype(np.int32)
+    bv = (rng.integers(-9, 9, bci.size) if np.issubdtype(dtype, np.integer)
+          else rng.uniform(-1, 1, bci.size)).astype(dtype)
+    rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, n_cols)
+    assert np.diff(rp).max() > 36_000
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
