@@ -347,8 +347,9 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     for (int i = threadIdx.x; i < s_n[l]; i += kBlockThreads) lists[l][s_base[l] + i] = s_list[l][i];
 }
 
+// counters: [0] medium rows, [1] huge rows, [2] small rows listed; [3], [4] next row to hand out
 __global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
-  if (threadIdx.x < 4) counters[threadIdx.x] = 0;
+  if (threadIdx.x < 8) counters[threadIdx.x] = 0;
   if (threadIdx.x == 0 && c_pos_last) *c_pos_last = 0;
 }
 
@@ -682,51 +683,54 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
 // counter, one at a time, so the workgroups stay evenly loaded.
 constexpr int kLdsBudget = 160 * 1024 - 1024;
 
-template <typename T, bool NUMERIC, int WORDS>
-__global__ __launch_bounds__(kHugeThreads) void spgemm_lds_bitmap_kernel(
+// THREADS: workgroup size.  ACC: LDS sums to provide (0: all the LDS that is left).
+// LIST, WORK: which of `counters` holds the length of `rows` and the next row to hand out.
+template <typename T, bool NUMERIC, int WORDS, int THREADS, int ACC, int LIST, int WORK>
+__global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
     int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, int *__restrict__ counters, int *__restrict__ c_pos,
     int *__restrict__ c_crd, T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
   constexpr int kGroups = WORDS / 4;
-  constexpr int kFixed = WORDS * 4 + (NUMERIC ? kGroups * 4 : 0) + (int)sizeof(ProductBatch<kHugeThreads, A>) + 512;
-  constexpr int kAccEntries = NUMERIC ? (kLdsBudget - kFixed) / (int)sizeof(A) : 1;
+  constexpr int kFixed = WORDS * 4 + (NUMERIC ? kGroups * 4 : 0) + (int)sizeof(ProductBatch<THREADS, A>) + 512;
+  constexpr int kAccEntries = !NUMERIC ? 1 : ACC > 0 ? ACC : (kLdsBudget - kFixed) / (int)sizeof(A);
+  constexpr int kWaves = THREADS / kWaveSize;
   __shared__ unsigned s_bits[WORDS];
   __shared__ int s_rank[NUMERIC ? kGroups : 1];  // rank of the first column of every group of four words
   __shared__ A s_acc[kAccEntries];
-  __shared__ ProductBatch<kHugeThreads, A> s_batch;
-  __shared__ int s_scan[kHugeWaves];
+  __shared__ ProductBatch<THREADS, A> s_batch;
+  __shared__ int s_scan[kWaves];
   __shared__ int s_next;
   const int tid = threadIdx.x;
-  const int n_rows = counters[1];
+  const int n_rows = counters[LIST];
   const int words = (N + 31) / 32;
   const int groups = (words + 3) / 4;
   A *acc = reinterpret_cast<A *>(c_val);
 
   for (;;) {
     __syncthreads();  // everyone is done with the previous row (and with s_next)
-    if (tid == 0) s_next = atomicAdd(&counters[3], 1);
-    for (int i = tid; i < 4 * groups; i += kHugeThreads) s_bits[i] = 0u;
+    if (tid == 0) s_next = atomicAdd(&counters[WORK], 1);
+    for (int i = tid; i < 4 * groups; i += THREADS) s_bits[i] = 0u;
     __syncthreads();
     const int idx = s_next;
     if (idx >= n_rows) return;  // the same for every thread
     const int row = rows[idx];
     const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
-    for_each_product<kHugeThreads, false, T, A>(
+    for_each_product<THREADS, false, T, A>(
         a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
         [&](int k, A) { atomicOr(&s_bits[k >> 5], 1u << (k & 31)); });
     __syncthreads();
 
     // distinct columns, and the rank of each group's first one
     int n = 0;
-    for (int base = 0; base < groups; base += kHugeThreads) {
+    for (int base = 0; base < groups; base += THREADS) {
       const int g = base + tid;
       int cnt = 0;
       if (g < groups)
         cnt = __popc(s_bits[4 * g]) + __popc(s_bits[4 * g + 1]) + __popc(s_bits[4 * g + 2]) + __popc(s_bits[4 * g + 3]);
       int total = 0;
-      const int at = block_exclusive_scan_n<kHugeWaves>(cnt, s_scan, total);
+      const int at = block_exclusive_scan_n<kWaves>(cnt, s_scan, total);
       if (NUMERIC && g < groups) s_rank[g] = n + at;
       n += total;
     }
@@ -738,7 +742,7 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_lds_bitmap_kernel(
     const int out = c_pos[row];
     const bool sums_in_lds = n <= kAccEntries;  // uniform
     __syncthreads();                            // s_rank is complete
-    for (int g = tid; g < groups; g += kHugeThreads) {
+    for (int g = tid; g < groups; g += THREADS) {
       int at = out + s_rank[g];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -751,12 +755,12 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_lds_bitmap_kernel(
       }
     }
     if (sums_in_lds) {
-      for (int e = tid; e < n; e += kHugeThreads) s_acc[e] = (A)0;
+      for (int e = tid; e < n; e += THREADS) s_acc[e] = (A)0;
     } else {
-      for (int e = tid; e < n; e += kHugeThreads) workgroup_store(&acc[out + e], (A)0);
+      for (int e = tid; e < n; e += THREADS) workgroup_store(&acc[out + e], (A)0);
     }
     __syncthreads();
-    for_each_product<kHugeThreads, true, T, A>(
+    for_each_product<THREADS, true, T, A>(
         a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
           const int w = k >> 5;
           int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (k & 31)) - 1u));
@@ -766,7 +770,7 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_lds_bitmap_kernel(
         });
     __syncthreads();
     if (sums_in_lds)
-      for (int e = tid; e < n; e += kHugeThreads) c_val[out + e] = (T)s_acc[e];
+      for (int e = tid; e < n; e += THREADS) c_val[out + e] = (T)s_acc[e];
   }
 }
 
@@ -790,7 +794,7 @@ inline SpgemmWorkspace spgemm_layout(char *base, int64_t M, int64_t N, size_t el
   ws.small_rows = reinterpret_cast<int *>(take((size_t)M * 4));
   ws.medium_rows = reinterpret_cast<int *>(take((size_t)M * 4));
   ws.huge_rows = reinterpret_cast<int *>(take((size_t)M * 4));
-  ws.counters = reinterpret_cast<int *>(take(16));
+  ws.counters = reinterpret_cast<int *>(take(32));
   ws.scan_totals = reinterpret_cast<int *>(take(((size_t)(M + 1) / kScanTile + 1) * 4));
   ws.huge_pool = huge_workgroups(N);
   ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
@@ -839,16 +843,23 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   spgemm_medium_kernel<T, NUMERIC, kSmallProducts, 2><<<medium_blocks, kBlockThreads, 0, stream>>>(
       a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.small_rows, ws.counters, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
-      a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
+  if (N <= 32 * 4096) {
+    // narrow enough for a bitmap in LDS beside other workgroups: no hashing, nothing to sort
+    spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kBlockThreads, kMediumProducts, 0, 4>
+        <<<medium_blocks, kBlockThreads, 0, stream>>>(N, a_pos, a_crd, a_val, b_pos, b_crd, b_val,
+                                                      ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
+  } else {
+    spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
+        a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
+  }
   SCORCH_HIP_CHECK(hipGetLastError());
   // one workgroup per CU's worth of LDS; more only queue up behind them
   const unsigned lds_pool = (unsigned)(M < 512 ? M : 512);
   if (N <= 32 * 4096)
-    spgemm_lds_bitmap_kernel<T, NUMERIC, 4096><<<lds_pool, kHugeThreads, 0, stream>>>(
+    spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
   else if (N <= 32 * 16384)
-    spgemm_lds_bitmap_kernel<T, NUMERIC, 16384><<<lds_pool, kHugeThreads, 0, stream>>>(
+    spgemm_lds_bitmap_kernel<T, NUMERIC, 16384, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
   else
     spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kHugeThreads, 0, stream>>>(
