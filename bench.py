@@ -90,6 +90,35 @@ def cpu_baseline(w, repeats=5):
                       "warm-up, whole native call incl. allocating and zeroing C"}
 
 
+def cpu_baseline_sddmm(w, repeats=5):
+    """The reference's sddmm_coo_float_prebuilt (oracle/_ref) or the C
+    restatement of it, on the host cores, coordinate mask, same inputs."""
+    from oracle import oracle as O
+    nnz, K = int(w["col_idx"].size), w["K"]
+    kind = "reference" if O.have_ref() else "port"
+    times = []
+    for i in range(repeats + 1):
+        t0 = time.perf_counter()
+        try:
+            if kind == "reference":
+                O.ref_sddmm_coo(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"], (w["M"], w["n_cols"]))
+            else:
+                O.sddmm_coo_f32(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])
+        except Exception as exc:  # module built for another host
+            if kind == "port":
+                raise
+            print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
+            kind = "port"
+            continue
+        if i:
+            times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {"value": round((2.0 * nnz * K + nnz) / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
+            "kind": kind, "ms_per_step": round(med * 1e3, 3),
+            "sample": f"full workload (nnz={nnz}, K={K}), median of {len(times)} calls after 1 warm-up, "
+                      "incl. wrapping the operands"}
+
+
 def _time_steps(fn, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -266,6 +295,8 @@ def side_workload(args, dev) -> int:
         out = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
                "ms_per_step": round(ms, 4), "ms_per_step_coo_mask": round(ms_coo, 4),
                "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K}}
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline_sddmm(w)
         if args.vendor:
             mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
             Bt = B.t().contiguous()
@@ -286,6 +317,8 @@ def side_workload(args, dev) -> int:
                           "features": N}}
         if args.vendor:
             out["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
+        if not args.no_cpu:
+            out["cpu_baseline"] = cpu_baseline(w)
     out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
                 "data": "synthetic", "higher_is_better": True,
                 "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
