@@ -315,6 +315,17 @@ def side_workload(args, dev) -> int:
                "ms_per_step": round(ms, 4),
                "config": {"workload": args.workload + "_fp32", "rows": M, "cols": K, "nnz": nnz,
                           "features": N}}
+        if args.graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                fn()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            out["ms_per_step_graph_replay"] = round(_time_steps(graph.replay, args.steps, args.warmup), 4)
         if args.vendor:
             out["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
         if not args.no_cpu:
@@ -343,6 +354,8 @@ def main() -> int:
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture one step in a HIP graph and time its replay (SpMM side workloads)")
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")

@@ -243,3 +243,40 @@ def test_matmul_normalises_a_transposed_csr_operand():
     out = scorch.matmul(A, b.cuda())
     assert torch.allclose(out.cpu(), a @ b, atol=1e-5)
     assert A.index.mode_order == [1, 0]          # the caller's tensor is left as it was
+
+
+# ---- HIP graphs -------------------------------------------------------------------------------------
+def test_steps_replay_from_a_hip_graph():
+    """The entry points only enqueue kernels on the caller's stream (no allocation,
+    no synchronisation, no memset), so a step can be captured once and replayed.
+    Each replay is checked against an eager call on fresh operand values, with
+    eager work and synchronisations between the replays."""
+    w = workloads.spmm_uniform()
+    M, K, N = w["M"], w["K"], w["N"]
+    rp, ci, v = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    B = dev(w["B"]).reshape(-1)
+    x = B[:K].clone()
+    spmm = lambda: H.spmm_csr_float_v2([M, N], [M, K], [[], [rp, ci]], v, [K, N], [[], []], B).storage.value
+    spmv = lambda: H.prebuilt_spmv_csr_f32([M], [M, K], [[], [rp, ci]], v, [K], [[]], x).storage.value
+    sddmm = lambda: H.sddmm_csr_float([M, K], [M, K], [[], [rp, ci]], v, [M, N], [[], []], B[:M * N],
+                                      [K, N], [[], []], B).storage.value
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up off the default stream, as graph capture wants it
+        for fn in (spmm, spmv, sddmm):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = (spmm(), spmv(), sddmm())
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    for _ in range(4):
+        B.copy_(torch.randn(B.shape, device="cuda", generator=gen))
+        x.copy_(torch.randn(x.shape, device="cuda", generator=gen))
+        eager = [fn().clone() for fn in (spmm, spmv, sddmm)]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want)
