@@ -42,6 +42,24 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef short short8v __attribute__((ext_vector_type(8)));
 typedef short4v __attribute__((address_space(3))) lds_short4v;
 
+// Combine a value over the four lanes that share a query (lanes n, n + 16,
+// n + 32, n + 48) with the row-swap instructions of gfx950: they stay in the
+// vector ALU, where a shuffle through LDS (ds_bpermute) would put two LDS round
+// trips into the middle of every key block's dependent chain.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the
+// even rows of its second, v_permlane32_swap the upper half of the first with the
+// lower half of the second; fed the same value twice, the two results hold, in
+// every lane, the value of the lane and of its partner.
+template <typename Op>
+__device__ __forceinline__ float combine_query_lanes(float x, Op op) {
+  const unsigned bits = __builtin_bit_cast(unsigned, x);
+  auto r = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  x = op(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+  const unsigned bits2 = __builtin_bit_cast(unsigned, x);
+  auto q = __builtin_amdgcn_permlane32_swap(bits2, bits2, false, false);
+  return op(__builtin_bit_cast(float, (unsigned)q[0]), __builtin_bit_cast(float, (unsigned)q[1]));
+}
+
 template <bool NEGATIVE_SCALE>
 __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
@@ -101,13 +119,14 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   bf16x8 k_stage[2][2], v_stage[2][2];
   auto load_tile = [&](auto set_tag, int it) {
     constexpr int kSet = decltype(set_tag)::value;
-    const int kb = block_col_idx[it];
+    // tile base: the same for every thread (scalar arithmetic); piece offset: fixed per thread
+    const size_t tile = (size_t)uniform(block_col_idx[it]) * (kAttnBlock * kAttnDim);
+    const __bf16 *k_tile = Kh + tile, *v_tile = Vh + tile;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int c = tid + u * kBlockThreads;
-      const size_t off = (size_t)(kb * kAttnBlock + (c >> 3)) * kAttnDim + (c & 7) * 8;
-      k_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(Kh + off);
-      v_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(Vh + off);
+      const int piece = (tid + u * kBlockThreads) * 8;  // tiles are contiguous: piece c starts at element 8 c
+      k_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(k_tile + piece);
+      v_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(v_tile + piece);
     }
   };
   auto store_tile = [&](auto set_tag) {  // register set p -> LDS buffer p
@@ -154,8 +173,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) mx = NEGATIVE_SCALE ? fminf(mx, st[t][r]) : fmaxf(mx, st[t][r]);
     mx *= scale_log2e;
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mx = combine_query_lanes(mx, [](float a, float b) { return fmaxf(a, b); });
     const float m_new = fmaxf(m_run, mx);
     // Rescale what has been accumulated only when some query's maximum moved
     // (after the first few key blocks it rarely does).
@@ -211,9 +229,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   }
 
   // Normalise and store O[query][16dt + 4g .. + 3] (8 bytes per tile and lane).
-  float l = l_run;
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
+  const float l = combine_query_lanes(l_run, [](float a, float b) { return a + b; });
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // block rows without key blocks give zeros
   __bf16 *out = O + head_off + (size_t)query * kAttnDim;
 #pragma unroll
