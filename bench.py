@@ -197,6 +197,37 @@ def probe_memory(args, dev) -> int:
     return 0
 
 
+def probe_compute(args, dev) -> int:
+    """Matrix-core and vector-ALU rates of this GPU, alone and in one loop, from
+    libscorch_probes.so (scorch_amd/csrc/probes/membench.hip).  One JSON line."""
+    import torch
+    from scorch_amd import build as hip_build
+    if not os.path.exists(hip_build.PROBES_PATH):
+        print("libscorch_probes.so is not built (python __graft_entry__.py)", file=sys.stderr)
+        return 1
+    P = ctypes.CDLL(hip_build.PROBES_PATH)
+    P.scorch_probe_compute.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    iters, rows = 4000, []
+    for per_simd in (1, 2, 4, 8):
+        workgroups = 256 * per_simd                       # 256 CUs x 4 SIMDs x per_simd wavefronts
+        waves = workgroups * 4
+        row = {"wavefronts_per_simd": per_simd}
+        for mode, name in ((0, "matrix"), (1, "vector"), (2, "both")):
+            call = lambda: P.scorch_probe_compute(mode, workgroups, iters, sink.data_ptr(), stream)
+            assert call() == 0
+            ms = _time_steps(call, 3, 1)
+            row[name + "_ms"] = round(ms, 4)
+            if mode != 1:
+                row[name + "_matrix_tflops"] = round(waves * iters * 8 * 16384 / ms / 1e9, 1)
+            if mode != 0:
+                row[name + "_vector_tflops"] = round(waves * iters * 64 * 64 * 2 / ms / 1e9, 1)
+        rows.append(row)
+    print(json.dumps({"probe": "compute", "iterations": iters, "rows": rows}))
+    return 0
+
+
 def side_workload(args, dev) -> int:
     """Times one of the other workloads (not the headline metric): same JSON
     shape, HIP-event time per step, algorithmic and gather-model bandwidth."""
@@ -359,6 +390,8 @@ def main() -> int:
     ap.add_argument("--probe-copy", action="store_true",
                     help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")
+    ap.add_argument("--probe-compute", action="store_true",
+                    help="measure matrix-core and vector-ALU throughput alone and in one loop")
     ap.add_argument("--probe-memory", action="store_true",
                     help="measure what the GPU sustains for a streaming read and for random row "
                          "gathers (kernels that only load): the ceilings the kernels are priced against")
@@ -394,6 +427,8 @@ def main() -> int:
 
     if args.probe_memory:
         return probe_memory(args, dev)
+    if args.probe_compute:
+        return probe_compute(args, dev)
     if args.workload != "gcn_powerlaw":
         return side_workload(args, dev)
 

@@ -1,7 +1,7 @@
-// Memory-system probes used by bench.py --probe: what this GPU sustains for a
-// streaming read and for random row gathers, measured with kernels that do
-// nothing else.  They give the ceilings the SpMM/SDDMM kernels are priced
-// against.  Built into libscorch_probes.so, separate from the product library.
+// Probes used by bench.py --probe-memory / --probe-compute: what this GPU
+// sustains for a streaming read, for random row gathers, and for matrix and
+// vector instructions alone and side by side, measured with kernels that do
+// nothing else.  They give the ceilings the kernels are priced against.  Built into libscorch_probes.so, separate from the product library.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -65,7 +65,57 @@ int launch_gather(const float *table, const int *idx, int64_t n_gathers, float *
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
+
+// Matrix and vector throughput.  MODE 0: eight independent v_mfma_f32_16x16x32_bf16
+// per iteration; MODE 1: 64 independent fp32 FMAs per lane and iteration; MODE 2:
+// both in the same loop.  Whether mode 2 takes the longer of the two times or
+// their sum says whether the matrix cores and the vector ALU of a SIMD run side
+// by side.
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float probe_floatx4 __attribute__((ext_vector_type(4)));
+
+template <int MODE>
+__global__ __launch_bounds__(256) void compute_kernel(float *sink, int iters) {
+  probe_bf16x8 a, b;
+  for (int j = 0; j < 8; ++j) {
+    a[j] = (__bf16)(float)(threadIdx.x & 3);
+    b[j] = (__bf16)1.0f;
+  }
+  probe_floatx4 acc[8];
+  for (int i = 0; i < 8; ++i) acc[i] = probe_floatx4{0.f, 0.f, 0.f, 0.f};
+  float x[16];
+  for (int i = 0; i < 16; ++i) x[i] = 1.0f + 0.001f * (threadIdx.x + i);
+  for (int it = 0; it < iters; ++it) {
+    if (MODE != 1) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+    }
+    if (MODE != 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] = __builtin_fmaf(x[i], 1.0001f, 0.5f);
+    }
+  }
+  float s = 0.f;
+  for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  for (int i = 0; i < 16; ++i) s += x[i];
+  if (s == 123.456f) sink[0] = s;  // keeps the work alive
+}
+
 }  // namespace
+
+// mode 0 / 1 / 2 as above; `workgroups` of 256 threads, `iters` loop iterations.
+// Per wavefront and iteration: 8 * 16384 matrix flops, 64 * 64 * 2 vector flops.
+PROBE_API int scorch_probe_compute(int mode, int workgroups, int iters, void *sink, void *stream) {
+  if (!sink || workgroups <= 0 || iters <= 0 || mode < 0 || mode > 2) return 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float *k = static_cast<float *>(sink);
+  if (mode == 0) compute_kernel<0><<<dim3((unsigned)workgroups), 256, 0, s>>>(k, iters);
+  else if (mode == 1) compute_kernel<1><<<dim3((unsigned)workgroups), 256, 0, s>>>(k, iters);
+  else compute_kernel<2><<<dim3((unsigned)workgroups), 256, 0, s>>>(k, iters);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
 
 // Reads `bytes` bytes (multiple of 16) once.  grid = number of 256-thread workgroups.
 PROBE_API int scorch_probe_stream_read(const void *src, int64_t bytes, int grid, void *sink, void *stream) {
