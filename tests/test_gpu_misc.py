@@ -245,6 +245,31 @@ def test_matmul_normalises_a_transposed_csr_operand():
     assert A.index.mode_order == [1, 0]          # the caller's tensor is left as it was
 
 
+def test_format_plumbing_stays_on_the_device():
+    """The formats either side of the kernels, built and converted on the device:
+    coordinate -> CSR (from_coo + to_sparse), CSR transpose, back to torch, and the
+    unfused chain SDDMM -> softmax -> SpMM fed from them (reference:
+    src/scorch/stensor.py:318-365, 785-896, 454-475)."""
+    torch.manual_seed(5)
+    n, d = 96, 32
+    dense = (torch.rand(n, n) * (torch.rand(n, n) < 0.15)).cuda()
+    coo = dense.to_sparse()
+    A = scorch.from_coo(indices=coo.indices(), values=coo.values(), shape=(n, n))
+    assert A.is_cuda and str(A.format) == "o,o"
+    A_csr = A.to_sparse("ds")
+    assert A_csr.is_cuda and all(t.is_cuda for lvl in A_csr.index.mode_indices for t in lvl)
+    assert torch.equal(A_csr.to_torch(in_place=False), dense)
+    At = A_csr.copy().change_mode_order([1, 0])
+    assert At.is_cuda and At.shape == (n, n)
+    q, k = torch.rand(n, d).cuda(), torch.rand(n, d).cuda()
+    scores = scorch.einsum("ij,ik,jk->ij", A_csr, q, k)
+    assert scores.is_cuda
+    want = dense * (q @ k.t())
+    assert torch.allclose(scores.to_torch(in_place=False), want, atol=1e-4)
+    out = scorch.matmul(A_csr, q)
+    assert out.is_cuda and torch.allclose(out, dense @ q, atol=1e-4)
+
+
 # ---- HIP graphs -------------------------------------------------------------------------------------
 def test_steps_replay_from_a_hip_graph():
     """The entry points only enqueue kernels on the caller's stream (no allocation,
