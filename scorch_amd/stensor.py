@@ -215,11 +215,24 @@ class STensor(torch.nn.Module):
             return self
         if self.dim() != 2:
             raise NotImplementedError("to_sparse handles matrices only")
+        target = str(fmt)
+        if not self.format.is_dense() and target in ("d,s", "o,o"):
+            # sparse -> sparse without a dense detour: the stored entries (explicit zeros
+            # included) are kept, sorted by (row, column); repeated coordinates are summed
+            rows, cols = self._coordinates()
+            rows, cols, values = _sorted_unique_entries(rows, cols, self.values, self.shape[1])
+            order = self.index.mode_order
+            if target == "o,o":
+                return STensor._coo(self.shape, [rows.to(torch.int32), cols.to(torch.int32)], values,
+                                    self._name, order)
+            pos = torch.zeros(self.shape[0] + 1, dtype=torch.int64, device=values.device)
+            if rows.numel():
+                pos[1:] = torch.cumsum(torch.bincount(rows, minlength=self.shape[0]), dim=0)
+            return STensor._csr(self.shape, pos.to(torch.int32), cols.to(torch.int32), values, self._name, order)
         if self.format.is_dense():
             dense = self.values.reshape(self.shape)
         else:
             dense = self._as_torch_sparse().to_dense()
-        target = str(fmt)
         if target == "d,s":
             return STensor.from_csr(dense.to_sparse_csr(), self._name)
         if target == "o,o":
@@ -227,6 +240,23 @@ class STensor(torch.nn.Module):
         if target == "d,d":
             return STensor.from_torch(dense, self._name)
         raise NotImplementedError(f"to_sparse: unsupported target format {fmt}")
+
+    def _coordinates(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(rows, cols) as int64 tensors of a 2-D "d,s" or "o,o" STensor, in storage order."""
+        idx = self.index.mode_indices
+        if str(self.format) == "d,s":
+            pos, crd = idx[1]
+            if crd.is_cuda and pos.dtype == torch.int32 and crd.numel() > 0:
+                from . import scorch_ops_hip
+                rows = scorch_ops_hip.csr_row_indices(pos.contiguous(), int(crd.numel())).to(torch.int64)
+            else:
+                counts = (pos[1:] - pos[:-1]).to(torch.int64)
+                rows = torch.repeat_interleave(
+                    torch.arange(self.shape[0], dtype=torch.int64, device=crd.device), counts)
+            return rows, crd.to(torch.int64)
+        if str(self.format) == "o,o":
+            return idx[0][0].to(torch.int64), idx[1][0].to(torch.int64)
+        raise NotImplementedError(f"no coordinates for format {self.format}")
 
     def change_mode_order(self, mode_order: List[int]) -> "STensor":
         """Re-store a matrix so that its physical mode order becomes ``mode_order``

@@ -270,6 +270,31 @@ def test_format_plumbing_stays_on_the_device():
     assert out.is_cuda and torch.allclose(out, dense @ q, atol=1e-4)
 
 
+def test_sparse_to_sparse_conversion_does_not_densify():
+    """Coordinate <-> CSR for a matrix far too large to materialise (2^20 x 2^20),
+    with a repeated coordinate (summed) and an explicit zero (kept)."""
+    n = 1 << 20
+    g = torch.Generator(device="cuda").manual_seed(9)
+    rows = torch.randint(0, n, (200_000,), device="cuda", generator=g)
+    cols = torch.randint(0, n, (200_000,), device="cuda", generator=g)
+    vals = torch.rand(200_000, device="cuda", generator=g)
+    rows[1], cols[1] = rows[0], cols[0]          # a repeated coordinate
+    vals[2] = 0.0                                # an explicit zero
+    A = scorch.from_coo(indices=torch.stack([rows, cols]), values=vals, shape=(n, n))
+    C = A.to_sparse("ds")
+    pos, crd = C.index.mode_indices[1]
+    assert C.is_cuda and pos.dtype == torch.int32 and pos.numel() == n + 1
+    keys = torch.unique(rows * n + cols)
+    assert int(pos[-1]) == keys.numel() == C.values.numel()
+    back = C.to_sparse("oo")
+    r2, c2 = back.index.mode_indices[0][0].long(), back.index.mode_indices[1][0].long()
+    assert torch.equal(r2 * n + c2, keys)        # sorted by (row, column), nothing dropped
+    assert torch.isclose(back.values.sum(), vals.sum(), rtol=1e-4)
+    x = torch.rand(n, 8, device="cuda", generator=g)
+    want = torch.zeros(n, 8, device="cuda").index_add_(0, rows, vals[:, None] * x[cols])
+    assert torch.allclose(scorch.matmul(C, x), want, atol=1e-4)
+
+
 # ---- HIP graphs -------------------------------------------------------------------------------------
 def test_steps_replay_from_a_hip_graph():
     """The entry points only enqueue kernels on the caller's stream (no allocation,
