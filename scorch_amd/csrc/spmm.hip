@@ -530,6 +530,9 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
   const int wide_ipc = spmm_split(M, nnz, N, sizeof(T)).items_per_chunk;
   if (ipc < wide_ipc) ipc = wide_ipc;  // never more carry records than the workspace holds
   const int64_t spans = (total + ipc - 1) / ipc;
+  if (spans > spmm_num_chunks(M, nnz, N, sizeof(T)))
+    return fail(SCORCH_HIP_ERUNTIME, "SpMM: %lld carry records exceed the workspace's %lld",
+                (long long)spans, (long long)spmm_num_chunks(M, nnz, N, sizeof(T)));
   int *carry_row = static_cast<int *>(workspace);
   T *carry_val = reinterpret_cast<T *>(
       static_cast<char *>(workspace) +
