@@ -40,6 +40,7 @@ constexpr int kMediumWorkgroups = 2048;
 constexpr int kMinHugeWorkgroups = 64;
 constexpr int kMaxHugeWorkgroups = 1024;
 constexpr size_t kHugeSlabBudget = (size_t)1 << 30;
+constexpr int kLdsBitmapColumns = 32 * 16384;  // widest B whose column bitmap fits LDS
 
 // Number of bitmap workgroups: as many slabs (N bits and N / 32 ranks) as fit
 // the budget, within [kMinHugeWorkgroups, kMaxHugeWorkgroups].
@@ -797,8 +798,10 @@ inline SpgemmWorkspace spgemm_layout(char *base, int64_t M, int64_t N, size_t el
   ws.counters = reinterpret_cast<int *>(take(32));
   ws.scan_totals = reinterpret_cast<int *>(take(((size_t)(M + 1) / kScanTile + 1) * 4));
   ws.huge_pool = huge_workgroups(N);
-  ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
-  ws.ranks = reinterpret_cast<int *>(take((size_t)ws.huge_pool * ((size_t)(N + 31) / 32) * 4));
+  // up to kLdsBitmapColumns columns the bitmap tier lives in LDS and needs no slabs
+  const size_t slab_words = N <= kLdsBitmapColumns ? 0 : (size_t)(N + 31) / 32;
+  ws.bitmaps = reinterpret_cast<unsigned *>(take((size_t)ws.huge_pool * slab_words * 4));
+  ws.ranks = reinterpret_cast<int *>(take((size_t)ws.huge_pool * slab_words * 4));
   (void)elem;  // no part of the workspace depends on the value type
   ws.total = off;
   return ws;
@@ -858,7 +861,7 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   if (N <= 32 * 4096)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
-  else if (N <= 32 * 16384)
+  else if (N <= kLdsBitmapColumns)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 16384, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
   else
