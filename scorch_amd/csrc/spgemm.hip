@@ -40,7 +40,7 @@ constexpr int kMediumWorkgroups = 2048;
 constexpr int kMinHugeWorkgroups = 64;
 constexpr int kMaxHugeWorkgroups = 1024;
 constexpr size_t kHugeSlabBudget = (size_t)1 << 30;
-constexpr int kLdsBitmapColumns = 32 * 16384;  // widest B whose column bitmap fits LDS
+constexpr int kLdsBitmapColumns = 8 * 32 * 16384;  // widest B served by the LDS bitmap (in up to 8 ranges of columns)
 
 // Number of bitmap workgroups: as many slabs (N bits and N / 32 ranks) as fit
 // the budget, within [kMinHugeWorkgroups, kMaxHugeWorkgroups].
@@ -705,73 +705,88 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   __shared__ int s_next;
   const int tid = threadIdx.x;
   const int n_rows = counters[LIST];
-  const int words = (N + 31) / 32;
-  const int groups = (words + 3) / 4;
+  constexpr int kRangeColumns = 32 * WORDS;
   A *acc = reinterpret_cast<A *>(c_val);
 
   for (;;) {
     __syncthreads();  // everyone is done with the previous row (and with s_next)
     if (tid == 0) s_next = atomicAdd(&counters[WORK], 1);
-    for (int i = tid; i < 4 * groups; i += THREADS) s_bits[i] = 0u;
     __syncthreads();
     const int idx = s_next;
     if (idx >= n_rows) return;  // the same for every thread
     const int row = rows[idx];
     const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
-    for_each_product<THREADS, false, T, A>(
-        a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
-        [&](int k, A) { atomicOr(&s_bits[k >> 5], 1u << (k & 31)); });
-    __syncthreads();
+    const int out = NUMERIC ? c_pos[row] : 0;
+    int done = 0;  // distinct columns found in the ranges before this one
 
-    // distinct columns, and the rank of each group's first one
-    int n = 0;
-    for (int base = 0; base < groups; base += THREADS) {
-      const int g = base + tid;
-      int cnt = 0;
-      if (g < groups)
-        cnt = __popc(s_bits[4 * g]) + __popc(s_bits[4 * g + 1]) + __popc(s_bits[4 * g + 2]) + __popc(s_bits[4 * g + 3]);
-      int total = 0;
-      const int at = block_exclusive_scan_n<kWaves>(cnt, s_scan, total);
-      if (NUMERIC && g < groups) s_rank[g] = n + at;
-      n += total;
-    }
-    if (!NUMERIC) {
-      if (tid == 0) c_pos[row] = n;
-      continue;
-    }
+    // B wider than the bitmap: one range of kRangeColumns columns after the other,
+    // walking the row's products again for each (ranges ascend, so the row comes
+    // out sorted all the same)
+    for (int c0 = 0; c0 < N; c0 += kRangeColumns) {
+      const int columns = N - c0 < kRangeColumns ? N - c0 : kRangeColumns;
+      const int groups = ((columns + 31) / 32 + 3) / 4;
+      if (c0 > 0) __syncthreads();  // the previous range's bits, ranks and sums have been used
+      for (int i = tid; i < 4 * groups; i += THREADS) s_bits[i] = 0u;
+      __syncthreads();
+      for_each_product<THREADS, false, T, A>(
+          a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A) {
+            const unsigned rel = (unsigned)(k - c0);
+            if (rel < (unsigned)columns) atomicOr(&s_bits[rel >> 5], 1u << (rel & 31));
+          });
+      __syncthreads();
 
-    const int out = c_pos[row];
-    const bool sums_in_lds = n <= kAccEntries;  // uniform
-    __syncthreads();                            // s_rank is complete
-    for (int g = tid; g < groups; g += THREADS) {
-      int at = out + s_rank[g];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        unsigned bits = s_bits[4 * g + i];
-        while (bits) {
-          const int bit = __ffs(bits) - 1;
-          bits &= bits - 1;
-          c_crd[at++] = (4 * g + i) * 32 + bit;
-        }
+      // distinct columns of the range, and the rank of each group's first one
+      int n = 0;
+      for (int base = 0; base < groups; base += THREADS) {
+        const int g = base + tid;
+        int cnt = 0;
+        if (g < groups)
+          cnt = __popc(s_bits[4 * g]) + __popc(s_bits[4 * g + 1]) + __popc(s_bits[4 * g + 2]) +
+                __popc(s_bits[4 * g + 3]);
+        int total = 0;
+        const int at = block_exclusive_scan_n<kWaves>(cnt, s_scan, total);
+        if (NUMERIC && g < groups) s_rank[g] = n + at;
+        n += total;
       }
+      if (NUMERIC && n > 0) {  // uniform
+        const int first = out + done;                // the range's place in the row's output
+        const bool sums_in_lds = n <= kAccEntries;  // uniform
+        __syncthreads();                            // s_rank is complete
+        for (int g = tid; g < groups; g += THREADS) {
+          int at = first + s_rank[g];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            unsigned bits = s_bits[4 * g + i];
+            while (bits) {
+              const int bit = __ffs(bits) - 1;
+              bits &= bits - 1;
+              c_crd[at++] = c0 + (4 * g + i) * 32 + bit;
+            }
+          }
+        }
+        if (sums_in_lds) {
+          for (int e = tid; e < n; e += THREADS) s_acc[e] = (A)0;
+        } else {
+          for (int e = tid; e < n; e += THREADS) workgroup_store(&acc[first + e], (A)0);
+        }
+        __syncthreads();
+        for_each_product<THREADS, true, T, A>(
+            a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
+              const unsigned rel = (unsigned)(k - c0);
+              if (rel >= (unsigned)columns) return;
+              const int w = (int)(rel >> 5);
+              int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (rel & 31)) - 1u));
+              for (int i = w & ~3; i < w; ++i) at += __popc(s_bits[i]);
+              if (sums_in_lds) atomic_accumulate<A>(&s_acc[at], product);
+              else __hip_atomic_fetch_add(&acc[first + at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            });
+        __syncthreads();
+        if (sums_in_lds)
+          for (int e = tid; e < n; e += THREADS) c_val[first + e] = (T)s_acc[e];
+      }
+      done += n;
     }
-    if (sums_in_lds) {
-      for (int e = tid; e < n; e += THREADS) s_acc[e] = (A)0;
-    } else {
-      for (int e = tid; e < n; e += THREADS) workgroup_store(&acc[out + e], (A)0);
-    }
-    __syncthreads();
-    for_each_product<THREADS, true, T, A>(
-        a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
-          const int w = k >> 5;
-          int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (k & 31)) - 1u));
-          for (int i = w & ~3; i < w; ++i) at += __popc(s_bits[i]);
-          if (sums_in_lds) atomic_accumulate<A>(&s_acc[at], product);
-          else __hip_atomic_fetch_add(&acc[out + at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        });
-    __syncthreads();
-    if (sums_in_lds)
-      for (int e = tid; e < n; e += THREADS) c_val[out + e] = (T)s_acc[e];
+    if (!NUMERIC && tid == 0) c_pos[row] = done;
   }
 }
 

@@ -92,11 +92,13 @@ def test_huge_rows_bitmap_path_and_all_three_mixed(oracle, dtype):
 
 @pytest.mark.parametrize("n_cols,dtype", [(100_000, np.float32), (100_000, np.float64), (300_000, np.float32),
                                           (300_000, np.int64), (600_000, np.float32), (600_000, np.float64),
-                                          (600_000, np.int32)])
+                                          (1_500_000, np.int32), (4_300_000, np.float32),
+                                          (4_300_000, np.float64), (4_300_000, np.int32)])
 def test_bitmap_tier_by_width(oracle, n_cols, dtype):
-    """Rows beyond 4096 products at three widths of B: bitmap in LDS (4096 and
-    16384 words) and in global memory.  One row has ~39,000 distinct columns,
-    more than the LDS accumulators hold; the others fit."""
+    """Rows beyond 4096 products at several widths of B: bitmap in LDS (4096 and
+    16384 words, the wider ones in two and three ranges of columns) and in
+    global memory.  One row has ~39,000 distinct columns, more than the LDS
+    accumulators hold at the narrow widths; the others fit."""
     rng = np.random.default_rng(7)
     lens = rng.integers(0, 4, 60)
     lens[[5, 31, 59]] = [500, 120, 60]
@@ -106,7 +108,10 @@ def test_bitmap_tier_by_width(oracle, n_cols, dtype):
           else rng.uniform(-1, 1, aci.size)).astype(dtype)
     b_lens = np.full(900, 100)
     brp = np.concatenate([[0], np.cumsum(b_lens)]).astype(np.int32)
-    bci = np.concatenate([np.sort(rng.choice(n_cols, 100, replace=False)) for _ in range(900)]).astype(np.int32)
+    def distinct_sorted(count):
+        cols = np.unique(rng.integers(0, n_cols, 2 * count))
+        return np.sort(rng.choice(cols, count, replace=False))
+    bci = np.concatenate([distinct_sorted(100) for _ in range(900)]).astype(np.int32)
     bv = (rng.integers(-9, 9, bci.size) if np.issubdtype(dtype, np.integer)
           else rng.uniform(-1, 1, bci.size)).astype(dtype)
     rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, n_cols)
