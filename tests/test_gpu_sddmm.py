@@ -85,6 +85,25 @@ def test_csr_rows_with_long_empty_stretches(oracle):
     assert oracle.rel_fro(val, oracle.sddmm_fp64(rows, ci, s, A, B)) <= TOL
 
 
+@pytest.mark.parametrize("K", [8, 64])
+def test_dense_operands_at_odd_element_offsets(oracle, K):
+    """A and B only 4-byte aligned (views one element into their buffers): K is a
+    multiple of four, but the 16-byte loads are not allowed."""
+    rng = np.random.default_rng(60 + K)
+    rp, ci, s = random_csr(rng, 150, 120, 0.1, dtype=np.float32)
+    A = rng.standard_normal((150, K)).astype(np.float32)
+    B = rng.standard_normal((120, K)).astype(np.float32)
+    big_a, big_b = torch.empty(150 * K + 1, device="cuda"), torch.empty(120 * K + 1, device="cuda")
+    big_a[1:].copy_(dev(A).reshape(-1))
+    big_b[1:].copy_(dev(B).reshape(-1))
+    assert big_a[1:].data_ptr() % 16 == 4
+    out = H.sddmm_csr_float([150, 120], [150, 120], [[], [dev(rp), dev(ci)]], dev(s), [150, K], [[], []],
+                            big_a[1:], [120, K], [[], []], big_b[1:])
+    rows = oracle.rows_of(rp)
+    want = oracle.sddmm_fp64(rows, ci, s, A, B)
+    assert oracle.rel_fro(host(out.storage.value), want) <= TOL
+
+
 def test_closed_forms():
     n = 64
     eye = np.eye(n, dtype=np.float32)

@@ -219,6 +219,33 @@ def test_dense_operand_beyond_two_to_the_31_elements():
     assert torch.equal(out, want)
 
 
+@pytest.mark.parametrize("N", [4, 64, 128, 256])
+def test_operands_at_odd_element_offsets(oracle, N):
+    """Dense and value operands that are only 4-byte aligned (views one element
+    into their buffers): the kernels must fall back to narrower loads, not fault
+    or read the wrong elements."""
+    rng = np.random.default_rng(40 + N)
+    rp, ci, v = random_csr(rng, 300, 200, 0.05, dtype=np.float32)
+    B = rng.standard_normal((200, N)).astype(np.float32)
+    big_b = torch.empty(200 * N + 1, device="cuda")
+    big_v = torch.empty(v.size + 1, device="cuda")
+    b_view, v_view = big_b[1:], big_v[1:]
+    b_view.copy_(dev(B).reshape(-1))
+    v_view.copy_(dev(v))
+    assert b_view.data_ptr() % 16 == 4 and v_view.data_ptr() % 8 == 4
+    out = H.spmm_csr_float_v2([300, N], [300, 200], [[], [dev(rp), dev(ci)]], v_view, [200, N], [[], []],
+                              b_view).storage.value
+    got = host(out).reshape(300, N)
+    assert oracle.rel_fro(got, oracle.spmm_fp64(rp, ci, v, B)) <= TOL
+    bias = rng.standard_normal(N).astype(np.float32)
+    big_bias = torch.empty(N + 1, device="cuda")
+    big_bias[1:].copy_(dev(bias))
+    fused = H.spmm_csr_bias_relu_float([300, N], [300, 200], [[], [dev(rp), dev(ci)]], v_view, [200, N],
+                                       [[], []], b_view, big_bias[1:]).storage.value
+    want = np.maximum(oracle.spmm_fp64(rp, ci, v, B) + bias, 0)
+    assert oracle.rel_fro(host(fused).reshape(300, N), want) <= TOL
+
+
 def test_uniform_workload_reference_size(oracle):
     """4096 x 4096 at 1 % density, N = 64: the reference's own CPU-runnable case."""
     w = workloads.spmm_uniform()
