@@ -10,14 +10,19 @@
 //
 //   up to 256 products   one wavefront, hash table of 512 slots in LDS
 //   up to 1024 products  one workgroup, hash table of 2048 slots in LDS
-//   up to 4096 products  one workgroup, hash table of 8192 slots in LDS (the
-//                        smaller table of the tier above lets more workgroups
-//                        share a CU)
-//   more                 one workgroup of 1024 threads with a bitmap over all N
-//                        columns in global memory (plus, in the numeric pass,
-//                        one rank per bitmap word, so that a column's place in
-//                        the row follows from its bit); a pool of such
-//                        workgroups walks the list of these rows
+//   up to 4096 products  B of at most 131,072 columns: a bitmap of the columns in LDS
+//                        (256 threads, see below); wider B: one workgroup, hash
+//                        table of 8192 slots in LDS
+//   more                 one workgroup of 1024 threads with a bitmap of the columns
+//                        in LDS, 524,288 columns at a time (B of up to 4.2 M
+//                        columns is covered in up to eight such ranges, walking the
+//                        row's products once more for each); wider B: a bitmap over
+//                        all N columns in global memory, one per workgroup of a pool
+//
+// A bitmap row needs neither hashing nor sorting: one walk over the products
+// sets the bits, a prefix sum over the bitmap gives every column its rank in
+// the row, and (numeric pass) a second walk adds each product at its column's
+// rank.
 //
 // Hash rows are emitted sorted: the wavefront version ranks every entry by
 // counting smaller keys (at most 256 of them), the workgroup version sorts in
