@@ -212,8 +212,8 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 // between groups is needed, since a row is summed by one group.  A row with many
 // nonzeros in the chunk would leave the other groups idle: such rows are summed
 // by all groups together (strided over its nonzeros, then combined with
-// shuffles in a fixed order).  Used for small N, and for large N when narrow
-// tiles let the B rows a tile gathers stay in one L2 (see use_narrow_tiles).
+// shuffles in a fixed order).  Used when a row of B is under 256 bytes (see
+// narrow_tile_bytes).
 constexpr int kGroupRowMax = 24;  // longer in-chunk rows are shared by all groups
 
 template <typename T, int VEC, int LPR, int EPI>
