@@ -15,11 +15,12 @@ reference's resolver moves on (prebuilt_kernels.py:96-101).
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
 from . import native
+from .utils import check_csr_indices, index_checks_enabled
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
@@ -79,10 +80,13 @@ def _flat(t: torch.Tensor, dtype: torch.dtype, what: str) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
 
 
-def _csr_parts(mode_indices, what: str):
+def _csr_parts(mode_indices, what: str, n_cols: Optional[int] = None):
     if len(mode_indices) != 2 or len(mode_indices[1]) != 2:
         raise ValueError(f"scorch_ops_hip: {what} is not a CSR (\"d,s\") operand")
-    return _index(mode_indices[1][0], what + " pos"), _index(mode_indices[1][1], what + " crd")
+    pos, crd = _index(mode_indices[1][0], what + " pos"), _index(mode_indices[1][1], what + " crd")
+    if n_cols is not None and index_checks_enabled():
+        check_csr_indices(pos, crd, n_cols, "scorch_ops_hip: " + what)
+    return pos, crd
 
 
 def _stream(dev: torch.device) -> int:
@@ -97,7 +101,7 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
     if int(B_shape[0]) != K or tuple(int(s) for s in result_shape) != (M, N):
         raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)} "
                          f"result{tuple(result_shape)}")
-    pos, crd = _csr_parts(A_mode_indices, "A")
+    pos, crd = _csr_parts(A_mode_indices, "A", K)
     a_val = _flat(A_values, dtype, "A values")
     b_val = _flat(B_values, dtype, "B values")
     if pos.numel() != M + 1 or b_val.numel() != K * N or crd.numel() != a_val.numel():
@@ -167,8 +171,8 @@ def _make_spgemm(dtype):
         M, K, N = int(A_shape[0]), int(A_shape[1]), int(B_shape[1])
         if int(B_shape[0]) != K:
             raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)}")
-        a_pos, a_crd = _csr_parts(A_mode_indices, "A")
-        b_pos, b_crd = _csr_parts(B_mode_indices, "B")
+        a_pos, a_crd = _csr_parts(A_mode_indices, "A", K)
+        b_pos, b_crd = _csr_parts(B_mode_indices, "B", N)
         a_val = _flat(A_values, dtype, "A values")
         b_val = _flat(B_values, dtype, "B values")
         if a_pos.numel() != M + 1 or b_pos.numel() != K + 1 or a_crd.numel() != a_val.numel() \
@@ -207,7 +211,7 @@ prebuilt_spmspm_csr_i64 = _make_spgemm(torch.int64)
 def _make_spmv(dtype):
     def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
         M, K = int(A_shape[0]), int(A_shape[1])
-        pos, crd = _csr_parts(A_mode_indices, "A")
+        pos, crd = _csr_parts(A_mode_indices, "A", K)
         a_val = _flat(A_values, dtype, "A values")
         x = _flat(B_values, dtype, "x values")
         if pos.numel() != M + 1 or x.numel() != K or crd.numel() != a_val.numel():
@@ -275,7 +279,7 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     mask entry in mask order: what the reference's generated kernel returns for
     this case (src/scorch/ops.py:638-666).  mode_indices = [[rows], [S's crd]]."""
     M, n_cols, K, a, b = _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values)
-    pos, crd = _csr_parts(S_mode_indices, "S")
+    pos, crd = _csr_parts(S_mode_indices, "S", n_cols)
     s_val = _flat(S_values, torch.float32, "S values")
     if pos.numel() != M + 1 or crd.numel() != s_val.numel():
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")

@@ -264,3 +264,22 @@ def test_change_mode_order_rejects_what_it_cannot_do():
         STensor.from_torch(torch.rand(3, 3)).change_mode_order([0, 0])
     with pytest.raises(NotImplementedError):
         STensor.from_torch(torch.rand(2, 3, 4)).change_mode_order([2, 0, 1])
+
+
+def test_check_csr_indices_names_what_is_wrong(monkeypatch):
+    from scorch_amd.utils import check_csr_indices, index_checks_enabled
+    pos = torch.tensor([0, 2, 2, 5], dtype=torch.int32)
+    crd = torch.tensor([0, 3, 1, 2, 3], dtype=torch.int32)
+    check_csr_indices(pos, crd, 4)                                   # well-formed: no exception
+    with pytest.raises(ValueError, match=r"outside \[0, 3\)"):
+        check_csr_indices(pos, crd, 3)
+    with pytest.raises(ValueError, match="decreases"):
+        check_csr_indices(torch.tensor([0, 3, 2, 5], dtype=torch.int32), crd, 4)
+    with pytest.raises(ValueError, match=r"row_ptr\[-1\] = 4"):
+        check_csr_indices(torch.tensor([0, 2, 2, 4], dtype=torch.int32), crd, 4)
+    with pytest.raises(ValueError, match=r"row_ptr\[0\] = 1"):
+        check_csr_indices(torch.tensor([1, 2, 2, 5], dtype=torch.int32), crd, 4)
+    monkeypatch.delenv("SCORCH_HIP_CHECK_INDICES", raising=False)
+    assert not index_checks_enabled()
+    monkeypatch.setenv("SCORCH_HIP_CHECK_INDICES", "1")
+    assert index_checks_enabled()
