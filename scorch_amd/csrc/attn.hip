@@ -10,9 +10,9 @@
 // Work split.  One workgroup (4 wavefronts) owns one head and one block row of
 // the mask, i.e. 64 queries; each wavefront owns 16 of them.  The workgroup
 // walks the block row's active key blocks.  For each, the 64 x 64 K tile and
-// the 64 x 64 V tile are staged in LDS once for all four wavefronts, both
-// row-major; the next tile's global loads are in flight while the current one
-// is consumed (two LDS buffers, one barrier per key block).  The second
+// the 64 x 64 V tile are put in LDS once for all four wavefronts, both
+// row-major; the next tile's loads are in flight while the current one is
+// consumed (two LDS buffers, one barrier per key block).  The second
 // product needs V by columns (eight keys of one feature per lane): that
 // operand is read with ds_read_b64_tr_b16, which hands each lane of a 16-lane
 // group one column of a 4 x 16 block whose rows the group's lanes address.
@@ -33,7 +33,6 @@ namespace scorch {
 
 constexpr int kAttnBlock = 64;  // mask block edge: queries per workgroup, keys per step
 constexpr int kAttnDim = 64;    // head dimension
-constexpr int kLdsRow = 72;     // LDS row length in bf16 (64 + 8 padding against bank conflicts)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -60,27 +59,39 @@ __device__ __forceinline__ float combine_query_lanes(float x, Op op) {
   return op(__builtin_bit_cast(float, (unsigned)q[0]), __builtin_bit_cast(float, (unsigned)q[1]));
 }
 
+// K and V tiles are written to LDS by the load itself (global_load_lds_dwordx4):
+// no staging registers, no LDS store instructions; with 90 VGPRs and 32 KB of
+// LDS per workgroup five workgroups share a CU.  Such a load puts lane L's 16
+// bytes at (wave-uniform base) + 16 L, so a wavefront instruction fills eight
+// whole 128-byte rows and rows cannot be padded against bank conflicts.  Instead
+// the 16-byte chunks of a row are permuted: chunk c of row r lies at position
+// c ^ (r & 7).  The permutation is applied on the way in (each lane fetches the
+// chunk that belongs at its LDS position) and undone by the readers' address
+// arithmetic.  (Staging through registers with padded rows: 118 VGPRs, 36 KB,
+// four workgroups per CU, 12 % slower.)
+constexpr int kTileBytes = kAttnBlock * kAttnDim * 2;  // 8 KB, rows of 128 bytes
+
 template <bool NEGATIVE_SCALE>
 __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
     const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O) {
-  __shared__ __attribute__((aligned(16))) __bf16 s_k[2][kAttnBlock][kLdsRow];   // [key][feature]
-  __shared__ __attribute__((aligned(16))) __bf16 s_v[2][kAttnBlock][kLdsRow];   // [key][feature]
+  __shared__ __attribute__((aligned(1024))) unsigned char s_k[2][kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_v[2][kTileBytes];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
   const int w = tid / kWaveSize;
-  const int g = lane >> 4;  // 16-lane group: which keys / features of a tile this lane holds
-  const int n = lane & 15;  // query within the wavefront's 16
-  // Workgroup -> (head, block row).  Workgroups are dealt to the 8 XCDs round
-  // robin by their linear id, and every XCD has its own 4 MB L2.  When the head
-  // count allows it, all workgroups of a head are given ids of one residue mod
-  // 8, so that a head's K and V (2 * S * 128 bytes) are fetched into one L2 only
-  // and an XCD works through its heads one after the other.
+  const int g = lane >> 4;
+  const int n = lane & 15;
   int head, rank;
   {
+    // Workgroups are dealt to the 8 XCDs round robin by their linear id, and every
+    // XCD has its own 4 MB L2.  When the head count allows it, all workgroups of a
+    // head are given ids of one residue mod 8, so that a head's K and V
+    // (2 * S * 128 bytes) are fetched into one L2 only and an XCD works through its
+    // heads one after the other.
     const int id = blockIdx.x;
     if (n_heads % 8 == 0) {
       const int xcd = id & 7, slot = id >> 3;
@@ -93,25 +104,21 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   }
   const int qb = n_blocks - 1 - rank;  // longest block rows first
   const size_t head_off = (size_t)head * (size_t)S * kAttnDim;
-  const __bf16 *Qh = Q + head_off, *Kh = K + head_off, *Vh = V + head_off;
+  const __bf16 *Qh = Q + head_off;
+  const unsigned char *Kb = reinterpret_cast<const unsigned char *>(K + head_off);
+  const unsigned char *Vb = reinterpret_cast<const unsigned char *>(V + head_off);
 
-  // B operand of S^T = K Q^T: this lane's query row, features 8g + 32s .. + 7.
   const int query = qb * kAttnBlock + w * 16 + n;
   bf16x8 q_op[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
     q_op[s] = *reinterpret_cast<const bf16x8 *>(Qh + (size_t)query * kAttnDim + 8 * g + 32 * s);
 
-  floatx4 o_acc[4];  // O^T tiles: o_acc[dt][r] = O[query][16 dt + 4g + r]
+  floatx4 o_acc[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) o_acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -3.0e38f;  // running maximum of scale * log2(e) * score, equal in the 4 lanes of a query
-  // Running sum of the (bf16-rounded) probabilities of query n, kept by the matrix
-  // core: a row of ones appended to V^T makes the second product add up P as
-  // well.  Matrix and vector instructions do not overlap on this chip, so two
-  // more matrix instructions (32 cycles) are cheaper than the sixteen additions
-  // (64 cycles) they replace.  Every element of l_acc holds the same value.
-  floatx4 l_acc = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -3.0e38f;
+  floatx4 l_acc = floatx4{0.f, 0.f, 0.f, 0.f};  // row sums of P, taken by the matrix core (ones row)
   bf16x8 ones;
 #pragma unroll
   for (int j = 0; j < 8; ++j) ones[j] = (__bf16)1.0f;
@@ -119,62 +126,52 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   const int kb_begin = block_row_ptr[qb];
   const int kb_end = block_row_ptr[qb + 1];
 
-  // Staging: a thread handles two 16-byte pieces of each tile; piece c covers
-  // row c / 8 (a key), features 8 (c % 8) .. + 7.  Tiles alternate between two
-  // register sets and two LDS buffers by parity: while tile `it` is consumed
-  // from LDS, tile it + 1 waits in registers and tile it + 2 is being fetched,
-  // so a fetch has a whole key block of work to hide behind.
-  bf16x8 k_stage[2][2], v_stage[2][2];
-  auto load_tile = [&](auto set_tag, int it) {
-    constexpr int kSet = decltype(set_tag)::value;
-    // tile base: the same for every thread (scalar arithmetic); piece offset: fixed per thread
-    const size_t tile = (size_t)uniform(block_col_idx[it]) * (kAttnBlock * kAttnDim);
-    const __bf16 *k_tile = Kh + tile, *v_tile = Vh + tile;
+  // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with two instructions
+  // of eight rows each.  Lane L of instruction u lands at row 16w + 8u + L / 8,
+  // position L % 8, which holds chunk (L % 8) ^ (row & 7) = (L % 8) ^ (L / 8).
+  const int src_in_tile = (16 * w + (lane >> 3)) * 128 + (((lane & 7) ^ (lane >> 3)) * 16);
+  auto load_tile = [&](auto buf_tag, int it) {
+    constexpr int kBuf = decltype(buf_tag)::value;
+    const size_t tile = (size_t)uniform(block_col_idx[it]) * kTileBytes;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int piece = (tid + u * kBlockThreads) * 8;  // tiles are contiguous: piece c starts at element 8 c
-      k_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(k_tile + piece);
-      v_stage[kSet][u] = *reinterpret_cast<const bf16x8 *>(v_tile + piece);
-    }
-  };
-  auto store_tile = [&](auto set_tag) {  // register set p -> LDS buffer p
-    constexpr int kSet = decltype(set_tag)::value;
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c = tid + u * kBlockThreads;
-      const int key = c >> 3, f0 = (c & 7) * 8;
-      *reinterpret_cast<bf16x8 *>(&s_k[kSet][key][f0]) = k_stage[kSet][u];
-      *reinterpret_cast<bf16x8 *>(&s_v[kSet][key][f0]) = v_stage[kSet][u];
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void *)(Kb + tile + src_in_tile + u * 1024),
+          (__attribute__((address_space(3))) void *)(&s_k[kBuf][(16 * w + 8 * u) * 128]), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void *)(Vb + tile + src_in_tile + u * 1024),
+          (__attribute__((address_space(3))) void *)(&s_v[kBuf][(16 * w + 8 * u) * 128]), 16, 0, 0);
     }
   };
   using Even = std::integral_constant<int, 0>;
   using Odd = std::integral_constant<int, 1>;
 
-  if (kb_begin < kb_end) {
-    load_tile(Even{}, kb_begin);
-    store_tile(Even{});
-    if (kb_begin + 1 < kb_end) load_tile(Odd{}, kb_begin + 1);
-  }
+  // Readers' offsets inside a tile.  K: row 16t + n, chunks g and g + 4 (positions
+  // g ^ (n & 7) and that ^ 4).  V^T: row 32s + 16h + 4g + n / 4, 8 bytes at feature
+  // 16dt + 4 (n % 4), i.e. chunk 2dt + (n % 4) / 2, half (n % 4) % 2.
+  const int k_off = n * 128 + ((g ^ (n & 7)) * 16);
+  const int v_row = 4 * g + (n >> 2);
+  const int v_swz = v_row & 7;
+  const int v_off = v_row * 128 + (n & 1) * 8;
+  const int v_chunk = (n & 3) >> 1;
+
+  if (kb_begin < kb_end) load_tile(Even{}, kb_begin);
   __syncthreads();
 
-  // One key block: tile `it` has parity P = decltype(tag)::value.
   auto key_block = [&](auto tag, int it) {
     constexpr int buf = decltype(tag)::value;
     using Other = std::integral_constant<int, buf ^ 1>;
-    if (it + 2 < kb_end) load_tile(tag, it + 2);  // this parity's registers are free again
+    if (it + 1 < kb_end) load_tile(Other{}, it + 1);  // its last readers passed the previous barrier
 
-    // S^T tile t: keys 16t .. 16t+15 (rows) x 16 queries (columns).
     floatx4 st[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g]);
-      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&s_k[buf][16 * t + n][8 * g + 32]);
+      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&s_k[buf][2048 * t + k_off]);
+      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&s_k[buf][2048 * t + (k_off ^ 64)]);
       st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_lo, q_op[0], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
       st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_hi, q_op[1], st[t], 0, 0, 0);
     }
 
-    // Online softmax for query n, in base 2: this lane holds keys 16t + 4g + r.
-    // With scale > 0 the maximum of the scaled scores is the scaled maximum.
     float mx = st[0][0];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -183,8 +180,6 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     mx *= scale_log2e;
     mx = combine_query_lanes(mx, [](float a, float b) { return fmaxf(a, b); });
     const float m_new = fmaxf(m_run, mx);
-    // Rescale what has been accumulated only when some query's maximum moved
-    // (after the first few key blocks it rarely does).
     if (__any(m_new > m_run)) {
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_acc[0] *= alpha;
@@ -195,8 +190,6 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     }
     m_run = m_new;
 
-    // P^T as the B operand of the second product: slot j of step s is key
-    // 32s + 16 (j / 4) + 4g + (j % 4).
     bf16x8 p_op[2];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -206,21 +199,13 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
 
-    // O^T tile dt: features 16dt .. 16dt+15 (rows) x 16 queries, contraction over
-    // the 64 keys.  A operand: lane (g, n) needs V[key][16dt + n] for the eight
-    // keys of its slots.  One transposing read covers four consecutive keys:
-    // lane i of the group addresses row key0 + i / 4, features 16dt + 4 (i % 4) .. + 3,
-    // and receives V[key0 .. key0 + 3][16dt + i].
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const int key0 = 32 * s + 4 * g + (n >> 2);
-        const int f0 = 16 * dt + 4 * (n & 3);
-        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_short4v *)&s_v[buf][key0][f0]);
-        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_short4v *)&s_v[buf][key0 + 16][f0]);
+        const int at = 4096 * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&s_v[buf][at]);
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&s_v[buf][at + 2048]);
         const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         const bf16x8 v_op = __builtin_bit_cast(bf16x8, packed);
         o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
@@ -228,8 +213,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 #pragma unroll
     for (int s = 0; s < 2; ++s) l_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, p_op[s], l_acc, 0, 0, 0);
 
-    if (it + 1 < kb_end) store_tile(Other{});
-    __syncthreads();
+    __syncthreads();  // waits for the loads issued above, and lets the next block overwrite this buffer
   };
 
   for (int it = kb_begin; it < kb_end; it += 2) {
@@ -237,7 +221,6 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     if (it + 1 < kb_end) key_block(Odd{}, it + 1);
   }
 
-  // Normalise and store O[query][16dt + 4g .. + 3] (8 bytes per tile and lane).
   const float l = l_acc[0];
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // block rows without key blocks give zeros
   __bf16 *out = O + head_off + (size_t)query * kAttnDim;
