@@ -212,7 +212,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 // between groups is needed, since a row is summed by one group.  A row with many
 // nonzeros in the chunk would leave the other groups idle: such rows are summed
 // by all groups together (strided over its nonzeros, then combined with
-// shuffles in a fixed order).  Used when a row of B is under 256 bytes (see
+// shuffles in a fixed order).  Used when a row of B is at most 256 bytes (see
 // narrow_tile_bytes).
 constexpr int kGroupRowMax = 24;  // longer in-chunk rows are shared by all groups
 
@@ -552,15 +552,15 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
   return SCORCH_HIP_OK;
 }
 
-// Narrow tiles pay off when N is small: a row of B is under 256 bytes, so
-// full-width tiles would leave most lanes idle.  Returns the tile width in
+// Narrow tiles pay off when N is small: a row of B is at most 256 bytes, so
+// full-width tiles would leave lanes idle or fall back to 4-byte loads.  Returns the tile width in
 // bytes, or 0 for wide tiles.  (Tiling a wide B by columns so that K narrow rows
 // stay in one XCD's L2 was measured and lost: the workgroups resident on an XCD
 // span several tiles at once and evict each other's slices.)
 inline int narrow_tile_bytes(int64_t K, int64_t N, int64_t nnz, size_t elem) {
   (void)K; (void)nnz;
   const int64_t row_bytes = N * (int64_t)elem;
-  return row_bytes < 256 ? (int)row_bytes : 0;
+  return row_bytes <= 256 ? (int)row_bytes : 0;
 }
 
 // Elements per lane.  Preferred: the widest vector (at most 16 bytes) that
