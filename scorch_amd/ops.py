@@ -15,8 +15,7 @@ exactly as the reference does at ops.py:256-293.)
 """
 from __future__ import annotations
 
-import time
-from typing import Any, List, Optional, Tuple, Union
+from typing import Any, Optional, Union
 
 import torch
 

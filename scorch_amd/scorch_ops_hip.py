@@ -15,7 +15,7 @@ reference's resolver moves on (prebuilt_kernels.py:96-101).
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import Optional
 
 import torch
 

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 import scorch_amd as scorch
-from gpu_util import dev, host
+from gpu_util import dev
 from scorch_amd import STensor, workloads
 from scorch_amd import scorch_ops_hip as H
 

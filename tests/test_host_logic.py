@@ -2,7 +2,6 @@
 tensor model, the prebuilt-kernel registry and the routing decisions of
 matmul / einsum.  Mirrors tests/test_scorch/test_prebuilt_kernel_registry.py
 and the format checks of the reference; runs without a GPU."""
-import numpy as np
 import pytest
 import torch
 
