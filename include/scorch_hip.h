@@ -260,6 +260,16 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_
 SCORCH_HIP_API int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr,
                                int32_t *row_idx, void *stream);
 
+/* The other direction: the CSR row pointer (M + 1 entries) of coordinates sorted
+ * by row, row_ptr[r] = number of entries in rows below r.  *unsorted, which the
+ * caller has set to 0, is set to 1 if a row coordinate lies outside [0, M) or
+ * below its predecessor; row_ptr is then meaningless.  With it a coordinate
+ * ("o,o") operand is handed to the CSR kernels, which is how this build serves
+ * the reference's spmm_coo_float (csrc/spmm.h:247-372) and spmspm_coo_float
+ * (csrc/kernels.h:397-497, bound at csrc/ops.cpp:140-143). */
+SCORCH_HIP_API int scorch_hip_coo_row_ptr(int64_t M, int64_t nnz, const int32_t *row_idx,
+                           int32_t *row_ptr, int32_t *unsorted, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

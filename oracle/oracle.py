@@ -176,6 +176,59 @@ def spgemm_csr_typed(a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, b_vals,
     return c_pos, c_crd, c_val
 
 
+def _runs(keys: np.ndarray):
+    """(start, end) of every run of equal neighbouring values, in order."""
+    if keys.size == 0:
+        return []
+    cuts = np.flatnonzero(keys[1:] != keys[:-1]) + 1
+    starts = np.concatenate([[0], cuts])
+    ends = np.concatenate([cuts, [keys.size]])
+    return list(zip(starts.tolist(), ends.tolist()))
+
+
+def spmm_coo_f32(row_idx, col_idx, vals, B, n_rows: int) -> np.ndarray:
+    """C = A @ B for A as coordinates (csrc/spmm.h:247-372): each run of equal
+    neighbouring rows is summed into a zeroed workspace, entry by entry, and the
+    workspace added to that row of C; repeated coordinates therefore add up and
+    the order of the runs does not matter beyond rounding.  fp32 throughout."""
+    rows, cols, vals = _c(row_idx, np.int32), _c(col_idx, np.int32), _c(vals, np.float32)
+    B = _c(B, np.float32)
+    C = np.zeros((n_rows, B.shape[1]), dtype=np.float32)
+    for lo, hi in _runs(rows):
+        wksp = np.zeros(B.shape[1], dtype=np.float32)
+        for p in range(lo, hi):
+            wksp += vals[p] * B[cols[p]]
+        C[rows[lo]] += wksp
+    return C
+
+
+def spgemm_coo_f32(a_row_idx, a_col_idx, a_vals, b_row_idx, b_col_idx, b_vals):
+    """C = A @ B, all three as coordinates (spmspm_coo_float_opt, csrc/kernels.h:397-497).
+    For each run of equal neighbouring rows of A, in A's order: every entry (i, j, v)
+    of the run adds v * B[j, k] to sums[k] for the entries of B whose row is j, in
+    B's storage order; the columns touched (cancelled sums included) are emitted in
+    ascending order.  Returns (row, col, val).  Small inputs only (Python loops)."""
+    a_rows, a_cols, a_vals = _c(a_row_idx, np.int32), _c(a_col_idx, np.int32), _c(a_vals, np.float32)
+    b_rows, b_cols, b_vals = _c(b_row_idx, np.int32), _c(b_col_idx, np.int32), _c(b_vals, np.float32)
+    by_row = {}
+    for p in range(b_rows.size):  # B's entries of each row, in storage order
+        by_row.setdefault(int(b_rows[p]), []).append(p)
+    out_r, out_c, out_v = [], [], []
+    for lo, hi in _runs(a_rows):
+        sums = {}
+        for p in range(lo, hi):
+            v = a_vals[p]
+            for q in by_row.get(int(a_cols[p]), ()):
+                k = int(b_cols[q])
+                sums[k] = np.float32(sums.get(k, np.float32(0)) + v * b_vals[q])
+        for k in sorted(sums):
+            out_r.append(int(a_rows[lo]))
+            out_c.append(k)
+            out_v.append(sums[k])
+    return (np.asarray(out_r, dtype=np.int32), np.asarray(out_c, dtype=np.int32),
+            np.asarray(out_v, dtype=np.float32))
+
+
 def spgemm_fp64(a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, b_vals, shape_a, n_cols):
     """(A @ B) as a dense float64 array (small cases) via scipy."""
     A = _scipy_csr(a_row_ptr, a_col_idx, a_vals, shape_a)
@@ -334,6 +387,31 @@ def ref_spgemm(symbol: str, a_row_ptr, a_col_idx, a_vals, b_row_ptr, b_col_idx, 
                              torch.from_numpy(_c(b_vals, a_vals.dtype)))
     idx = out.storage.index.mode_indices[1]
     return idx[0].numpy().copy(), idx[1].numpy().copy(), out.storage.value.numpy().copy()
+
+
+def ref_spmm_coo(row_idx, col_idx, vals, B, n_rows: int) -> np.ndarray:
+    """Call the reference's spmm_coo_float on numpy inputs."""
+    import torch
+    m = ref_module()
+    B = _c(B, np.float32)
+    a_idx = [[torch.from_numpy(_c(row_idx, np.int32))], [torch.from_numpy(_c(col_idx, np.int32))]]
+    out = m.spmm_coo_float([n_rows, B.shape[1]], [n_rows, B.shape[0]], a_idx,
+                           torch.from_numpy(_c(vals, np.float32)), list(B.shape), [[], []],
+                           torch.from_numpy(B).reshape(-1))
+    return out.storage.value.numpy().reshape(n_rows, B.shape[1]).copy()
+
+
+def ref_spgemm_coo(a_row_idx, a_col_idx, a_vals, b_row_idx, b_col_idx, b_vals, shape_a, n_cols):
+    """Call the reference's spmspm_coo_float; returns (row, col, val)."""
+    import torch
+    m = ref_module()
+    M, K = shape_a
+    t = lambda a, dt: torch.from_numpy(_c(a, dt))
+    out = m.spmspm_coo_float([M, n_cols], [M, K], [[t(a_row_idx, np.int32)], [t(a_col_idx, np.int32)]],
+                             t(a_vals, np.float32), [K, n_cols],
+                             [[t(b_row_idx, np.int32)], [t(b_col_idx, np.int32)]], t(b_vals, np.float32))
+    idx = out.storage.index.mode_indices
+    return idx[0][0].numpy().copy(), idx[1][0].numpy().copy(), out.storage.value.numpy().copy()
 
 
 def ref_sddmm_coo(row_idx, col_idx, svals, A, B, shape):

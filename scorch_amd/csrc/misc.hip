@@ -224,6 +224,33 @@ __global__ __launch_bounds__(kBlockThreads) void csr_row_indices_kernel(
   row_idx[p] = lo;
 }
 
+// ---- coordinate rows -> CSR row pointer -------------------------------------------
+// row_ptr[r] = number of entries whose row is below r, found by bisection in the
+// sorted row coordinates (every thread one r: the work is the same whatever the
+// gaps between rows).  The same threads look at the coordinates themselves, one
+// pair of neighbours each, and raise *unsorted if a row lies outside [0, M) or
+// below its predecessor; row_ptr is meaningless then.
+__global__ __launch_bounds__(kBlockThreads) void coo_row_ptr_kernel(
+    int M, int64_t nnz, const int *__restrict__ row_idx, int *__restrict__ row_ptr,
+    int *__restrict__ unsorted) {
+  const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+  const int64_t first = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  for (int64_t r = first; r <= M; r += stride) {
+    int64_t lo = 0, hi = nnz;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (row_idx[mid] < r) lo = mid + 1; else hi = mid;
+    }
+    row_ptr[r] = (int)lo;
+  }
+  bool bad = false;
+  for (int64_t p = first; p < nnz; p += stride) {
+    const int row = row_idx[p];
+    bad |= row < 0 || row >= M || (p > 0 && row_idx[p - 1] > row);
+  }
+  if (bad) *unsorted = 1;  // every writer stores the same value
+}
+
 }  // namespace scorch
 
 extern "C" {
@@ -277,6 +304,23 @@ int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr, i
   const dim3 grid((unsigned)((waves + scorch::kWavesPerBlock - 1) / scorch::kWavesPerBlock));
   scorch::csr_row_indices_kernel<<<grid, scorch::kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
       (int)M, nnz, row_ptr, row_idx);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_coo_row_ptr(int64_t M, int64_t nnz, const int32_t *row_idx, int32_t *row_ptr,
+                           int32_t *unsorted, void *stream) {
+  const char *fn = "scorch_hip_coo_row_ptr";
+  if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
+  if (M >= INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  SCORCH_REQUIRE(row_ptr != nullptr && unsorted != nullptr, "%s: NULL output", fn);
+  SCORCH_REQUIRE(nnz == 0 || row_idx != nullptr, "%s: row_idx is NULL", fn);
+  const int64_t items = M + 1 > nnz ? M + 1 : nnz;
+  int64_t blocks = (items + scorch::kBlockThreads - 1) / scorch::kBlockThreads;
+  if (blocks > 65536) blocks = 65536;  // the kernel strides
+  scorch::coo_row_ptr_kernel<<<dim3((unsigned)blocks), scorch::kBlockThreads, 0,
+                               static_cast<hipStream_t>(stream)>>>((int)M, nnz, row_idx, row_ptr, unsorted);
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }

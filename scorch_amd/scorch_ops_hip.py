@@ -323,6 +323,67 @@ def csr_row_indices(row_ptr: torch.Tensor, nnz: int) -> torch.Tensor:
     return rows
 
 
+def coo_row_ptr(row_idx: torch.Tensor, n_rows: int) -> Optional[torch.Tensor]:
+    """CSR row pointer (int32[n_rows + 1]) of coordinates sorted by row, or None
+    if they are not sorted or lie outside [0, n_rows).  One host read of a flag."""
+    rows = _index(row_idx, "row coordinates")
+    dev = _device_of(rows)
+    pos = torch.empty(n_rows + 1, dtype=torch.int32, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = native.lib().scorch_hip_coo_row_ptr(n_rows, rows.numel(), rows.data_ptr(), pos.data_ptr(),
+                                                 flag.data_ptr(), _stream(dev))
+    native.check(rc)
+    return None if int(flag.item()) else pos
+
+
+def _coo_as_csr(mode_indices, values, n_rows: int, what: str):
+    """(pos, crd, values) of a coordinate ("o,o") operand in row order.  Entries
+    already grouped by ascending row (what STensor produces) are used as they
+    are; anything else is first sorted by row, keeping the order inside a row."""
+    if len(mode_indices) != 2 or len(mode_indices[0]) != 1 or len(mode_indices[1]) != 1:
+        raise ValueError(f"scorch_ops_hip: {what} is not a coordinate (\"o,o\") operand")
+    rows, cols = _index(mode_indices[0][0], what + " rows"), _index(mode_indices[1][0], what + " columns")
+    if rows.numel() != cols.numel() or rows.numel() != values.numel():
+        raise ValueError(f"scorch_ops_hip: {what}: coordinate and value arrays differ in length")
+    pos = coo_row_ptr(rows, n_rows)
+    if pos is None:
+        if rows.numel() and (int(rows.min()) < 0 or int(rows.max()) >= n_rows):
+            raise ValueError(f"scorch_ops_hip: {what} has a row coordinate outside [0, {n_rows})")
+        rows, order = torch.sort(rows, stable=True)
+        cols, values = cols[order].contiguous(), values[order].contiguous()
+        pos = coo_row_ptr(rows, n_rows)
+    return pos, cols, values
+
+
+def spmm_coo_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+    """C = A @ B for A in coordinate form, fp32, dense result; repeated
+    coordinates add up (reference: csrc/spmm.h:247-372).  The coordinates are
+    turned into a row pointer on the device and the CSR kernel does the rest."""
+    a_val = _flat(A_values, torch.float32, "A values")
+    pos, crd, a_val = _coo_as_csr(A_mode_indices, a_val, int(A_shape[0]), "A")
+    return _spmm(torch.float32, result_shape, A_shape, [[], [pos, crd]], a_val, B_shape, B_mode_indices,
+                 B_values)
+
+
+def spmspm_coo_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+    """C = A @ B, all in coordinate form, fp32 (reference: csrc/kernels.h:397-497):
+    the result lists every structurally non-zero (row, column) once, rows
+    ascending and columns ascending inside a row, sums that cancel included.
+    Runs the CSR kernels between two index conversions on the device.  Where
+    the reference emits one group of entries per run of equal rows in A, rows
+    that are not grouped in A are merged here."""
+    a_val = _flat(A_values, torch.float32, "A values")
+    b_val = _flat(B_values, torch.float32, "B values")
+    a_pos, a_crd, a_val = _coo_as_csr(A_mode_indices, a_val, int(A_shape[0]), "A")
+    b_pos, b_crd, b_val = _coo_as_csr(B_mode_indices, b_val, int(B_shape[0]), "B")
+    out = prebuilt_spmspm_csr_f32(result_shape, A_shape, [[], [a_pos, a_crd]], a_val, B_shape,
+                                  [[], [b_pos, b_crd]], b_val)
+    c_pos, c_crd = out.storage.index.mode_indices[1]
+    rows = csr_row_indices(c_pos, int(c_crd.numel()))
+    return Tensor(out.storage.value, [[rows], [c_crd]])
+
+
 def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,
                           block_col_idx: torch.Tensor, scale: float, block: int = 64) -> torch.Tensor:
     """softmax(scale * q k^T over a block mask) v for q, k, v of shape (H, S, D),

@@ -6,7 +6,7 @@ Run once, in a container that holds the reference sources, after
 oracle/_ref/scorch_ops.so.  The outputs stored here come from that module
 (symbols spmm_csr_float_v2, prebuilt_spmm_csr_{f32,f64,i32,i64},
 spmm_csr_bias[_relu]_float, prebuilt_spmspm_csr_{f32,f64,i32,i64}, sddmm_coo_float_prebuilt,
-prebuilt_spmv_csr_{f32,f64,i32,i64}); the inputs come from this script's own
+prebuilt_spmv_csr_{f32,f64,i32,i64}, spmm_coo_float, spmspm_coo_float); the inputs come from this script's own
 seeded numpy generators.  The file holds data only.
 
 The cases re-express, with numpy's generator instead of torch's, the seeded and
@@ -192,6 +192,41 @@ def main() -> None:
     crp, cci, cv = O.ref_spgemm("spmspm_csr_float", arp, aci, av, brp, bci, bv, (2, 2), 3)
     put("spgemm_cancel", a_row_ptr=arp, a_col_idx=aci, a_vals=av, b_row_ptr=brp, b_col_idx=bci, b_vals=bv,
         n_cols=np.int64(3), c_row_ptr=crp, c_col_idx=cci, c_vals=cv)
+
+    # ---- coordinate-form operands: spmm_coo_float, spmspm_coo_float ------------
+    def coo_of(rp, ci):
+        return np.repeat(np.arange(rp.size - 1, dtype=np.int32), np.diff(rp)), ci
+
+    rng = np.random.default_rng(41)
+    rp, ci, v = random_csr(rng, 37, 29, 0.15, empty_rows=(0, 11))
+    r, c = coo_of(rp, ci)
+    B = dense(rng, (29, 21))
+    put("spmm_coo", row_idx=r, col_idx=c, vals=v, B=B, n_rows=np.int64(37), C=O.ref_spmm_coo(r, c, v, B, 37))
+    # the same entries with runs of rows out of order and some coordinates repeated
+    order = np.concatenate([np.flatnonzero(r >= 20), np.flatnonzero(r < 20), np.flatnonzero(r == 3)])
+    r2, c2, v2 = r[order], c[order], v[order]
+    put("spmm_coo_unsorted", row_idx=r2, col_idx=c2, vals=v2, B=B, n_rows=np.int64(37),
+        C=O.ref_spmm_coo(r2, c2, v2, B, 37))
+
+    rng = np.random.default_rng(42)
+    arp, aci, av = random_csr(rng, 33, 27, 0.12, empty_rows=(4,))
+    # (the reference sizes this kernel's per-column workspace by B's row count, so B must not be wider than tall)
+    brp, bci, bv = random_csr(rng, 27, 25, 0.15, empty_rows=(0, 9))
+    ar, ac = coo_of(arp, aci)
+    br, bc = coo_of(brp, bci)
+    shuffle = rng.permutation(br.size)  # the reference scans all of B for every entry of A: any order
+    br, bc, bv = br[shuffle], bc[shuffle], bv[shuffle]
+    cr, cc, cv = O.ref_spgemm_coo(ar, ac, av, br, bc, bv, (33, 27), 25)
+    put("spgemm_coo", a_row_idx=ar, a_col_idx=ac, a_vals=av, b_row_idx=br, b_col_idx=bc, b_vals=bv,
+        shape=np.array([33, 27, 25], np.int64), c_row_idx=cr, c_col_idx=cc, c_vals=cv)
+    # cancellation (the entry stays) and a coordinate of B stored twice (the two add up)
+    ar = np.array([0, 0, 1], np.int32); ac = np.array([0, 1, 1], np.int32)
+    av = np.array([1.0, -1.0, 2.0], np.float32)
+    br = np.array([0, 0, 1, 1, 1], np.int32); bc = np.array([0, 2, 0, 1, 1], np.int32)
+    bv = np.array([3.0, 5.0, 3.0, 7.0, 0.5], np.float32)
+    cr, cc, cv = O.ref_spgemm_coo(ar, ac, av, br, bc, bv, (2, 3), 3)
+    put("spgemm_coo_cancel", a_row_idx=ar, a_col_idx=ac, a_vals=av, b_row_idx=br, b_col_idx=bc, b_vals=bv,
+        shape=np.array([2, 3, 3], np.int64), c_row_idx=cr, c_col_idx=cc, c_vals=cv)
 
     np.savez_compressed(OUT, **data)
     print(f"wrote {OUT}: {len(data)} arrays, {os.path.getsize(OUT) / 1024:.1f} KiB")

@@ -186,3 +186,50 @@ def test_graph_squared_power_law(oracle):
     from scorch_amd import workloads
     w = workloads.gcn_powerlaw(M=20000, N=4, seed=21, max_degree=3000)
     check(oracle, w["row_ptr"], w["col_idx"], w["vals"], w["row_ptr"], w["col_idx"], w["vals"], 20000)
+
+
+# ---- all three in coordinate form (the reference's spmspm_coo_float) -----------------------
+def hip_spgemm_coo(ar, ac, av, br, bc, bv, shape):
+    M, K, N = (int(x) for x in shape)
+    out = H.spmspm_coo_float([M, N], [M, K], [[dev(ar)], [dev(ac)]], dev(av), [K, N], [[dev(br)], [dev(bc)]],
+                             dev(bv))
+    idx = out.storage.index.mode_indices
+    return host(idx[0][0]), host(idx[1][0]), host(out.storage.value)
+
+
+@pytest.mark.parametrize("name", ["spgemm_coo", "spgemm_coo_cancel"])
+def test_golden_coordinate_operands(golden, name):
+    c = golden.case(name)
+    r, k, v = hip_spgemm_coo(c["a_row_idx"], c["a_col_idx"], c["a_vals"], c["b_row_idx"], c["b_col_idx"],
+                             c["b_vals"], c["shape"])
+    assert r.dtype == np.int32 and k.dtype == np.int32
+    assert np.array_equal(r, c["c_row_idx"]) and np.array_equal(k, c["c_col_idx"])
+    np.testing.assert_allclose(v, c["c_vals"], rtol=1e-5, atol=1e-6)
+
+
+def test_coordinate_operands_give_the_csr_product(oracle):
+    rng = np.random.default_rng(73)
+    arp, aci, av = random_csr(rng, 900, 700, 0.01, empty_rows=(0,))
+    brp, bci, bv = random_csr(rng, 700, 1500, 0.01, empty_rows=(5,))
+    ar = np.repeat(np.arange(900, dtype=np.int32), np.diff(arp))
+    br = np.repeat(np.arange(700, dtype=np.int32), np.diff(brp))
+    shuffle = rng.permutation(br.size)  # B in any storage order
+    r, k, v = hip_spgemm_coo(ar, aci, av, br[shuffle], bci[shuffle], bv[shuffle], (900, 700, 1500))
+    wrp, wci, _ = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, 1500)
+    assert np.array_equal(r, np.repeat(np.arange(900, dtype=np.int32), np.diff(wrp)))
+    assert np.array_equal(k, wci)
+    _, _, ref64 = oracle.spgemm_csr_typed(arp, aci, av.astype(np.float64), brp, bci, bv.astype(np.float64), 1500)
+    assert oracle.rel_fro(v, ref64) <= 1e-5
+
+
+def test_coordinate_stensors_multiply_on_the_device():
+    torch.manual_seed(3)
+    a_t = torch.rand(40, 30) * (torch.rand(40, 30) < 0.1)
+    b_t = torch.rand(30, 20) * (torch.rand(30, 20) < 0.15)
+    a = STensor.from_torch(a_t, "A").to_sparse("oo").to("cuda")
+    b = STensor.from_torch(b_t, "B").to_sparse("oo").to("cuda")
+    out = scorch.matmul(a, b)
+    assert isinstance(out, STensor) and str(out.format) == "o,o" and out.shape == (40, 20)
+    assert torch.allclose(out.to_torch().cpu(), a_t @ b_t, atol=1e-5)
+    dense = scorch.matmul(a, STensor.from_torch(b_t, "B").to("cuda"))
+    assert isinstance(dense, torch.Tensor) and torch.allclose(dense.cpu(), a_t @ b_t, atol=1e-5)

@@ -335,3 +335,51 @@ def test_spmv_full_size_and_reproducible():
     A64 = torch.sparse_csr_tensor(rp.long(), ci.long(), v.double(), size=(M, M))
     ref = torch.mv(A64, x.double())
     assert (torch.linalg.norm(y.double() - ref) / torch.linalg.norm(ref)).item() <= TOL
+
+
+# ---- A in coordinate form (the reference's spmm_coo_float) ------------------------------
+def hip_spmm_coo(row_idx, col_idx, vals, B, n_rows):
+    out = H.spmm_coo_float([n_rows, B.shape[1]], [n_rows, B.shape[0]], [[dev(row_idx)], [dev(col_idx)]], dev(vals),
+                           list(B.shape), [[], []], dev(B).reshape(-1))
+    assert out.storage.index.mode_indices == [[], []]
+    return host(out.storage.value).reshape(n_rows, B.shape[1])
+
+
+@pytest.mark.parametrize("name", ["spmm_coo", "spmm_coo_unsorted"])
+def test_golden_coordinate_operand(golden, name):
+    c = golden.case(name)
+    got = hip_spmm_coo(c["row_idx"], c["col_idx"], c["vals"], c["B"], int(c["n_rows"]))
+    np.testing.assert_allclose(got, c["C"], rtol=1e-4, atol=1e-5)  # the reference's own output
+
+
+def test_coordinate_operand_in_any_order_with_repeats(oracle):
+    rng = np.random.default_rng(71)
+    rp, ci, v = random_csr(rng, 3000, 2000, 0.004, empty_rows=(0, 2999))
+    r = np.repeat(np.arange(3000, dtype=np.int32), np.diff(rp))
+    B = rng.standard_normal((2000, 96)).astype(np.float32)
+    ref64 = oracle.spmm_fp64(rp, ci, v, B)
+    assert oracle.rel_fro(hip_spmm_coo(r, ci, v, B, 3000), ref64) <= TOL
+    order = rng.permutation(r.size)  # shuffled, every entry twice
+    got = hip_spmm_coo(np.tile(r[order], 2), np.tile(ci[order], 2), np.tile(v[order], 2), B, 3000)
+    assert oracle.rel_fro(got, 2 * ref64) <= TOL
+
+
+def test_coordinate_operand_checks_row_range():
+    B = np.ones((4, 8), np.float32)
+    with pytest.raises(ValueError, match="outside"):
+        hip_spmm_coo(np.array([0, 5], np.int32), np.array([1, 1], np.int32), np.ones(2, np.float32), B, 4)
+
+
+def test_coordinate_row_pointer(oracle):
+    rng = np.random.default_rng(72)
+    rows = np.sort(rng.integers(0, 50_000, 400_000)).astype(np.int32)
+    pos = H.coo_row_ptr(dev(rows), 50_000)
+    assert np.array_equal(host(pos), np.searchsorted(rows, np.arange(50_001)).astype(np.int32))
+    # far more rows than entries, and no entries at all
+    few = np.array([7, 7, 999_999], np.int32)
+    assert np.array_equal(host(H.coo_row_ptr(dev(few), 1_000_000)),
+                          np.searchsorted(few, np.arange(1_000_001)).astype(np.int32))
+    assert not host(H.coo_row_ptr(dev(np.zeros(0, np.int32)), 9)).any()
+    assert H.coo_row_ptr(dev(np.array([3, 2], np.int32)), 9) is None      # descending
+    assert H.coo_row_ptr(dev(np.array([3, 9], np.int32)), 9) is None      # out of range
+    assert H.coo_row_ptr(dev(np.array([-1, 2], np.int32)), 9) is None

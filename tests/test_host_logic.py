@@ -132,9 +132,15 @@ def test_resolve_prebuilt_gates():
     spgemm = resolve_prebuilt_matmul(A, A)
     assert spgemm.symbol_name == "prebuilt_spmspm_csr_f32" and str(spgemm.output_format) == "d,s"
     assert resolve_prebuilt_matmul(A, A, output_format="ds").symbol_name == "prebuilt_spmspm_csr_f32"
-    # coordinate-format products are in the table but have no device symbol
+    # coordinate-format products, fp32 only (reference: prebuilt_kernels.py:64-79)
     coo = STensor.from_torch(a).to_sparse("oo")
-    assert resolve_prebuilt_matmul(coo, coo) is None and resolve_prebuilt_matmul(coo, B) is None
+    both = resolve_prebuilt_matmul(coo, coo)
+    assert both.symbol_name == "spmspm_coo_float" and str(both.output_format) == "o,o"
+    mixed = resolve_prebuilt_matmul(coo, B)
+    assert mixed.symbol_name == "spmm_coo_float" and str(mixed.output_format) == "d,d"
+    assert resolve_prebuilt_matmul(coo, coo, output_format="ds") is None
+    coo64 = STensor.from_torch(a.double()).to_sparse("oo")
+    assert resolve_prebuilt_matmul(coo64, coo64) is None
 
 
 def test_resolve_prebuilt_fused():

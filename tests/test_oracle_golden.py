@@ -140,3 +140,33 @@ def test_spgemm_keeps_entries_that_cancel_to_zero(golden):
     c = golden.case("spgemm_cancel")
     assert c["c_row_ptr"].tolist() == [0, 3, 5] and c["c_col_idx"].tolist() == [0, 1, 2, 0, 1]
     assert c["c_vals"][0] == 0.0                      # 1*3 + (-1)*3, stored all the same
+
+
+@pytest.mark.parametrize("name", ["spmm_coo", "spmm_coo_unsorted"])
+def test_spmm_coo_matches_reference_output(golden, oracle, name):
+    c = golden.case(name)
+    got = oracle.spmm_coo_f32(c["row_idx"], c["col_idx"], c["vals"], c["B"], int(c["n_rows"]))
+    np.testing.assert_allclose(got, c["C"], rtol=FP_RTOL, atol=FP_ATOL)
+
+
+def test_spmm_coo_fixture_does_not_depend_on_the_order_of_runs(golden):
+    # the unsorted case repeats row 3's entries: that row doubles, the others agree with the sorted case
+    a, b = golden.case("spmm_coo"), golden.case("spmm_coo_unsorted")
+    expect = a["C"].copy()
+    expect[3] *= 2
+    np.testing.assert_allclose(b["C"], expect, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["spgemm_coo", "spgemm_coo_cancel"])
+def test_spgemm_coo_matches_reference_output(golden, oracle, name):
+    c = golden.case(name)
+    r, k, v = oracle.spgemm_coo_f32(c["a_row_idx"], c["a_col_idx"], c["a_vals"], c["b_row_idx"],
+                                    c["b_col_idx"], c["b_vals"])
+    assert np.array_equal(r, c["c_row_idx"]) and np.array_equal(k, c["c_col_idx"])
+    np.testing.assert_allclose(v, c["c_vals"], rtol=FP_RTOL, atol=FP_ATOL)
+
+
+def test_spgemm_coo_keeps_cancelled_entries_and_adds_repeated_ones(golden):
+    c = golden.case("spgemm_coo_cancel")
+    assert list(c["c_row_idx"]) == [0, 0, 0, 1, 1] and list(c["c_col_idx"]) == [0, 1, 2, 0, 1]
+    assert list(c["c_vals"]) == [0.0, -7.5, 5.0, 6.0, 15.0]  # 3 - 3; -(7 + 0.5); 5; 2 * 3; 2 * 7.5

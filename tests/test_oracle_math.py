@@ -251,3 +251,49 @@ def test_spgemm_identity_and_empty_operands(oracle):
     rp, ci, v = oracle.spgemm_csr_typed(np.zeros(6, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32),
                                         brp, bci, bv, 33)
     assert rp.tolist() == [0] * 6 and ci.size == 0 and v.size == 0
+
+
+def _coo(rp, ci):
+    return np.repeat(np.arange(rp.size - 1, dtype=np.int32), np.diff(rp)), ci
+
+
+def test_spmm_coo_is_the_csr_product_and_adds_repeated_coordinates(oracle):
+    rng = np.random.default_rng(61)
+    rp, ci, v = random_csr(rng, 40, 30, 0.2, empty_rows=(0, 7))
+    B = rng.standard_normal((30, 13)).astype(np.float32)
+    r, c = _coo(rp, ci)
+    dense = np.zeros((40, 30))
+    np.add.at(dense, (r, c), v.astype(np.float64))
+    got = oracle.spmm_coo_f32(r, c, v, B, 40)
+    assert oracle.rel_fro(got, dense @ B.astype(np.float64)) < 1e-6
+    np.testing.assert_allclose(got, oracle.spmm_csr_typed(rp, ci, v, B), rtol=2e-6, atol=1e-6)
+    # any order of the entries, every entry twice: twice the product
+    order = rng.permutation(r.size)
+    twice = oracle.spmm_coo_f32(np.tile(r[order], 2), np.tile(c[order], 2), np.tile(v[order], 2), B, 40)
+    assert oracle.rel_fro(twice, 2 * (dense @ B.astype(np.float64))) < 1e-6
+
+
+def test_spgemm_coo_is_the_csr_product_in_coordinates(oracle):
+    rng = np.random.default_rng(62)
+    arp, aci, av = random_csr(rng, 35, 28, 0.15, empty_rows=(2,))
+    brp, bci, bv = random_csr(rng, 28, 50, 0.12, empty_rows=(0,))
+    ar, ac = _coo(arp, aci)
+    br, bc = _coo(brp, bci)
+    shuffle = rng.permutation(br.size)  # B in any order
+    r, k, v = oracle.spgemm_coo_f32(ar, ac, av, br[shuffle], bc[shuffle], bv[shuffle])
+    crp, cci, cv = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, 50)
+    assert np.array_equal(r, np.repeat(np.arange(35, dtype=np.int32), np.diff(crp)))
+    assert np.array_equal(k, cci)
+    np.testing.assert_allclose(v, cv, rtol=1e-5, atol=1e-6)
+    full = oracle.spgemm_fp64(arp, aci, av, brp, bci, bv, (35, 28), 50)
+    assert oracle.rel_fro(v, full[r, k]) < 1e-6
+    assert np.count_nonzero(full) <= r.size  # nothing structural is missing
+
+
+def test_spgemm_coo_emits_one_group_per_run_of_rows(oracle):
+    # row 1 appears in two separate runs of A: two groups of output entries, as in the reference's loop
+    ar = np.array([1, 0, 1], np.int32); ac = np.array([0, 0, 1], np.int32)
+    av = np.array([2.0, 3.0, 5.0], np.float32)
+    br = np.array([0, 1], np.int32); bc = np.array([1, 1], np.int32); bv = np.array([1.0, 10.0], np.float32)
+    r, k, v = oracle.spgemm_coo_f32(ar, ac, av, br, bc, bv)
+    assert list(r) == [1, 0, 1] and list(k) == [1, 1, 1] and list(v) == [2.0, 3.0, 50.0]

@@ -104,3 +104,36 @@ def test_spgemm(ref, suffix, dtype):
         assert np.array_equal(got[2], want[2])
     else:
         np.testing.assert_allclose(got[2], want[2], rtol=1e-6 if dtype == np.float32 else 1e-14)
+
+
+def _coo(rp, ci):
+    return np.repeat(np.arange(rp.size - 1, dtype=np.int32), np.diff(rp)), ci
+
+
+@pytest.mark.parametrize("seed,N", [(30, 17), (31, 64)])
+def test_spmm_coo(ref, seed, N):
+    rng = np.random.default_rng(seed)
+    rp, ci, v = random_csr(rng, 80, 60, 0.1, empty_rows=(0, 41))
+    r, c = _coo(rp, ci)
+    B = rng.standard_normal((60, N)).astype(np.float32)
+    np.testing.assert_allclose(ref.spmm_coo_f32(r, c, v, B, 80), ref.ref_spmm_coo(r, c, v, B, 80),
+                               rtol=2e-6, atol=1e-6)
+    runs = np.concatenate([np.flatnonzero(r >= 50), np.flatnonzero(r < 50), np.flatnonzero(r == 7)])
+    np.testing.assert_allclose(ref.spmm_coo_f32(r[runs], c[runs], v[runs], B, 80),
+                               ref.ref_spmm_coo(r[runs], c[runs], v[runs], B, 80), rtol=2e-6, atol=1e-5)
+
+
+@pytest.mark.parametrize("seed", [32, 33])
+def test_spgemm_coo(ref, seed):
+    # B no wider than tall: the reference sizes this kernel's per-column arrays by B's row count
+    rng = np.random.default_rng(seed)
+    arp, aci, av = random_csr(rng, 50, 40, 0.1, empty_rows=(3,))
+    brp, bci, bv = random_csr(rng, 40, 38, 0.12, empty_rows=(0, 20))
+    ar, ac = _coo(arp, aci)
+    br, bc = _coo(brp, bci)
+    shuffle = rng.permutation(br.size)
+    br, bc, bv = br[shuffle], bc[shuffle], bv[shuffle]
+    r, k, v = ref.spgemm_coo_f32(ar, ac, av, br, bc, bv)
+    wr, wk, wv = ref.ref_spgemm_coo(ar, ac, av, br, bc, bv, (50, 40), 38)
+    assert np.array_equal(r, wr) and np.array_equal(k, wk)
+    np.testing.assert_allclose(v, wv, rtol=2e-6, atol=1e-6)
