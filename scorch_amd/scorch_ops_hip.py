@@ -148,6 +148,22 @@ spmm_csr_double = _make_spmm(torch.float64)
 prebuilt_spmm_csr_i32 = _make_spmm(torch.int32)
 prebuilt_spmm_csr_i64 = _make_spmm(torch.int64)
 
+# The reference also binds its CPU tiling experiments of the same fp32 product under
+# names of their own (csrc/ops.cpp:121-160; called from its benchmark scripts and
+# tests/test_scorch/test_perf_large.py).  A tiling for caches and SIMD units of a host
+# has no meaning here: every name runs the one device kernel, tile arguments ignored.
+SPMM_CSR_FLOAT_VARIANTS = ("optimized", "turbo", "ultra", "apex", "untiled", "direct", "neon", "row_panel",
+                           "k_parallel", "sorted_rows", "neon2", "neon4", "tiled_neon")
+for _variant in SPMM_CSR_FLOAT_VARIANTS:
+    globals()["spmm_csr_float_" + _variant] = _make_spmm(torch.float32)
+del _variant
+
+
+def spmm_csr_float_tiled_i_k(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
+                             B_values, i_tile_size: int = 0, k_tile_size: int = 0):
+    return _spmm(torch.float32, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
+                 B_values)
+
 
 def spmm_csr_bias_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices,
                         B_values, bias):

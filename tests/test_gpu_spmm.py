@@ -383,3 +383,43 @@ def test_coordinate_row_pointer(oracle):
     assert H.coo_row_ptr(dev(np.array([3, 2], np.int32)), 9) is None      # descending
     assert H.coo_row_ptr(dev(np.array([3, 9], np.int32)), 9) is None      # out of range
     assert H.coo_row_ptr(dev(np.array([-1, 2], np.int32)), 9) is None
+
+
+def test_every_spmm_name_the_reference_binds_runs_the_device_kernel(golden):
+    """reference: csrc/ops.cpp:107-164 (the fp32 CSR x dense names, with their tile arguments)"""
+    c = golden.case("spmm_rect")
+    M, (K, N) = c["row_ptr"].size - 1, c["B"].shape
+    args = ([M, N], [M, K], [[], [dev(c["row_ptr"]), dev(c["col_idx"])]], dev(c["vals"]), [K, N], [[], []],
+            dev(c["B"]).reshape(-1))
+    expect = host(H.spmm_csr_float_v2(*args).storage.value)
+    names = ["spmm_csr_float", "prebuilt_spmm_csr_f32"] + ["spmm_csr_float_" + v for v in H.SPMM_CSR_FLOAT_VARIANTS]
+    assert len(names) == 15
+    for name in names:
+        assert np.array_equal(host(getattr(H, name)(*args).storage.value), expect), name
+    for name in ("spmm_csr_float_v2", "spmm_csr_float_turbo", "spmm_csr_float_apex"):
+        assert np.array_equal(host(getattr(H, name)(*args, tile_size=128).storage.value), expect)
+    tiled = H.spmm_csr_float_tiled_i_k(*args, i_tile_size=64, k_tile_size=32)
+    assert np.array_equal(host(tiled.storage.value), expect)
+
+
+def test_direct_calls_on_a_large_square_like_the_references_perf_test():
+    """reference: tests/test_scorch/test_perf_large.py:15-35,52-73 -- n = 1024, 95 % sparse, seed 7,
+    the native symbols called directly with STensor parts, checked against torch.sparse.mm."""
+    import scorch_amd as scorch
+    generator = torch.Generator().manual_seed(7)
+    n = 1024
+    a_dense = torch.rand((n, n), generator=generator, dtype=torch.float32)
+    b_dense = torch.rand((n, n), generator=generator, dtype=torch.float32)
+    a_dense = a_dense * (torch.rand((n, n), generator=generator) > 0.95)
+    reference = torch.sparse.mm(a_dense.to_sparse_csr(), b_dense)
+    a = scorch.STensor.from_torch(a_dense, "A").to_sparse("ds").to("cuda")
+    b = scorch.STensor.from_torch(b_dense, "B").to("cuda")
+    args = [[n, n]]
+    for tensor in (a, b):
+        args += [list(tensor.shape), tensor.index.mode_indices, tensor.values]
+    for name in ("spmm_csr_float_untiled", "spmm_csr_float", "spmm_csr_float_optimized", "spmm_csr_float_turbo",
+                 "spmm_csr_float_ultra", "spmm_csr_float_apex", "spmm_csr_float_tiled_i_k", "spmm_csr_float_v2"):
+        result = getattr(H, name)(*args).storage.value
+        assert torch.allclose(result.cpu().view_as(reference), reference, atol=1e-3, rtol=1e-3), name
+    out = scorch.matmul(a, b)
+    assert torch.allclose(out.cpu(), reference, atol=1e-3, rtol=1e-3)
