@@ -10,7 +10,7 @@ their neighbours) as hand-written HIP for AMD MI355X, behind Scorch's own
 from .format import LevelFormat, LevelType, TensorFormat, parse_format
 from .stensor import STensor
 from .storage import TensorIndex, TensorStorage
-from .ops import einsum, matmul, spmm_bias_act
+from .ops import einsum, matmul, matmul_wksp, precompile_kernels, spmm_bias_act, spmv
 from .trace import compile
 
 from_torch = STensor.from_torch
@@ -20,5 +20,5 @@ from_csr = STensor.from_csr
 __version__ = "0.1.0"
 
 __all__ = ["STensor", "TensorFormat", "TensorIndex", "TensorStorage", "LevelFormat", "LevelType",
-           "parse_format", "compile", "einsum", "matmul", "spmm_bias_act", "from_torch", "from_coo", "from_csr",
+           "parse_format", "compile", "einsum", "matmul", "matmul_wksp", "precompile_kernels", "spmm_bias_act", "spmv", "from_torch", "from_coo", "from_csr",
            "__version__"]

@@ -15,12 +15,12 @@ exactly as the reference does at ops.py:256-293.)
 """
 from __future__ import annotations
 
-from typing import Any, Optional, Union
+from typing import Any, List, Optional, Union
 
 import torch
 
 from . import scorch_ops_hip
-from .format import parse_format
+from .format import TensorFormat, parse_format
 from .prebuilt_kernels import (_timed, execute_prebuilt_binary_kernel, resolve_prebuilt_fused,
                                resolve_prebuilt_matmul)
 from .stensor import STensor
@@ -76,6 +76,58 @@ def _run_prebuilt_matmul(a: STensor, b: STensor, requested_format, time_dict):
     return _wrap(result_cpp, result_shape, resolved.output_format)
 
 
+def _as_format(result: STensor, requested) -> STensor:
+    """`result` re-stored in the requested format (on its device)."""
+    if requested is None:
+        return result
+    fmt = parse_format(requested)
+    if str(fmt) == str(result.format):
+        return result
+    if fmt.is_dense():
+        return STensor.from_torch(result.to_torch().contiguous())
+    return result.to_sparse(fmt)
+
+
+def _run_converted_matmul(a: STensor, b: STensor, requested, time_dict) -> Optional[STensor]:
+    """Matrix products of 2-D operands in any mix of "d,d", "d,s" and "o,o" (and a
+    sparse matrix times a dense vector) that no registry entry takes as they
+    are: the operands are re-stored, on the device, in the formats a prebuilt
+    kernel takes, and its result in the format asked for.  The reference sends
+    these combinations to its code generator (ops.py:358-367); the contraction
+    is the same, so the values agree to rounding.  ``eval_time`` covers the
+    kernel, as it does for a direct hit."""
+    kinds = ("d,d", "d,s", "o,o")
+    if a.dim() != 2 or str(a.format) not in kinds or a.values.dtype != b.values.dtype:
+        return None
+    if b.dim() == 1:
+        if not b.format.is_dense() or a.format.is_dense():
+            return None
+        natural = _run_prebuilt_matmul(a.to_sparse("ds"), b, None, time_dict)
+        return None if natural is None else _as_format(natural, requested)
+    if b.dim() != 2 or str(b.format) not in kinds:
+        return None
+    if a.format.is_dense():
+        if b.format.is_dense():
+            return None
+        # A B = (B^T A^T)^T with B^T in CSR, i.e. B stored by columns
+        _require_device(a, b)
+        bt = b.copy().to_sparse("ds").change_mode_order([1, 0])
+        pos, crd = bt.index.mode_indices[1]
+        bt = STensor.from_csr_arrays(pos, crd, bt.values, (b.shape[1], b.shape[0]))
+        at = STensor.from_torch(a.to_torch(in_place=False).t().contiguous())
+        natural = _run_prebuilt_matmul(bt, at, None, time_dict)
+        if natural is None:
+            return None
+        natural = STensor.from_torch(natural.to_torch().t().contiguous())
+    else:
+        left = a.to_sparse("ds")
+        right = b if b.format.is_dense() else b.to_sparse("ds")
+        natural = _run_prebuilt_matmul(left, right, None, time_dict)
+        if natural is None:
+            return None
+    return _as_format(natural, requested)
+
+
 def matmul(a: Union[torch.Tensor, STensor], b: Union[torch.Tensor, STensor],
            **kwargs: Any) -> Union[torch.Tensor, STensor]:
     """Matrix product.  Keyword arguments as in the reference: ``format`` /
@@ -112,6 +164,8 @@ def matmul(a: Union[torch.Tensor, STensor], b: Union[torch.Tensor, STensor],
 
     if kwargs.get("use_cache", True):
         result = _run_prebuilt_matmul(a, b, requested, time_dict)
+        if result is None:
+            result = _run_converted_matmul(a, b, requested, time_dict)
         if result is None:
             raise _not_prebuilt(f"matmul({a.format} x {b.format}, {a.values.dtype}, format={requested})")
     else:
@@ -178,6 +232,8 @@ def einsum(expression: str, *tensors: Optional[Union[torch.Tensor, STensor]],
             return torch.matmul(a.to_torch(in_place=False), b.to_torch(in_place=False))
         result = _run_prebuilt_matmul(a, b, requested, time_dict)
         if result is None:
+            result = _run_converted_matmul(a, b, requested, time_dict)
+        if result is None:
             raise _not_prebuilt(f"einsum({expression!r}) with formats {a.format} x {b.format}")
         return result.to_torch() if result.format.is_dense() else result
 
@@ -185,10 +241,56 @@ def einsum(expression: str, *tensors: Optional[Union[torch.Tensor, STensor]],
         a, b = operands
         result = _run_prebuilt_matmul(a, b, requested, time_dict)
         if result is None:
+            result = _run_converted_matmul(a, b, requested, time_dict)
+        if result is None:
             raise _not_prebuilt(f"einsum({expression!r}) with formats {a.format} x {b.format}")
         return result.to_torch() if result.format.is_dense() else result
 
     raise _not_prebuilt(f"einsum({expression!r})")
+
+
+def spmv(a: STensor, b: STensor, output_format: Optional[Union[TensorFormat, str, List[str]]] = None,
+         **kwargs: Any) -> STensor:
+    """Sparse matrix times dense vector; an STensor in format "d", as the
+    reference's function of this name returns (ops.py:48-136)."""
+    if output_format is not None and not parse_format(output_format).is_dense():
+        raise _not_prebuilt(f"spmv with output format {output_format}")
+    time_dict = kwargs.get("time_dict", None)
+    result = _run_prebuilt_matmul(a, b, None, time_dict)
+    if result is None:
+        result = _run_converted_matmul(a, b, None, time_dict)
+    if result is None:
+        raise _not_prebuilt(f"spmv({a.format} x {b.format}, {a.values.dtype})")
+    return result
+
+
+def matmul_wksp(a: Union[torch.Tensor, STensor], b: Union[torch.Tensor, STensor],
+                output_format: Optional[Union[TensorFormat, str, List[str]]] = None,
+                **kwargs: Any) -> STensor:
+    """Matrix product of two sparse operands; torch tensors are made sparse
+    first and the result is an STensor, "d,s" unless another format is asked for
+    (reference: ops.py:139-245, a generated kernel with a row workspace; here
+    the CSR x CSR kernel, which keeps a row's sums in LDS, does the work)."""
+    if isinstance(a, torch.Tensor):
+        a = STensor.from_torch(a).to_sparse()
+    if isinstance(b, torch.Tensor):
+        b = STensor.from_torch(b).to_sparse()
+    fmt = parse_format("ds" if output_format is None else output_format)
+    time_dict = kwargs.get("time_dict", None)
+    result = _run_prebuilt_matmul(a, b, fmt, time_dict)
+    if result is None:
+        result = _run_converted_matmul(a, b, fmt, time_dict)
+    if result is None:
+        raise _not_prebuilt(f"matmul_wksp({a.format} x {b.format}, {a.values.dtype}, format={fmt})")
+    return result
+
+
+def precompile_kernels() -> None:
+    """The reference generates and compiles its common matmul kernels ahead of
+    use (ops.py:933-945).  Here they are built with the package; this loads
+    the library so that a missing build shows up now and not at the first product."""
+    from . import native
+    native.lib()
 
 
 def spmm_bias_act(a: STensor, b: Union[torch.Tensor, STensor], bias: torch.Tensor,

@@ -345,3 +345,58 @@ def test_steps_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         for got, want in zip(captured, eager):
             assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("a_fmt,b_fmt", [("oo", "dd"), ("ds", "oo"), ("oo", "ds"), ("oo", "oo"), ("dd", "ds"),
+                                         ("dd", "oo"), ("ds", "ds")])
+@pytest.mark.parametrize("out_fmt", [None, "dd", "ds", "oo"])
+def test_matmul_in_every_mix_of_matrix_formats(a_fmt, b_fmt, out_fmt, dtype):
+    """What the reference's matmul accepts (ops.py:248-372: any format pair, an
+    optional result format), served by re-storing operands and result around the
+    prebuilt kernels."""
+    torch.manual_seed(11)
+    a_t = (torch.rand(37, 29) * (torch.rand(37, 29) < 0.15)).to(dtype)
+    b_t = (torch.rand(29, 23) * (torch.rand(29, 23) < 0.2)).to(dtype)
+    expect = a_t.double() @ b_t.double()
+
+    def stored(t, fmt, name):
+        s = STensor.from_torch(t, name)
+        return (s if fmt == "dd" else s.to_sparse(fmt)).to("cuda")
+
+    a, b = stored(a_t, a_fmt, "A"), stored(b_t, b_fmt, "B")
+    kwargs = {} if out_fmt is None else {"format": out_fmt}
+    out = scorch.matmul(a, b, **kwargs)
+    if isinstance(out, STensor):
+        assert out_fmt is None or str(out.format) == str(scorch.parse_format(out_fmt))
+        assert out.values.is_cuda and out.shape == (37, 23)
+        got = out.to_torch()
+    else:
+        assert out_fmt in (None, "dd") and out.is_cuda
+        got = out
+    assert torch.allclose(got.cpu().double(), expect, atol=1e-5)
+    same = scorch.einsum("ik,kj->ij", a, b, **kwargs)
+    same = same.to_torch() if isinstance(same, STensor) else same
+    assert torch.equal(same.cpu(), got.cpu())
+
+
+def test_spmv_matmul_wksp_and_precompile_follow_the_reference_signatures():
+    """reference: src/scorch/ops.py:48-136 (spmv), :139-245 (matmul_wksp), :933-945"""
+    torch.manual_seed(12)
+    a_t = torch.rand(40, 31) * (torch.rand(40, 31) < 0.2)
+    b_t = torch.rand(31, 18) * (torch.rand(31, 18) < 0.2)
+    x_t = torch.rand(31)
+    scorch.precompile_kernels()
+    a = STensor.from_torch(a_t, "A").to_sparse("ds").to("cuda")
+    y = scorch.spmv(a, STensor.from_torch(x_t, "x").to("cuda"))
+    assert isinstance(y, STensor) and str(y.format) == "d" and y.shape == (40,)
+    assert torch.allclose(y.to_torch().cpu(), a_t @ x_t, atol=1e-5)
+    y_coo = scorch.spmv(a.to_sparse("oo"), STensor.from_torch(x_t, "x").to("cuda"))
+    assert torch.allclose(y_coo.to_torch().cpu(), a_t @ x_t, atol=1e-5)
+    times = {}
+    c = scorch.matmul_wksp(a_t.cuda(), b_t.cuda(), time_dict=times)
+    assert isinstance(c, STensor) and str(c.format) == "d,s" and times["eval_time"] > 0
+    assert torch.allclose(c.to_torch().cpu(), a_t @ b_t, atol=1e-5)
+    d = scorch.matmul_wksp(a, STensor.from_torch(b_t, "B").to_sparse("ds").to("cuda"), output_format="dd")
+    assert isinstance(d, STensor) and d.format.is_dense()
+    assert torch.allclose(d.to_torch().cpu(), a_t @ b_t, atol=1e-5)

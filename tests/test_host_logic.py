@@ -201,14 +201,18 @@ def test_host_sparse_operands_are_refused_not_computed():
 def test_expressions_outside_the_path_raise_not_implemented():
     a, b = sparse_dense_pair()
     A = STensor.from_torch(a).to_sparse("ds")
-    with pytest.raises(NotImplementedError):
-        scorch.matmul(A, A, format="dd")         # CSR x CSR -> dense is the code generator's
     with pytest.raises(RuntimeError, match="HIP devices only"):
         scorch.matmul(A, A)                      # CSR x CSR -> CSR has a kernel, on the device
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.matmul(A, A, format="dd")         # the same kernel, its result re-stored
+    with pytest.raises(RuntimeError, match="HIP devices only"):
+        scorch.matmul(A, b, format="ds")
     with pytest.raises(NotImplementedError):
         scorch.einsum("ij,ij->ij", A, A)
     with pytest.raises(NotImplementedError):
-        scorch.matmul(A, b, format="ds")
+        scorch.matmul(A, STensor.from_torch(b.double()))   # operands of different types
+    with pytest.raises(NotImplementedError):
+        scorch.einsum("ijk,kl->ijl", STensor.from_torch(torch.rand(2, 3, 4)), A)
     with pytest.raises(NotImplementedError):
         scorch.einsum("ij,jk->ik", A, b, compile_only=True)
     with pytest.raises(NotImplementedError):
