@@ -72,6 +72,25 @@ def test_softmax_every_row_length_tier(oracle):
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-12)
 
 
+def test_softmax_full_size(oracle):
+    """The headline graph's pattern (1,048,576 rows, 17 M entries, rows up to 50,000 entries):
+    against the restatement, and every non-empty row sums to one."""
+    w = workloads.gcn_powerlaw(N=1)
+    rng = np.random.default_rng(5)
+    vals = (rng.standard_normal(w["col_idx"].size) * 6).astype(np.float32)
+    rp = dev(w["row_ptr"])
+    out = H.softmax_csr_float(rp, dev(vals), 0.5)
+    assert torch.equal(out, H.softmax_csr_float(rp, dev(vals), 0.5))  # same bits on every run
+    got = host(out)
+    want = oracle.softmax_csr_f32(w["row_ptr"], vals, 0.5)
+    assert oracle.rel_fro(got, want.astype(np.float64)) <= TOL
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-9)
+    rows = torch.repeat_interleave(torch.arange(w["M"], device="cuda"), (rp[1:] - rp[:-1]).long())
+    sums = torch.zeros(w["M"], dtype=torch.float64, device="cuda").index_add_(0, rows, out.double())
+    nonempty = (rp[1:] > rp[:-1])
+    assert torch.allclose(sums[nonempty], torch.ones_like(sums[nonempty]), rtol=1e-5)
+
+
 def test_softmax_with_empty_rows_and_large_values(oracle):
     rp = np.array([0, 0, 4, 4, 5], np.int32)
     vals = np.array([1000.0, 1001.0, 999.0, 1000.5, -3.0], np.float32)

@@ -181,6 +181,16 @@ def test_sparse_stensor_spgemm_does_not_call_torch_matmul(use_cache, monkeypatch
     assert torch.allclose(out.to_torch().cpu(), expected, atol=1e-5)
 
 
+@pytest.mark.parametrize("nodes", [131072, 524288])
+def test_graph_squared_at_the_benchmark_sizes(oracle, nodes):
+    """A @ A for the benchmark's graphs (bench.py --workload spgemm_powerlaw and four times as
+    many nodes): 30 M and 120 M result entries, structure bit for bit, values against fp64."""
+    from scorch_amd import workloads
+    w = workloads.gcn_powerlaw(M=nodes, N=4, max_degree=5000)
+    rp, _, _ = check(oracle, w["row_ptr"], w["col_idx"], w["vals"], w["row_ptr"], w["col_idx"], w["vals"], nodes)
+    assert rp[-1] > 200 * nodes
+
+
 def test_graph_squared_power_law(oracle):
     """A @ A for a power-law graph: rows from one entry to tens of thousands."""
     from scorch_amd import workloads
