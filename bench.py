@@ -255,6 +255,25 @@ def side_workload(args, dev) -> int:
                           "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
                           "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
         return 0
+    if args.workload == "softmax_rows":
+        # every row --row-length entries long, or a causal mask (row i has i + 1) with --row-length 0
+        import numpy as np
+        M = args.rows if args.rows != 1 << 20 else 8192
+        lens = np.full(M, args.row_length, np.int64) if args.row_length > 0 else np.arange(1, M + 1, dtype=np.int64)
+        pos = t(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+        nnz = int(lens.sum())
+        val = torch.randn(nnz, device="cuda")
+        ms = _time_steps(lambda: H.softmax_csr_float(pos, val, 1.0), args.steps, args.warmup)
+        algo = 8 * nnz + 4 * (M + 1)
+        print(json.dumps({"metric": "CSR row softmax GFLOP/s (4 flops per entry)",
+                          "value": round(4.0 * nnz / ms / 1e6, 2), "unit": "GFLOP/s", "ms_per_step": round(ms, 4),
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
+                          "data": "synthetic", "higher_is_better": True,
+                          "config": {"workload": "softmax_rows_fp32", "rows": M, "nnz": nnz,
+                                     "row_length": args.row_length if args.row_length > 0 else "causal"},
+                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                          "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}))
+        return 0
     if args.workload in ("spmv_powerlaw", "softmax_powerlaw"):
         w = workloads.gcn_powerlaw(M=args.rows, N=1)
         M, nnz = w["M"], int(w["col_idx"].size)
@@ -377,11 +396,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--rows", type=int, default=1 << 20, help="nodes of the graph (default: the headline size)")
     ap.add_argument("--features", type=int, default=128)
+    ap.add_argument("--row-length", type=int, default=0,
+                    help="softmax_rows: entries per row (0: a causal mask, row i has i + 1 entries)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="gcn_powerlaw",
                     choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
                              "attention_blocksparse", "spgemm_powerlaw", "spmv_powerlaw",
-                             "softmax_powerlaw"],
+                             "softmax_powerlaw", "softmax_rows"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")

@@ -230,9 +230,15 @@ SCORCH_HIP_API int scorch_hip_spgemm_csr_numeric_i64(int64_t M, int64_t K, int64
  * benchmark (_sparse_softmax_csr_vectorized,
  * bench/bench_sparse_transformer.py:277-297, applied to scores * scale at
  * :362-368); it has no native kernel for it.
+ * `workspace` (256-byte aligned, scorch_hip_softmax_csr_workspace_bytes; 0
+ * bytes, and then it may be NULL, for nnz <= 4096) holds the list of rows
+ * longer than 4096 entries between the two kernels; not to be shared by calls
+ * that may overlap in time.
  * ---------------------------------------------------------------------- */
+SCORCH_HIP_API size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz);
 SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr,
-                               const float *vals, float scale, float *out, void *stream);
+                               const float *vals, float scale, float *out, void *workspace,
+                               size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * Fused block-sparse attention, bf16 in / bf16 out, fp32 accumulation:

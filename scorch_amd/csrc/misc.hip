@@ -20,19 +20,26 @@ char *error_buffer() {
 //                                    (only when G < 16);
 //   up to kSoftmaxRegs * 64 entries  one wavefront per row, the workgroup's four
 //                                    wavefronts sharing those rows out;
-//   up to 2048 entries               the whole workgroup, one row after the other.
+//   up to 4096 entries               the whole workgroup, one row after the other.
 // In all of these a row sits in registers between the phases and is read from
-// memory once.  Rows beyond 2048 entries are left to softmax_csr_giant_kernel:
-// workgroups of 1024 threads that look through 1024 row lengths each and sweep
-// the giant rows among them, the first 8192 entries in registers and the rest
-// re-read from cache.
+// memory once.  Rows beyond 4096 entries are only noted, in a list in the
+// caller's workspace (one atomic per workgroup that has any), and
+// softmax_csr_giant_kernel then deals them out, one row at a time, to
+// workgroups of 1024 threads (the first 8192 entries in registers, the rest
+// re-read from cache; the next row's entries are requested before the current
+// row's phases start): however such rows are placed in the matrix, few among
+// many short ones or all of them long, they are spread over the whole chip.
+// Values are loaded raw and scaled at their first use, so that a row's loads
+// are all issued before any of them is waited for.
 constexpr int kSoftmaxRegs = 4;
-constexpr int kSoftmaxBlockRegs = 8;
+constexpr int kSoftmaxBlockRegs = 16;
+constexpr int kSoftmaxGiantRegs = 8;
 constexpr int kSoftmaxQuarter = kWaveSize / 4;
 constexpr int kSoftmaxQuarterRowMax = kSoftmaxRegs * kSoftmaxQuarter;
 constexpr int kSoftmaxWaveRowMax = kSoftmaxRegs * kWaveSize;
 constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
 constexpr int kSoftmaxGiantThreads = 1024;
+constexpr int kSoftmaxGiantBlocks = 1024;  // most workgroups the giant-row kernel starts
 constexpr float kSoftmaxLowest = -3.402823466e38f;
 
 // Lanes per row: the smallest power of two, between 2 and 64, whose groups hold
@@ -44,17 +51,27 @@ inline int softmax_group_width(int64_t M, int64_t nnz) {
   return g;
 }
 
-// The three phases for entries [lo, hi) by a team of TEAM threads (this one is
-// number t); `reduce(value, take_max)` combines a value over the team.
-template <int TEAM, int REGS, bool TAIL, typename Reduce>
-__device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *vals, float scale,
-                                            float *out, Reduce reduce) {
-  float v[REGS];
-  float mx = kSoftmaxLowest;
+// A row's entries [lo, hi) for a team of TEAM threads (this one is number t):
+// the first REGS * TEAM of them are read into registers, raw ...
+template <int TEAM, int REGS>
+__device__ __forceinline__ void softmax_load(int lo, int hi, int t, const float *vals, float (&v)[REGS]) {
 #pragma unroll
   for (int u = 0; u < REGS; ++u) {
     const int p = lo + t + u * TEAM;
-    v[u] = p < hi ? vals[p] * scale : kSoftmaxLowest;
+    v[u] = p < hi ? vals[p] : 0.0f;
+  }
+}
+
+// ... and the three phases on them; `reduce(value, take_max)` combines a value
+// over the team.  TAIL: the row may be longer than the registers hold; the
+// rest is read again in every phase.
+template <int TEAM, int REGS, bool TAIL, typename Reduce>
+__device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const float *vals, float scale,
+                                               float *out, float (&v)[REGS], Reduce reduce) {
+  float mx = kSoftmaxLowest;
+#pragma unroll
+  for (int u = 0; u < REGS; ++u) {
+    v[u] = lo + t + u * TEAM < hi ? v[u] * scale : kSoftmaxLowest;
     mx = fmaxf(mx, v[u]);
   }
   const int rest = lo + REGS * TEAM + t;  // this thread's first entry beyond the registers
@@ -85,6 +102,14 @@ __device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *
   }
 }
 
+template <int TEAM, int REGS, bool TAIL, typename Reduce>
+__device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *vals, float scale,
+                                            float *out, Reduce reduce) {
+  float v[REGS];
+  softmax_load<TEAM, REGS>(lo, hi, t, vals, v);
+  softmax_finish<TEAM, REGS, TAIL>(lo, hi, t, vals, scale, out, v, reduce);
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float softmax_shuffle_reduce(float v, bool take_max) {
 #pragma unroll
@@ -99,14 +124,17 @@ template <int G>
 __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                                     const int *__restrict__ row_ptr,
                                                                     const float *vals, float scale,
-                                                                    float *out) {
+                                                                    float *out, int *giant_count,
+                                                                    int *__restrict__ giant_rows) {
   constexpr int kRows = kBlockThreads / G;  // rows per workgroup
   __shared__ float s_red[kWavesPerBlock];
   __shared__ int s_lo[kRows], s_hi[kRows];
-  // row slots left to the quarter wavefronts [0], the wavefronts [1] and the workgroup [2]
-  __shared__ int s_list[3][kRows];
-  __shared__ int s_count[3];
-  if (threadIdx.x < 3) s_count[threadIdx.x] = 0;
+  // row slots left to the quarter wavefronts [0], the wavefronts [1] and the workgroup [2];
+  // [3]: rows left to the giant-row kernel
+  __shared__ int s_list[4][kRows];
+  __shared__ int s_count[4];
+  __shared__ int s_giant_base;
+  if (threadIdx.x < 4) s_count[threadIdx.x] = 0;
   __syncthreads();
   const int slot = threadIdx.x / G;
   const int t = threadIdx.x % G;
@@ -123,6 +151,8 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
       s_lo[slot] = lo;
       s_hi[slot] = hi;
       s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
+    } else if (t == 0) {
+      s_list[3][atomicAdd(&s_count[3], 1)] = (int)row;
     }
     hi = lo;
   }
@@ -130,7 +160,12 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   __syncthreads();
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int n_quarter = s_count[0], n_wave = s_count[1], n_block = s_count[2];
+  const int n_quarter = s_count[0], n_wave = s_count[1], n_block = s_count[2], n_giant = s_count[3];
+  if (n_giant > 0) {  // uniform over the workgroup; rows are independent, so the list's order is free
+    if (threadIdx.x == 0) s_giant_base = atomicAdd(giant_count, n_giant);
+    __syncthreads();
+    if ((int)threadIdx.x < n_giant) giant_rows[s_giant_base + threadIdx.x] = s_list[3][threadIdx.x];
+  }
   if (G < kSoftmaxQuarter) {
     constexpr int kTeams = kBlockThreads / kSoftmaxQuarter;
     for (int base = 0; base < n_quarter; base += kTeams) {  // uniform over the workgroup
@@ -168,40 +203,68 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   }
 }
 
+__global__ void softmax_reset_kernel(int *giant_count) {
+  if (threadIdx.x == 0) *giant_count = 0;
+}
+
 __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel(
-    int M, const int *__restrict__ row_ptr, const float *vals, float scale, float *out) {
+    const int *__restrict__ row_ptr, const float *vals, float scale, float *out,
+    const int *__restrict__ giant_count, const int *__restrict__ giant_rows) {
   constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
   __shared__ float s_red[kWaves];
-  __shared__ int s_lo[kSoftmaxGiantThreads], s_hi[kSoftmaxGiantThreads];
-  __shared__ int s_count;
-  if (threadIdx.x == 0) s_count = 0;
-  __syncthreads();
-  const int64_t row = (int64_t)blockIdx.x * kSoftmaxGiantThreads + threadIdx.x;
-  if (row < M) {
-    const int lo = row_ptr[row], hi = row_ptr[row + 1];
-    if (hi - lo > kSoftmaxBlockRowMax) {
-      const int k = atomicAdd(&s_count, 1);  // rows are independent: their order is free
-      s_lo[k] = lo;
-      s_hi[k] = hi;
-    }
-  }
-  __syncthreads();
-  const int n = s_count;
+  const int n = *giant_count;
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  for (int i = 0; i < n; ++i) {  // uniform over the workgroup
-    softmax_row<kSoftmaxGiantThreads, kSoftmaxBlockRegs, true>(
-        s_lo[i], s_hi[i], (int)threadIdx.x, vals, scale, out, [&](float v, bool take_max) {
-          v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
-          __syncthreads();
-          if (lane == 0) s_red[w] = v;
-          __syncthreads();
-          float r = s_red[0];
+  const int t = (int)threadIdx.x;
+  auto reduce = [&](float v, bool take_max) {
+    v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
+    __syncthreads();
+    if (lane == 0) s_red[w] = v;
+    __syncthreads();
+    float r = s_red[0];
 #pragma unroll
-          for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
-          return r;
-        });
+    for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
+    return r;
+  };
+  // The next row's first entries are requested before this row's phases begin,
+  // so that its memory latency passes behind their barriers.  (out may alias
+  // vals: rows do not overlap, so the early read sees the row unchanged.)
+  int i = blockIdx.x;
+  if (i >= n) return;
+  int row = giant_rows[i];
+  int lo = row_ptr[row], hi = row_ptr[row + 1];
+  float v[kSoftmaxGiantRegs];
+  softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo, hi, t, vals, v);
+  for (;;) {  // uniform over the workgroup
+    const int i_next = i + gridDim.x;
+    int lo_next = 0, hi_next = 0;
+    float v_next[kSoftmaxGiantRegs];
+    if (i_next < n) {
+      const int row_next = giant_rows[i_next];
+      lo_next = row_ptr[row_next];
+      hi_next = row_ptr[row_next + 1];
+    }
+    softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo_next, hi_next, t, vals, v_next);
+    softmax_finish<kSoftmaxGiantThreads, kSoftmaxGiantRegs, true>(lo, hi, t, vals, scale, out, v, reduce);
+    if (i_next >= n) break;
+    i = i_next;
+    lo = lo_next;
+    hi = hi_next;
+#pragma unroll
+    for (int u = 0; u < kSoftmaxGiantRegs; ++u) v[u] = v_next[u];
   }
+}
+
+// Rows the giant-row list must have room for: a row is listed only if it has
+// more than kSoftmaxBlockRowMax entries.
+inline int64_t softmax_giant_capacity(int64_t M, int64_t nnz) {
+  const int64_t by_entries = nnz / (kSoftmaxBlockRowMax + 1);
+  return by_entries < M ? by_entries : M;
+}
+
+inline size_t softmax_workspace_bytes(int64_t M, int64_t nnz) {
+  const int64_t rows = softmax_giant_capacity(M, nnz);
+  return rows > 0 ? 256 + ((size_t)rows * sizeof(int) + 255) / 256 * 256 : 0;
 }
 
 // ---- CSR -> coordinate rows ---------------------------------------------------
@@ -259,8 +322,14 @@ int scorch_hip_abi_version(void) { return SCORCH_HIP_ABI_VERSION; }
 
 const char *scorch_hip_last_error(void) { return scorch::error_buffer(); }
 
+size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz) {
+  if (M <= 0 || nnz <= 0) return 0;
+  return scorch::softmax_workspace_bytes(M, nnz);
+}
+
 int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, const float *vals,
-                               float scale, float *out, void *stream) {
+                               float scale, float *out, void *workspace, size_t workspace_bytes,
+                               void *stream) {
   const char *fn = "scorch_hip_softmax_csr_f32";
   if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
   if (M >= INT32_MAX || nnz > INT32_MAX)
@@ -268,23 +337,41 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
   SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
   if (M == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
+  const size_t need = scorch::softmax_workspace_bytes(M, nnz);
+  if (need > 0 && (!workspace || workspace_bytes < need))
+    return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
+                        workspace ? workspace_bytes : (size_t)0);
+  SCORCH_REQUIRE(need == 0 || scorch::aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // workspace: the number of giant rows, then (256 bytes on) their row numbers
+  int *giant_count = static_cast<int *>(workspace);
+  int *giant_rows = need > 0 ? giant_count + 64 : nullptr;
+  if (need > 0) {
+    scorch::softmax_reset_kernel<<<1, scorch::kWaveSize, 0, s>>>(giant_count);
+    SCORCH_HIP_CHECK(hipGetLastError());
+  }
   const int g = scorch::softmax_group_width(M, nnz);
   const int64_t rows_per_block = scorch::kBlockThreads / g;
   const dim3 grid((unsigned)((M + rows_per_block - 1) / rows_per_block));
   const int m = (int)M;
+#define SCORCH_SOFTMAX(G)                                                                               \
+  scorch::softmax_csr_kernel<G><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out, \
+                                                                       giant_count, giant_rows)
   switch (g) {
-    case 2: scorch::softmax_csr_kernel<2><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
-    case 4: scorch::softmax_csr_kernel<4><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
-    case 8: scorch::softmax_csr_kernel<8><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
-    case 16: scorch::softmax_csr_kernel<16><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
-    case 32: scorch::softmax_csr_kernel<32><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
-    default: scorch::softmax_csr_kernel<64><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out); break;
+    case 2: SCORCH_SOFTMAX(2); break;
+    case 4: SCORCH_SOFTMAX(4); break;
+    case 8: SCORCH_SOFTMAX(8); break;
+    case 16: SCORCH_SOFTMAX(16); break;
+    case 32: SCORCH_SOFTMAX(32); break;
+    default: SCORCH_SOFTMAX(64); break;
   }
+#undef SCORCH_SOFTMAX
   SCORCH_HIP_CHECK(hipGetLastError());
-  if (nnz > scorch::kSoftmaxBlockRowMax) {  // else no row can be that long
-    const dim3 giant_grid((unsigned)((M + scorch::kSoftmaxGiantThreads - 1) / scorch::kSoftmaxGiantThreads));
-    scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(m, row_ptr, vals, scale, out);
+  if (need > 0) {  // else no row can be that long
+    const int64_t most = scorch::softmax_giant_capacity(M, nnz);
+    const dim3 giant_grid((unsigned)(most < scorch::kSoftmaxGiantBlocks ? most : scorch::kSoftmaxGiantBlocks));
+    scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(
+        row_ptr, vals, scale, out, giant_count, giant_rows);
     SCORCH_HIP_CHECK(hipGetLastError());
   }
   return SCORCH_HIP_OK;

@@ -51,7 +51,9 @@ SIGNATURES = {
     "scorch_hip_spmv_csr_f64": (ctypes.c_int, _SPMV),
     "scorch_hip_spmv_csr_i32": (ctypes.c_int, _SPMV),
     "scorch_hip_spmv_csr_i64": (ctypes.c_int, _SPMV),
-    "scorch_hip_softmax_csr_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr, _ptr]),
+    "scorch_hip_softmax_csr_workspace_bytes": (_size, [_i64, _i64]),
+    "scorch_hip_softmax_csr_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr, _ptr, _size,
+                                                  _ptr]),
     "scorch_hip_attn_blocksparse_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_float, _ptr, _ptr]),
     "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),

@@ -319,10 +319,14 @@ def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float 
     v = _flat(values, torch.float32, "values")
     dev = _device_of(pos, v)
     out = torch.empty_like(v)
+    L = native.lib()
     with torch.cuda.device(dev):
-        rc = native.lib().scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(),
-                                                     v.data_ptr(), float(scale), out.data_ptr(),
-                                                     _stream(dev))
+        stream = _stream(dev)
+        need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, v.numel())
+        ws = _workspace(dev, stream, need) if need else None
+        rc = L.scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
+                                          float(scale), out.data_ptr(), ws.data_ptr() if need else None,
+                                          ws.numel() if need else 0, stream)
     native.check(rc)
     return out
 

@@ -112,8 +112,14 @@ def test_spmv_softmax_rows_reject_bad_arguments(L):
     assert L.scorch_hip_spmv_csr_i64(0, 4, 0, FAKE, NULL, NULL, NULL, NULL, NULL, 0, NULL) == native.OK
     assert L.scorch_hip_spmv_csr_f32(4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL, 0, NULL) == native.EWORKSPACE
     assert L.scorch_hip_spmv_csr_workspace_bytes(1000, 5000, 4) % 256 == 0
-    assert L.scorch_hip_softmax_csr_f32(4, 4, NULL, FAKE, 1.0, FAKE, NULL) == native.EINVAL
-    assert L.scorch_hip_softmax_csr_f32(4, 4, FAKE, NULL, 1.0, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_softmax_csr_f32(4, 4, NULL, FAKE, 1.0, FAKE, NULL, 0, NULL) == native.EINVAL
+    assert L.scorch_hip_softmax_csr_f32(4, 4, FAKE, NULL, 1.0, FAKE, NULL, 0, NULL) == native.EINVAL
+    # rows longer than 4096 entries are possible from nnz = 4097 on: a workspace is needed then
+    assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4096) == 0
+    assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4097) == 512
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 17_000_000) == 256 + 16640
+    assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, NULL, 0, NULL) == native.EWORKSPACE
+    assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, FAKE, 256, NULL) == native.EWORKSPACE
     assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL
     assert L.scorch_hip_csr_row_indices(0, 4, FAKE, FAKE, NULL) == native.EINVAL
 

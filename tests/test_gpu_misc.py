@@ -57,10 +57,10 @@ def test_softmax_against_oracle(oracle):
 
 def test_softmax_every_row_length_tier(oracle):
     """Row lengths chosen around each hand-over of the kernel: lane groups, quarter
-    wavefronts, wavefronts, the workgroup (up to 2048 entries) and the giant-row
+    wavefronts, wavefronts, the workgroup (up to 4096 entries) and the giant-row
     kernel (first 8192 entries in registers, the rest re-read)."""
-    lens = np.array([0, 1, 7, 8, 9, 16, 17, 63, 64, 65, 255, 256, 257, 0, 2047, 2048, 2049, 3,
-                     8191, 8192, 8193, 20000, 5, 0], np.int64)
+    lens = np.array([0, 1, 7, 8, 9, 16, 17, 63, 64, 65, 255, 256, 257, 0, 2047, 2048, 2049, 3, 4095, 4096,
+                     4097, 8191, 8192, 8193, 20000, 5, 0], np.int64)
     rng = np.random.default_rng(3)
     for mean_pad in (0, 400):  # few short rows -> narrow groups; many -> group width follows the mean
         all_lens = np.concatenate([lens, np.full(mean_pad, 2, np.int64)])
@@ -89,6 +89,35 @@ def test_softmax_full_size(oracle):
     sums = torch.zeros(w["M"], dtype=torch.float64, device="cuda").index_add_(0, rows, out.double())
     nonempty = (rp[1:] > rp[:-1])
     assert torch.allclose(sums[nonempty], torch.ones_like(sums[nonempty]), rtol=1e-5)
+
+
+@pytest.mark.parametrize("n_rows,length", [(300, 5000), (2100, 4097), (40, 9000)])
+def test_softmax_many_long_rows(oracle, n_rows, length):
+    """Every row beyond the workgroup tier: more listed rows than the giant-row kernel has
+    workgroups (it walks the list), fewer, and rows longer than its registers hold."""
+    rng = np.random.default_rng(n_rows)
+    rp = (np.arange(n_rows + 1, dtype=np.int64) * length).astype(np.int32)
+    vals = (rng.standard_normal(int(rp[-1])) * 3).astype(np.float32)
+    got = host(H.softmax_csr_float(dev(rp), dev(vals), 0.7))
+    want = oracle.softmax_csr_f32(rp, vals, 0.7)
+    assert oracle.rel_fro(got, want.astype(np.float64)) <= TOL
+    np.testing.assert_allclose(got.reshape(n_rows, length).sum(axis=1), 1.0, rtol=1e-5)
+
+
+def test_softmax_in_place(oracle):
+    """out may alias vals, also for rows that are re-read and for prefetched ones"""
+    lens = np.array([3, 9000, 5000, 12, 20000, 300, 4500, 0, 70], np.int64)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    vals = (np.random.default_rng(8).standard_normal(int(rp[-1])) * 3).astype(np.float32)
+    v = dev(vals)
+    pos = dev(rp)
+    L = H.native.lib()
+    need = L.scorch_hip_softmax_csr_workspace_bytes(len(lens), v.numel())
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    rc = L.scorch_hip_softmax_csr_f32(len(lens), v.numel(), pos.data_ptr(), v.data_ptr(), 0.5, v.data_ptr(),
+                                      ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert oracle.rel_fro(host(v), oracle.softmax_csr_fp64(rp, vals, 0.5)) <= TOL
 
 
 def test_softmax_with_empty_rows_and_large_values(oracle):
