@@ -21,7 +21,10 @@ namespace scorch {
 
 constexpr int kEntriesPerWave = 256;
 
-template <int GS, int VEC, bool COO>
+// LONG: K exceeds what the group's lanes cover with one load each (GS * VEC
+// elements); the vectors are then read four such pieces at a time, all eight
+// loads requested before the first product.
+template <int GS, int VEC, bool COO, bool LONG>
 __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
     int M, int K, int64_t nnz, const int *__restrict__ rows /* row_idx (COO) or row_ptr (CSR) */,
     const int *__restrict__ col_idx, const float *__restrict__ mask_vals,
@@ -74,11 +77,33 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
       const float *a = A + (size_t)r * (size_t)K;
       const float *b = B + (size_t)c * (size_t)K;
       float dot = 0.0f;
-      for (int k = t * VEC; k < K; k += GS * VEC) {
-        const VecT av = *reinterpret_cast<const VecT *>(a + k);
-        const VecT bv = *reinterpret_cast<const VecT *>(b + k);
+      if (!LONG) {
+        for (int k = t * VEC; k < K; k += GS * VEC) {
+          const VecT av = *reinterpret_cast<const VecT *>(a + k);
+          const VecT bv = *reinterpret_cast<const VecT *>(b + k);
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
+          for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
+        }
+      } else {
+        constexpr int kPieces = 4;
+        for (int k0 = t * VEC; k0 < K; k0 += kPieces * GS * VEC) {
+          VecT av[kPieces], bv[kPieces];
+#pragma unroll
+          for (int u = 0; u < kPieces; ++u) {
+            const int k = k0 + u * GS * VEC;
+            if (k < K) {
+              av[u] = *reinterpret_cast<const VecT *>(a + k);
+              bv[u] = *reinterpret_cast<const VecT *>(b + k);
+            } else {
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) av[u].v[v] = bv[u].v[v] = 0.0f;
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < kPieces; ++u)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) dot += av[u].v[v] * bv[u].v[v];
+        }
       }
 #pragma unroll
       for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
@@ -102,17 +127,18 @@ int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
   const int per_lane = vec4 ? 4 : 1;
   const int64_t lanes_needed = (K + per_lane - 1) / per_lane;
 
-#define SCORCH_SDDMM_LAUNCH(GS, VEC)                                                             \
-  sddmm_kernel<GS, VEC, COO><<<grid, kBlockThreads, 0, stream>>>(M, K, nnz, rows, col_idx,       \
-                                                                mask_vals, A, B, out_vals,      \
-                                                                out_row_idx)
-#define SCORCH_SDDMM_PICK(VEC)                                       \
-  do {                                                               \
-    if (lanes_needed <= 4) SCORCH_SDDMM_LAUNCH(4, VEC);              \
-    else if (lanes_needed <= 8) SCORCH_SDDMM_LAUNCH(8, VEC);         \
-    else if (lanes_needed <= 16) SCORCH_SDDMM_LAUNCH(16, VEC);       \
-    else if (lanes_needed <= 32) SCORCH_SDDMM_LAUNCH(32, VEC);       \
-    else SCORCH_SDDMM_LAUNCH(64, VEC);                               \
+#define SCORCH_SDDMM_LAUNCH(GS, VEC, LONG)                                                         \
+  sddmm_kernel<GS, VEC, COO, LONG><<<grid, kBlockThreads, 0, stream>>>(M, K, nnz, rows, col_idx,   \
+                                                                      mask_vals, A, B, out_vals,  \
+                                                                      out_row_idx)
+#define SCORCH_SDDMM_PICK(VEC)                                              \
+  do {                                                                      \
+    if (lanes_needed <= 4) SCORCH_SDDMM_LAUNCH(4, VEC, false);              \
+    else if (lanes_needed <= 8) SCORCH_SDDMM_LAUNCH(8, VEC, false);         \
+    else if (lanes_needed <= 16) SCORCH_SDDMM_LAUNCH(16, VEC, false);       \
+    else if (lanes_needed <= 32) SCORCH_SDDMM_LAUNCH(32, VEC, false);       \
+    else if (lanes_needed <= 64) SCORCH_SDDMM_LAUNCH(64, VEC, false);       \
+    else SCORCH_SDDMM_LAUNCH(64, VEC, true);                                \
   } while (0)
 
   if (vec4) SCORCH_SDDMM_PICK(4); else SCORCH_SDDMM_PICK(1);

@@ -43,7 +43,7 @@ def test_golden_csr(golden, oracle, name):
 
 
 # K chosen to hit every group width (4..64 lanes per entry), the scalar path (K % 4 != 0) and K > 256
-@pytest.mark.parametrize("K", [1, 2, 5, 8, 13, 16, 32, 64, 96, 128, 200, 256, 260, 512])
+@pytest.mark.parametrize("K", [1, 2, 5, 8, 13, 16, 32, 64, 65, 96, 128, 200, 256, 257, 260, 512, 1024, 1100, 1101])
 def test_inner_dimensions(oracle, K):
     rng = np.random.default_rng(K)
     rp, ci, s = random_csr(rng, 211, 157, 0.07, empty_rows=(0, 7, 210))
