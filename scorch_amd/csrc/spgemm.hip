@@ -8,7 +8,10 @@
 // is processed depends on an upper bound of its size, the number of products
 // it sums (sum over its entries of the length of the B row they select):
 //
+//   up to 32 products    a quarter wavefront, hash table of 64 slots in LDS
 //   up to 256 products   one wavefront, hash table of 512 slots in LDS
+//                        (a wavefront takes four consecutive rows: the first kind
+//                        all at once, then the second kind one after the other)
 //   up to 1024 products  one workgroup, hash table of 2048 slots in LDS
 //   up to 4096 products  B of at most 131,072 columns: a bitmap of the columns in LDS
 //                        (256 threads, see below); wider B: one workgroup, hash
@@ -37,7 +40,7 @@
 
 namespace scorch {
 
-constexpr int kTinyProducts = 256;
+constexpr int kTinyProducts = 256;     // wavefront tier (512 slots)
 constexpr int kTinySlots = 512;
 constexpr int kSmallProducts = 1024;   // workgroup tier 1 (2048 slots)
 constexpr int kMediumProducts = 4096;  // workgroup tier 2 (8192 slots)
@@ -150,7 +153,8 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &to
 // The products of a row are the entries of the B rows its A entries select.  B
 // rows are often much shorter than a wavefront, so handing one B row to a team
 // at a time wastes most lanes and chains three dependent loads per A entry.
-// Instead the team (TEAM = 64: one wavefront, TEAM = 256: the workgroup) takes
+// Instead the team (TEAM = 16: a quarter wavefront, 64: one wavefront, 256 or
+// 1024: the workgroup) takes
 // TEAM entries of A at once -- thread t reads entry t, its B row's start and
 // length -- turns the lengths into offsets with a prefix sum, and then walks the
 // batch's products flat: product x belongs to the entry e with off[e] <= x <
@@ -163,22 +167,25 @@ struct ProductBatch {
   A a_val[TEAM];
 };
 
+// Teams of up to a wavefront (64 lanes, or an aligned part of one) need no
+// barrier: a wavefront's LDS operations complete in program order.
 template <int TEAM>
 __device__ __forceinline__ void team_sync() {
-  if (TEAM == kWaveSize) wave_lds_sync(); else __syncthreads();
+  if (TEAM <= kWaveSize) wave_lds_sync(); else __syncthreads();
 }
 
 template <int TEAM>
 __device__ __forceinline__ int team_exclusive_scan(int v, int *scratch, int &total) {
-  if (TEAM != kWaveSize) return block_exclusive_scan_n<TEAM / kWaveSize>(v, scratch, total);
+  if (TEAM > kWaveSize) return block_exclusive_scan_n<TEAM / kWaveSize>(v, scratch, total);
   const int lane = wave_lane();
+  const int t = lane % TEAM;
   int incl = v;
 #pragma unroll
-  for (int off = 1; off < kWaveSize; off <<= 1) {
+  for (int off = 1; off < TEAM; off <<= 1) {
     const int up = __shfl_up(incl, off);
-    if (lane >= off) incl += up;
+    if (t >= off) incl += up;
   }
-  total = __shfl(incl, kWaveSize - 1);
+  total = __shfl(incl, lane - t + TEAM - 1);
   return incl - v;
 }
 
@@ -359,66 +366,132 @@ __global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
   if (threadIdx.x == 0 && c_pos_last) *c_pos_last = 0;
 }
 
-// ---- rows of at most kTinyProducts products: one wavefront each ---------------------
-template <typename T, bool NUMERIC>
-__global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
-    int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+// ---- rows of at most kMicroProducts products: a quarter wavefront each -----------------
+// Most rows of a very sparse product have a few dozen products: a wavefront each
+// would mean a wavefront's start-up and its chain of dependent loads (A's row,
+// B's row pointers, B's entries) for every such row.  Sixteen lanes do the same
+// steps on tables a quarter the size, four rows to a wavefront.  The teams of a
+// wavefront take different numbers of steps; all synchronisation is the
+// wavefront's own program order, and shuffles and ballots only look at a
+// team's own lanes.
+constexpr int kMicroTeam = 16;
+constexpr int kMicroProducts = 32;
+constexpr int kMicroSlots = 64;
+
+// What TEAMS teams keep in LDS for their rows: the hash table, the compacted
+// entries and the batch of A entries being walked.
+template <typename A, bool NUMERIC, int TEAM, int TEAMS, int SLOTS, int PRODUCTS>
+struct TeamTables {
+  int keys[TEAMS][SLOTS];
+  A vals[TEAMS][NUMERIC ? SLOTS : 1];
+  int ck[TEAMS][NUMERIC ? PRODUCTS : 1];
+  A cv[TEAMS][NUMERIC ? PRODUCTS : 1];
+  ProductBatch<TEAM, A> batch[TEAMS];
+};
+
+// One row of C by team number `team` of TEAM lanes (a wavefront or an aligned
+// part of one; this lane is its number t): hash the row's products, count or
+// compact the occupied slots, sort by rank.
+template <typename T, bool NUMERIC, int TEAM, int TEAMS, int SLOTS, int PRODUCTS>
+__device__ __forceinline__ void spgemm_team_row(
+    TeamTables<typename Acc<T>::type, NUMERIC, TEAM, TEAMS, SLOTS, PRODUCTS> &lds, int team, int t, int row,
+    const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
-    const int *__restrict__ products, int *__restrict__ c_pos, int *__restrict__ c_crd,
-    T *__restrict__ c_val) {
+    int *__restrict__ c_pos, int *__restrict__ c_crd, T *__restrict__ c_val) {
   using A = typename Acc<T>::type;
-  __shared__ int s_keys[kWavesPerBlock][kTinySlots];
-  __shared__ A s_vals[kWavesPerBlock][NUMERIC ? kTinySlots : 1];
-  __shared__ int s_ck[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
-  __shared__ A s_cv[kWavesPerBlock][NUMERIC ? kTinyProducts : 1];
-  __shared__ ProductBatch<kWaveSize, A> s_batch[kWavesPerBlock];
-
   const int lane = wave_lane();
-  const int w = threadIdx.x / kWaveSize;
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + w;
-  if (row >= M) return;
-  if (products[row] > kTinyProducts) return;  // a workgroup kernel owns this row
 
-  for (int s = lane; s < kTinySlots; s += kWaveSize) {
-    s_keys[w][s] = -1;
-    if (NUMERIC) s_vals[w][s] = (A)0;
+  for (int s = t; s < SLOTS; s += TEAM) {
+    lds.keys[team][s] = -1;
+    if (NUMERIC) lds.vals[team][s] = (A)0;
   }
   wave_lds_sync();
 
-  for_each_product<kWaveSize, NUMERIC, T, A>(
-      a_pos[row], a_pos[row + 1], lane, a_crd, a_val, b_pos, b_crd, b_val, s_batch[w], nullptr,
+  for_each_product<TEAM, NUMERIC, T, A>(
+      a_pos[row], a_pos[row + 1], t, a_crd, a_val, b_pos, b_crd, b_val, lds.batch[team], nullptr,
       [&](int col, A product) {
-        const int slot = hash_insert(s_keys[w], kTinySlots - 1, col);
-        if (NUMERIC) atomic_accumulate<A>(&s_vals[w][slot], product);
+        const int slot = hash_insert(lds.keys[team], SLOTS - 1, col);
+        if (NUMERIC) atomic_accumulate<A>(&lds.vals[team][slot], product);
       });
   wave_lds_sync();
 
   // Count the occupied slots; in the numeric pass, also compact them.
   int n = 0;
-  for (int base = 0; base < kTinySlots; base += kWaveSize) {
-    const int key = s_keys[w][base + lane];
-    const unsigned long long occupied = __ballot(key != -1);
+  for (int base = 0; base < SLOTS; base += TEAM) {
+    const int key = lds.keys[team][base + t];
+    unsigned long long occupied = __ballot(key != -1) >> (lane - t);  // the team's lanes from bit 0
+    if (TEAM < kWaveSize) occupied &= (1ull << (TEAM % kWaveSize)) - 1ull;
     if (NUMERIC && key != -1) {
-      const int at = n + __popcll(occupied & ((1ull << lane) - 1ull));
-      s_ck[w][at] = key;
-      s_cv[w][at] = s_vals[w][base + lane];
+      const int at = n + __popcll(occupied & ((1ull << t) - 1ull));
+      lds.ck[team][at] = key;
+      lds.cv[team][at] = lds.vals[team][base + t];
     }
     n += __popcll(occupied);
   }
   if (!NUMERIC) {
-    if (lane == 0) c_pos[row] = n;
+    if (t == 0) c_pos[row] = n;
     return;
   }
   wave_lds_sync();
 
   // Rank = number of smaller keys (keys are distinct): the sorted position.
   const int out = c_pos[row];
-  for (int e = lane; e < n; e += kWaveSize) {
-    const int key = s_ck[w][e];
+  for (int e = t; e < n; e += TEAM) {
+    const int key = lds.ck[team][e];
     int rank = 0;
-    for (int x = 0; x < n; ++x) rank += s_ck[w][x] < key ? 1 : 0;
+    for (int x = 0; x < n; ++x) rank += lds.ck[team][x] < key ? 1 : 0;
     c_crd[out + rank] = key;
-    c_val[out + rank] = (T)s_cv[w][e];
+    c_val[out + rank] = (T)lds.cv[team][e];
+  }
+}
+
+// A wavefront takes four consecutive rows: those of at most kMicroProducts
+// products by its four quarters at once, then those of up to kTinyProducts one
+// after the other with all its lanes (rows beyond that belong to the workgroup
+// kernels).  The two kinds of table share the wavefront's LDS.
+// QUARTERS = false: one row per wavefront, all lanes on it whatever its size; for
+// matrices of too few rows to fill the chip four to a wavefront.
+template <typename T, bool NUMERIC, bool QUARTERS>
+__global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
+    int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
+    const int *__restrict__ products, int *__restrict__ c_pos, int *__restrict__ c_crd,
+    T *__restrict__ c_val) {
+  using A = typename Acc<T>::type;
+  constexpr int kQuarters = kWaveSize / kMicroTeam;
+  if (!QUARTERS) {
+    __shared__ TeamTables<A, NUMERIC, kWaveSize, kWavesPerBlock, kTinySlots, kTinyProducts> one;
+    const int w = threadIdx.x / kWaveSize;
+    const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + w;
+    if (row >= M || products[row] > kTinyProducts) return;
+    spgemm_team_row<T, NUMERIC, kWaveSize, kWavesPerBlock, kTinySlots, kTinyProducts>(
+        one, w, wave_lane(), (int)row, a_pos, a_crd, a_val, b_pos, b_crd, b_val, c_pos, c_crd, c_val);
+    return;
+  }
+  union Tables {
+    TeamTables<A, NUMERIC, kWaveSize, 1, kTinySlots, kTinyProducts> wave;
+    TeamTables<A, NUMERIC, kMicroTeam, kQuarters, kMicroSlots, kMicroProducts> quarter;
+  };
+  __shared__ Tables lds[kWavesPerBlock];
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + w) * kQuarters;
+  if (first >= M) return;
+  const int q = lane / kMicroTeam;
+  const int64_t mine = first + q;
+  const int bound = mine < M ? products[mine] : INT_MAX;
+  if (bound <= kMicroProducts)
+    spgemm_team_row<T, NUMERIC, kMicroTeam, kQuarters, kMicroSlots, kMicroProducts>(
+        lds[w].quarter, q, lane % kMicroTeam, (int)mine, a_pos, a_crd, a_val, b_pos, b_crd, b_val, c_pos, c_crd,
+        c_val);
+#pragma unroll
+  for (int i = 0; i < kQuarters; ++i) {
+    const int b = __shfl(bound, i * kMicroTeam);  // uniform
+    if (b > kMicroProducts && b <= kTinyProducts) {
+      wave_lds_sync();  // the tables' previous users are done
+      spgemm_team_row<T, NUMERIC, kWaveSize, 1, kTinySlots, kTinyProducts>(
+          lds[w].wave, 0, lane, (int)(first + i), a_pos, a_crd, a_val, b_pos, b_crd, b_val, c_pos, c_crd, c_val);
+    }
   }
 }
 
@@ -858,9 +931,17 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
                                                                 ws.small_rows, ws.medium_rows,
                                                                 ws.huge_rows, ws.counters);
   SCORCH_HIP_CHECK(hipGetLastError());
-  const unsigned tiny_blocks = (unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock);
-  spgemm_tiny_kernel<T, NUMERIC><<<tiny_blocks, kBlockThreads, 0, stream>>>(
-      M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
+  // four rows to a wavefront once that still leaves every wavefront slot of the chip a wavefront
+  if ((int64_t)M >= 4 * 8192) {
+    const int64_t rows_per_block = kWavesPerBlock * (kWaveSize / kMicroTeam);
+    const unsigned tiny_blocks = (unsigned)(((int64_t)M + rows_per_block - 1) / rows_per_block);
+    spgemm_tiny_kernel<T, NUMERIC, true><<<tiny_blocks, kBlockThreads, 0, stream>>>(
+        M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
+  } else {
+    const unsigned tiny_blocks = (unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock);
+    spgemm_tiny_kernel<T, NUMERIC, false><<<tiny_blocks, kBlockThreads, 0, stream>>>(
+        M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
+  }
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned medium_blocks = (unsigned)(M < kMediumWorkgroups ? M : kMediumWorkgroups);
   spgemm_medium_kernel<T, NUMERIC, kSmallProducts, 2><<<medium_blocks, kBlockThreads, 0, stream>>>(

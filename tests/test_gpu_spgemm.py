@@ -191,6 +191,28 @@ def test_graph_squared_at_the_benchmark_sizes(oracle, nodes):
     assert rp[-1] > 200 * nodes
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_many_rows_of_few_products(oracle, dtype):
+    """Enough rows (>= 32,768) for wavefronts to take four rows each: rows of 0 to 32 products go
+    to quarter wavefronts, their neighbours of up to 256 to the whole wavefront in turn, a few
+    beyond that to the workgroup kernels.  Tridiagonal-like with denser stretches."""
+    M = 40_003
+    rng = np.random.default_rng(31)
+    lens = rng.integers(0, 4, M)
+    lens[rng.integers(0, M, 3000)] = rng.integers(4, 17, 3000)   # up to 16 x 16 = 256 products
+    lens[rng.integers(0, M, 40)] = rng.integers(300, 900, 40)    # beyond the wavefront tier
+    lens[[0, M - 1]] = [0, 3]
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([np.sort(rng.choice(M, int(n), replace=False)) for n in lens]).astype(np.int32)
+    vals = (rng.integers(-9, 9, cols.size) if np.issubdtype(dtype, np.integer)
+            else rng.uniform(-1, 1, cols.size)).astype(dtype)
+    products = np.zeros(M, np.int64)
+    np.add.at(products, np.repeat(np.arange(M), lens), lens[cols])
+    assert (products <= 32).sum() > 30_000 and ((products > 32) & (products <= 256)).sum() > 300
+    assert (products > 256).sum() >= 30 and (products == 0).any()
+    check(oracle, rp, cols, vals, rp, cols, vals, M)
+
+
 def test_graph_squared_power_law(oracle):
     """A @ A for a power-law graph: rows from one entry to tens of thousands."""
     from scorch_amd import workloads
