@@ -14,6 +14,22 @@ Three layers, from most to least trusted as ground truth:
 * the C restatement in ``scorch_oracle.c`` (``liboracle.so``), wrapped by the
   plain functions below.  It follows the reference loop by loop and is what
   gets timed as the CPU baseline when ``_ref`` is absent.
+
+What pins each restatement (tests/test_oracle_golden.py, test_oracle_math.py,
+test_oracle_ref.py):
+
+* spmm_csr_f32_v2, spmm_csr_typed, spmm_csr_bias_act_f32, sddmm_coo_f32,
+  sddmm_csr_f32, spmv_csr_typed, spgemm_csr_typed, spmm_coo_f32,
+  spgemm_coo_f32: the reference's own outputs (golden fixtures written by its
+  compiled native module, and that module live where it is built), plus closed
+  forms and brute force.
+* softmax_csr_f32 / softmax_csr_fp64 and attention_dense_fp64 /
+  attention_blocksparse_fp64: PARITY UNPINNED against the reference -- it has
+  no native kernel, test or stored vector for the row softmax or for fused
+  attention (it composes them from torch operations in a benchmark script).
+  They are pinned by mathematics only: scipy.special.softmax, shift
+  invariance, rows summing to one, and the SDDMM -> softmax -> SpMM pipeline
+  equalling masked dense attention.
 """
 from __future__ import annotations
 

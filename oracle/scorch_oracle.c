@@ -12,6 +12,12 @@
  * workspace) follows the reference so that timing it is a fair stand-in for
  * timing the reference itself.
  *
+ * Pinned against the reference's own outputs (golden fixtures and, where it
+ * is built, its compiled module): every routine here except
+ * oracle_softmax_csr_f32, which is PARITY UNPINNED -- the reference has no
+ * native row softmax and no test vector for one; that routine is pinned by
+ * mathematics only (scipy's softmax, shift invariance, rows summing to one).
+ *
  * Build: see oracle/Makefile (flags follow the reference's setup.py:9-14,50:
  * -O3 -ffast-math -funroll-loops -fopenmp).
  */
