@@ -373,21 +373,29 @@ def test_steps_replay_from_a_hip_graph():
     spmv = lambda: H.prebuilt_spmv_csr_f32([M], [M, K], [[], [rp, ci]], v, [K], [[]], x).storage.value
     sddmm = lambda: H.sddmm_csr_float([M, K], [M, K], [[], [rp, ci]], v, [M, N], [[], []], B[:M * N],
                                       [K, N], [[], []], B).storage.value
+    # row softmax over a pattern with rows for every tier, the listed (giant) ones included:
+    # their count in the workspace has to start from zero in every replay
+    lens = np.concatenate([np.full(300, 5), [9000, 70, 5000, 300, 12000], np.full(50, 40)])
+    s_rp = dev(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+    s_val = torch.empty(int(lens.sum()), device="cuda")
+    softmax = lambda: H.softmax_csr_float(s_rp, s_val, 0.5)
+    steps = (spmm, spmv, sddmm, softmax)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):  # warm-up off the default stream, as graph capture wants it
-        for fn in (spmm, spmv, sddmm):
+        for fn in steps:
             fn()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        captured = (spmm(), spmv(), sddmm())
+        captured = tuple(fn() for fn in steps)
     gen = torch.Generator(device="cuda").manual_seed(17)
     for _ in range(4):
         B.copy_(torch.randn(B.shape, device="cuda", generator=gen))
         x.copy_(torch.randn(x.shape, device="cuda", generator=gen))
-        eager = [fn().clone() for fn in (spmm, spmv, sddmm)]
+        s_val.copy_(torch.randn(s_val.shape, device="cuda", generator=gen) * 3)
+        eager = [fn().clone() for fn in steps]
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
