@@ -89,8 +89,37 @@ def _csr_parts(mode_indices, what: str, n_cols: Optional[int] = None):
     return pos, crd
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(dev: torch.device) -> int:
+    """Handle of torch's current stream on `dev` (the raw getter costs a fraction of
+    a microsecond; building a Stream object, several)."""
+    if _raw_stream is not None:
+        return _raw_stream(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _on_device:
+    """``with _on_device(dev):`` makes `dev` the current device like
+    ``torch.cuda.device`` does, but costs next to nothing when it already is."""
+    __slots__ = ("index", "previous")
+
+    def __init__(self, dev: torch.device):
+        self.index = dev.index
+        self.previous = -1
+
+    def __enter__(self):
+        current = torch.cuda.current_device()
+        if current != self.index:
+            self.previous = current
+            torch.cuda.set_device(self.index)
+        return self
+
+    def __exit__(self, *exc):
+        if self.previous >= 0:
+            torch.cuda.set_device(self.previous)
+        return False
 
 
 # ---- SpMM ----------------------------------------------------------------------
@@ -110,7 +139,7 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
     nnz = a_val.numel()
     out = torch.empty(M * N, dtype=dtype, device=dev)
     L = native.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         stream = _stream(dev)
         need = L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, a_val.element_size())
         ws = _workspace(dev, stream, need)
@@ -196,7 +225,7 @@ def _make_spgemm(dtype):
             raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
         dev = _device_of(a_pos, a_crd, a_val, b_pos, b_crd, b_val)
         L = native.lib()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             stream = _stream(dev)
             need = L.scorch_hip_spgemm_csr_workspace_bytes(M, N, a_val.element_size())
             ws = _workspace(dev, stream, need)
@@ -235,7 +264,7 @@ def _make_spmv(dtype):
         dev = _device_of(pos, crd, a_val, x)
         y = torch.empty(M, dtype=dtype, device=dev)
         L = native.lib()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             stream = _stream(dev)
             ws = _workspace(dev, stream, L.scorch_hip_spmv_csr_workspace_bytes(M, a_val.numel(),
                                                                               a_val.element_size()))
@@ -281,7 +310,7 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
         raise ValueError("scorch_ops_hip: S index and value lengths differ")
     dev = _device_of(row, col, s_val, a, b)
     out = torch.empty_like(s_val)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = native.lib().scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(),
                                                    col.data_ptr(), s_val.data_ptr(), a.data_ptr(),
                                                    b.data_ptr(), out.data_ptr(), _stream(dev))
@@ -302,7 +331,7 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     dev = _device_of(pos, crd, s_val, a, b)
     out = torch.empty_like(s_val)
     rows = torch.empty_like(crd)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = native.lib().scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(),
                                                    crd.data_ptr(), s_val.data_ptr(), a.data_ptr(),
                                                    b.data_ptr(), out.data_ptr(), rows.data_ptr(),
@@ -320,7 +349,7 @@ def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float 
     dev = _device_of(pos, v)
     out = torch.empty_like(v)
     L = native.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         stream = _stream(dev)
         need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, v.numel())
         ws = _workspace(dev, stream, need) if need else None
@@ -336,7 +365,7 @@ def csr_row_indices(row_ptr: torch.Tensor, nnz: int) -> torch.Tensor:
     pos = _index(row_ptr, "row_ptr")
     dev = _device_of(pos)
     rows = torch.empty(nnz, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = native.lib().scorch_hip_csr_row_indices(pos.numel() - 1, nnz, pos.data_ptr(),
                                                      rows.data_ptr(), _stream(dev))
     native.check(rc)
@@ -350,7 +379,7 @@ def coo_row_ptr(row_idx: torch.Tensor, n_rows: int) -> Optional[torch.Tensor]:
     dev = _device_of(rows)
     pos = torch.empty(n_rows + 1, dtype=torch.int32, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = native.lib().scorch_hip_coo_row_ptr(n_rows, rows.numel(), rows.data_ptr(), pos.data_ptr(),
                                                  flag.data_ptr(), _stream(dev))
     native.check(rc)
@@ -422,7 +451,7 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     if brp.numel() != S // block + 1:
         raise ValueError("scorch_ops_hip: block_row_ptr length does not match S / block")
     out = torch.empty_like(q)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),
                                                            bci.data_ptr(), q.data_ptr(), k.data_ptr(),
                                                            v.data_ptr(), float(scale), out.data_ptr(),
