@@ -30,7 +30,8 @@ HIPCC_FLAGS = [
     # floating-point atomic adds (SpGEMM accumulators) as the hardware's add instructions, not
     # compare-and-swap loops; their targets are LDS and ordinary device memory
     "-munsafe-fp-atomics",
-    "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
+    # (an unroll request the optimizer declines, e.g. in a loop it has already restructured, is no news)
+    "-fvisibility=hidden", "-Wall", "-Wno-unused-function", "-Wno-pass-failed",
 ]
 
 
