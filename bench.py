@@ -396,6 +396,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--rows", type=int, default=1 << 20, help="nodes of the graph (default: the headline size)")
     ap.add_argument("--features", type=int, default=128)
+    ap.add_argument("--window", type=int, default=0,
+                    help="gcn_powerlaw: draw a node's neighbours from this many nodes around it instead of from "
+                         "all nodes (same degrees; shows what the kernel does when rows share neighbours)")
     ap.add_argument("--row-length", type=int, default=0,
                     help="softmax_rows: entries per row (0: a causal mask, row i has i + 1 entries)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -454,7 +457,7 @@ def main() -> int:
         return side_workload(args, dev)
 
     t0 = time.time()
-    w = workloads.gcn_powerlaw(M=args.rows, N=args.features)
+    w = workloads.gcn_powerlaw(M=args.rows, N=args.features, window=args.window)
     M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
     print(f"[bench] generated {WORKLOAD}: M={M} nnz={nnz} N={N} in {time.time() - t0:.1f}s", file=sys.stderr)
 
@@ -508,7 +511,8 @@ def main() -> int:
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": WORKLOAD, "rows": M, "cols": K, "nnz": nnz, "features": N,
                    "degree": "zipf(2.1) scaled to mean 16, cap 50000, + self-loops",
-                   "values": "D^-1/2 (A+I) D^-1/2", "seed": workloads.SEEDS["gcn_powerlaw"]},
+                   "values": "D^-1/2 (A+I) D^-1/2", "seed": workloads.SEEDS["gcn_powerlaw"],
+                   **({"neighbour_window": args.window} if args.window else {})},
         "hbm_gbps_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
         "hbm_frac_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "event_ms_per_step": round(event_ms_per_step, 4),

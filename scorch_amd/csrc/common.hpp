@@ -82,6 +82,18 @@ __device__ __forceinline__ int wave_lane() { return threadIdx.x & (kWaveSize - 1
 // wave-uniform so that addresses built from it use scalar arithmetic.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Workgroups are dealt to the 8 XCDs round robin by their linear id, and every
+// XCD has its own L2.  xcd_contiguous renumbers the n workgroups of a launch (n a
+// multiple of 8, see round_up_8; a kernel lets the surplus ones find nothing to
+// do) so that XCD x works through the contiguous range [x n/8, (x + 1) n/8) in
+// order: the wavefronts resident on one XCD then work on neighbouring pieces of
+// the input, and rows of the gathered operand that neighbouring pieces share
+// are found in that XCD's L2 instead of being fetched into all eight.
+__device__ __forceinline__ int64_t xcd_contiguous(int64_t id, int64_t n) {
+  return (id & 7) * (n >> 3) + (id >> 3);
+}
+inline int64_t round_up_8(int64_t n) { return (n + 7) / 8 * 8; }
+
 // Orders LDS traffic inside one wavefront: writes by any lane before this point
 // are seen by reads of any lane after it.  Enough when the LDS region is
 // private to the wavefront (the hardware runs one wavefront's LDS instructions

@@ -32,7 +32,8 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
     int *__restrict__ out_row_idx) {
   using VecT = Vec<float, VEC>;
   const int lane = wave_lane();
-  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  // the grid is a multiple of 8 workgroups; every XCD takes a contiguous eighth of the entries
+  const int64_t wave = xcd_contiguous(blockIdx.x, gridDim.x) * kWavesPerBlock + threadIdx.x / kWaveSize;
   const int64_t first = wave * kEntriesPerWave;
   if (first >= nnz) return;
   const int64_t last = first + kEntriesPerWave < nnz ? first + kEntriesPerWave : nnz;
@@ -122,7 +123,7 @@ int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
                  const float *mask_vals, const float *A, const float *B, float *out_vals,
                  int *out_row_idx, hipStream_t stream) {
   const int64_t waves = (nnz + kEntriesPerWave - 1) / kEntriesPerWave;
-  const dim3 grid((unsigned)((waves + kWavesPerBlock - 1) / kWavesPerBlock));
+  const dim3 grid((unsigned)round_up_8((waves + kWavesPerBlock - 1) / kWavesPerBlock));
   const bool vec4 = K % 4 == 0 && aligned_to(A, 16) && aligned_to(B, 16);
   const int per_lane = vec4 ? 4 : 1;
   const int64_t lanes_needed = (K + per_lane - 1) / per_lane;

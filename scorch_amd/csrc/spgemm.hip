@@ -462,7 +462,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
   if (!QUARTERS) {
     __shared__ TeamTables<A, NUMERIC, kWaveSize, kWavesPerBlock, kTinySlots, kTinyProducts> one;
     const int w = threadIdx.x / kWaveSize;
-    const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + w;
+    const int64_t row = xcd_contiguous(blockIdx.x, gridDim.x) * kWavesPerBlock + w;
     if (row >= M || products[row] > kTinyProducts) return;
     spgemm_team_row<T, NUMERIC, kWaveSize, kWavesPerBlock, kTinySlots, kTinyProducts>(
         one, w, wave_lane(), (int)row, a_pos, a_crd, a_val, b_pos, b_crd, b_val, c_pos, c_crd, c_val);
@@ -475,7 +475,9 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
   __shared__ Tables lds[kWavesPerBlock];
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int64_t first = ((int64_t)blockIdx.x * kWavesPerBlock + w) * kQuarters;
+  // (the grid is a multiple of 8 workgroups: neighbouring rows, which may well select the same
+  // rows of B, go to one XCD)
+  const int64_t first = (xcd_contiguous(blockIdx.x, gridDim.x) * kWavesPerBlock + w) * kQuarters;
   if (first >= M) return;
   const int q = lane / kMicroTeam;
   const int64_t mine = first + q;
@@ -934,11 +936,11 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   // four rows to a wavefront once that still leaves every wavefront slot of the chip a wavefront
   if ((int64_t)M >= 4 * 8192) {
     const int64_t rows_per_block = kWavesPerBlock * (kWaveSize / kMicroTeam);
-    const unsigned tiny_blocks = (unsigned)(((int64_t)M + rows_per_block - 1) / rows_per_block);
+    const unsigned tiny_blocks = (unsigned)round_up_8(((int64_t)M + rows_per_block - 1) / rows_per_block);
     spgemm_tiny_kernel<T, NUMERIC, true><<<tiny_blocks, kBlockThreads, 0, stream>>>(
         M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
   } else {
-    const unsigned tiny_blocks = (unsigned)((M + kWavesPerBlock - 1) / kWavesPerBlock);
+    const unsigned tiny_blocks = (unsigned)round_up_8(((int64_t)M + kWavesPerBlock - 1) / kWavesPerBlock);
     spgemm_tiny_kernel<T, NUMERIC, false><<<tiny_blocks, kBlockThreads, 0, stream>>>(
         M, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.products, c_pos, c_crd, c_val);
   }

@@ -57,7 +57,11 @@ __device__ __forceinline__ TileMap map_workgroup(int64_t id, int n_tiles, int64_
     m.block = slot % blocks_per_tile;
   } else {
     m.tile = (int)(id / blocks_per_tile);
-    m.block = id % blocks_per_tile;
+    const int64_t rem = id % blocks_per_tile;
+    // rem & 7 is the XCD when blocks_per_tile is a multiple of 8 (the SpMM launchers
+    // see to that): every XCD gets one contiguous eighth of the chunks, so that B
+    // rows shared by neighbouring rows of A are found in its L2
+    m.block = (blocks_per_tile & 7) == 0 ? xcd_contiguous(rem, blocks_per_tile) : rem;
   }
   return m;
 }
@@ -495,7 +499,8 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
       align_up((size_t)spmm_num_chunks(M, nnz, N, sizeof(T)) * sizeof(int), 256));
   const int tile = kWaveSize * VEC;
   const int n_tiles = (N + tile - 1) / tile;
-  const int64_t blocks_per_tile = (chunks + kWavesPerBlock - 1) / kWavesPerBlock;
+  // a multiple of 8 (see map_workgroup); workgroups past the last chunk find nothing to do
+  const int64_t blocks_per_tile = round_up_8((chunks + kWavesPerBlock - 1) / kWavesPerBlock);
   if (blocks_per_tile * n_tiles > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
@@ -537,7 +542,7 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
   T *carry_val = reinterpret_cast<T *>(
       static_cast<char *>(workspace) +
       align_up((size_t)spmm_num_chunks(M, nnz, N, sizeof(T)) * sizeof(int), 256));
-  const int64_t blocks_per_tile = (spans + kWavesPerBlock - 1) / kWavesPerBlock;
+  const int64_t blocks_per_tile = round_up_8((spans + kWavesPerBlock - 1) / kWavesPerBlock);
   if (blocks_per_tile * n_tiles > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
@@ -662,7 +667,8 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_merge_kernel(
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int64_t span = (int64_t)blockIdx.x * kWavesPerBlock + w;
+  // the grid is a multiple of 8 workgroups; every XCD takes a contiguous eighth of the spans
+  const int64_t span = xcd_contiguous(blockIdx.x, gridDim.x) * kWavesPerBlock + w;
   int64_t d0 = span * kSpmvItems;
   if (d0 >= total_items) return;  // nothing here uses workgroup barriers
   int64_t d1 = d0 + kSpmvItems;
@@ -778,7 +784,7 @@ int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t 
   int *carry_row = static_cast<int *>(workspace);
   T *carry_val = reinterpret_cast<T *>(static_cast<char *>(workspace) +
                                        align_up((size_t)spans * sizeof(int), 256));
-  const int64_t blocks = (spans + kWavesPerBlock - 1) / kWavesPerBlock;
+  const int64_t blocks = round_up_8((spans + kWavesPerBlock - 1) / kWavesPerBlock);
   spmv_merge_kernel<T><<<dim3((unsigned)blocks), kBlockThreads, 0, s>>>(
       (int)M, row_ptr, col_idx, vals, x, y, M + nnz, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());

@@ -57,7 +57,7 @@ def spmm_uniform(M: int = 4096, K: int = 4096, N: int = 64, density: float = 0.0
 
 def gcn_powerlaw(M: int = 1 << 20, N: int = 128, seed: int = SEEDS["gcn_powerlaw"],
                  zipf_a: float = 2.1, mean_degree: float = 16.0,
-                 max_degree: int = 50_000) -> Dict[str, np.ndarray]:
+                 max_degree: int = 50_000, window: int = 0) -> Dict[str, np.ndarray]:
     """Power-law graph with the GCN normalisation D^-1/2 (A + I) D^-1/2.
 
     Out-degrees are Zipf(``zipf_a``) draws capped at ``max_degree``, rescaled to
@@ -66,6 +66,10 @@ def gcn_powerlaw(M: int = 1 << 20, N: int = 128, seed: int = SEEDS["gcn_powerlaw
     ``deg`` is the row length of A + I and each entry is
     ``deg[row]^-1/2 * deg[col]^-1/2`` (the edge weight of
     bench/bench_gcn.py:248-258).  Features are N(0, 1).
+
+    ``window`` > 0 draws a node's neighbours from the ``window`` nodes around it
+    (wrapping at the ends) instead of from all nodes: the same degrees and entry
+    count, but rows that lie close together share neighbours.
     """
     rng = _rng(seed)
     cap = min(max_degree, M - 1) if M > 1 else 0
@@ -74,7 +78,10 @@ def gcn_powerlaw(M: int = 1 << 20, N: int = 128, seed: int = SEEDS["gcn_powerlaw
     deg = np.floor(scaled + rng.random(M)).astype(np.int64)
     deg = np.clip(deg, 0, cap)
     rows = np.repeat(np.arange(M, dtype=np.int32), deg)
-    cols = rng.integers(0, M, size=rows.size, dtype=np.int64).astype(np.int32)
+    cols = rng.integers(0, M, size=rows.size, dtype=np.int64)
+    if window > 0:
+        cols = (rows.astype(np.int64) + cols % window - window // 2) % M
+    cols = cols.astype(np.int32)
     loops = np.arange(M, dtype=np.int32)
     rows = np.concatenate([rows, loops])
     cols = np.concatenate([cols, loops])
