@@ -425,9 +425,8 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
 
 // Shape of the work split.  A chunk holds up to 256 merge items (what the LDS
 // slices hold); a wavefront walks chunks_per_wave consecutive chunks and leaves
-// one carry.  Small problems use smaller chunks, one per wavefront, so that
-// they are spread over more, shorter wavefronts; large ones use several chunks
-// per wavefront, which divides the number of carries the fix-up must fold.
+// one carry.  Small problems use smaller chunks, so that they are spread over
+// more, shorter wavefronts.
 struct SpmmSplit {
   int items_per_chunk;
   int chunks_per_wave;
@@ -443,15 +442,12 @@ inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   sp.items_per_chunk = kMinItemsPerWave;
   while (sp.items_per_chunk < kItemsPerWave && sp.items_per_chunk * 2 <= per_wave)
     sp.items_per_chunk *= 2;
+  // One chunk per wavefront.  (The kernel can walk several consecutive chunks and
+  // leave one carry for all of them; that halves the carries the fix-up folds but
+  // widens the stretch of rows an XCD has in flight, which costs more in L2 hits on
+  // matrices whose neighbouring rows share columns -- 0.81 against 0.69 ms with two
+  // chunks on the 4,096-neighbour graph -- than it saves: nothing on the headline graph.)
   sp.chunks_per_wave = 1;
-  if (sp.items_per_chunk == kItemsPerWave) {
-    const int64_t chunks_per_slot = per_wave / kItemsPerWave;  // chunks per resident wavefront
-    // Keep at least four rounds of wavefronts so that the last, partly filled
-    // round stays a small share of the run (measured: 2-3 chunks per wavefront
-    // are as fast as 1 at 18 M items and halve the carries; 8 cost 4 %).
-    const int cpw = (int)(chunks_per_slot / 4);
-    sp.chunks_per_wave = cpw < 1 ? 1 : (cpw > 4 ? 4 : cpw);
-  }
   const int64_t span_items = (int64_t)sp.items_per_chunk * sp.chunks_per_wave;
   sp.spans = (total + span_items - 1) / span_items;
   return sp;
