@@ -69,3 +69,19 @@ def test_sae_decoder_topk():
     assert (np.diff(w["row_ptr"]) == 8).all() and rows_sorted_unique(w["row_ptr"], w["col_idx"])
     assert (w["vals"] > 0).all() and w["B"].shape == (512, 32)
     assert abs(w["B"].std() - 0.125) < 0.01
+
+
+def test_gcn_powerlaw_neighbour_window():
+    """window > 0: every neighbour lies within window / 2 of its row (wrapping), the degrees keep their
+    shape, and the normalisation is unchanged."""
+    M, W = 5000, 64
+    w = workloads.gcn_powerlaw(M=M, N=4, seed=3, max_degree=400, window=W)
+    rows = np.repeat(np.arange(M), np.diff(w["row_ptr"]))
+    gap = np.abs(w["col_idx"].astype(np.int64) - rows)
+    gap = np.minimum(gap, M - gap)
+    assert gap.max() <= W // 2 and (gap == 0).sum() == M          # self-loops included
+    assert np.all(np.diff(w["row_ptr"]) >= 1) and np.diff(w["row_ptr"]).max() <= W
+    d = np.diff(w["row_ptr"]).astype(np.float64)
+    np.testing.assert_allclose(w["vals"], 1 / np.sqrt(d[rows] * d[w["col_idx"]]), rtol=1e-6)
+    plain = workloads.gcn_powerlaw(M=M, N=4, seed=3, max_degree=400)
+    assert np.abs(plain["col_idx"].astype(np.int64) - np.repeat(np.arange(M), np.diff(plain["row_ptr"]))).max() > M // 4
