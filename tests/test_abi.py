@@ -122,6 +122,10 @@ def test_spmv_softmax_rows_reject_bad_arguments(L):
     assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, FAKE, 256, NULL) == native.EWORKSPACE
     assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL
     assert L.scorch_hip_csr_row_indices(0, 4, FAKE, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_coo_row_ptr(4, 4, FAKE, NULL, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_coo_row_ptr(4, 4, FAKE, FAKE, NULL, NULL) == native.EINVAL
+    assert L.scorch_hip_coo_row_ptr(4, 4, NULL, FAKE, FAKE, NULL) == native.EINVAL
+    assert L.scorch_hip_coo_row_ptr(-1, 0, NULL, FAKE, FAKE, NULL) == native.EINVAL
 
 
 def test_check_raises_with_the_library_message(L):
@@ -147,3 +151,33 @@ def test_attention_rejects_unsupported_shapes(L):
     assert call(q=NULL) == native.EINVAL
     assert call(o=ctypes.c_void_p(0x1008)) == native.EINVAL      # not 16-byte aligned
     assert call(H=0, q=NULL, k=NULL, v=NULL, o=NULL) == native.OK
+
+
+def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 and as C++11, and a C program linked
+    against the library reads the ABI version and a workspace size (no GPU involved)."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = os.path.join(root, "include", "scorch_hip.h")
+    gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+    if not gcc or not gxx:
+        pytest.skip("no host compiler")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", header], check=True)
+    subprocess.run([gxx, "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", header], check=True)
+    src = tmp_path / "host.c"
+    src.write_text(
+        '#include <stdio.h>\n#include "scorch_hip.h"\n'
+        "int main(void) {\n"
+        '  printf("%d %zu\\n", scorch_hip_abi_version(),\n'
+        "         scorch_hip_spmm_csr_workspace_bytes(1000, 5000, 64, 4));\n"
+        "  return scorch_hip_last_error() == NULL;\n}\n")
+    lib_dir = os.path.dirname(native.library_path())
+    exe = tmp_path / "host"
+    subprocess.run([gcc, "-std=c99", "-I", os.path.join(root, "include"), str(src), "-L", lib_dir,
+                    "-l:libscorch_hip.so", "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib", "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) == native.lib().scorch_hip_abi_version()
+    assert int(out[1]) == native.lib().scorch_hip_spmm_csr_workspace_bytes(1000, 5000, 64, 4)
