@@ -647,8 +647,8 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
 // sums the products of the r-th row the chunk touches.  A row with many entries
 // in the chunk is summed by the whole wavefront instead (strided partial sums,
 // butterfly reduction).  The part of the last row that continues in the next
-// chunk becomes a carry, folded into y by spmm_fixup_kernel exactly as for SpMM,
-// so the summation order is fixed and results are bit-reproducible.
+// chunk becomes a carry, folded into y by spmv_fixup_kernel in a fixed order,
+// so results are bit-reproducible.
 constexpr int kSpmvItems = 512;
 constexpr int kSpmvLaneRowMax = 32;  // longer in-chunk rows are summed by the whole wavefront
 
@@ -751,6 +751,63 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_merge_kernel(
   }
 }
 
+// The carries of SpMV are single values, so a wavefront per chunk (spmm_fixup_kernel)
+// would leave 63 lanes idle.  Here a thread looks at one chunk: if it heads a run
+// of equal carry rows it adds the run, in chunk order, to y.  Runs of more than
+// kSpmvShortRun carries (a row spread over that many wavefronts) are then taken
+// one after the other by the whole wavefront: lane l sums members l, l + 64, ...
+// and the lanes' sums are combined in a fixed order.  Same result on every run.
+constexpr int kSpmvShortRun = 32;
+
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void spmv_fixup_kernel(int64_t spans,
+                                                                   const int *__restrict__ carry_row,
+                                                                   const T *__restrict__ carry_val,
+                                                                   T *__restrict__ y) {
+  using A = typename Acc<T>::type;
+  const int lane = wave_lane();
+  const int64_t c = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  int row = -1;
+  if (c < spans) {
+    row = carry_row[c];
+    if (row >= 0 && c > 0 && carry_row[c - 1] == row) row = -1;  // not the head of its run
+  }
+  bool long_run = false;
+  if (row >= 0) {
+    A sum = (A)0;
+    int64_t e = c;
+    for (; e < spans && e < c + kSpmvShortRun && carry_row[e] == row; ++e) sum += (A)carry_val[e];
+    long_run = e == c + kSpmvShortRun && e < spans && carry_row[e] == row;
+    if (!long_run) y[row] = (T)(sum + (A)y[row]);
+  }
+  unsigned long long pending = __ballot(long_run);
+  while (pending) {  // uniform over the wavefront
+    const int owner = __ffsll(pending) - 1;
+    pending &= pending - 1;
+    const int64_t start = c - lane + owner;
+    const int r = __shfl(row, owner);
+    // End of the run by a 64-way search: its members are consecutive, so "same row"
+    // holds up to the end and nowhere after.  `last` is a known member, `stop` the
+    // first position known to lie beyond (or the end of the list).
+    int64_t last = start, stop = spans;
+    while (stop - last > 1) {
+      const int64_t step = (stop - last + kWaveSize) / (kWaveSize + 1);
+      const int64_t probe = last + (int64_t)(lane + 1) * step;
+      const bool same = probe < stop && carry_row[probe] == r;
+      const int members = __popcll(__ballot(same));  // lanes 0 .. members - 1
+      const int64_t reached = last + (int64_t)members * step;
+      if (members < kWaveSize && reached + step < stop) stop = reached + step;  // lane `members` saw the end
+      last = reached;
+    }
+    const int64_t end = last + 1;
+    A part = (A)0;
+    for (int64_t e = start + lane; e < end; e += kWaveSize) part += (A)carry_val[e];
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) part += (A)__shfl_xor((T)part, off);
+    if (lane == owner) y[r] = (T)(part + (A)y[r]);
+  }
+}
+
 inline int64_t spmv_num_spans(int64_t M, int64_t nnz) {
   return (M + nnz + kSpmvItems - 1) / kSpmvItems;
 }
@@ -784,8 +841,8 @@ int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t 
   spmv_merge_kernel<T><<<dim3((unsigned)blocks), kBlockThreads, 0, s>>>(
       (int)M, row_ptr, col_idx, vals, x, y, M + nnz, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  spmm_fixup_kernel<T, 1, kEpiNone><<<dim3((unsigned)blocks), kBlockThreads, 0, s>>>(
-      1, spans, 1, blocks, carry_row, carry_val, y, nullptr);
+  spmv_fixup_kernel<T><<<dim3((unsigned)((spans + kBlockThreads - 1) / kBlockThreads)), kBlockThreads, 0, s>>>(
+      spans, carry_row, carry_val, y);
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }

@@ -325,6 +325,30 @@ def test_spmv_row_length_distributions(oracle, name, dtype):
     assert not got[np.diff(rp) == 0].any()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
+def test_spmv_rows_spread_over_many_wavefronts(oracle, dtype):
+    """Rows whose carries form long runs (a row of 40,000 entries spans ~80 wavefronts, one of
+    600,000 over a thousand), next to ordinary ones and at both ends of the matrix."""
+    from gpu_util import hip_spmv
+    rng = np.random.default_rng(5)
+    lens = rng.integers(0, 6, 300)
+    lens[[0, 57, 58, 299]] = [40_000, 600_000, 17_000, 33_000]
+    K = 700_000
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, int(n), replace=False)) for n in lens]).astype(np.int32)
+    if np.issubdtype(dtype, np.integer):
+        v, x = rng.integers(-1000, 1000, ci.size).astype(dtype), rng.integers(-1000, 1000, K).astype(dtype)
+    else:
+        v, x = rng.uniform(-1, 1, ci.size).astype(dtype), rng.standard_normal(K).astype(dtype)
+    got = hip_spmv(rp, ci, v, x)
+    assert np.array_equal(got, hip_spmv(rp, ci, v, x))
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(got, oracle.spmv_csr_typed(rp, ci, v, x))
+    else:
+        ref64 = oracle.spmm_fp64(rp, ci, v, x.reshape(-1, 1)).reshape(-1)
+        assert oracle.rel_fro(got, ref64) <= (TOL if dtype == np.float32 else 1e-13)
+
+
 def test_spmv_full_size_and_reproducible():
     w = workloads.gcn_powerlaw(N=1)
     M = w["M"]
