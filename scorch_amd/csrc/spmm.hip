@@ -768,17 +768,22 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_fixup_kernel(int64_t spans
   const int lane = wave_lane();
   const int64_t c = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
   int row = -1;
-  if (c < spans) {
-    row = carry_row[c];
-    if (row >= 0 && c > 0 && carry_row[c - 1] == row) row = -1;  // not the head of its run
-  }
   bool long_run = false;
-  if (row >= 0) {
-    A sum = (A)0;
-    int64_t e = c;
-    for (; e < spans && e < c + kSpmvShortRun && carry_row[e] == row; ++e) sum += (A)carry_val[e];
-    long_run = e == c + kSpmvShortRun && e < spans && carry_row[e] == row;
-    if (!long_run) y[row] = (T)(sum + (A)y[row]);
+  if (c < spans) {
+    // everything the usual case needs (a run of one) is requested at once
+    row = carry_row[c];
+    const int before = c > 0 ? carry_row[c - 1] : -1;
+    const int after = c + 1 < spans ? carry_row[c + 1] : -1;
+    A sum = (A)carry_val[c];
+    if (row >= 0 && before == row) row = -1;  // not the head of its run
+    if (row >= 0) {
+      if (after == row) {
+        int64_t e = c + 1;
+        for (; e < spans && e < c + kSpmvShortRun && carry_row[e] == row; ++e) sum += (A)carry_val[e];
+        long_run = e == c + kSpmvShortRun && e < spans && carry_row[e] == row;
+      }
+      if (!long_run) y[row] = (T)(sum + (A)y[row]);
+    }
   }
   unsigned long long pending = __ballot(long_run);
   while (pending) {  // uniform over the wavefront
