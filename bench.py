@@ -255,6 +255,63 @@ def side_workload(args, dev) -> int:
                           "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
                           "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
         return 0
+    if args.workload == "gcn_forward":
+        # The two-layer GCN forward pass of the reference's graph benchmark
+        # (bench/bench_gcn.py:320-357) on the headline graph: linear -> A_hat x -> + bias
+        # -> relu -> linear -> A_hat x -> + bias -> log_softmax, once with the separate
+        # steps and once through @compile, which routes matmul + bias (+ relu) to the fused kernel.
+        import torch.nn.functional as F
+        import scorch_amd as scorch
+        w = workloads.gcn_powerlaw(M=args.rows, N=args.features)
+        M, nnz = w["M"], int(w["col_idx"].size)
+        hidden, classes = 128, 64
+        adj = scorch.STensor.from_csr_arrays(t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), (M, M))
+        x0 = t(w["B"])
+        gen = torch.Generator(device="cuda").manual_seed(5)
+        weights = {"w1": torch.randn(hidden, args.features, device="cuda", generator=gen) * 0.1,
+                   "b1": torch.randn(hidden, device="cuda", generator=gen) * 0.1,
+                   "w2": torch.randn(classes, hidden, device="cuda", generator=gen) * 0.1,
+                   "b2": torch.randn(classes, device="cuda", generator=gen) * 0.1}
+
+        def unfused():
+            h = F.linear(x0, weights["w1"])
+            h = scorch.matmul(adj, h, format="dd") + weights["b1"]
+            h = F.linear(F.relu(h), weights["w2"])
+            return F.log_softmax(scorch.matmul(adj, h, format="dd") + weights["b2"], dim=1)
+
+        @scorch.compile
+        def spmm_bias_relu(a, h, bias):
+            return torch.relu(scorch.matmul(a, h, format="dd") + bias)
+
+        @scorch.compile
+        def spmm_bias(a, h, bias):
+            return scorch.matmul(a, h, format="dd") + bias
+
+        def fused():
+            h = spmm_bias_relu(adj, F.linear(x0, weights["w1"]), weights["b1"])
+            return F.log_softmax(spmm_bias(adj, F.linear(h, weights["w2"]), weights["b2"]), dim=1)
+
+        a_t = torch.sparse_csr_tensor(adj.index.mode_indices[1][0], adj.index.mode_indices[1][1], adj.values,
+                                      size=(M, M))
+
+        def vendor():
+            h = F.relu(torch.sparse.mm(a_t, F.linear(x0, weights["w1"])) + weights["b1"])
+            return F.log_softmax(torch.sparse.mm(a_t, F.linear(h, weights["w2"])) + weights["b2"], dim=1)
+
+        err = float((fused() - unfused()).abs().max())
+        ms_fused = _time_steps(fused, args.steps, args.warmup)
+        ms_unfused = _time_steps(unfused, args.steps, args.warmup)
+        out = {"metric": "two-layer GCN forward passes per second", "value": round(1e3 / ms_fused, 2),
+               "unit": "1/s", "ms_per_step": round(ms_fused, 4), "ms_per_step_unfused": round(ms_unfused, 4),
+               "max_abs_difference_fused_unfused": err, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+               "dtype": "f32", "data": "synthetic", "higher_is_better": True,
+               "config": {"workload": "gcn_forward_fp32", "rows": M, "nnz": nnz, "features": args.features,
+                          "hidden": hidden, "classes": classes}}
+        if args.vendor:
+            out["vendor_library"] = _vendor_time("torch.sparse.mm in the same forward pass", vendor, args.steps,
+                                                 args.warmup)
+        print(json.dumps(out))
+        return 0
     if args.workload == "softmax_rows":
         # every row --row-length entries long, or a causal mask (row i has i + 1) with --row-length 0
         import numpy as np
@@ -405,7 +462,7 @@ def main() -> int:
     ap.add_argument("--workload", default="gcn_powerlaw",
                     choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
                              "attention_blocksparse", "spgemm_powerlaw", "spmv_powerlaw",
-                             "softmax_powerlaw", "softmax_rows"],
+                             "softmax_powerlaw", "softmax_rows", "gcn_forward"],
                     help="gcn_powerlaw is the headline line; the others time the parity workloads")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")
