@@ -245,7 +245,41 @@ def side_workload(args, dev) -> int:
         ms = _time_steps(fn, args.steps, args.warmup)
         flops = 4.0 * nnz * D * Hh
         algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
-        print(json.dumps({"metric": "fused block-sparse attention TFLOP/s", "value": round(flops / ms / 1e9, 2),
+        extra = {}
+        if args.vendor:
+            # (a) the composition the reference's benchmark uses, per head and in fp32, on this
+            # package's own kernels: SDDMM -> row softmax -> SpMM (bench_sparse_transformer.py:354-372)
+            import numpy as np
+            blk = w["block"]
+            rows_b = np.repeat(np.arange(brp.numel() - 1), np.diff(w["block_row_ptr"]))
+            dense_blocks = np.zeros((S // blk, S // blk), bool)
+            dense_blocks[rows_b, w["block_col_idx"]] = True
+            mask = torch.from_numpy(np.kron(dense_blocks, np.ones((blk, blk), bool))).to(dev)
+            csr = mask.to(torch.float32).to_sparse_csr()
+            pos, crd = csr.crow_indices().to(torch.int32), csr.col_indices().to(torch.int32)
+            ones = torch.ones(crd.numel(), device=dev)
+            qf, kf, vf = q.float(), k.float(), v.float()
+
+            def unfused():
+                outs = []
+                for h in range(Hh):
+                    sc = H.sddmm_csr_float([S, S], [S, S], [[], [pos, crd]], ones, [S, D], [[], []],
+                                           qf[h].reshape(-1), [S, D], [[], []], kf[h].reshape(-1))
+                    p = H.softmax_csr_float(pos, sc.storage.value, float(w["scale"]))
+                    outs.append(H.spmm_csr_float_v2([S, D], [S, S], [[], [pos, crd]], p, [S, D], [[], []],
+                                                    vf[h].reshape(-1)).storage.value)
+                return outs
+
+            extra["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM per head (this package, fp32)",
+                                                          unfused, max(args.steps // 4, 2), 1)
+            # (b) torch's dense attention with the same mask
+            import torch.nn.functional as F
+            extra["vendor_library"] = _vendor_time(
+                "F.scaled_dot_product_attention(bf16, dense boolean mask)",
+                lambda: F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask[None, None],
+                                                       scale=float(w["scale"])), max(args.steps // 4, 2), 1)
+        print(json.dumps({**extra,
+                          "metric": "fused block-sparse attention TFLOP/s", "value": round(flops / ms / 1e9, 2),
                           "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
                           "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
                           "higher_is_better": True,
