@@ -74,136 +74,152 @@ __device__ __forceinline__ T apply_epilogue(typename Acc<T>::type acc, T bias) {
   return r;
 }
 
+// Chunk boundaries.  Chunk c nominally covers the merged positions [c * items,
+// (c + 1) * items).  A boundary that falls inside a row moves forward to just
+// after the row's end marker when that is at most `snap` items away: the row
+// is then summed by one chunk and leaves no carry.  Most rows are short, so
+// most boundaries snap, and carries remain for rows that really span chunks.
+// The result depends on the nominal position only, so the two chunks on either
+// side of a boundary agree on it.  x: rows finished before the boundary, y:
+// nonzeros before it.
+constexpr int kSnapItems = 64;
+
+struct Boundary {
+  int x, y;
+};
+
+__device__ __forceinline__ Boundary chunk_boundary(int64_t d, int M, int64_t total_items,
+                                                   const int *__restrict__ row_ptr, int snap) {
+  Boundary b;
+  if (d >= total_items) {
+    b.x = M;
+    b.y = (int)(total_items - M);
+    return b;
+  }
+  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
+  b.x = wave_count_below(M, d, row_end_key);
+  b.y = uniform((int)(d - b.x));
+  if (b.x < M) {
+    const int begin = uniform(row_ptr[b.x]), end = uniform(row_ptr[b.x + 1]);
+    const int64_t after_marker = (int64_t)end + b.x + 1;
+    if (begin < b.y && after_marker - d <= snap) {  // the row is under way and nearly done
+      b.x += 1;
+      b.y = end;
+    }
+  }
+  return b;
+}
+
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
-    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int chunks_per_wave,
-    int n_tiles, int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
+    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
+    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
+  constexpr int kSlots = kItemsPerWave + kSnapItems;
 
-  __shared__ int s_col[kWavesPerBlock][kItemsPerWave];
-  __shared__ T s_val[kWavesPerBlock][kItemsPerWave];
-  __shared__ int s_rp[kWavesPerBlock][kItemsPerWave + 2];
+  __shared__ int s_col[kWavesPerBlock][kSlots];
+  __shared__ T s_val[kWavesPerBlock][kSlots];
+  __shared__ int s_rp[kWavesPerBlock][kSlots + 2];
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
   const TileMap where = map_workgroup(blockIdx.x, n_tiles, blocks_per_tile);
-  const int64_t span = where.block * kWavesPerBlock + w;  // this wavefront's share
+  const int64_t chunk = where.block * kWavesPerBlock + w;
   const int col0 = (where.tile * kWaveSize + lane) * VEC;
   const bool active = col0 < N;
 
-  // The wavefront owns chunks_per_wave consecutive chunks of the merged
-  // sequence, [span_d0, span_d1); spans past the end are empty.
-  const int64_t span_items = (int64_t)items_per_chunk * chunks_per_wave;
-  int64_t span_d0 = span * span_items;
-  span_d0 = span_d0 < total_items ? span_d0 : total_items;
-  int64_t span_d1 = span_d0 + span_items;
-  span_d1 = span_d1 < total_items ? span_d1 : total_items;
+  const int64_t d0 = chunk * items_per_chunk;
+  if (d0 >= total_items) return;  // only wave-level synchronisation below
+  const Boundary from = chunk_boundary(d0, M, total_items, row_ptr, snap);
+  const Boundary to = chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
+  const int x0 = from.x, y0 = from.y, x1 = to.x, y1 = to.y;
+  const int n_nz = y1 - y0;
+  const int n_rows = x1 - x0;
 
-  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
-  const int span_x0 = wave_count_below(M, span_d0, row_end_key);  // rows finished before the span
-  const int span_y0 = uniform((int)(span_d0 - span_x0));          // its first nonzero
-  // Row span_x0 began in an earlier span iff its first nonzero precedes
-  // span_y0: then its store is a partial sum and its epilogue is the fix-up's.
-  const bool carry_in = uniform(row_ptr[span_x0 < M ? span_x0 : M]) < span_y0;
+  // Stage the chunk's slice of A in LDS: coalesced loads now, broadcast reads later.
+  for (int k = lane; k < n_nz; k += kWaveSize) {
+    s_col[w][k] = col_idx[y0 + k];
+    s_val[w][k] = vals[y0 + k];
+  }
+  // s_rp[k] = row_ptr[x0 + k] for k = 0 .. n_rows + 1 (clamped at M).
+  for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
+    const int r = x0 + k < M ? x0 + k : M;
+    s_rp[w][k] = row_ptr[r];
+  }
+  wave_lds_sync();  // the slices are private to this wavefront
+
+  // Row x0 began in an earlier chunk iff its first nonzero precedes y0: then
+  // its store is a partial sum and its epilogue is the fix-up's.
+  const bool carry_in = uniform(s_rp[w][0]) < y0;
 
   T bias_v[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) bias_v[v] = (EPI != kEpiNone && active) ? bias[col0 + v] : (T)0;
 
-  A acc[VEC];  // carried in registers from chunk to chunk
+  A acc[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
 
-  int x = span_x0;        // next row to finish
-  int y = span_y0;        // next nonzero to consume
-  int last_row_start = 0; // row_ptr[x] after the last chunk
+  int x = x0;  // next row to finish
+  int next_end = uniform(s_rp[w][1]);
 
-  for (int sub = 0; sub < chunks_per_wave; ++sub) {
-    int64_t d1 = span_d0 + (int64_t)(sub + 1) * items_per_chunk;
-    d1 = d1 < span_d1 ? d1 : span_d1;
-    // The chunk starts where the walk stands, (x, y); only its end needs a search.
-    const int x0 = x, y0 = y;
-    const int x1 = wave_count_below(M, d1, row_end_key);  // rows finished by the chunk's end
-    const int y1 = uniform((int)(d1 - x1));
-    const int n_nz = y1 - y0;
-    const int n_rows = x1 - x0;
-
-    // Stage the chunk's slice of A in LDS: coalesced loads now, broadcast reads later.
-    for (int k = lane; k < n_nz; k += kWaveSize) {
-      s_col[w][k] = col_idx[y0 + k];
-      s_val[w][k] = vals[y0 + k];
-    }
-    // s_rp[k] = row_ptr[x0 + k] for k = 0 .. n_rows + 1 (clamped at M).
-    for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
-      const int r = x0 + k < M ? x0 + k : M;
-      s_rp[w][k] = row_ptr[r];
-    }
-    wave_lds_sync();  // the slices are private to this wavefront
-
-    int next_end = uniform(s_rp[w][1]);
-
-    auto flush_row = [&]() {
-      if (active) {
-        const bool partial = carry_in && x == span_x0;
-        VecT o;
-#pragma unroll
-        for (int v = 0; v < VEC; ++v)
-          o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
-        *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
-      }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
-      ++x;
-      next_end = uniform(s_rp[w][x - x0 + 1]);
-    };
-
-    auto gather = [&](int k) -> VecT {
-      const int j = uniform(s_col[w][k]);
-      VecT b;
-      if (active) {
-        b = *reinterpret_cast<const VecT *>(B + (size_t)j * (size_t)N + col0);
-      } else {
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) b.v[v] = (T)0;
-      }
-      return b;
-    };
-
-    auto consume = [&](int k, const VecT &b) {
-      while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
-      const A a = (A)s_val[w][k];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
-    };
-
-    int k = 0;
-    for (; k + kGather <= n_nz; k += kGather) {
-      VecT b[kGather];
-#pragma unroll
-      for (int u = 0; u < kGather; ++u) b[u] = gather(k + u);
-#pragma unroll
-      for (int u = 0; u < kGather; ++u) consume(k + u, b[u]);
-    }
-    for (; k < n_nz; ++k) consume(k, gather(k));
-    while (x < x1) flush_row();  // markers after the chunk's last nonzero
-    y = y1;
-    last_row_start = uniform(s_rp[w][n_rows]);  // row_ptr[x1]
-    wave_lds_sync();  // the LDS slices are rewritten by the next chunk
-  }
-
-  // Whatever is left belongs to row x, whose marker lies in a later span.
-  if (span * span_items < total_items) {
-    const int tail = y - (last_row_start > span_y0 ? last_row_start : span_y0);
-    if (where.tile == 0 && lane == 0) carry_row[span] = tail > 0 ? x : -1;
-    if (tail > 0 && active) {
+  auto flush_row = [&]() {
+    if (active) {
+      const bool partial = carry_in && x == x0;
       VecT o;
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];
-      *reinterpret_cast<VecT *>(carry_val + (size_t)span * (size_t)N + col0) = o;
+      for (int v = 0; v < VEC; ++v)
+        o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
+      *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
     }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+    ++x;
+    next_end = uniform(s_rp[w][x - x0 + 1]);
+  };
+
+  auto gather = [&](int k) -> VecT {
+    const int j = uniform(s_col[w][k]);
+    VecT b;
+    if (active) {
+      b = *reinterpret_cast<const VecT *>(B + (size_t)j * (size_t)N + col0);
+    } else {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) b.v[v] = (T)0;
+    }
+    return b;
+  };
+
+  auto consume = [&](int k, const VecT &b) {
+    while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
+    const A a = (A)s_val[w][k];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
+  };
+
+  int k = 0;
+  for (; k + kGather <= n_nz; k += kGather) {
+    VecT b[kGather];
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) b[u] = gather(k + u);
+#pragma unroll
+    for (int u = 0; u < kGather; ++u) consume(k + u, b[u]);
+  }
+  for (; k < n_nz; ++k) consume(k, gather(k));
+  while (x < x1) flush_row();  // markers after the chunk's last nonzero
+
+  // Whatever is left belongs to row x1, whose marker lies in a later chunk.
+  const int row_start = uniform(s_rp[w][n_rows]);  // row_ptr[x1]
+  const int tail = y1 - (row_start > y0 ? row_start : y0);
+  if (where.tile == 0 && lane == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
+  if (tail > 0 && active) {
+    VecT o;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];
+    *reinterpret_cast<VecT *>(carry_val + (size_t)chunk * (size_t)N + col0) = o;
   }
 }
 
@@ -224,15 +240,16 @@ template <typename T, int VEC, int LPR, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
-    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int n_tiles,
+    const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
     int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int G = kWaveSize / LPR;
+  constexpr int kSlots = kItemsPerWave + kSnapItems;
 
-  __shared__ int s_col[kWavesPerBlock][kItemsPerWave];
-  __shared__ T s_val[kWavesPerBlock][kItemsPerWave];
-  __shared__ int s_rp[kWavesPerBlock][kItemsPerWave + 2];
+  __shared__ int s_col[kWavesPerBlock][kSlots];
+  __shared__ T s_val[kWavesPerBlock][kSlots];
+  __shared__ int s_rp[kWavesPerBlock][kSlots + 2];
 
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
@@ -243,16 +260,11 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
   const int col0 = (where.tile * LPR + t) * VEC;
   const bool active = col0 < N;
 
-  int64_t d0 = span * items_per_chunk;
+  const int64_t d0 = span * items_per_chunk;
   if (d0 >= total_items) return;  // only wave-level synchronisation below
-  int64_t d1 = d0 + items_per_chunk;
-  d1 = d1 < total_items ? d1 : total_items;
-
-  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
-  const int x0 = wave_count_below(M, d0, row_end_key);
-  const int x1 = wave_count_below(M, d1, row_end_key);
-  const int y0 = uniform((int)(d0 - x0));
-  const int y1 = uniform((int)(d1 - x1));
+  const Boundary from = chunk_boundary(d0, M, total_items, row_ptr, snap);
+  const Boundary to = chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
+  const int x0 = from.x, y0 = from.y, x1 = to.x, y1 = to.y;
   const int n_nz = y1 - y0;
   const int n_rows = x1 - x0;
 
@@ -352,85 +364,103 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
 }
 
 
-// One wavefront per (chunk, column tile).  The first chunk of each run of
-// equal carry_row values sums the run in chunk order and folds it into C.
+// End of the run of equal carry rows that starts at `start` (a member): a 64-way
+// search by the whole wavefront.  The members of a run are consecutive, so
+// "same row" holds up to the end and nowhere after.
+__device__ __forceinline__ int64_t carry_run_end(const int *__restrict__ carry_row, int64_t start,
+                                                 int64_t num_chunks, int row) {
+  const int lane = wave_lane();
+  int64_t last = start, stop = num_chunks;  // a known member; the first position known to lie beyond
+  while (stop - last > 1) {
+    const int64_t step = (stop - last + kWaveSize) / (kWaveSize + 1);
+    const int64_t probe = last + (int64_t)(lane + 1) * step;
+    const bool same = probe < stop && carry_row[probe] == row;
+    const int members = __popcll(__ballot(same));  // lanes 0 .. members - 1
+    const int64_t reached = last + (int64_t)members * step;
+    if (members < kWaveSize && reached + step < stop) stop = reached + step;  // lane `members` saw the end
+    last = reached;
+  }
+  return last + 1;
+}
+
+// Folds the carries into C.  A wavefront looks at kFixupChunks consecutive
+// chunks' carry rows (one lane each, one load); those that head a run of equal
+// rows are then taken one after the other by the whole wavefront, lanes on
+// columns: the run is summed in chunk order and added to the row of C, with
+// the epilogue.  Few chunks leave a carry (see chunk_boundary), so most
+// wavefronts only look: fewer, wider-looking wavefronts cost less to start,
+// while a matrix of long rows, where every chunk leaves a carry, still has
+// its heads spread over many wavefronts.
+constexpr int kFixupChunks = 8;
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
-    int N, int64_t num_chunks, int n_tiles, int64_t blocks_per_tile,
-    const int *__restrict__ carry_row, const T *__restrict__ carry_val, T *__restrict__ C,
-    const T *__restrict__ bias) {
+    int N, int64_t num_chunks, const int *__restrict__ carry_row, const T *__restrict__ carry_val,
+    T *__restrict__ C, const T *__restrict__ bias) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   const int lane = wave_lane();
-  const TileMap where = map_workgroup(blockIdx.x, n_tiles, blocks_per_tile);
-  const int64_t chunk = where.block * kWavesPerBlock + threadIdx.x / kWaveSize;
-  if (chunk >= num_chunks) return;
-  // One coalesced load answers three questions: lane 0 holds the previous
-  // chunk's carry row, lane 1 this chunk's, lanes 2.. the following ones.
-  const int64_t first_probe = chunk - 1 + lane;
-  const int seen = (first_probe >= 0 && first_probe < num_chunks) ? carry_row[first_probe] : -2;
-  const int row = __builtin_amdgcn_readlane(seen, 1);
-  if (row < 0) return;
-  if (__builtin_amdgcn_readlane(seen, 0) == row) return;  // not the head of its run
-  // End of the run: 62 entries are already here, then 64 per step.
-  const unsigned long long differs = ~(__ballot(lane >= 2 && seen == row) | 3ull);
-  const int matched = differs ? __ffsll(differs) - 3 : kWaveSize - 2;
-  int64_t end = chunk + 1 + matched;
-  if (matched == kWaveSize - 2) {
-    for (;;) {
-      const int64_t probe = end + lane;
-      const bool same = probe < num_chunks && carry_row[probe] == row;
-      const unsigned long long differs_here = ~__ballot(same);
-      const int run = differs_here ? __ffsll(differs_here) - 1 : kWaveSize;
-      end += run;
-      if (run < kWaveSize) break;
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  const int64_t c = wave * kFixupChunks + lane;
+  int row = -1, after = -1;
+  if (lane < kFixupChunks && c < num_chunks) {
+    row = carry_row[c];
+    after = c + 1 < num_chunks ? carry_row[c + 1] : -1;
+    if (row >= 0 && c > 0 && carry_row[c - 1] == row) row = -1;  // not the head of its run
+  }
+  unsigned long long pending = __ballot(row >= 0);
+  while (pending) {  // uniform over the wavefront
+    const int owner = __ffsll(pending) - 1;
+    pending &= pending - 1;
+    const int r = __shfl(row, owner);
+    const int64_t start = c - lane + owner;
+    // a run of one, the usual case, needs no search
+    const int64_t end = __shfl(after, owner) != r ? start + 1 : carry_run_end(carry_row, start, num_chunks, r);
+    for (int col0 = lane * VEC; col0 < N; col0 += kWaveSize * VEC) {
+      VecT *dst = reinterpret_cast<VecT *>(C + (size_t)r * (size_t)N + col0);
+      VecT o = *dst;  // issued before the carries so that both are in flight together
+      A sum[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) sum[v] = (A)0;
+      int64_t e = start;
+      constexpr int kBatch = 32;  // loads in flight: a long row spans hundreds of chunks
+      for (; e + kBatch <= end; e += kBatch) {
+        VecT part[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+          part[u] = *reinterpret_cast<const VecT *>(carry_val + (size_t)(e + u) * (size_t)N + col0);
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) sum[v] += (A)part[u].v[v];
+      }
+      for (; e < end; ++e) {
+        const VecT part = *reinterpret_cast<const VecT *>(carry_val + (size_t)e * (size_t)N + col0);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) sum[v] += (A)part.v[v];
+      }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        const T b = EPI != kEpiNone ? bias[col0 + v] : (T)0;
+        o.v[v] = apply_epilogue<T, EPI>(sum[v] + (A)o.v[v], b);
+      }
+      *dst = o;
     }
   }
-  const int col0 = (where.tile * kWaveSize + lane) * VEC;
-  if (col0 >= N) return;
-
-  VecT *dst = reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0);
-  VecT o = *dst;  // issued before the carries so that both are in flight together
-
-  A sum[VEC];
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) sum[v] = (A)0;
-  int64_t c = chunk;
-  constexpr int kBatch = 32;  // loads in flight: a long row spans hundreds of chunks
-  for (; c + kBatch <= end; c += kBatch) {
-    VecT part[kBatch];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-      part[u] = *reinterpret_cast<const VecT *>(carry_val + (size_t)(c + u) * (size_t)N + col0);
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) sum[v] += (A)part[u].v[v];
-  }
-  for (; c < end; ++c) {
-    const VecT part = *reinterpret_cast<const VecT *>(carry_val + (size_t)c * (size_t)N + col0);
-#pragma unroll
-    for (int v = 0; v < VEC; ++v) sum[v] += (A)part.v[v];
-  }
-
-#pragma unroll
-  for (int v = 0; v < VEC; ++v) {
-    const T b = EPI != kEpiNone ? bias[col0 + v] : (T)0;
-    o.v[v] = apply_epilogue<T, EPI>(sum[v] + (A)o.v[v], b);
-  }
-  *dst = o;
 }
 
 // ---- host side ----------------------------------------------------------------
 
-// Shape of the work split.  A chunk holds up to 256 merge items (what the LDS
-// slices hold); a wavefront walks chunks_per_wave consecutive chunks and leaves
-// one carry.  Small problems use smaller chunks, so that they are spread over
-// more, shorter wavefronts.
+// Shape of the work split.  A chunk holds nominally up to 256 merge items, one
+// chunk per wavefront; small problems use smaller chunks, so that they are
+// spread over more, shorter wavefronts.  (A wavefront that walked two or more
+// consecutive chunks with one carry for all of them was measured: the same
+// time on a graph with uniform neighbours, slower -- 0.81 against 0.69 ms on the
+// 4,096-neighbour graph -- where neighbouring rows share columns, because an XCD
+// then has a wider stretch of rows in flight than its L2 covers.)
 struct SpmmSplit {
   int items_per_chunk;
-  int chunks_per_wave;
-  int64_t spans;  // wavefronts with work = carry records
+  int snap;        // see chunk_boundary
+  int64_t spans;   // chunks = wavefronts with work = carry records
 };
 
 inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
@@ -442,14 +472,8 @@ inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   sp.items_per_chunk = kMinItemsPerWave;
   while (sp.items_per_chunk < kItemsPerWave && sp.items_per_chunk * 2 <= per_wave)
     sp.items_per_chunk *= 2;
-  // One chunk per wavefront.  (The kernel can walk several consecutive chunks and
-  // leave one carry for all of them; that halves the carries the fix-up folds but
-  // widens the stretch of rows an XCD has in flight, which costs more in L2 hits on
-  // matrices whose neighbouring rows share columns -- 0.81 against 0.69 ms with two
-  // chunks on the 4,096-neighbour graph -- than it saves: nothing on the headline graph.)
-  sp.chunks_per_wave = 1;
-  const int64_t span_items = (int64_t)sp.items_per_chunk * sp.chunks_per_wave;
-  sp.spans = (total + span_items - 1) / span_items;
+  sp.snap = sp.items_per_chunk < kSnapItems ? sp.items_per_chunk : kSnapItems;
+  sp.spans = (total + sp.items_per_chunk - 1) / sp.items_per_chunk;
   return sp;
 }
 
@@ -504,11 +528,12 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
-      split.chunks_per_wave, n_tiles, blocks_per_tile, carry_row, carry_val);
+      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
-  spmm_fixup_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
-      N, chunks, n_tiles, blocks_per_tile, carry_row, carry_val, C, bias);
+  const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
+  spmm_fixup_kernel<T, VEC, EPI><<<dim3((unsigned)((chunks + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
+                                   stream>>>(N, chunks, carry_row, carry_val, C, bias);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
   return SCORCH_HIP_OK;
@@ -543,12 +568,12 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
   spmm_grouped_kernel<T, VEC, LPR, EPI><<<dim3((unsigned)(blocks_per_tile * n_tiles)), kBlockThreads, 0, stream>>>(
-      M, N, row_ptr, col_idx, vals, B, C, bias, total, ipc, n_tiles, blocks_per_tile, carry_row,
-      carry_val);
+      M, N, row_ptr, col_idx, vals, B, C, bias, total, ipc, ipc < kSnapItems ? ipc : kSnapItems, n_tiles,
+      blocks_per_tile, carry_row, carry_val);
   SCORCH_HIP_CHECK(hipGetLastError());
-  const int fix_tiles = (N + kWaveSize - 1) / kWaveSize;
-  spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)(blocks_per_tile * fix_tiles)), kBlockThreads, 0, stream>>>(
-      N, spans, fix_tiles, blocks_per_tile, carry_row, carry_val, C, bias);
+  const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
+  spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((spans + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
+                                 stream>>>(N, spans, carry_row, carry_val, C, bias);
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }
@@ -791,20 +816,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_fixup_kernel(int64_t spans
     pending &= pending - 1;
     const int64_t start = c - lane + owner;
     const int r = __shfl(row, owner);
-    // End of the run by a 64-way search: its members are consecutive, so "same row"
-    // holds up to the end and nowhere after.  `last` is a known member, `stop` the
-    // first position known to lie beyond (or the end of the list).
-    int64_t last = start, stop = spans;
-    while (stop - last > 1) {
-      const int64_t step = (stop - last + kWaveSize) / (kWaveSize + 1);
-      const int64_t probe = last + (int64_t)(lane + 1) * step;
-      const bool same = probe < stop && carry_row[probe] == r;
-      const int members = __popcll(__ballot(same));  // lanes 0 .. members - 1
-      const int64_t reached = last + (int64_t)members * step;
-      if (members < kWaveSize && reached + step < stop) stop = reached + step;  // lane `members` saw the end
-      last = reached;
-    }
-    const int64_t end = last + 1;
+    const int64_t end = carry_run_end(carry_row, start, spans, r);
     A part = (A)0;
     for (int64_t e = start + lane; e < end; e += kWaveSize) part += (A)carry_val[e];
 #pragma unroll
