@@ -27,12 +27,12 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
 WORKLOAD = "gcn_powerlaw_spmm_fp32"
 
 # Bytes through the L2-to-fabric boundary per launch of the dominant kernel at
-# the headline size: FETCH_SIZE (4,293,887 KiB x 2.0, the factor a 1 GiB copy
-# kernel gives for this counter) + WRITE_SIZE (557,973 KiB x 1.0) from two
+# the headline size: FETCH_SIZE (4,292,650 KiB x 2.0, the factor a 1 GiB copy
+# kernel gives for this counter) + WRITE_SIZE (539,816 KiB x 1.0) from two
 # rocprofv3 --pmc runs of this script.  It is a measured constant, valid for
 # the default workload only; the summary with the commands is
 # profiles/spmm_merge_kernel_gcn_powerlaw.md.
-MEASURED_TRAFFIC_BYTES = 9_365_165_000
+MEASURED_TRAFFIC_BYTES = 9_344_118_000
 
 
 def algorithmic_bytes(M, K, N, nnz):
