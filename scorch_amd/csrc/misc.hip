@@ -26,8 +26,8 @@ char *error_buffer() {
 // caller's workspace (one atomic per workgroup that has any), and
 // softmax_csr_giant_kernel then deals them out, one row at a time, to
 // workgroups of 1024 threads (the first 8192 entries in registers, the rest
-// re-read from cache; the next row's entries are requested before the current
-// row's phases start): however such rows are placed in the matrix, few among
+// read twice: a running maximum and sum first, the write second; the next
+// row's entries are requested before the current row's phases start): however such rows are placed in the matrix, few among
 // many short ones or all of them long, they are spread over the whole chip.
 // Values are loaded raw and scaled at their first use, so that a row's loads
 // are all issued before any of them is waited for.
@@ -64,7 +64,7 @@ __device__ __forceinline__ void softmax_load(int lo, int hi, int t, const float 
 
 // ... and the three phases on them; `reduce(value, take_max)` combines a value
 // over the team.  TAIL: the row may be longer than the registers hold; the
-// rest is read again in every phase.
+// rest is read once for maximum and sum together and once more for the write.
 template <int TEAM, int REGS, bool TAIL, typename Reduce>
 __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const float *vals, float scale,
                                                float *out, float (&v)[REGS], Reduce reduce) {
@@ -75,20 +75,27 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
     mx = fmaxf(mx, v[u]);
   }
   const int rest = lo + REGS * TEAM + t;  // this thread's first entry beyond the registers
+  // The entries beyond the registers are read twice, not three times: the first
+  // sweep keeps a running maximum and the sum of exponentials relative to it
+  // (rescaled whenever the maximum moves: one exponential per entry either way).
+  float tail_max = mx, tail_sum = 0.0f;
   if (TAIL) {
 #pragma unroll 8
-    for (int p = rest; p < hi; p += TEAM) mx = fmaxf(mx, vals[p] * scale);
+    for (int p = rest; p < hi; p += TEAM) {
+      const float x = vals[p] * scale;
+      const float e = expf(-fabsf(x - tail_max));
+      const bool higher = x > tail_max;
+      tail_sum = higher ? tail_sum * e + 1.0f : tail_sum + e;
+      tail_max = higher ? x : tail_max;
+    }
+    mx = tail_max;
   }
   mx = reduce(mx, true);
-  float sum = 0.0f;
+  float sum = TAIL ? tail_sum * expf(tail_max - mx) : 0.0f;
 #pragma unroll
   for (int u = 0; u < REGS; ++u) {
     v[u] = lo + t + u * TEAM < hi ? expf(v[u] - mx) : 0.0f;
     sum += v[u];
-  }
-  if (TAIL) {
-#pragma unroll 8
-    for (int p = rest; p < hi; p += TEAM) sum += expf(vals[p] * scale - mx);
   }
   sum = reduce(sum, false);
 #pragma unroll
