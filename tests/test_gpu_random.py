@@ -91,6 +91,68 @@ def test_spgemm_random(oracle, seed):
                                    atol=1e-3 if dtype == np.float32 else 1e-10)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_spgemm_random_many_short_rows(oracle, seed):
+    """More than 32,768 rows, so that wavefronts take four rows each (quarters for rows of at most
+    32 products); mixes of empty, tiny and a few long rows, operands of different shapes."""
+    rng = np.random.default_rng(4000 + seed)
+    M = int(rng.integers(33_000, 60_000))
+    K, N = int(rng.integers(50, 3000)), int(rng.integers(50, 5000))
+    dtype = DTYPES[seed % 4]
+    a_lens = rng.choice([0, 1, 2, 3, 5, 9], size=M, p=[0.2, 0.3, 0.2, 0.15, 0.1, 0.05])
+    a_lens[rng.integers(0, M, 30)] = rng.integers(10, min(K, 200), 30)
+    a_lens = np.minimum(a_lens, K)
+    arp = np.concatenate([[0], np.cumsum(a_lens)]).astype(np.int32)
+    aci = np.concatenate([np.sort(rng.choice(K, int(n), replace=False)) for n in a_lens if n] or
+                         [np.zeros(0, np.int64)]).astype(np.int32)
+    av = draw_dense(rng, aci.size, dtype)
+    brp, bci, bv = random_csr(rng, K, N, float(rng.choice([0.002, 0.01, 0.05])), dtype=dtype)
+    rp, ci, v = hip_spgemm(arp, aci, av, brp, bci, bv, N)
+    wrp, wci, wv = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, N)
+    assert np.array_equal(rp, wrp) and np.array_equal(ci, wci)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(v, wv)
+    else:
+        _, _, ref64 = oracle.spgemm_csr_typed(arp, aci, av.astype(np.float64), brp, bci, bv.astype(np.float64), N)
+        assert oracle.rel_fro(v, ref64) <= (1e-5 if dtype == np.float32 else 1e-13)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_coordinate_products_random(oracle, seed):
+    """spmm_coo_float and spmspm_coo_float on shuffled, partly repeated coordinates."""
+    import torch
+    from gpu_util import dev, host
+    from scorch_amd import scorch_ops_hip as H
+    rng = np.random.default_rng(5000 + seed)
+    M, K, N = int(rng.integers(1, 300)), int(rng.integers(1, 300)), int(rng.integers(1, 200))
+    arp, aci, av = random_csr(rng, M, K, draw_density(rng, K))
+    ar = np.repeat(np.arange(M, dtype=np.int32), np.diff(arp))
+    if seed % 2:  # any order, some entries twice
+        pick = np.concatenate([rng.permutation(ar.size), rng.integers(0, max(ar.size, 1), ar.size // 3)]) \
+            if ar.size else np.zeros(0, np.int64)
+        ar, aci, av = ar[pick], aci[pick], av[pick]
+    B = draw_dense(rng, (K, N), np.float32)
+    got = host(H.spmm_coo_float([M, N], [M, K], [[dev(ar)], [dev(aci)]], dev(av), [K, N], [[], []],
+                                dev(B).reshape(-1)).storage.value).reshape(M, N)
+    dense_a = np.zeros((M, K))
+    np.add.at(dense_a, (ar, aci), av.astype(np.float64))
+    ref = dense_a @ B.astype(np.float64)
+    assert oracle.rel_fro(got, ref) <= 1e-5
+    brp, bci, bv = random_csr(rng, K, N, draw_density(rng, N))
+    br = np.repeat(np.arange(K, dtype=np.int32), np.diff(brp))
+    shuffle = rng.permutation(br.size)
+    out = H.spmspm_coo_float([M, N], [M, K], [[dev(ar)], [dev(aci)]], dev(av), [K, N],
+                             [[dev(br[shuffle])], [dev(bci[shuffle])]], dev(bv[shuffle]))
+    r, c = (host(level[0]) for level in out.storage.index.mode_indices)
+    dense_b = np.zeros((K, N))
+    dense_b[br, bci] = bv
+    full = dense_a @ dense_b
+    structure = (np.abs(dense_a) > 0).astype(np.float64) @ (np.abs(dense_b) > 0)
+    wr, wc = np.nonzero(structure)                                # every structural entry, row-major
+    assert np.array_equal(r, wr.astype(np.int32)) and np.array_equal(c, wc.astype(np.int32))
+    assert oracle.rel_fro(host(out.storage.value), full[wr, wc]) <= 1e-5
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_softmax_random(oracle, seed):
     """Row lengths from a heavy-tailed draw (so that every tier of the kernel and
