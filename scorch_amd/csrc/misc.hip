@@ -32,6 +32,9 @@ char *error_buffer() {
 // Values are loaded raw and scaled at their first use, so that a row's loads
 // are all issued before any of them is waited for.
 constexpr int kSoftmaxRegs = 4;
+// rows a lane group of G lanes has in flight (whole wavefronts take fewer: their
+// workgroup's rows are long, and what the later tiers take they take one after the other)
+constexpr int softmax_team_rows(int G) { return G == kWaveSize ? 2 : 4; }
 constexpr int kSoftmaxBlockRegs = 16;
 constexpr int kSoftmaxGiantRegs = 8;
 constexpr int kSoftmaxQuarter = kWaveSize / 4;
@@ -133,7 +136,13 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                                     const float *vals, float scale,
                                                                     float *out, int *giant_count,
                                                                     int *__restrict__ giant_rows) {
-  constexpr int kRows = kBlockThreads / G;  // rows per workgroup
+  // A lane group takes kTeamRows rows, one from each block of 256 / G consecutive rows
+  // the workgroup owns, and requests the entries of all of them before it works on the
+  // first: these rows are short, and with one row in flight per group the kernel waits on
+  // memory latency rather than bandwidth.
+  constexpr int kGroups = kBlockThreads / G;
+  constexpr int kTeamRows = softmax_team_rows(G);
+  constexpr int kRows = kGroups * kTeamRows;  // rows per workgroup
   __shared__ float s_red[kWavesPerBlock];
   __shared__ int s_lo[kRows], s_hi[kRows];
   // row slots left to the quarter wavefronts [0], the wavefronts [1] and the workgroup [2];
@@ -143,27 +152,36 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   __shared__ int s_giant_base;
   if (threadIdx.x < 4) s_count[threadIdx.x] = 0;
   __syncthreads();
-  const int slot = threadIdx.x / G;
   const int t = threadIdx.x % G;
-  const int64_t row = (int64_t)blockIdx.x * kRows + slot;
-  int lo = 0, hi = 0;
-  if (row < M) {
-    lo = row_ptr[row];
-    hi = row_ptr[row + 1];
-  }
-  const int len = hi - lo;
-  if (len > G * kSoftmaxRegs) {
-    if (t == 0 && len <= kSoftmaxBlockRowMax) {
-      const int tier = len > kSoftmaxWaveRowMax ? 2 : (len > kSoftmaxQuarterRowMax || G >= kSoftmaxQuarter);
-      s_lo[slot] = lo;
-      s_hi[slot] = hi;
-      s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
-    } else if (t == 0) {
-      s_list[3][atomicAdd(&s_count[3], 1)] = (int)row;
+  int lo[kTeamRows], hi[kTeamRows];
+#pragma unroll
+  for (int j = 0; j < kTeamRows; ++j) {
+    const int slot = j * kGroups + threadIdx.x / G;
+    const int64_t row = (int64_t)blockIdx.x * kRows + slot;
+    lo[j] = hi[j] = 0;
+    if (row < M) {
+      lo[j] = row_ptr[row];
+      hi[j] = row_ptr[row + 1];
     }
-    hi = lo;
+    const int len = hi[j] - lo[j];
+    if (len > G * kSoftmaxRegs) {
+      if (t == 0 && len <= kSoftmaxBlockRowMax) {
+        const int tier = len > kSoftmaxWaveRowMax ? 2 : (len > kSoftmaxQuarterRowMax || G >= kSoftmaxQuarter);
+        s_lo[slot] = lo[j];
+        s_hi[slot] = hi[j];
+        s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
+      } else if (t == 0) {
+        s_list[3][atomicAdd(&s_count[3], 1)] = (int)row;
+      }
+      hi[j] = lo[j];
+    }
   }
-  softmax_row<G, kSoftmaxRegs, false>(lo, hi, t, vals, scale, out, softmax_shuffle_reduce<G>);
+  float v[kTeamRows][kSoftmaxRegs];
+#pragma unroll
+  for (int j = 0; j < kTeamRows; ++j) softmax_load<G, kSoftmaxRegs>(lo[j], hi[j], t, vals, v[j]);
+#pragma unroll
+  for (int j = 0; j < kTeamRows; ++j)
+    softmax_finish<G, kSoftmaxRegs, false>(lo[j], hi[j], t, vals, scale, out, v[j], softmax_shuffle_reduce<G>);
   __syncthreads();
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
@@ -171,7 +189,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   if (n_giant > 0) {  // uniform over the workgroup; rows are independent, so the list's order is free
     if (threadIdx.x == 0) s_giant_base = atomicAdd(giant_count, n_giant);
     __syncthreads();
-    if ((int)threadIdx.x < n_giant) giant_rows[s_giant_base + threadIdx.x] = s_list[3][threadIdx.x];
+    for (int i = threadIdx.x; i < n_giant; i += kBlockThreads) giant_rows[s_giant_base + i] = s_list[3][i];
   }
   if (G < kSoftmaxQuarter) {
     constexpr int kTeams = kBlockThreads / kSoftmaxQuarter;
@@ -358,7 +376,7 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
     SCORCH_HIP_CHECK(hipGetLastError());
   }
   const int g = scorch::softmax_group_width(M, nnz);
-  const int64_t rows_per_block = scorch::kBlockThreads / g;
+  const int64_t rows_per_block = scorch::kBlockThreads / g * scorch::softmax_team_rows(g);
   const dim3 grid((unsigned)((M + rows_per_block - 1) / rows_per_block));
   const int m = (int)M;
 #define SCORCH_SOFTMAX(G)                                                                               \

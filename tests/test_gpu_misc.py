@@ -104,6 +104,20 @@ def test_softmax_many_long_rows(oracle, n_rows, length):
     np.testing.assert_allclose(got.reshape(n_rows, length).sum(axis=1), 1.0, rtol=1e-5)
 
 
+def test_softmax_long_rows_among_very_short_ones(oracle):
+    """A mean row length of two (lane groups of two, 512 rows to a workgroup) with every row of
+    one stretch far beyond the workgroup tier: more listed rows in one workgroup than it has threads."""
+    rng = np.random.default_rng(12)
+    lens = np.full(700_000, 1, np.int64)
+    lens[1024:1024 + 300] = 4100 + rng.integers(0, 50, 300)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    vals = (rng.standard_normal(int(rp[-1])) * 2).astype(np.float32)
+    got = host(H.softmax_csr_float(dev(rp), dev(vals), 1.0))
+    want = oracle.softmax_csr_f32(rp, vals, 1.0)
+    assert oracle.rel_fro(got, want.astype(np.float64)) <= TOL
+    assert np.all(got[:1024] == 1.0)
+
+
 def test_softmax_in_place(oracle):
     """out may alias vals, also for rows that are re-read and for prefetched ones"""
     lens = np.array([3, 9000, 5000, 12, 20000, 300, 4500, 0, 70], np.int64)
