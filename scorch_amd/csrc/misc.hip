@@ -20,6 +20,7 @@ char *error_buffer() {
 //                                    (only when G < 16);
 //   up to kSoftmaxRegs * 64 entries  one wavefront per row, the workgroup's four
 //                                    wavefronts sharing those rows out;
+//   up to 1024 entries               the same with sixteen entries per lane;
 //   up to 4096 entries               the whole workgroup, one row after the other.
 // In all of these a row sits in registers between the phases and is read from
 // memory once.  Rows beyond 4096 entries are only noted, in a list in the
@@ -40,6 +41,7 @@ constexpr int kSoftmaxGiantRegs = 8;
 constexpr int kSoftmaxQuarter = kWaveSize / 4;
 constexpr int kSoftmaxQuarterRowMax = kSoftmaxRegs * kSoftmaxQuarter;
 constexpr int kSoftmaxWaveRowMax = kSoftmaxRegs * kWaveSize;
+constexpr int kSoftmaxLongWaveRowMax = kSoftmaxBlockRegs * kWaveSize;
 constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
 constexpr int kSoftmaxGiantThreads = 1024;
 constexpr int kSoftmaxGiantBlocks = 1024;  // most workgroups the giant-row kernel starts
@@ -145,12 +147,12 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   constexpr int kRows = kGroups * kTeamRows;  // rows per workgroup
   __shared__ float s_red[kWavesPerBlock];
   __shared__ int s_lo[kRows], s_hi[kRows];
-  // row slots left to the quarter wavefronts [0], the wavefronts [1] and the workgroup [2];
-  // [3]: rows left to the giant-row kernel
-  __shared__ int s_list[4][kRows];
-  __shared__ int s_count[4];
+  // row slots left to the quarter wavefronts [0], the wavefronts with few [1] and with many
+  // [2] entries per lane, and the workgroup [3]; [4]: rows left to the giant-row kernel
+  __shared__ int s_list[5][kRows];
+  __shared__ int s_count[5];
   __shared__ int s_giant_base;
-  if (threadIdx.x < 4) s_count[threadIdx.x] = 0;
+  if (threadIdx.x < 5) s_count[threadIdx.x] = 0;
   __syncthreads();
   const int t = threadIdx.x % G;
   int lo[kTeamRows], hi[kTeamRows];
@@ -166,12 +168,14 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
     const int len = hi[j] - lo[j];
     if (len > G * kSoftmaxRegs) {
       if (t == 0 && len <= kSoftmaxBlockRowMax) {
-        const int tier = len > kSoftmaxWaveRowMax ? 2 : (len > kSoftmaxQuarterRowMax || G >= kSoftmaxQuarter);
+        const int tier = len > kSoftmaxLongWaveRowMax ? 3
+                         : len > kSoftmaxWaveRowMax   ? 2
+                                                      : (len > kSoftmaxQuarterRowMax || G >= kSoftmaxQuarter);
         s_lo[slot] = lo[j];
         s_hi[slot] = hi[j];
         s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
       } else if (t == 0) {
-        s_list[3][atomicAdd(&s_count[3], 1)] = (int)row;
+        s_list[4][atomicAdd(&s_count[4], 1)] = (int)row;
       }
       hi[j] = lo[j];
     }
@@ -185,11 +189,12 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   __syncthreads();
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
-  const int n_quarter = s_count[0], n_wave = s_count[1], n_block = s_count[2], n_giant = s_count[3];
+  const int n_quarter = s_count[0], n_wave = s_count[1], n_long_wave = s_count[2], n_block = s_count[3],
+            n_giant = s_count[4];
   if (n_giant > 0) {  // uniform over the workgroup; rows are independent, so the list's order is free
     if (threadIdx.x == 0) s_giant_base = atomicAdd(giant_count, n_giant);
     __syncthreads();
-    for (int i = threadIdx.x; i < n_giant; i += kBlockThreads) giant_rows[s_giant_base + i] = s_list[3][i];
+    for (int i = threadIdx.x; i < n_giant; i += kBlockThreads) giant_rows[s_giant_base + i] = s_list[4][i];
   }
   if (G < kSoftmaxQuarter) {
     constexpr int kTeams = kBlockThreads / kSoftmaxQuarter;
@@ -212,8 +217,15 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                   softmax_shuffle_reduce<kWaveSize>);
     }
   }
-  for (int i = 0; i < n_block; ++i) {  // uniform over the workgroup
+  // up to 1024 entries: still one wavefront per row, sixteen entries per lane, so that the four
+  // wavefronts work on four such rows at once and need no barriers
+  for (int i = w; i < n_long_wave; i += kWavesPerBlock) {
     const int k = s_list[2][i];
+    softmax_row<kWaveSize, kSoftmaxBlockRegs, false>(s_lo[k], s_hi[k], lane, vals, scale, out,
+                                                     softmax_shuffle_reduce<kWaveSize>);
+  }
+  for (int i = 0; i < n_block; ++i) {  // uniform over the workgroup
+    const int k = s_list[3][i];
     softmax_row<kBlockThreads, kSoftmaxBlockRegs, false>(
         s_lo[k], s_hi[k], (int)threadIdx.x, vals, scale, out, [&](float v, bool take_max) {
           v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts

@@ -59,8 +59,8 @@ def test_softmax_every_row_length_tier(oracle):
     """Row lengths chosen around each hand-over of the kernel: lane groups, quarter
     wavefronts, wavefronts, the workgroup (up to 4096 entries) and the giant-row
     kernel (first 8192 entries in registers, the rest re-read)."""
-    lens = np.array([0, 1, 7, 8, 9, 16, 17, 63, 64, 65, 255, 256, 257, 0, 2047, 2048, 2049, 3, 4095, 4096,
-                     4097, 8191, 8192, 8193, 20000, 5, 0], np.int64)
+    lens = np.array([0, 1, 7, 8, 9, 16, 17, 63, 64, 65, 255, 256, 257, 0, 1023, 1024, 1025, 2047, 2048, 2049, 3,
+                     4095, 4096, 4097, 8191, 8192, 8193, 20000, 5, 0], np.int64)
     rng = np.random.default_rng(3)
     for mean_pad in (0, 400):  # few short rows -> narrow groups; many -> group width follows the mean
         all_lens = np.concatenate([lens, np.full(mean_pad, 2, np.int64)])
