@@ -378,14 +378,14 @@ constexpr int kMicroTeam = 16;
 constexpr int kMicroProducts = 32;
 constexpr int kMicroSlots = 64;
 
-// What TEAMS teams keep in LDS for their rows: the hash table, the compacted
-// entries and the batch of A entries being walked.
+// What TEAMS teams keep in LDS for their rows: the hash table (its occupied slots
+// are later compacted to the front of the same arrays: less LDS, more wavefronts
+// per CU, and these rows are bound by how many are in flight) and the batch of A
+// entries being walked.
 template <typename A, bool NUMERIC, int TEAM, int TEAMS, int SLOTS, int PRODUCTS>
 struct TeamTables {
   int keys[TEAMS][SLOTS];
   A vals[TEAMS][NUMERIC ? SLOTS : 1];
-  int ck[TEAMS][NUMERIC ? PRODUCTS : 1];
-  A cv[TEAMS][NUMERIC ? PRODUCTS : 1];
   ProductBatch<TEAM, A> batch[TEAMS];
 };
 
@@ -415,16 +415,23 @@ __device__ __forceinline__ void spgemm_team_row(
       });
   wave_lds_sync();
 
-  // Count the occupied slots; in the numeric pass, also compact them.
+  // Count the occupied slots; in the numeric pass, also compact them, in place: a
+  // step's TEAM slots are read by all lanes before any is written, and entry
+  // number `at` never lies beyond the slot it came from.
   int n = 0;
   for (int base = 0; base < SLOTS; base += TEAM) {
     const int key = lds.keys[team][base + t];
+    A val = (A)0;
+    if (NUMERIC) val = lds.vals[team][base + t];
     unsigned long long occupied = __ballot(key != -1) >> (lane - t);  // the team's lanes from bit 0
     if (TEAM < kWaveSize) occupied &= (1ull << (TEAM % kWaveSize)) - 1ull;
-    if (NUMERIC && key != -1) {
-      const int at = n + __popcll(occupied & ((1ull << t) - 1ull));
-      lds.ck[team][at] = key;
-      lds.cv[team][at] = lds.vals[team][base + t];
+    if (NUMERIC) {
+      wave_lds_sync();  // everyone has read this step's slots
+      if (key != -1) {
+        const int at = n + __popcll(occupied & ((1ull << t) - 1ull));
+        lds.keys[team][at] = key;
+        lds.vals[team][at] = val;
+      }
     }
     n += __popcll(occupied);
   }
@@ -437,11 +444,11 @@ __device__ __forceinline__ void spgemm_team_row(
   // Rank = number of smaller keys (keys are distinct): the sorted position.
   const int out = c_pos[row];
   for (int e = t; e < n; e += TEAM) {
-    const int key = lds.ck[team][e];
+    const int key = lds.keys[team][e];
     int rank = 0;
-    for (int x = 0; x < n; ++x) rank += lds.ck[team][x] < key ? 1 : 0;
+    for (int x = 0; x < n; ++x) rank += lds.keys[team][x] < key ? 1 : 0;
     c_crd[out + rank] = key;
-    c_val[out + rank] = (T)lds.cv[team][e];
+    c_val[out + rank] = (T)lds.vals[team][e];
   }
 }
 
