@@ -189,6 +189,39 @@ __device__ __forceinline__ int team_exclusive_scan(int v, int *scratch, int &tot
   return incl - v;
 }
 
+constexpr int kProductsInFlight = 4;
+
+// One step of the walk over a batch's products: products x0, x0 + TEAM, ... (U of
+// them) of this thread.  Their bisections interleave and their loads from B are all
+// issued before the first is used; a step of one product waits out a whole memory
+// round trip for it.  PARTIAL: the batch may end within the step; slots beyond its
+// last product read that product again and hand nothing to fn.
+template <int TEAM, bool NUMERIC, int U, bool PARTIAL, typename T, typename A, typename Fn>
+__device__ __forceinline__ void product_step(int x0, int total, const int *__restrict__ b_crd,
+                                             const T *__restrict__ b_val,
+                                             const ProductBatch<TEAM, A> &batch, Fn &fn) {
+  int q[U], e[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int x = PARTIAL ? min(x0 + u * TEAM, total - 1) : x0 + u * TEAM;
+    e[u] = 0;  // the last entry whose offset is <= x (entries without products share an offset)
+#pragma unroll
+    for (int step = TEAM / 2; step > 0; step >>= 1)
+      if (batch.off[e[u] + step] <= x) e[u] += step;
+    q[u] = batch.b_lo[e[u]] + (x - batch.off[e[u]]);
+  }
+  int col[U];
+  A b[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    col[u] = b_crd[q[u]];
+    b[u] = NUMERIC ? (A)b_val[q[u]] : (A)0;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (!PARTIAL || x0 + u * TEAM < total) fn(col[u], NUMERIC ? batch.a_val[e[u]] * b[u] : (A)0);
+}
+
 // fn(column, product) for every product of A entries [a_lo, a_hi); `t` is the
 // thread's number in the team.  Uniform over the team.
 template <int TEAM, bool NUMERIC, typename T, typename A, typename Fn>
@@ -196,6 +229,7 @@ __device__ __forceinline__ void for_each_product(int a_lo, int a_hi, int t, cons
                                                  const T *__restrict__ a_val, const int *__restrict__ b_pos,
                                                  const int *__restrict__ b_crd, const T *__restrict__ b_val,
                                                  ProductBatch<TEAM, A> &batch, int *scan_scratch, Fn fn) {
+  constexpr int U = kProductsInFlight;
   for (int base = a_lo; base < a_hi; base += TEAM) {
     const int p = base + t;
     int lo = 0, len = 0;
@@ -213,15 +247,13 @@ __device__ __forceinline__ void for_each_product(int a_lo, int a_hi, int t, cons
     batch.b_lo[t] = lo;
     if (NUMERIC) batch.a_val[t] = av;
     team_sync<TEAM>();
-#pragma unroll 8
-    for (int x = t; x < total; x += TEAM) {
-      int e = 0;  // the last entry whose offset is <= x (entries without products share an offset)
-#pragma unroll
-      for (int step = TEAM / 2; step > 0; step >>= 1)
-        if (batch.off[e + step] <= x) e += step;
-      const int q = batch.b_lo[e] + (x - batch.off[e]);
-      fn(b_crd[q], NUMERIC ? batch.a_val[e] * (A)b_val[q] : (A)0);
-    }
+    int x = 0;  // the team's first product of the step
+    for (; x + U * TEAM <= total; x += U * TEAM)
+      product_step<TEAM, NUMERIC, U, false, T, A>(x + t, total, b_crd, b_val, batch, fn);
+    if (x + TEAM < total)  // more than one product a thread is left
+      product_step<TEAM, NUMERIC, U, true, T, A>(x + t, total, b_crd, b_val, batch, fn);
+    else if (x + t < total)
+      product_step<TEAM, NUMERIC, 1, false, T, A>(x + t, total, b_crd, b_val, batch, fn);
   }
 }
 
