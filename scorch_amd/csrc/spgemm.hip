@@ -314,6 +314,11 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
 // waiting on a long dependent chain.  The three row lists are gathered in LDS
 // first and appended to the global lists with one atomic per list and
 // workgroup: thousands of atomics on one counter would serialise in the L2.
+// Rows beyond kMediumProducts products come in two classes: the workgroups that
+// take them get them one at a time from a counter, and the longest rows decide
+// when that kernel ends, so those of at least kGiantProducts are listed apart
+// (from the back of the same array) and handed out first.
+constexpr int kGiantProducts = 16384;
 constexpr int kBoundsLongRow = 64;
 constexpr int kBoundsRows = 256;
 
@@ -324,16 +329,17 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
   constexpr int G = 8;  // lanes per row
   constexpr int kStep = kBlockThreads / G;
   __shared__ int s_long[kBoundsRows];
-  __shared__ int s_list[3][kBoundsRows];  // counters' order: medium, huge, small
-  __shared__ int s_n[4];                  // [3]: long rows queued
-  __shared__ int s_base[3];
+  __shared__ int s_list[4][kBoundsRows];  // medium, huge, small, giant
+  __shared__ int s_n[5];                  // [4]: long rows queued
+  __shared__ int s_base[4];
   __shared__ long long s_part[kWavesPerBlock];
-  if (threadIdx.x < 4) s_n[threadIdx.x] = 0;
+  if (threadIdx.x < 5) s_n[threadIdx.x] = 0;
   __syncthreads();
   auto file_row = [&](int row, long long sum) {
     const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
     products[row] = bound;
-    const int list = bound > kMediumProducts ? 1 : bound > kSmallProducts ? 0 : bound > kTinyProducts ? 2 : -1;
+    const int list = bound >= kGiantProducts ? 3 : bound > kMediumProducts ? 1 : bound > kSmallProducts ? 0
+                     : bound > kTinyProducts ? 2 : -1;
     if (list >= 0) s_list[list][atomicAdd(&s_n[list], 1)] = row;
   };
 
@@ -348,7 +354,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     }
     const bool is_long = hi - lo > kBoundsLongRow;
     if (is_long) {
-      if (t == 0) s_long[atomicAdd(&s_n[3], 1)] = (int)row;
+      if (t == 0) s_long[atomicAdd(&s_n[4], 1)] = (int)row;
       hi = lo;
     }
     long long sum = 0;
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
   }
   __syncthreads();
 
-  const int n_long = s_n[3];
+  const int n_long = s_n[4];
   for (int i = 0; i < n_long; ++i) {  // uniform over the workgroup
     const int r = s_long[i];
     long long part = 0;
@@ -383,16 +389,22 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     }
   }
   __syncthreads();
-  if (threadIdx.x < 3 && s_n[threadIdx.x] > 0)
-    s_base[threadIdx.x] = atomicAdd(&counters[threadIdx.x], s_n[threadIdx.x]);
+  if (threadIdx.x < 4 && s_n[threadIdx.x] > 0)
+    s_base[threadIdx.x] = atomicAdd(&counters[threadIdx.x < 3 ? threadIdx.x : 5], s_n[threadIdx.x]);
   __syncthreads();
   int *const lists[3] = {medium_rows, huge_rows, small_rows};
 #pragma unroll
   for (int l = 0; l < 3; ++l)
     for (int i = threadIdx.x; i < s_n[l]; i += kBlockThreads) lists[l][s_base[l] + i] = s_list[l][i];
+  for (int i = threadIdx.x; i < s_n[3]; i += kBlockThreads) huge_rows[M - 1 - (s_base[3] + i)] = s_list[3][i];
 }
 
-// counters: [0] medium rows, [1] huge rows, [2] small rows listed; [3], [4] next row to hand out
+// Entry `idx` of the rows beyond kMediumProducts products, the giant ones first.
+__device__ __forceinline__ int huge_row(const int *__restrict__ rows, int M, int n_giant, int idx) {
+  return idx < n_giant ? rows[M - 1 - idx] : rows[idx - n_giant];
+}
+
+// counters: [0] medium rows, [1] huge rows, [2] small rows, [5] giant rows listed; [3], [4] next row to hand out
 __global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
   if (threadIdx.x < 8) counters[threadIdx.x] = 0;
   if (threadIdx.x == 0 && c_pos_last) *c_pos_last = 0;
@@ -711,7 +723,7 @@ constexpr int kHugeEmitWords = 256;  // bitmap words emitted per step (at most 8
 
 template <typename T, bool NUMERIC>
 __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
-    int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    int M, int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, const int *__restrict__ counters, unsigned *__restrict__ bitmaps,
     int *__restrict__ ranks, int *__restrict__ c_pos, int *__restrict__ c_crd, T *__restrict__ c_val) {
@@ -720,7 +732,8 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
   __shared__ ProductBatch<kHugeThreads, A> s_batch;
   __shared__ int s_cols[NUMERIC ? kHugeEmitWords * 32 : 1];
   const int tid = threadIdx.x;
-  const int n_rows = counters[1];
+  const int n_giant = counters[5];
+  const int n_rows = counters[1] + n_giant;
   if ((int)blockIdx.x >= n_rows) return;
 
   const int words = (N + 31) / 32;
@@ -732,7 +745,7 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
   __syncthreads();
 
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
-    const int row = rows[idx];
+    const int row = huge_row(rows, M, n_giant, idx);
     const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
     for_each_product<kHugeThreads, false, T, A>(
         a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A) {
@@ -807,7 +820,7 @@ constexpr int kLdsBudget = 160 * 1024 - 1024;
 // LIST, WORK: which of `counters` holds the length of `rows` and the next row to hand out.
 template <typename T, bool NUMERIC, int WORDS, int THREADS, int ACC, int LIST, int WORK>
 __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
-    int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
+    int M, int N, const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, int *__restrict__ counters, int *__restrict__ c_pos,
     int *__restrict__ c_crd, T *__restrict__ c_val) {
@@ -823,7 +836,8 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   __shared__ int s_scan[kWaves];
   __shared__ int s_next;
   const int tid = threadIdx.x;
-  const int n_rows = counters[LIST];
+  const int n_giant = LIST == 1 ? counters[5] : 0;  // only the list of the longest rows has the class
+  const int n_rows = counters[LIST] + n_giant;
   constexpr int kRangeColumns = 32 * WORDS;
   A *acc = reinterpret_cast<A *>(c_val);
 
@@ -833,7 +847,7 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
     __syncthreads();
     const int idx = s_next;
     if (idx >= n_rows) return;  // the same for every thread
-    const int row = rows[idx];
+    const int row = LIST == 1 ? huge_row(rows, M, n_giant, idx) : rows[idx];
     const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
     const int out = NUMERIC ? c_pos[row] : 0;
     int done = 0;  // distinct columns found in the ranges before this one
@@ -991,7 +1005,7 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   if (N <= 32 * 4096) {
     // narrow enough for a bitmap in LDS beside other workgroups: no hashing, nothing to sort
     spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kBlockThreads, kMediumProducts, 0, 4>
-        <<<medium_blocks, kBlockThreads, 0, stream>>>(N, a_pos, a_crd, a_val, b_pos, b_crd, b_val,
+        <<<medium_blocks, kBlockThreads, 0, stream>>>(M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val,
                                                       ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   } else {
     spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
@@ -1002,13 +1016,13 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   const unsigned lds_pool = (unsigned)(M < 512 ? M : 512);
   if (N <= 32 * 4096)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
-        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
+        M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
   else if (N <= kLdsBitmapColumns)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 16384, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
-        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
+        M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
   else
     spgemm_huge_kernel<T, NUMERIC><<<ws.huge_pool, kHugeThreads, 0, stream>>>(
-        N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
+        M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, ws.bitmaps,
         ws.ranks, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (!NUMERIC) {
