@@ -308,10 +308,11 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
 }
 
 // ---- pass 0: products per row, and the lists of rows too big for a wavefront ----
-// A workgroup takes kBoundsRows consecutive rows, eight lanes per row; rows of A
-// with more than kBoundsLongRow entries are queued in LDS and summed by the whole
-// workgroup afterwards, so that a hub row does not leave its neighbours' lanes
-// waiting on a long dependent chain.  The three row lists are gathered in LDS
+// A workgroup takes up to kBoundsRows consecutive rows, eight lanes per row; rows
+// of A with more than kBoundsLongRow entries are queued in LDS and summed
+// afterwards, by a wavefront each or, beyond kBoundsWaveRow entries, by the whole
+// workgroup one after the other, so that a hub row does not leave its neighbours'
+// lanes waiting on a long dependent chain.  The three row lists are gathered in LDS
 // first and appended to the global lists with one atomic per list and
 // workgroup: thousands of atomics on one counter would serialise in the L2.
 // Rows beyond kMediumProducts products come in two classes: the workgroups that
@@ -320,20 +321,29 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
 // (from the back of the same array) and handed out first.
 constexpr int kGiantProducts = 16384;
 constexpr int kBoundsLongRow = 64;
+constexpr int kBoundsWaveRow = 2048;
 constexpr int kBoundsRows = 256;
 
+// Rows to a workgroup: fewer for matrices that would not fill the chip otherwise
+// (their rows tend to be the long ones, which a workgroup takes a few at a time).
+inline int bounds_rows_per_group(int64_t M) {
+  const int64_t rows = (M / 1024 + 31) / 32 * 32;
+  return (int)(rows < 32 ? 32 : rows > kBoundsRows ? kBoundsRows : rows);
+}
+
 __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
-    int M, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
+    int M, int rows_per_group, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
     const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ small_rows,
     int *__restrict__ medium_rows, int *__restrict__ huge_rows, int *__restrict__ counters) {
   constexpr int G = 8;  // lanes per row
   constexpr int kStep = kBlockThreads / G;
   __shared__ int s_long[kBoundsRows];
+  __shared__ int s_very_long[kBoundsRows];
   __shared__ int s_list[4][kBoundsRows];  // medium, huge, small, giant
-  __shared__ int s_n[5];                  // [4]: long rows queued
+  __shared__ int s_n[6];                  // [4], [5]: long and very long rows queued
   __shared__ int s_base[4];
   __shared__ long long s_part[kWavesPerBlock];
-  if (threadIdx.x < 5) s_n[threadIdx.x] = 0;
+  if (threadIdx.x < 6) s_n[threadIdx.x] = 0;
   __syncthreads();
   auto file_row = [&](int row, long long sum) {
     const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
@@ -344,8 +354,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
   };
 
   const int t = threadIdx.x % G;
-  const int64_t first = (int64_t)blockIdx.x * kBoundsRows;
-  for (int it = 0; it < kBoundsRows / kStep; ++it) {
+  const int64_t first = (int64_t)blockIdx.x * rows_per_group;
+  for (int it = 0; it < rows_per_group / kStep; ++it) {
     const int64_t row = first + it * kStep + threadIdx.x / G;
     int lo = 0, hi = 0;
     if (row < M) {
@@ -354,7 +364,10 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     }
     const bool is_long = hi - lo > kBoundsLongRow;
     if (is_long) {
-      if (t == 0) s_long[atomicAdd(&s_n[4], 1)] = (int)row;
+      if (t == 0) {
+        if (hi - lo > kBoundsWaveRow) s_very_long[atomicAdd(&s_n[5], 1)] = (int)row;
+        else s_long[atomicAdd(&s_n[4], 1)] = (int)row;
+      }
       hi = lo;
     }
     long long sum = 0;
@@ -369,8 +382,21 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
   __syncthreads();
 
   const int n_long = s_n[4];
-  for (int i = 0; i < n_long; ++i) {  // uniform over the workgroup
+  for (int i = threadIdx.x / kWaveSize; i < n_long; i += kWavesPerBlock) {  // uniform over the wavefront
     const int r = s_long[i];
+    long long part = 0;
+#pragma unroll 4
+    for (int p = a_pos[r] + wave_lane(); p < a_pos[r + 1]; p += kWaveSize) {
+      const int j = a_crd[p];
+      part += b_pos[j + 1] - b_pos[j];
+    }
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) part += __shfl_xor(part, off);
+    if (wave_lane() == 0) file_row(r, part);
+  }
+  const int n_very_long = s_n[5];
+  for (int i = 0; i < n_very_long; ++i) {  // uniform over the workgroup
+    const int r = s_very_long[i];
     long long part = 0;
 #pragma unroll 4
     for (int p = a_pos[r] + (int)threadIdx.x; p < a_pos[r + 1]; p += kBlockThreads) {
@@ -838,6 +864,7 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   const int tid = threadIdx.x;
   const int n_giant = LIST == 1 ? counters[5] : 0;  // only the list of the longest rows has the class
   const int n_rows = counters[LIST] + n_giant;
+  if ((int)blockIdx.x >= n_rows) return;  // more workgroups than rows: no need to queue at the counter
   constexpr int kRangeColumns = 32 * WORDS;
   A *acc = reinterpret_cast<A *>(c_val);
 
@@ -981,8 +1008,9 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
                const SpgemmWorkspace &ws, hipStream_t stream) {
   spgemm_reset_kernel<<<1, 64, 0, stream>>>(ws.counters, NUMERIC ? nullptr : c_pos + M);
   SCORCH_HIP_CHECK(hipGetLastError());
-  const unsigned row_groups = (unsigned)(((int64_t)M + kBoundsRows - 1) / kBoundsRows);
-  spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, a_pos, a_crd, b_pos, ws.products,
+  const int rows_per_group = bounds_rows_per_group(M);
+  const unsigned row_groups = (unsigned)(((int64_t)M + rows_per_group - 1) / rows_per_group);
+  spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, rows_per_group, a_pos, a_crd, b_pos, ws.products,
                                                                 ws.small_rows, ws.medium_rows,
                                                                 ws.huge_rows, ws.counters);
   SCORCH_HIP_CHECK(hipGetLastError());
