@@ -334,7 +334,8 @@ inline int bounds_rows_per_group(int64_t M) {
 __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
     int M, int rows_per_group, const int *__restrict__ a_pos, const int *__restrict__ a_crd,
     const int *__restrict__ b_pos, int *__restrict__ products, int *__restrict__ small_rows,
-    int *__restrict__ medium_rows, int *__restrict__ huge_rows, int *__restrict__ counters) {
+    int *__restrict__ medium_rows, int *__restrict__ huge_rows, int *__restrict__ counters,
+    const int *__restrict__ c_pos_if_narrow) {
   constexpr int G = 8;  // lanes per row
   constexpr int kStep = kBlockThreads / G;
   __shared__ int s_long[kBoundsRows];
@@ -348,8 +349,12 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_bounds_kernel(
   auto file_row = [&](int row, long long sum) {
     const int bound = sum > INT_MAX ? INT_MAX : (int)sum;
     products[row] = bound;
-    const int list = bound >= kGiantProducts ? 3 : bound > kMediumProducts ? 1 : bound > kSmallProducts ? 0
+    int list = bound >= kGiantProducts ? 3 : bound > kMediumProducts ? 1 : bound > kSmallProducts ? 0
                      : bound > kTinyProducts ? 2 : -1;
+    // The numeric pass knows the row's length: a row of many products but at most
+    // kMediumProducts distinct columns fits the sums of the tier below, whose
+    // smaller workgroups share a compute unit (B no wider than its bitmap).
+    if (list == 1 && c_pos_if_narrow && c_pos_if_narrow[row + 1] - c_pos_if_narrow[row] <= kMediumProducts) list = 0;
     if (list >= 0) s_list[list][atomicAdd(&s_n[list], 1)] = row;
   };
 
@@ -1012,7 +1017,8 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   const unsigned row_groups = (unsigned)(((int64_t)M + rows_per_group - 1) / rows_per_group);
   spgemm_bounds_kernel<<<row_groups, kBlockThreads, 0, stream>>>(M, rows_per_group, a_pos, a_crd, b_pos, ws.products,
                                                                 ws.small_rows, ws.medium_rows,
-                                                                ws.huge_rows, ws.counters);
+                                                                ws.huge_rows, ws.counters,
+                                                                NUMERIC && N <= 32 * 4096 ? c_pos : nullptr);
   SCORCH_HIP_CHECK(hipGetLastError());
   // four rows to a wavefront once that still leaves every wavefront slot of the chip a wavefront
   if ((int64_t)M >= 4 * 8192) {
