@@ -143,6 +143,27 @@ def test_clustered_columns_fall_back_to_the_whole_row_sort(oracle, dtype):
     assert list(np.diff(rp)) == [451, 1801, 300]
 
 
+@pytest.mark.parametrize("n,dtype", [(3000, np.float32), (3000, np.float64), (3000, np.int32),
+                                     (140_000, np.float32)])
+def test_many_products_on_few_distinct_columns(oracle, n, dtype):
+    """A band of 69 entries per row, squared: 4761 products per row on 137 distinct
+    columns.  The symbolic pass files such rows by their products; the numeric pass,
+    which knows their length, gives them to the tier of at most 4096 output entries
+    when B is no wider than that tier's bitmap (n = 3000; not at n = 140,000)."""
+    half = 34
+    rng = np.random.default_rng(23)
+    rows = np.arange(n)[:, None]
+    cols = rows + np.arange(-half, half + 1)[None, :]
+    keep = (cols >= 0) & (cols < n)
+    lens = keep.sum(axis=1)
+    arp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    aci = cols[keep].astype(np.int32)
+    av = (rng.integers(-9, 9, aci.size) if np.issubdtype(dtype, np.integer)
+          else rng.uniform(-1, 1, aci.size)).astype(dtype)
+    rp, _, _ = check(oracle, arp, aci, av, arp, aci, av, n)
+    assert np.diff(rp).max() == 4 * half + 1 and lens.max() ** 2 > 4096
+
+
 def test_structure_is_the_same_on_every_run_and_inputs_untouched(oracle):
     rng = np.random.default_rng(4)
     arp, aci, av = random_csr(rng, 300, 300, 0.05)
