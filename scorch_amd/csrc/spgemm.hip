@@ -602,6 +602,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   const int tid = threadIdx.x;
   const int n_rows = counters[COUNTER];
 
+  // (rows handed out one at a time through a counter, as in the bitmap tiers, measured
+  // slower: these rows are short enough for the counter's round trip to show)
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
     const int row = rows[idx];
     for (int s = tid; s < kSlots; s += kBlockThreads) {
@@ -618,12 +620,13 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
         });
     __syncthreads();
 
-    // Each thread owns a contiguous run of slots; an exclusive scan of the
-    // per-thread counts places the occupied ones.
+    // Each thread owns kRun slots, a workgroup's width apart (neighbouring threads
+    // on neighbouring LDS banks); an exclusive scan of the per-thread counts
+    // places the occupied ones.
     constexpr int kRun = kSlots / kBlockThreads;
     int mine = 0, key_min = INT_MAX, key_max = -1;
     for (int s = 0; s < kRun; ++s) {
-      const int key = s_keys[tid * kRun + s];
+      const int key = s_keys[s * kBlockThreads + tid];
       if (key != -1) {
         ++mine;
         key_min = key < key_min ? key : key_min;
@@ -651,7 +654,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) s_cnt[bkt] = 0;
     __syncthreads();
     for (int s = 0; s < kRun; ++s) {
-      const int key = s_keys[tid * kRun + s];
+      const int key = s_keys[s * kBlockThreads + tid];
       if (key != -1) atomicAdd(&s_cnt[(key - key_min) >> shift], 1);
     }
     __syncthreads();
@@ -673,11 +676,11 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       }
       __syncthreads();
       for (int s = 0; s < kRun; ++s) {
-        const int key = s_keys[tid * kRun + s];
+        const int key = s_keys[s * kBlockThreads + tid];
         if (key != -1) {
           const int pos = atomicAdd(&s_cnt[(key - key_min) >> shift], 1);  // ends as the bucket's end
           s_ck[pos] = key;
-          s_cv[pos] = s_vals[tid * kRun + s];
+          s_cv[pos] = s_vals[s * kBlockThreads + tid];
         }
       }
       __syncthreads();
@@ -698,10 +701,10 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       __syncthreads();
     } else {
       for (int s = 0; s < kRun; ++s) {
-        const int key = s_keys[tid * kRun + s];
+        const int key = s_keys[s * kBlockThreads + tid];
         if (key != -1) {
           s_ck[at] = key;
-          s_cv[at] = s_vals[tid * kRun + s];
+          s_cv[at] = s_vals[s * kBlockThreads + tid];
           ++at;
         }
       }
