@@ -876,11 +876,19 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   constexpr int kRangeColumns = 32 * WORDS;
   A *acc = reinterpret_cast<A *>(c_val);
 
-  for (;;) {
+  // The longest rows are handed out through a counter, one at a time, so that the
+  // workgroups stay evenly loaded; the rows of the tier below are short enough
+  // for the counter's round trip to show, and are taken in fixed strides.
+  for (int turn = 0;; ++turn) {
     __syncthreads();  // everyone is done with the previous row (and with s_next)
-    if (tid == 0) s_next = atomicAdd(&counters[WORK], 1);
-    __syncthreads();
-    const int idx = s_next;
+    int idx;
+    if (LIST == 1) {
+      if (tid == 0) s_next = atomicAdd(&counters[WORK], 1);
+      __syncthreads();
+      idx = s_next;
+    } else {
+      idx = (int)blockIdx.x + turn * (int)gridDim.x;
+    }
     if (idx >= n_rows) return;  // the same for every thread
     const int row = LIST == 1 ? huge_row(rows, M, n_giant, idx) : rows[idx];
     const int a_lo = a_pos[row], a_hi = a_pos[row + 1];
