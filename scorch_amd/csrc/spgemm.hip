@@ -162,8 +162,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &to
 // lanes read consecutive entries of a B row.
 template <int TEAM, typename A>
 struct ProductBatch {
-  int off[TEAM];  // first product of each entry within the batch
-  int b_lo[TEAM];
+  int index[2 * TEAM];  // [e]: first product of entry e within the batch; [TEAM + e]: where its B row starts
   A a_val[TEAM];
 };
 
@@ -207,8 +206,8 @@ __device__ __forceinline__ void product_step(int x0, int total, const int *__res
     e[u] = 0;  // the last entry whose offset is <= x (entries without products share an offset)
 #pragma unroll
     for (int step = TEAM / 2; step > 0; step >>= 1)
-      if (batch.off[e[u] + step] <= x) e[u] += step;
-    q[u] = batch.b_lo[e[u]] + (x - batch.off[e[u]]);
+      if (batch.index[e[u] + step] <= x) e[u] += step;
+    q[u] = batch.index[TEAM + e[u]] + (x - batch.index[e[u]]);
   }
   int col[U];
   A b[U];
@@ -243,8 +242,8 @@ __device__ __forceinline__ void for_each_product(int a_lo, int a_hi, int t, cons
     int total = 0;
     const int first = team_exclusive_scan<TEAM>(len, scan_scratch, total);
     team_sync<TEAM>();  // the previous batch has been read by everyone
-    batch.off[t] = first;
-    batch.b_lo[t] = lo;
+    batch.index[t] = first;
+    batch.index[TEAM + t] = lo;
     if (NUMERIC) batch.a_val[t] = av;
     team_sync<TEAM>();
     int x = 0;  // the team's first product of the step
@@ -516,8 +515,88 @@ __device__ __forceinline__ void spgemm_team_row(
   }
   wave_lds_sync();
 
-  // Rank = number of smaller keys (keys are distinct): the sorted position.
   const int out = c_pos[row];
+  // Whole wavefronts with more than a key per lane sort by buckets: counting
+  // ranks below costs n compares per key, half of this tier's time at 256 keys a
+  // row.  The keys' range is cut into 2 * TEAM equal power-of-two intervals; a
+  // prefix sum of the bucket counts (kept where the batch's indices were) places
+  // the buckets, the entries are scattered bucket by bucket into the tables'
+  // upper halves (free: n <= PRODUCTS <= SLOTS / 2), and an entry's rank is
+  // its bucket's start plus the smaller keys in its bucket.  Crowded buckets
+  // (clustered columns) leave the row to the rank count.
+  if (TEAM == kWaveSize && 2 * PRODUCTS <= SLOTS && n > TEAM) {
+    constexpr int kBuckets = 2 * TEAM;
+    constexpr int kPerLane = PRODUCTS / TEAM;
+    constexpr int kCrowd = 16;
+    int *const cnt = lds.batch[team].index;
+    int key[kPerLane], pos[kPerLane];
+    int key_min = INT_MAX, key_max = -1;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+      const int e = t + i * TEAM;
+      key[i] = e < n ? lds.keys[team][e] : -1;
+      if (e < n) {
+        key_min = key[i] < key_min ? key[i] : key_min;
+        key_max = key[i] > key_max ? key[i] : key_max;
+      }
+    }
+#pragma unroll
+    for (int off = TEAM / 2; off > 0; off >>= 1) {
+      const int lo = __shfl_xor(key_min, off), hi = __shfl_xor(key_max, off);
+      key_min = lo < key_min ? lo : key_min;
+      key_max = hi > key_max ? hi : key_max;
+    }
+    int shift = 0;
+    while (((key_max - key_min) >> shift) >= kBuckets) ++shift;
+    cnt[t] = 0;
+    cnt[TEAM + t] = 0;
+    wave_lds_sync();
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i)
+      if (t + i * TEAM < n) pos[i] = atomicAdd(&cnt[(key[i] - key_min) >> shift], 1);
+    wave_lds_sync();
+    const int c0 = cnt[2 * t], c1 = cnt[2 * t + 1];  // lane t places buckets 2t and 2t + 1
+    int unused = 0;
+    const int before = team_exclusive_scan<TEAM>(c0 + c1, nullptr, unused);
+    int crowd = c0 > c1 ? c0 : c1;
+#pragma unroll
+    for (int off = TEAM / 2; off > 0; off >>= 1) {
+      const int other = __shfl_xor(crowd, off);
+      crowd = other > crowd ? other : crowd;
+    }
+    if (crowd <= kCrowd) {  // uniform
+      wave_lds_sync();  // everyone has read the counts
+      cnt[2 * t] = before;
+      cnt[2 * t + 1] = before + c0;
+      wave_lds_sync();
+#pragma unroll
+      for (int i = 0; i < kPerLane; ++i) {
+        const int e = t + i * TEAM;
+        if (e < n) {
+          const int p = PRODUCTS + cnt[(key[i] - key_min) >> shift] + pos[i];
+          lds.keys[team][p] = key[i];
+          lds.vals[team][p] = lds.vals[team][e];
+        }
+      }
+      wave_lds_sync();
+#pragma unroll
+      for (int i = 0; i < kPerLane; ++i) {
+        const int e = t + i * TEAM;
+        if (e < n) {
+          const int k = lds.keys[team][PRODUCTS + e];
+          const int b = (k - key_min) >> shift;
+          const int lo = cnt[b], hi = b + 1 < kBuckets ? cnt[b + 1] : n;
+          int rank = lo;
+          for (int x = lo; x < hi; ++x) rank += lds.keys[team][PRODUCTS + x] < k ? 1 : 0;
+          c_crd[out + rank] = k;
+          c_val[out + rank] = (T)lds.vals[team][PRODUCTS + e];
+        }
+      }
+      return;
+    }
+  }
+
+  // Rank = number of smaller keys (keys are distinct): the sorted position.
   for (int e = t; e < n; e += TEAM) {
     const int key = lds.keys[team][e];
     int rank = 0;
