@@ -164,6 +164,35 @@ def test_many_products_on_few_distinct_columns(oracle, n, dtype):
     assert np.diff(rp).max() == 4 * half + 1 and lens.max() ** 2 > 4096
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+def test_wavefront_rows_sorted_by_buckets_and_by_rank(oracle, dtype):
+    """Rows of 65 to 256 output entries (a wavefront each) are sorted by buckets over
+    their column range, unless the columns crowd a few buckets: row 0 spreads 200
+    columns evenly, row 1 has a run of 120 consecutive columns and two far outliers
+    (one bucket would hold the whole run: the rank count takes over), row 2 puts
+    exactly 17 columns into one bucket, one more than a bucket may hold, row 3 has
+    64 entries (rank count by size) and row 4 has 256, each column hit twice."""
+    n_cols = 1 << 20
+    rng = np.random.default_rng(29)
+    b_cols = [np.sort(rng.choice(n_cols, 200, replace=False)),
+              np.concatenate([[5], np.arange(1000, 1120), [900_000]]),
+              np.concatenate([np.arange(0, 17), np.arange(1, 100) * 8192]),
+              np.sort(rng.choice(n_cols, 64, replace=False)),
+              np.sort(rng.choice(n_cols, 128, replace=False)),
+              np.sort(rng.choice(n_cols, 128, replace=False))]
+    b_cols[5][:64] = b_cols[4][:64]          # half of row 4's columns come from both B rows
+    b_cols[5] = np.unique(b_cols[5])
+    brp = np.concatenate([[0], np.cumsum([c.size for c in b_cols])]).astype(np.int32)
+    bci = np.concatenate(b_cols).astype(np.int32)
+    draw = (lambda k: rng.integers(1, 9, k)) if np.issubdtype(dtype, np.integer) else (lambda k: rng.uniform(0.5, 1.5, k))
+    bv = draw(bci.size).astype(dtype)
+    arp = np.array([0, 1, 2, 3, 4, 6], np.int32)
+    aci = np.array([0, 1, 2, 3, 4, 5], np.int32)
+    av = draw(aci.size).astype(dtype)
+    rp, ci, _ = check(oracle, arp, aci, av, brp, bci, bv, n_cols)
+    assert list(np.diff(rp)[:4]) == [200, 122, 116, 64] and 128 < np.diff(rp)[4] <= 256
+
+
 def test_structure_is_the_same_on_every_run_and_inputs_untouched(oracle):
     rng = np.random.default_rng(4)
     arp, aci, av = random_csr(rng, 300, 300, 0.05)
