@@ -923,10 +923,9 @@ __global__ __launch_bounds__(kHugeThreads) void spgemm_huge_kernel(
 // Atomics on a bitmap in global memory all land on a few hundred cache lines and
 // queue up in the L2's atomic units (the 13.7 M products of a power-law square
 // spend 0.4 ms there per walk).  For N up to 32 * WORDS columns the bitmap lives
-// in LDS instead, with one rank per four bitmap words, and so do the row's sums
-// when the row has at most kAccEntries distinct columns (else they are added
-// into the output with global atomics as above).  Rows are handed out through a
-// counter, one at a time, so the workgroups stay evenly loaded.
+// in LDS instead, with one rank per four bitmap words, and so do the sums of the
+// row's first kAccEntries output entries (the others are added into the output
+// with global atomics as above).
 constexpr int kLdsBudget = 160 * 1024 - 1024;
 
 // THREADS: workgroup size.  ACC: LDS sums to provide (0: all the LDS that is left).
@@ -1004,26 +1003,29 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
         n += total;
       }
       if (NUMERIC && n > 0) {  // uniform
-        const int first = out + done;                // the range's place in the row's output
-        const bool sums_in_lds = n <= kAccEntries;  // uniform
-        __syncthreads();                            // s_rank is complete
+        const int first = out + done;  // the range's place in the row's output
+        // The first kAccEntries output entries have their sums, and before that their
+        // column indices, in LDS; entries beyond go straight to the output: a
+        // thread's columns lie far apart there (single 4-byte stores), and sums added
+        // with global atomics queue up in the L2's atomic units.
+        const int in_lds = n < kAccEntries ? n : kAccEntries;
+        __syncthreads();  // s_rank is complete
         for (int g = tid; g < groups; g += THREADS) {
-          int at = first + s_rank[g];
+          int at = s_rank[g];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             unsigned bits = s_bits[4 * g + i];
             while (bits) {
               const int bit = __ffs(bits) - 1;
               bits &= bits - 1;
-              c_crd[at++] = c0 + (4 * g + i) * 32 + bit;
+              const int col = c0 + (4 * g + i) * 32 + bit;
+              c_crd[first + at] = col;
+              ++at;
             }
           }
         }
-        if (sums_in_lds) {
-          for (int e = tid; e < n; e += THREADS) s_acc[e] = (A)0;
-        } else {
-          for (int e = tid; e < n; e += THREADS) workgroup_store(&acc[first + e], (A)0);
-        }
+        for (int e = in_lds + tid; e < n; e += THREADS) workgroup_store(&acc[first + e], (A)0);
+        for (int e = tid; e < in_lds; e += THREADS) s_acc[e] = (A)0;
         __syncthreads();
         for_each_product<THREADS, true, T, A>(
             a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
@@ -1032,12 +1034,11 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
               const int w = (int)(rel >> 5);
               int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (rel & 31)) - 1u));
               for (int i = w & ~3; i < w; ++i) at += __popc(s_bits[i]);
-              if (sums_in_lds) atomic_accumulate<A>(&s_acc[at], product);
+              if (at < kAccEntries) atomic_accumulate<A>(&s_acc[at], product);
               else __hip_atomic_fetch_add(&acc[first + at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             });
         __syncthreads();
-        if (sums_in_lds)
-          for (int e = tid; e < n; e += THREADS) c_val[first + e] = (T)s_acc[e];
+        for (int e = tid; e < in_lds; e += THREADS) c_val[first + e] = (T)s_acc[e];
       }
       done += n;
     }
