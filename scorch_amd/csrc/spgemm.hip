@@ -128,25 +128,46 @@ __device__ __forceinline__ int block_exclusive_scan_n(int v, int *scratch, int &
   return before + incl - v;
 }
 
-// Maximum (or minimum) of one int per thread over a 256-thread workgroup.
-template <bool MAX>
-__device__ __forceinline__ int block_reduce_int(int v, int *scratch) {
-#pragma unroll
-  for (int off = kWaveSize / 2; off > 0; off >>= 1) {
-    const int o = __shfl_xor(v, off);
-    v = MAX ? (o > v ? o : v) : (o < v ? o : v);
-  }
-  __syncthreads();  // scratch may still be read from a previous call
-  if (wave_lane() == 0) scratch[threadIdx.x / kWaveSize] = v;
-  __syncthreads();
-  int r = scratch[0];
-#pragma unroll
-  for (int i = 1; i < kWavesPerBlock; ++i) r = MAX ? (scratch[i] > r ? scratch[i] : r) : (scratch[i] < r ? scratch[i] : r);
-  return r;
-}
-
 __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &total) {
   return block_exclusive_scan_n<kWavesPerBlock>(v, scratch, total);
+}
+
+// Exclusive scan of `v` over a 256-thread workgroup and, behind the same two
+// barriers, the workgroup's minimum of `lo` and maximum of `hi`.
+__device__ __forceinline__ int block_scan_min_max(int v, int &total, int &lo, int &hi, int *scan_scratch,
+                                                  int *min_scratch, int *max_scratch) {
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  int incl = v;
+#pragma unroll
+  for (int off = 1; off < kWaveSize; off <<= 1) {
+    const int up = __shfl_up(incl, off);
+    if (lane >= off) incl += up;
+  }
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) {
+    const int l = __shfl_xor(lo, off), h = __shfl_xor(hi, off);
+    lo = l < lo ? l : lo;
+    hi = h > hi ? h : hi;
+  }
+  __syncthreads();  // the scratch arrays may still be read from a previous call
+  if (lane == kWaveSize - 1) scan_scratch[w] = incl;
+  if (lane == 0) {
+    min_scratch[w] = lo;
+    max_scratch[w] = hi;
+  }
+  __syncthreads();
+  int before = 0, all = 0;
+#pragma unroll
+  for (int i = 0; i < kWavesPerBlock; ++i) {
+    const int part = scan_scratch[i];
+    if (i < w) before += part;
+    all += part;
+    lo = min_scratch[i] < lo ? min_scratch[i] : lo;
+    hi = max_scratch[i] > hi ? max_scratch[i] : hi;
+  }
+  total = all;
+  return before + incl - v;
 }
 
 // ---- walking the products of one row of C ------------------------------------------------
@@ -674,7 +695,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   __shared__ int s_ck[NUMERIC ? PRODUCTS : 1];
   __shared__ A s_cv[NUMERIC ? PRODUCTS : 1];
   __shared__ int s_scan[kWavesPerBlock + 1];
-  __shared__ int s_red[kWavesPerBlock];
+  __shared__ int s_red[2][kWavesPerBlock];
   __shared__ int s_cnt[NUMERIC ? kBuckets : 1];
   __shared__ ProductBatch<kBlockThreads, A> s_batch;
 
@@ -689,6 +710,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       s_keys[s] = -1;
       if (NUMERIC) s_vals[s] = (A)0;
     }
+    if (NUMERIC)
+      for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) s_cnt[bkt] = 0;
     __syncthreads();
 
     for_each_product<kBlockThreads, NUMERIC, T, A>(
@@ -713,7 +736,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       }
     }
     int n = 0;
-    int at = block_exclusive_scan(mine, s_scan, n);
+    int at = block_scan_min_max(mine, n, key_min, key_max, s_scan, s_red[0], s_red[1]);
     if (!NUMERIC) {
       if (tid == 0) c_pos[row] = n;
       __syncthreads();
@@ -723,16 +746,13 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     // Sorting the row's (column, value) pairs.  First choice: buckets.  The
     // columns' range [min, max] is cut into kBuckets equal power-of-two intervals
     // (about two entries each when the columns are spread evenly), a prefix sum of
-    // the bucket counts places the buckets, and a thread sorts each bucket by
-    // insertion.  If some bucket is crowded (clustered columns), a bitonic sort
+    // the bucket counts places the buckets, the entries are scattered bucket by
+    // bucket, and an entry's rank is its bucket's start plus the smaller keys in
+    // its bucket.  If some bucket is crowded (clustered columns), a bitonic sort
     // of the whole row takes over.
-    key_min = block_reduce_int<false>(key_min, s_red);
-    key_max = block_reduce_int<true>(key_max, s_red);
     int shift = 0;
     while (((key_max - key_min) >> shift) >= kBuckets) ++shift;  // n > 0 here: the row has products
-    for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) s_cnt[bkt] = 0;
-    __syncthreads();
-    for (int s = 0; s < kRun; ++s) {
+    for (int s = 0; s < kRun; ++s) {  // (the counts were cleared with the tables)
       const int key = s_keys[s * kBlockThreads + tid];
       if (key != -1) atomicAdd(&s_cnt[(key - key_min) >> shift], 1);
     }
@@ -744,9 +764,8 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       run_total += c;
       crowd = c > crowd ? c : crowd;
     }
-    int unused = 0;
-    int start = block_exclusive_scan(run_total, s_scan, unused);
-    crowd = block_reduce_int<true>(crowd, s_red);
+    int unused = 0, unused_min = 0;
+    int start = block_scan_min_max(run_total, unused, unused_min, crowd, s_scan, s_red[0], s_red[1]);
     if (crowd <= kBucketCrowd) {
       for (int i = 0; i < kBucketRun; ++i) {  // counts -> first positions
         const int c = s_cnt[tid * kBucketRun + i];
@@ -763,21 +782,18 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
         }
       }
       __syncthreads();
-      for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) {
+      const int out = c_pos[row];
+      for (int e = tid; e < n; e += kBlockThreads) {
+        const int key = s_ck[e];
+        const int bkt = (key - key_min) >> shift;
         const int lo = bkt ? s_cnt[bkt - 1] : 0, hi = s_cnt[bkt];
-        for (int i = lo + 1; i < hi; ++i) {
-          const int key = s_ck[i];
-          const A val = s_cv[i];
-          int j = i;
-          for (; j > lo && s_ck[j - 1] > key; --j) {
-            s_ck[j] = s_ck[j - 1];
-            s_cv[j] = s_cv[j - 1];
-          }
-          s_ck[j] = key;
-          s_cv[j] = val;
-        }
+        int rank = lo;
+        for (int x = lo; x < hi; ++x) rank += s_ck[x] < key ? 1 : 0;
+        c_crd[out + rank] = key;
+        c_val[out + rank] = (T)s_cv[e];
       }
       __syncthreads();
+      continue;
     } else {
       for (int s = 0; s < kRun; ++s) {
         const int key = s_keys[s * kBlockThreads + tid];
