@@ -83,15 +83,27 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
   // The entries beyond the registers are read twice, not three times: the first
   // sweep keeps a running maximum and the sum of exponentials relative to it
   // (rescaled whenever the maximum moves: one exponential per entry either way).
+  constexpr int kTailBatch = 8;
   float tail_max = mx, tail_sum = 0.0f;
   if (TAIL) {
-#pragma unroll 8
-    for (int p = rest; p < hi; p += TEAM) {
-      const float x = vals[p] * scale;
-      const float e = expf(-fabsf(x - tail_max));
-      const bool higher = x > tail_max;
-      tail_sum = higher ? tail_sum * e + 1.0f : tail_sum + e;
-      tail_max = higher ? x : tail_max;
+    // (kTailBatch loads are issued together in both sweeps: out may alias vals, so
+    // the compiler would not move a load above the store of the entry before)
+    for (int p0 = rest; p0 < hi; p0 += kTailBatch * TEAM) {
+      float raw[kTailBatch];
+#pragma unroll
+      for (int u = 0; u < kTailBatch; ++u) {
+        const int p = p0 + u * TEAM;
+        raw[u] = p < hi ? vals[p] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < kTailBatch; ++u) {
+        if (p0 + u * TEAM >= hi) break;
+        const float x = raw[u] * scale;
+        const float e = expf(-fabsf(x - tail_max));
+        const bool higher = x > tail_max;
+        tail_sum = higher ? tail_sum * e + 1.0f : tail_sum + e;
+        tail_max = higher ? x : tail_max;
+      }
     }
     mx = tail_max;
   }
@@ -109,8 +121,19 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
     if (p < hi) out[p] = v[u] / sum;
   }
   if (TAIL) {
-#pragma unroll 8
-    for (int p = rest; p < hi; p += TEAM) out[p] = expf(vals[p] * scale - mx) / sum;
+    for (int p0 = rest; p0 < hi; p0 += kTailBatch * TEAM) {
+      float raw[kTailBatch];
+#pragma unroll
+      for (int u = 0; u < kTailBatch; ++u) {
+        const int p = p0 + u * TEAM;
+        raw[u] = p < hi ? vals[p] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < kTailBatch; ++u) {
+        const int p = p0 + u * TEAM;
+        if (p < hi) out[p] = expf(raw[u] * scale - mx) / sum;
+      }
+    }
   }
 }
 
