@@ -957,7 +957,7 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   constexpr int kFixed = WORDS * 4 + (NUMERIC ? kGroups * 4 : 0) + (int)sizeof(ProductBatch<THREADS, A>) + 512;
   constexpr int kAccEntries = !NUMERIC ? 1 : ACC > 0 ? ACC : (kLdsBudget - kFixed) / (int)sizeof(A);
   constexpr int kWaves = THREADS / kWaveSize;
-  __shared__ unsigned s_bits[WORDS];
+  __shared__ __align__(16) unsigned s_bits[WORDS];
   __shared__ int s_rank[NUMERIC ? kGroups : 1];  // rank of the first column of every group of four words
   __shared__ A s_acc[kAccEntries];
   __shared__ ProductBatch<THREADS, A> s_batch;
@@ -1047,9 +1047,16 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
             a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
               const unsigned rel = (unsigned)(k - c0);
               if (rel >= (unsigned)columns) return;
-              const int w = (int)(rel >> 5);
-              int at = s_rank[w >> 2] + __popc(s_bits[w] & ((1u << (rel & 31)) - 1u));
-              for (int i = w & ~3; i < w; ++i) at += __popc(s_bits[i]);
+              // rank = the group's + the bits below the column's in the group's four words,
+              // which come in one read (a loop over the words before the column's
+              // would chain up to three more LDS round trips)
+              const int w = (int)(rel >> 5), sub = w & 3;
+              const uint4 grp = *reinterpret_cast<const uint4 *>(&s_bits[w & ~3]);
+              const unsigned below = (1u << (rel & 31)) - 1u;
+              const int at = s_rank[w >> 2] + __popc(grp.x & (sub == 0 ? below : ~0u)) +
+                             __popc(grp.y & (sub == 1 ? below : sub > 1 ? ~0u : 0u)) +
+                             __popc(grp.z & (sub == 2 ? below : sub > 2 ? ~0u : 0u)) +
+                             __popc(grp.w & (sub == 3 ? below : 0u));
               if (at < kAccEntries) atomic_accumulate<A>(&s_acc[at], product);
               else __hip_atomic_fetch_add(&acc[first + at], product, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             });
