@@ -969,6 +969,10 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
   if ((int)blockIdx.x >= n_rows) return;  // more workgroups than rows: no need to queue at the counter
   constexpr int kRangeColumns = 32 * WORDS;
   A *acc = reinterpret_cast<A *>(c_val);
+  // B with no more columns than the LDS holds sums: the numeric pass keeps a sum
+  // per column and walks the row's products once (bits and sums together)
+  // instead of twice (bits, then sums at their ranks).
+  const bool sums_by_column = NUMERIC && N <= kAccEntries && N <= kRangeColumns;
 
   // The longest rows are handed out through a counter, one at a time, so that the
   // workgroups stay evenly loaded; the rows of the tier below are short enough
@@ -997,12 +1001,22 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
       const int groups = ((columns + 31) / 32 + 3) / 4;
       if (c0 > 0) __syncthreads();  // the previous range's bits, ranks and sums have been used
       for (int i = tid; i < 4 * groups; i += THREADS) s_bits[i] = 0u;
+      if (sums_by_column)
+        for (int i = tid; i < columns; i += THREADS) s_acc[i] = (A)0;
       __syncthreads();
-      for_each_product<THREADS, false, T, A>(
-          a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A) {
-            const unsigned rel = (unsigned)(k - c0);
-            if (rel < (unsigned)columns) atomicOr(&s_bits[rel >> 5], 1u << (rel & 31));
-          });
+      if (sums_by_column) {
+        for_each_product<THREADS, true, T, A>(
+            a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A product) {
+              atomicOr(&s_bits[k >> 5], 1u << (k & 31));
+              atomic_accumulate<A>(&s_acc[k], product);
+            });
+      } else {
+        for_each_product<THREADS, false, T, A>(
+            a_lo, a_hi, tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan, [&](int k, A) {
+              const unsigned rel = (unsigned)(k - c0);
+              if (rel < (unsigned)columns) atomicOr(&s_bits[rel >> 5], 1u << (rel & 31));
+            });
+      }
       __syncthreads();
 
       // distinct columns of the range, and the rank of each group's first one
@@ -1036,10 +1050,12 @@ __global__ __launch_bounds__(THREADS) void spgemm_lds_bitmap_kernel(
               bits &= bits - 1;
               const int col = c0 + (4 * g + i) * 32 + bit;
               c_crd[first + at] = col;
+              if (sums_by_column) c_val[first + at] = (T)s_acc[col];
               ++at;
             }
           }
         }
+        if (sums_by_column) break;  // uniform; the only range: the row is complete
         for (int e = in_lds + tid; e < n; e += THREADS) workgroup_store(&acc[first + e], (A)0);
         for (int e = tid; e < in_lds; e += THREADS) s_acc[e] = (A)0;
         __syncthreads();
