@@ -193,6 +193,27 @@ def test_wavefront_rows_sorted_by_buckets_and_by_rank(oracle, dtype):
     assert list(np.diff(rp)[:4]) == [200, 122, 116, 64] and 128 < np.diff(rp)[4] <= 256
 
 
+@pytest.mark.parametrize("n_cols", [3000, 15_000, 16_500, 31_000, 34_000])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64])
+def test_bitmap_tiers_around_the_widths_that_fit_sums_by_column(oracle, n_cols, dtype):
+    """B no wider than the sums a workgroup keeps in LDS (about 32 K four-byte or
+    16 K eight-byte values with 1024 threads, 4096 with 256) has its rows summed by
+    column in one walk; wider, by rank in two.  Rows of about 2,000, 6,000 and
+    40,000 products on either side of those widths, some columns hit many times."""
+    rng = np.random.default_rng(31)
+    lens = rng.integers(0, 3, 40)
+    lens[[3, 17, 39]] = [20, 60, 400]
+    arp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    aci = np.concatenate([np.sort(rng.choice(500, int(n), replace=False)) for n in lens]).astype(np.int32)
+    b_cols = [np.sort(rng.choice(n_cols, 100, replace=False)) for _ in range(500)]
+    brp = np.arange(501, dtype=np.int32) * 100
+    bci = np.concatenate(b_cols).astype(np.int32)
+    draw = (lambda k: rng.integers(-9, 9, k)) if np.issubdtype(dtype, np.integer) else (lambda k: rng.uniform(-1, 1, k))
+    av, bv = draw(aci.size).astype(dtype), draw(bci.size).astype(dtype)
+    rp, _, _ = check(oracle, arp, aci, av, brp, bci, bv, n_cols)
+    assert np.diff(rp)[39] > 2000
+
+
 def test_structure_is_the_same_on_every_run_and_inputs_untouched(oracle):
     rng = np.random.default_rng(4)
     arp, aci, av = random_csr(rng, 300, 300, 0.05)
