@@ -132,8 +132,9 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *scratch, int &to
   return block_exclusive_scan_n<kWavesPerBlock>(v, scratch, total);
 }
 
-// Exclusive scan of `v` over a 256-thread workgroup and, behind the same two
+// Exclusive scan of `v` over a workgroup of WAVES wavefronts and, behind the same two
 // barriers, the workgroup's minimum of `lo` and maximum of `hi`.
+template <int WAVES>
 __device__ __forceinline__ int block_scan_min_max(int v, int &total, int &lo, int &hi, int *scan_scratch,
                                                   int *min_scratch, int *max_scratch) {
   const int lane = wave_lane();
@@ -159,7 +160,7 @@ __device__ __forceinline__ int block_scan_min_max(int v, int &total, int &lo, in
   __syncthreads();
   int before = 0, all = 0;
 #pragma unroll
-  for (int i = 0; i < kWavesPerBlock; ++i) {
+  for (int i = 0; i < WAVES; ++i) {
     const int part = scan_scratch[i];
     if (i < w) before += part;
     all += part;
@@ -680,8 +681,10 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_tiny_kernel(
 }
 
 // ---- rows of at most PRODUCTS products: one workgroup each, 2 * PRODUCTS hash slots ----
-template <typename T, bool NUMERIC, int PRODUCTS, int COUNTER>
-__global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
+// THREADS: workgroup size (the tables of the larger form leave room for one workgroup per
+// CU: it is given 1024 threads rather than 256).
+template <typename T, bool NUMERIC, int PRODUCTS, int COUNTER, int THREADS>
+__global__ __launch_bounds__(THREADS) void spgemm_medium_kernel(
     const int *__restrict__ a_pos, const int *__restrict__ a_crd, const T *__restrict__ a_val,
     const int *__restrict__ b_pos, const int *__restrict__ b_crd, const T *__restrict__ b_val,
     const int *__restrict__ rows, const int *__restrict__ counters, int *__restrict__ c_pos,
@@ -694,10 +697,10 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   __shared__ A s_vals[NUMERIC ? kSlots : 1];
   __shared__ int s_ck[NUMERIC ? PRODUCTS : 1];
   __shared__ A s_cv[NUMERIC ? PRODUCTS : 1];
-  __shared__ int s_scan[kWavesPerBlock + 1];
-  __shared__ int s_red[2][kWavesPerBlock];
+  __shared__ int s_scan[(THREADS / kWaveSize) + 1];
+  __shared__ int s_red[2][(THREADS / kWaveSize)];
   __shared__ int s_cnt[NUMERIC ? kBuckets : 1];
-  __shared__ ProductBatch<kBlockThreads, A> s_batch;
+  __shared__ ProductBatch<THREADS, A> s_batch;
 
   const int tid = threadIdx.x;
   const int n_rows = counters[COUNTER];
@@ -706,15 +709,15 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
   // slower: these rows are short enough for the counter's round trip to show)
   for (int idx = blockIdx.x; idx < n_rows; idx += gridDim.x) {
     const int row = rows[idx];
-    for (int s = tid; s < kSlots; s += kBlockThreads) {
+    for (int s = tid; s < kSlots; s += THREADS) {
       s_keys[s] = -1;
       if (NUMERIC) s_vals[s] = (A)0;
     }
     if (NUMERIC)
-      for (int bkt = tid; bkt < kBuckets; bkt += kBlockThreads) s_cnt[bkt] = 0;
+      for (int bkt = tid; bkt < kBuckets; bkt += THREADS) s_cnt[bkt] = 0;
     __syncthreads();
 
-    for_each_product<kBlockThreads, NUMERIC, T, A>(
+    for_each_product<THREADS, NUMERIC, T, A>(
         a_pos[row], a_pos[row + 1], tid, a_crd, a_val, b_pos, b_crd, b_val, s_batch, s_scan,
         [&](int col, A product) {
           const int slot = hash_insert(s_keys, kSlots - 1, col);
@@ -725,10 +728,10 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     // Each thread owns kRun slots, a workgroup's width apart (neighbouring threads
     // on neighbouring LDS banks); an exclusive scan of the per-thread counts
     // places the occupied ones.
-    constexpr int kRun = kSlots / kBlockThreads;
+    constexpr int kRun = kSlots / THREADS;
     int mine = 0, key_min = INT_MAX, key_max = -1;
     for (int s = 0; s < kRun; ++s) {
-      const int key = s_keys[s * kBlockThreads + tid];
+      const int key = s_keys[s * THREADS + tid];
       if (key != -1) {
         ++mine;
         key_min = key < key_min ? key : key_min;
@@ -736,7 +739,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       }
     }
     int n = 0;
-    int at = block_scan_min_max(mine, n, key_min, key_max, s_scan, s_red[0], s_red[1]);
+    int at = block_scan_min_max<THREADS / kWaveSize>(mine, n, key_min, key_max, s_scan, s_red[0], s_red[1]);
     if (!NUMERIC) {
       if (tid == 0) c_pos[row] = n;
       __syncthreads();
@@ -753,11 +756,11 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
     int shift = 0;
     while (((key_max - key_min) >> shift) >= kBuckets) ++shift;  // n > 0 here: the row has products
     for (int s = 0; s < kRun; ++s) {  // (the counts were cleared with the tables)
-      const int key = s_keys[s * kBlockThreads + tid];
+      const int key = s_keys[s * THREADS + tid];
       if (key != -1) atomicAdd(&s_cnt[(key - key_min) >> shift], 1);
     }
     __syncthreads();
-    constexpr int kBucketRun = kBuckets / kBlockThreads;
+    constexpr int kBucketRun = kBuckets / THREADS;
     int run_total = 0, crowd = 0;
     for (int i = 0; i < kBucketRun; ++i) {
       const int c = s_cnt[tid * kBucketRun + i];
@@ -765,7 +768,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       crowd = c > crowd ? c : crowd;
     }
     int unused = 0, unused_min = 0;
-    int start = block_scan_min_max(run_total, unused, unused_min, crowd, s_scan, s_red[0], s_red[1]);
+    int start = block_scan_min_max<THREADS / kWaveSize>(run_total, unused, unused_min, crowd, s_scan, s_red[0], s_red[1]);
     if (crowd <= kBucketCrowd) {
       for (int i = 0; i < kBucketRun; ++i) {  // counts -> first positions
         const int c = s_cnt[tid * kBucketRun + i];
@@ -774,16 +777,16 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       }
       __syncthreads();
       for (int s = 0; s < kRun; ++s) {
-        const int key = s_keys[s * kBlockThreads + tid];
+        const int key = s_keys[s * THREADS + tid];
         if (key != -1) {
           const int pos = atomicAdd(&s_cnt[(key - key_min) >> shift], 1);  // ends as the bucket's end
           s_ck[pos] = key;
-          s_cv[pos] = s_vals[s * kBlockThreads + tid];
+          s_cv[pos] = s_vals[s * THREADS + tid];
         }
       }
       __syncthreads();
       const int out = c_pos[row];
-      for (int e = tid; e < n; e += kBlockThreads) {
+      for (int e = tid; e < n; e += THREADS) {
         const int key = s_ck[e];
         const int bkt = (key - key_min) >> shift;
         const int lo = bkt ? s_cnt[bkt - 1] : 0, hi = s_cnt[bkt];
@@ -796,21 +799,21 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       continue;
     } else {
       for (int s = 0; s < kRun; ++s) {
-        const int key = s_keys[s * kBlockThreads + tid];
+        const int key = s_keys[s * THREADS + tid];
         if (key != -1) {
           s_ck[at] = key;
-          s_cv[at] = s_vals[s * kBlockThreads + tid];
+          s_cv[at] = s_vals[s * THREADS + tid];
           ++at;
         }
       }
       int padded = 1;
       while (padded < n) padded <<= 1;
       __syncthreads();
-      for (int e = n + tid; e < padded; e += kBlockThreads) s_ck[e] = INT_MAX;
+      for (int e = n + tid; e < padded; e += THREADS) s_ck[e] = INT_MAX;
       __syncthreads();
       for (int size = 2; size <= padded; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
-          for (int e = tid; e < padded / 2; e += kBlockThreads) {
+          for (int e = tid; e < padded / 2; e += THREADS) {
             const int lo = 2 * e - (e & (stride - 1));
             const int hi = lo + stride;
             const bool ascending = (lo & size) == 0;
@@ -828,7 +831,7 @@ __global__ __launch_bounds__(kBlockThreads) void spgemm_medium_kernel(
       }
     }
     const int out = c_pos[row];
-    for (int e = tid; e < n; e += kBlockThreads) {
+    for (int e = tid; e < n; e += THREADS) {
       c_crd[out + e] = s_ck[e];
       c_val[out + e] = (T)s_cv[e];
     }
@@ -1163,7 +1166,7 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   }
   SCORCH_HIP_CHECK(hipGetLastError());
   const unsigned medium_blocks = (unsigned)(M < kMediumWorkgroups ? M : kMediumWorkgroups);
-  spgemm_medium_kernel<T, NUMERIC, kSmallProducts, 2><<<medium_blocks, kBlockThreads, 0, stream>>>(
+  spgemm_medium_kernel<T, NUMERIC, kSmallProducts, 2, kBlockThreads><<<medium_blocks, kBlockThreads, 0, stream>>>(
       a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.small_rows, ws.counters, c_pos, c_crd, c_val);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (N <= 32 * 4096) {
@@ -1172,7 +1175,10 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
         <<<medium_blocks, kBlockThreads, 0, stream>>>(M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val,
                                                       ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   } else {
-    spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0><<<medium_blocks, kBlockThreads, 0, stream>>>(
+    // tables for 4096 products leave room for one workgroup per CU: as many threads as still fit
+    // beside them (with 8-byte sums, no more than 256)
+    constexpr int kThreads = sizeof(typename Acc<T>::type) > 4 ? kBlockThreads : kHugeThreads;
+    spgemm_medium_kernel<T, NUMERIC, kMediumProducts, 0, kThreads><<<medium_blocks, kThreads, 0, stream>>>(
         a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.medium_rows, ws.counters, c_pos, c_crd, c_val);
   }
   SCORCH_HIP_CHECK(hipGetLastError());
