@@ -1187,6 +1187,11 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   if (N <= 32 * 4096)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 4096, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
+  else if (!NUMERIC && N > 32 * 16384 && N <= 32 * 32768)
+    // the symbolic pass keeps no ranks or sums: its bitmap can be twice as wide, one range instead of two
+    spgemm_lds_bitmap_kernel<T, NUMERIC, NUMERIC ? 16384 : 32768, kHugeThreads, 0, 1, 3>
+        <<<lds_pool, kHugeThreads, 0, stream>>>(M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows,
+                                                ws.counters, c_pos, c_crd, c_val);
   else if (N <= kLdsBitmapColumns)
     spgemm_lds_bitmap_kernel<T, NUMERIC, 16384, kHugeThreads, 0, 1, 3><<<lds_pool, kHugeThreads, 0, stream>>>(
         M, N, a_pos, a_crd, a_val, b_pos, b_crd, b_val, ws.huge_rows, ws.counters, c_pos, c_crd, c_val);
