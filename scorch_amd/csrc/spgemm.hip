@@ -739,7 +739,8 @@ __global__ __launch_bounds__(THREADS) void spgemm_medium_kernel(
       }
     }
     int n = 0;
-    int at = block_scan_min_max<THREADS / kWaveSize>(mine, n, key_min, key_max, s_scan, s_red[0], s_red[1]);
+    int at = NUMERIC ? block_scan_min_max<THREADS / kWaveSize>(mine, n, key_min, key_max, s_scan, s_red[0], s_red[1])
+                     : block_exclusive_scan_n<THREADS / kWaveSize>(mine, s_scan, n);
     if (!NUMERIC) {
       if (tid == 0) c_pos[row] = n;
       __syncthreads();
