@@ -117,6 +117,50 @@ def test_spgemm_random_many_short_rows(oracle, seed):
         assert oracle.rel_fro(v, ref64) <= (1e-5 if dtype == np.float32 else 1e-13)
 
 
+def _rows_of(rng, rows, cols, lens, clustered):
+    """Sorted distinct column indices for rows of the given lengths; clustered rows draw theirs
+    from a window twice their length."""
+    out = []
+    for n in lens:
+        n = int(min(n, cols))
+        if clustered and n and rng.random() < 0.5:
+            span = min(cols, 2 * n)
+            start = int(rng.integers(0, cols - span + 1))
+            out.append(start + np.sort(rng.choice(span, n, replace=False)))
+        else:
+            out.append(np.sort(rng.choice(cols, n, replace=False)))
+    row_ptr = np.concatenate([[0], np.cumsum([c.size for c in out])]).astype(np.int32)
+    return row_ptr, np.concatenate(out or [np.zeros(0, np.int64)]).astype(np.int32)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_spgemm_random_across_the_tiers(oracle, seed):
+    """Operands drawn so that result rows land in every tier (a few entries to tens of
+    thousands), B from 100 to 1,048,576 columns wide (sums by column, LDS bitmap in one or more
+    ranges, hash tables), columns spread or clustered, mostly short rows with a few heavy ones."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = DTYPES[seed % 4]
+    M = int(rng.choice([3, 50, 700, 5000, 40000]))
+    K = int(rng.choice([40, 900, 6000]))
+    N = int(rng.choice([100, 3000, 20000, 140000, 600000, 1 << 20]))
+    a_lens = rng.integers(0, 6, M)
+    if rng.random() < 0.6:
+        heavy = rng.choice(M, min(M, 6), replace=False)
+        a_lens[heavy] = rng.integers(10, min(K, 400) + 1, heavy.size)
+    b_lens = rng.integers(0, 2 * int(rng.choice([2, 20, 120])) + 1, K)
+    arp, aci = _rows_of(rng, M, K, a_lens, False)
+    brp, bci = _rows_of(rng, K, N, b_lens, rng.random() < 0.4)
+    av, bv = draw_dense(rng, aci.size, dtype), draw_dense(rng, bci.size, dtype)
+    rp, ci, v = hip_spgemm(arp, aci, av, brp, bci, bv, N)
+    wrp, wci, wv = oracle.spgemm_csr_typed(arp, aci, av, brp, bci, bv, N)
+    assert np.array_equal(rp, wrp) and np.array_equal(ci, wci), (M, K, N)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(v, wv)
+    else:
+        _, _, ref64 = oracle.spgemm_csr_typed(arp, aci, av.astype(np.float64), brp, bci, bv.astype(np.float64), N)
+        assert oracle.rel_fro(v, ref64) <= (1e-5 if dtype == np.float32 else 1e-13)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_coordinate_products_random(oracle, seed):
     """spmm_coo_float and spmspm_coo_float on shuffled, partly repeated coordinates."""
