@@ -155,79 +155,6 @@ def vendor_spmm(pos, crd, val, B2d, steps, warmup):
     return {"call": "torch.sparse.mm(csr, dense)", "ms_per_step": round(ms, 4)}
 
 
-def probe_memory(args, dev) -> int:
-    """Streaming-read and random-row-gather rates of this GPU, from
-    libscorch_probes.so (scorch_amd/csrc/probes/membench.hip).  One JSON line."""
-    import numpy as np
-    import torch
-    from scorch_amd import build as hip_build
-    path = hip_build.PROBES_PATH
-    if not os.path.exists(path):
-        print("libscorch_probes.so is not built (python __graft_entry__.py)", file=sys.stderr)
-        return 1
-    P = ctypes.CDLL(path)
-    vp, i64 = ctypes.c_void_p, ctypes.c_int64
-    P.scorch_probe_stream_read.argtypes = [vp, i64, ctypes.c_int, vp, vp]
-    P.scorch_probe_gather_rows.argtypes = [vp, vp, i64, ctypes.c_int, ctypes.c_int, vp, vp]
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    table = torch.zeros(1 << 29, dtype=torch.float32, device=dev)      # 2 GiB
-    sink = torch.zeros(4, dtype=torch.float32, device=dev)
-    results = {"probe": "memory", "stream_read": [], "gather": []}
-    for mib in (2048, 512, 128):
-        for grid in (2048, 8192, 65536):
-            call = lambda: P.scorch_probe_stream_read(table.data_ptr(), mib << 20, grid, sink.data_ptr(), stream)
-            assert call() == 0
-            ms = _time_steps(call, args.steps, args.warmup)
-            results["stream_read"].append({"MiB": mib, "workgroups": grid, "ms": round(ms, 4),
-                                           "GBps": round((mib << 20) / ms / 1e6, 1)})
-    n = 1 << 24                                                         # 16 M gathers
-    rng = np.random.Generator(np.random.PCG64(7))
-    for rows in (1 << 20, 1 << 18, 1 << 16, 1 << 13):
-        idx = torch.from_numpy(rng.integers(0, rows, size=n, dtype=np.int64).astype(np.int32)).to(dev)
-        for row_bytes in (256, 512, 1024):
-            for in_flight in (4, 8, 16):
-                call = lambda: P.scorch_probe_gather_rows(table.data_ptr(), idx.data_ptr(), n, row_bytes,
-                                                          in_flight, sink.data_ptr(), stream)
-                assert call() == 0
-                ms = _time_steps(call, max(3, args.steps // 4), 1)
-                results["gather"].append({"table_rows": rows, "row_bytes": row_bytes,
-                                          "footprint_MiB": rows * row_bytes >> 20, "in_flight": in_flight,
-                                          "ms": round(ms, 4), "GBps": round(n * row_bytes / ms / 1e6, 1)})
-    print(json.dumps(results))
-    return 0
-
-
-def probe_compute(args, dev) -> int:
-    """Matrix-core and vector-ALU rates of this GPU, alone and in one loop, from
-    libscorch_probes.so (scorch_amd/csrc/probes/membench.hip).  One JSON line."""
-    import torch
-    from scorch_amd import build as hip_build
-    if not os.path.exists(hip_build.PROBES_PATH):
-        print("libscorch_probes.so is not built (python __graft_entry__.py)", file=sys.stderr)
-        return 1
-    P = ctypes.CDLL(hip_build.PROBES_PATH)
-    P.scorch_probe_compute.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
-    sink = torch.zeros(4, dtype=torch.float32, device=dev)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    iters, rows = 4000, []
-    for per_simd in (1, 2, 4, 8):
-        workgroups = 256 * per_simd                       # 256 CUs x 4 SIMDs x per_simd wavefronts
-        waves = workgroups * 4
-        row = {"wavefronts_per_simd": per_simd}
-        for mode, name in ((0, "matrix"), (1, "vector"), (2, "both")):
-            call = lambda: P.scorch_probe_compute(mode, workgroups, iters, sink.data_ptr(), stream)
-            assert call() == 0
-            ms = _time_steps(call, 3, 1)
-            row[name + "_ms"] = round(ms, 4)
-            if mode != 1:
-                row[name + "_matrix_tflops"] = round(waves * iters * 8 * 16384 / ms / 1e9, 1)
-            if mode != 0:
-                row[name + "_vector_tflops"] = round(waves * iters * 64 * 64 * 2 / ms / 1e9, 1)
-        rows.append(row)
-    print(json.dumps({"probe": "compute", "iterations": iters, "rows": rows}))
-    return 0
-
-
 def side_workload(args, dev) -> int:
     """Times one of the other workloads (not the headline metric): same JSON
     shape, HIP-event time per step, algorithmic and gather-model bandwidth."""
@@ -502,14 +429,6 @@ def main() -> int:
                     help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replay (SpMM side workloads)")
-    ap.add_argument("--probe-copy", action="store_true",
-                    help="run plain 1 GiB device copies instead (calibrates rocprofv3's FETCH_SIZE / "
-                         "WRITE_SIZE counters against a kernel of known traffic)")
-    ap.add_argument("--probe-compute", action="store_true",
-                    help="measure matrix-core and vector-ALU throughput alone and in one loop")
-    ap.add_argument("--probe-memory", action="store_true",
-                    help="measure what the GPU sustains for a streaming read and for random row "
-                         "gathers (kernels that only load): the ceilings the kernels are priced against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (the kernel shards by rows "
@@ -529,21 +448,6 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    if args.probe_copy:
-        n = 1 << 28                                  # 1 GiB of fp32 read, 1 GiB written per copy
-        src = torch.ones(n, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(args.warmup + args.steps):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"probe": "copy", "read_bytes_per_launch": 4 * n,
-                          "write_bytes_per_launch": 4 * n, "launches": args.warmup + args.steps}))
-        return 0
-
-    if args.probe_memory:
-        return probe_memory(args, dev)
-    if args.probe_compute:
-        return probe_compute(args, dev)
     if args.workload != "gcn_powerlaw":
         return side_workload(args, dev)
 

@@ -12,16 +12,15 @@ import os
 import shutil
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libscorch_hip.so")
-# memory-system probes for bench.py --probe; not part of the product library
-PROBES_SRC = os.path.join(SRC_DIR, "probes", "membench.hip")
-PROBES_PATH = os.path.join(PKG_DIR, "libscorch_probes.so")
+OBJ_DIR = os.path.join(SRC_DIR, "obj")  # one object per source, rebuilt only when stale
 
 HIPCC_FLAGS = [
-    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
     # packed fp32 instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA results stay in ordinary vector registers: the attention kernel feeds them
@@ -39,50 +38,65 @@ def sources():
     return sorted(glob.glob(os.path.join(SRC_DIR, "*.hip")))
 
 
-def _stale() -> bool:
-    if not os.path.exists(LIB_PATH):
-        return True
-    built = os.path.getmtime(LIB_PATH)
-    deps = sources() + glob.glob(os.path.join(SRC_DIR, "*.hpp")) + [
+def _headers():
+    return glob.glob(os.path.join(SRC_DIR, "*.hpp")) + [
         os.path.join(os.path.dirname(PKG_DIR), "include", "scorch_hip.h")]
+
+
+def _newer(target, deps) -> bool:
+    """True if `target` is missing or older than any of `deps`."""
+    if not os.path.exists(target):
+        return True
+    built = os.path.getmtime(target)
     return any(os.path.getmtime(d) > built for d in deps)
 
 
-def _hipcc(srcs, out, verbose):
+def _run_hipcc(args, verbose):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
-        raise RuntimeError(f"hipcc not found: cannot build {os.path.basename(out)}")
-    tmp = out + ".tmp"
-    cmd = [hipcc] + HIPCC_FLAGS + list(srcs) + ["-o", tmp]
+        raise RuntimeError("hipcc not found: cannot build libscorch_hip.so")
+    cmd = [hipcc] + list(args)
     if verbose:
-        print(" ".join(cmd))
+        print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # the host pass does not know the packed-fp32 feature name and says so: harmless
     noise = [l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and l.strip()]
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + "\n".join(noise))
     if verbose and noise:
-        print("\n".join(noise))
-    os.replace(tmp, out)
-    return out
+        print("\n".join(noise), flush=True)
+
+
+def _object_of(src) -> str:
+    return os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(src))[0] + ".o")
+
+
+def _compile(src, verbose):
+    obj = _object_of(src)
+    tmp = obj + ".tmp"
+    _run_hipcc(HIPCC_FLAGS + ["-c", src, "-o", tmp], verbose)
+    os.replace(tmp, obj)
+    return obj
 
 
 def build_library(force: bool = False, verbose: bool = False) -> str:
-    """Build libscorch_hip.so if it is missing or older than its sources
-    (always when ``force``).  Returns the library path."""
-    if not force and not _stale():
-        return LIB_PATH
-    return _hipcc(sources(), LIB_PATH, verbose)
-
-
-def build_probes(force: bool = False, verbose: bool = False) -> str:
-    """Build libscorch_probes.so (bench.py --probe) if missing, stale or forced."""
-    if not force and os.path.exists(PROBES_PATH) \
-            and os.path.getmtime(PROBES_PATH) >= os.path.getmtime(PROBES_SRC):
-        return PROBES_PATH
-    return _hipcc([PROBES_SRC], PROBES_PATH, verbose)
+    """Build libscorch_hip.so: every source that is newer than its object (all of
+    them when ``force``) is compiled, the sources side by side, and the objects
+    are linked.  Returns the library path."""
+    srcs = sources()
+    headers = _headers()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    todo = [s for s in srcs if force or _newer(_object_of(s), [s] + headers)]
+    if todo:
+        with ThreadPoolExecutor(max_workers=min(len(todo), os.cpu_count() or 1)) as pool:
+            list(pool.map(lambda s: _compile(s, verbose), todo))
+    objs = [_object_of(s) for s in srcs]
+    if todo or _newer(LIB_PATH, objs):
+        tmp = LIB_PATH + ".tmp"
+        _run_hipcc(["-shared", "-fPIC", "--offload-arch=gfx950", "-fvisibility=hidden"] + objs + ["-o", tmp], verbose)
+        os.replace(tmp, LIB_PATH)
+    return LIB_PATH
 
 
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv, verbose=True))
-    print(build_probes(force="--force" in sys.argv, verbose=True))

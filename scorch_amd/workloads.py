@@ -55,37 +55,75 @@ def spmm_uniform(M: int = 4096, K: int = 4096, N: int = 64, density: float = 0.0
             "col_idx": cols, "vals": vals, "B": B}
 
 
+def _degrees_with_mean(z: np.ndarray, mean_degree: float, cap: int, rng: np.random.Generator) -> np.ndarray:
+    """Integer degrees proportional to ``z``, capped at ``cap``, whose mean after
+    the cap is ``mean_degree``: the scale factor is found by bisection on the mean
+    of the capped values, then rounded stochastically (floor(x + u), u ~ U[0, 1))."""
+    if cap <= 0 or z.size == 0:
+        return np.zeros(z.size, dtype=np.int64)
+    target = min(mean_degree, float(cap))
+    lo, hi = 0.0, 1.0
+    while np.minimum(z * hi, cap).mean() < target and hi < 1e12:
+        hi *= 2.0
+    for _ in range(60):
+        mid = 0.5 * (lo + hi)
+        if np.minimum(z * mid, cap).mean() < target:
+            lo = mid
+        else:
+            hi = mid
+    scaled = np.minimum(z * hi, cap)
+    return np.clip(np.floor(scaled + rng.random(z.size)).astype(np.int64), 0, cap)
+
+
+def _distinct_neighbours(deg: np.ndarray, M: int, window: int, rng: np.random.Generator):
+    """``deg[i]`` distinct neighbours for node i, uniform over the nodes (or over
+    the ``window`` nodes around i): draw, drop repeats, and top up the rows that
+    lost entries until none is short.  Returns row-sorted (rows, cols), int32."""
+    def draw(rows):
+        cols = rng.integers(0, M, size=rows.size, dtype=np.int64)
+        if window > 0:
+            cols = (rows.astype(np.int64) + cols % window - window // 2) % M
+        return cols.astype(np.int32)
+
+    rows = np.repeat(np.arange(M, dtype=np.int32), deg)
+    rows, cols = _dedupe_sorted(rows, draw(rows), M)
+    for _ in range(200):
+        have = np.bincount(rows, minlength=M)
+        short = np.nonzero(have < deg)[0]
+        if short.size == 0:
+            break
+        r_new = np.repeat(short.astype(np.int32), (deg[short] - have[short]).astype(np.int64))
+        rows, cols = _dedupe_sorted(np.concatenate([rows, r_new]), np.concatenate([cols, draw(r_new)]), M)
+    return rows, cols
+
+
 def gcn_powerlaw(M: int = 1 << 20, N: int = 128, seed: int = SEEDS["gcn_powerlaw"],
                  zipf_a: float = 2.1, mean_degree: float = 16.0,
                  max_degree: int = 50_000, window: int = 0) -> Dict[str, np.ndarray]:
     """Power-law graph with the GCN normalisation D^-1/2 (A + I) D^-1/2.
 
-    Out-degrees are Zipf(``zipf_a``) draws capped at ``max_degree``, rescaled to
-    ``mean_degree`` with stochastic rounding and capped again; neighbours are
-    uniform over the nodes; a self-loop is added to every node that lacks one;
+    Out-degrees are Zipf(``zipf_a``) draws capped at ``max_degree``, rescaled so
+    that their mean *after* the cap is ``mean_degree`` (stochastic rounding);
+    every node gets that many distinct neighbours, uniform over the nodes (drawn
+    without replacement); a self-loop is added to every node that lacks one;
     ``deg`` is the row length of A + I and each entry is
     ``deg[row]^-1/2 * deg[col]^-1/2`` (the edge weight of
-    bench/bench_gcn.py:248-258).  Features are N(0, 1).
+    bench/bench_gcn.py:248-258).  Features are N(0, 1).  At the default size:
+    17,825,865 entries with the default seed (16 per node + the self-loops).
 
     ``window`` > 0 draws a node's neighbours from the ``window`` nodes around it
-    (wrapping at the ends) instead of from all nodes: the same degrees and entry
-    count, but rows that lie close together share neighbours.
+    (wrapping at the ends) instead of from all nodes, at most ``window`` of them:
+    rows that lie close together then share neighbours.
     """
     rng = _rng(seed)
     cap = min(max_degree, M - 1) if M > 1 else 0
-    z = np.minimum(rng.zipf(zipf_a, size=M), max(cap, 1)).astype(np.float64)
-    scaled = z * (mean_degree / z.mean())
-    deg = np.floor(scaled + rng.random(M)).astype(np.int64)
-    deg = np.clip(deg, 0, cap)
-    rows = np.repeat(np.arange(M, dtype=np.int32), deg)
-    cols = rng.integers(0, M, size=rows.size, dtype=np.int64)
     if window > 0:
-        cols = (rows.astype(np.int64) + cols % window - window // 2) % M
-    cols = cols.astype(np.int32)
+        cap = min(cap, window - 1)
+    z = np.minimum(rng.zipf(zipf_a, size=M), max(cap, 1)).astype(np.float64)
+    deg = _degrees_with_mean(z, mean_degree, cap, rng)
+    rows, cols = _distinct_neighbours(deg, M, window, rng)
     loops = np.arange(M, dtype=np.int32)
-    rows = np.concatenate([rows, loops])
-    cols = np.concatenate([cols, loops])
-    rows, cols = _dedupe_sorted(rows, cols, M)
+    rows, cols = _dedupe_sorted(np.concatenate([rows, loops]), np.concatenate([cols, loops]), M)
     row_ptr = csr_from_sorted_rows(rows, M)
     d = np.diff(row_ptr).astype(np.float32)
     inv_sqrt = (1.0 / np.sqrt(d)).astype(np.float32)

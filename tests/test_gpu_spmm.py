@@ -255,9 +255,13 @@ def test_uniform_workload_reference_size(oracle):
                                rtol=1e-4, atol=1e-5)
 
 
-def test_sae_decoder_workload(oracle):
-    """Sparse-autoencoder decoder shape (32 entries per row, N = 4096) at a quarter of the rows."""
-    w = workloads.sae_decoder(M=1024)
+@pytest.mark.parametrize("M", [1024, 4096])
+def test_sae_decoder_workload(oracle, M):
+    """Sparse-autoencoder decoder shape (32 entries per row, K = 16,384, N = 4096): at a quarter of the
+    rows, and at the full 4096 rows that `bench.py --workload sae_decoder` times (the work split
+    depends on the size, so the two take different chunk sizes)."""
+    w = workloads.sae_decoder(M=M)
+    assert w["K"] == 16_384 and w["N"] == 4096 and w["col_idx"].size == 32 * M
     got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
     assert oracle.rel_fro(got, oracle.spmm_fp64(w["row_ptr"], w["col_idx"], w["vals"], w["B"])) <= TOL
 
