@@ -104,6 +104,26 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_i64(int64_t M, int64_t K, int64_t N, int6
                             const int64_t *B, int64_t *C,
                             void *workspace, size_t workspace_bytes, void *stream);
 
+/* scorch_hip_spmm_csr_f32 for callers that cannot allocate device memory or
+ * hand over a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Same kernels and bit-identical results; the carry records live in a static
+ * device array of SCORCH_HIP_STATIC_SCRATCH_BYTES inside the library (every
+ * GPU the library has run on holds its copy until the process ends) instead of
+ * a workspace argument, and the call makes no hipMalloc / hipFree.
+ *   - Shapes whose scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, 4) exceeds
+ *     SCORCH_HIP_STATIC_SCRATCH_BYTES are refused with SCORCH_HIP_EWORKSPACE
+ *     (the 1,048,576-row, 17.8 M-entry, N = 128 product needs 38 MB and fits).
+ *   - All calls on one GPU share that GPU's array: calls that may overlap in
+ *     time on one GPU (two streams, two host threads) race on it.  Calls on one
+ *     stream are ordered and safe.
+ *   - The first call on a device looks the array's address up
+ *     (hipGetSymbolAddress); make that call outside a graph capture. */
+#define SCORCH_HIP_STATIC_SCRATCH_BYTES ((size_t)48 << 20)
+SCORCH_HIP_API int scorch_hip_spmm_csr_f32_static(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                   const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                   const float *B, float *C, void *stream);
+
 /* Benchmarking aid: scorch_hip_spmm_csr_f32 with each of its two kernels
  * bracketed by HIP events on `stream`.  Waits for the work to finish and
  * reports the durations in milliseconds: kernel_ms[0] the merge-path SpMM

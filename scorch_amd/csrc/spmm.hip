@@ -29,6 +29,8 @@
 // placed on XCDs so that a tile's slice of B stays in one L2 (map_workgroup).
 #include "common.hpp"
 
+#include <mutex>
+
 namespace scorch {
 
 constexpr int kItemsPerWave = 256;  // most merge items (row ends + nonzeros) per wavefront
@@ -876,6 +878,37 @@ int spmv_entry(const char *fn, int64_t M, int64_t K, int64_t nnz, const int32_t 
   return SCORCH_HIP_OK;
 }
 
+// ---- the entry point that allocates nothing --------------------------------------------------
+// Scratch for scorch_hip_spmm_csr_f32_static: the carry records that the other
+// entry points keep in the caller's workspace live in this array instead.  Every
+// GPU the library runs on holds its own copy, at its own address, until the
+// process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels are given the address that call returns.
+constexpr size_t kStaticScratchBytes = SCORCH_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];  // per device, filled on the first call there
+static std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`.
+static int static_scratch(const char *fn, void **out) {
+  int device = -1;
+  SCORCH_HIP_CHECK(hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: device ordinal %d is beyond the %d this library tracks", fn,
+                device, kMaxDevices);
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void *ptr = nullptr;
+    SCORCH_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(SCORCH_HIP_ERUNTIME, "%s: hipGetSymbolAddress returned a null address", fn);
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return SCORCH_HIP_OK;
+}
+
 }  // namespace scorch
 
 extern "C" {
@@ -954,6 +987,29 @@ int scorch_hip_spmm_csr_bias_act_f32(int64_t M, int64_t K, int64_t N, int64_t nn
                                                            B, bias, C, workspace, workspace_bytes,
                                                            stream);
   return scorch::fail(SCORCH_HIP_EINVAL, "%s: unknown activation %d", fn, act);
+}
+
+int scorch_hip_spmm_csr_f32_static(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                   const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                   const float *B, float *C, void *stream) {
+  const char *fn = "scorch_hip_spmm_csr_f32_static";
+  if (M < 0 || K < 0 || N < 0 || nnz < 0)
+    return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld K=%lld N=%lld nnz=%lld)", fn,
+                        (long long)M, (long long)K, (long long)N, (long long)nnz);
+  const size_t need = scorch::spmm_workspace_bytes(M, nnz, N, sizeof(float));
+  if (need > scorch::kStaticScratchBytes)
+    return scorch::fail(SCORCH_HIP_EWORKSPACE,
+                        "%s: this shape needs %zu bytes of scratch, the library's static buffer holds %zu; "
+                        "use scorch_hip_spmm_csr_f32 with a workspace of the caller's",
+                        fn, need, scorch::kStaticScratchBytes);
+  void *ws = nullptr;
+  if (M > 0 && N > 0)
+    if (int rc = scorch::static_scratch(fn, &ws)) return rc;
+  // nothing in the scratch has to start at zero: every chunk writes its carry row, and a carry
+  // value is read only where the carry row written in the same launch says there is one
+  return scorch::spmm_entry<float, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, nullptr, C,
+                                                     ws ? ws : (void *)nullptr,
+                                                     scorch::kStaticScratchBytes, stream);
 }
 
 }  // extern "C"

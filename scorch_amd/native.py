@@ -32,6 +32,7 @@ SIGNATURES = {
     "scorch_hip_spmm_csr_f64": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_i32": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_i64": (ctypes.c_int, _SPMM),
+    "scorch_hip_spmm_csr_f32_static": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "scorch_hip_spmm_csr_f32_timed": (ctypes.c_int, _SPMM + [ctypes.POINTER(ctypes.c_float)]),
     "scorch_hip_spmm_csr_bias_act_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr]),

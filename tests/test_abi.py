@@ -82,6 +82,18 @@ def test_spmm_rejects_bad_arguments(L):
     assert spmm(L, ws=ctypes.c_void_p(0x1010)) == native.EINVAL  # not 256-byte aligned
 
 
+def test_static_scratch_spmm_rejects_sizes_beyond_its_buffer(L):
+    f = L.scorch_hip_spmm_csr_f32_static
+    limit = int(re.search(r"#define SCORCH_HIP_STATIC_SCRATCH_BYTES \(\(size_t\)(\d+) << 20\)",
+                          open(HEADER).read()).group(1)) << 20
+    assert L.scorch_hip_spmm_csr_workspace_bytes(1 << 20, 60_000_000, 512, 4) > limit
+    assert f(1 << 20, 1 << 20, 512, 60_000_000, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EWORKSPACE
+    assert b"static buffer" in L.scorch_hip_last_error()
+    assert f(-1, 4, 4, 4, FAKE, FAKE, FAKE, FAKE, FAKE, NULL) == native.EINVAL
+    # the headline product fits
+    assert L.scorch_hip_spmm_csr_workspace_bytes(1 << 20, 17_825_865, 128, 4) <= limit
+
+
 def test_spmm_empty_output_is_a_no_op(L):
     assert spmm(L, M=0, nnz=0, C=NULL, ws=NULL) == native.OK
     assert spmm(L, N=0, C=NULL, ws=NULL) == native.OK
