@@ -1,18 +1,29 @@
-"""Headline benchmark: CSR SpMM, fp32, on the GCN-style power-law graph
-(1,048,576 nodes, N = 128 features) on one MI355X.
+"""Benchmark of the CSR sparse x dense kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--workload NAME]
 
-A step is one C = A @ B through the C ABI of libscorch_hip.so with A, B
-resident in HBM (the output buffer comes from torch's caching allocator).
-Prints ONE JSON line: whole-job GFLOP/s (2 * nnz * N flops per step, the
-reference's convention, tools/benchmark_spmm_variants.py:127-129), the memory
-roofline of the dominant kernel and the CPU baseline timed on this host.
+With no --workload the line is the headline: CSR SpMM, fp32, on the GCN-style
+power-law graph (1,048,576 nodes, N = 128 features), W untimed warm-up steps and
+then exactly K timed steps between two device synchronisations.  A step is one
+C = A @ B through the C ABI of libscorch_hip.so with A and B resident in HBM (the
+output buffer comes from torch's caching allocator).  `value` is whole-job
+GFLOP/s (2 * nnz * N flops per step, the reference's convention,
+tools/benchmark_spmm_variants.py:127-129).  The same line carries, under
+"configs", one record for each of the other four benchmark configurations
+(SpMM 4096^2, SDDMM 65,536^2, fused block-sparse attention, the
+sparse-autoencoder decoder), every one with the roofline of its dominant kernel
+and the reference's CPU path timed on this host.  --workload NAME prints that
+workload's record alone.
+
+Per-kernel durations are measured in this process with HIP events on the launch
+stream (scorch_hip_timing_begin / _end); what is computed once per operand
+(index inspection, chunk boundaries, the column-tile copy of a reused dense
+operand) happens in the warm-up calls, whose wall times are listed in
+"warmup_ms".
 """
 from __future__ import annotations
 
 import argparse
-import ctypes
 import json
 import os
 import statistics
@@ -23,38 +34,62 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
-WORKLOAD = "gcn_powerlaw_spmm_fp32"
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+HEADLINE = "gcn_powerlaw"
+CONFIG_WORKLOADS = ("spmm_uniform", "sddmm_uniform", "attention_blocksparse", "sae_decoder")
 
-# Bytes through the L2-to-fabric boundary per launch of the dominant kernel at
-# the headline size: FETCH_SIZE (4,292,650 KiB x 2.0, the factor a 1 GiB copy
-# kernel gives for this counter) + WRITE_SIZE (539,816 KiB x 1.0) from two
-# rocprofv3 --pmc runs of this script.  It is a measured constant, valid for
-# the default workload only; the summary with the commands is
-# profiles/spmm_merge_kernel_gcn_powerlaw.md.
-MEASURED_TRAFFIC_BYTES = 9_344_118_000
+# Bytes through the L2-to-fabric boundary per launch of each configuration's
+# dominant kernel at its default size: FETCH_SIZE (KiB, x 2.0: the factor a
+# 1 GiB device copy gives for this counter on gfx950) + WRITE_SIZE (KiB, x 1.0)
+# from two rocprofv3 --pmc runs of `python3 bench.py --workload NAME --no-cpu`.
+# Measured constants: valid for the default sizes and for the kernels as they
+# stood at the named commit only (null for anything else); the summaries with
+# the commands are the named files.
+MEASURED_TRAFFIC = {
+    # filled in from the profiles named; see profiles/*.md
+}
 
 
-def algorithmic_bytes(M, K, N, nnz):
+def measured_traffic(name, default_size):
+    rec = MEASURED_TRAFFIC.get(name)
+    if rec is None or not default_size:
+        return None, None
+    return rec["bytes"], {"commit": rec["commit"], "profile": rec["profile"]}
+
+
+def spmm_algorithmic_bytes(M, K, N, nnz):
     """Every array touched once: col_idx + vals, row_ptr, B, C (fp32 / int32)."""
     return 8 * nnz + 4 * (M + 1) + 4 * K * N + 4 * M * N
 
 
-def gather_bytes(M, N, nnz):
+def spmm_gather_bytes(M, N, nnz):
     """No-reuse model: a B row re-read for every nonzero."""
     return 8 * nnz + 4 * (M + 1) + 4 * nnz * N + 4 * M * N
 
 
-def cpu_baseline(w, repeats=5):
+# ---- CPU baselines: the reference's own kernels (oracle/_ref) on the host cores ------------------
+def _timed_calls(fn, repeats):
+    times = []
+    for i in range(repeats + 1):
+        t0 = time.perf_counter()
+        out = fn()
+        dt = time.perf_counter() - t0
+        del out
+        if i:
+            times.append(dt)
+    return statistics.median(times)
+
+
+def cpu_baseline_spmm(w, repeats=5):
     """The reference's spmm_csr_float_v2 (oracle/_ref, compiled from the
     reference's sources) or, where that module is absent, this repository's C
-    restatement of it, timed on the host cores on the same inputs.  The timed
-    region is the whole native call, as the reference's own eval_time is: it
-    includes allocating and zero-filling C."""
+    restatement of it, on the host cores and the same inputs.  The timed region
+    is the whole native call, as the reference's own eval_time is: it includes
+    allocating and zero-filling C."""
     from oracle import oracle as O
     M, N, nnz = w["M"], w["N"], int(w["col_idx"].size)
-    flops = 2.0 * nnz * N
-    kind, times = "port", []
+    kind, med = "port", None
     if O.have_ref():
         try:
             import torch
@@ -62,29 +97,15 @@ def cpu_baseline(w, repeats=5):
             pos, crd = torch.from_numpy(w["row_ptr"]), torch.from_numpy(w["col_idx"])
             val, Bf = torch.from_numpy(w["vals"]), torch.from_numpy(w["B"]).reshape(-1)
             args = ([M, N], [M, w["K"]], [[], [pos, crd]], val, [w["K"], N], [[], []], Bf)
-            for i in range(repeats + 1):
-                t0 = time.perf_counter()
-                out = mod.spmm_csr_float_v2(*args)
-                dt = time.perf_counter() - t0
-                del out
-                if i:
-                    times.append(dt)
+            med = _timed_calls(lambda: mod.spmm_csr_float_v2(*args), repeats)
             kind = "reference"
         except Exception as exc:  # module built for another host
-            print(f"[bench] reference module unusable here ({exc}); timing the C restatement",
-                  file=sys.stderr)
-            times = []
-    if not times:
+            print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
+    if med is None:
         import numpy as np
         out = np.empty((M, N), dtype=np.float32)
-        for i in range(repeats + 1):
-            t0 = time.perf_counter()
-            O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"], out=out)
-            dt = time.perf_counter() - t0
-            if i:
-                times.append(dt)
-    med = statistics.median(times)
-    return {"value": round(flops / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
+        med = _timed_calls(lambda: O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"], out=out), repeats)
+    return {"value": round(2.0 * nnz * N / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
             "kind": kind, "ms_per_step": round(med * 1e3, 3),
             "sample": f"full workload (M={M}, nnz={nnz}, N={N}), median of {repeats} calls after 1 "
                       "warm-up, whole native call incl. allocating and zeroing C"}
@@ -96,126 +117,368 @@ def cpu_baseline_sddmm(w, repeats=5):
     from oracle import oracle as O
     nnz, K = int(w["col_idx"].size), w["K"]
     kind = "reference" if O.have_ref() else "port"
-    times = []
-    for i in range(repeats + 1):
-        t0 = time.perf_counter()
-        try:
-            if kind == "reference":
-                O.ref_sddmm_coo(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"], (w["M"], w["n_cols"]))
-            else:
-                O.sddmm_coo_f32(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])
-        except Exception as exc:  # module built for another host
-            if kind == "port":
-                raise
-            print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
-            kind = "port"
-            continue
-        if i:
-            times.append(time.perf_counter() - t0)
-    med = statistics.median(times)
+
+    def ref():
+        return O.ref_sddmm_coo(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"], (w["M"], w["n_cols"]))
+
+    def port():
+        return O.sddmm_coo_f32(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])
+
+    try:
+        med = _timed_calls(ref if kind == "reference" else port, repeats)
+    except Exception as exc:  # module built for another host
+        if kind == "port":
+            raise
+        print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
+        kind, med = "port", _timed_calls(port, repeats)
     return {"value": round((2.0 * nnz * K + nnz) / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
             "kind": kind, "ms_per_step": round(med * 1e3, 3),
-            "sample": f"full workload (nnz={nnz}, K={K}), median of {len(times)} calls after 1 warm-up, "
+            "sample": f"full workload (nnz={nnz}, K={K}), median of {repeats} calls after 1 warm-up, "
                       "incl. wrapping the operands"}
 
 
-def _time_steps(fn, steps, warmup):
+def cpu_baseline_attention(w, heads=2):
+    """The per-head composition of the reference's attention benchmark
+    (bench/bench_sparse_transformer.py:354-372) on the host cores, fp32, for a
+    sample of the heads: its SDDMM and SpMM kernels (oracle/_ref, or the C
+    restatements where that module is absent) with the CSR row softmax between
+    them (the oracle's C restatement of the benchmark's torch composition)."""
+    import numpy as np
+    from oracle import oracle as O
+    from scorch_amd import workloads
+    S, D, H = w["S"], w["D"], w["H"]
+    pos, crd = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], w["block"])
+    rows = np.repeat(np.arange(S, dtype=np.int32), np.diff(pos))
+    ones = np.ones(crd.size, np.float32)
+    kind = "reference" if O.have_ref() else "port"
+
+    def head(h, use_ref):
+        q, k, v = (np.ascontiguousarray(w[n][h]) for n in ("q", "k", "v"))
+        if use_ref:
+            s = O.ref_sddmm_coo(rows, crd, ones, q, k, (S, S))[2]
+            p = O.softmax_csr_f32(pos, s, float(w["scale"]))
+            return O.ref_spmm("spmm_csr_float_v2", pos, crd, p, v)
+        s = O.sddmm_coo_f32(rows, crd, ones, q, k)
+        p = O.softmax_csr_f32(pos, s, float(w["scale"]))
+        return O.spmm_csr_f32_v2(pos, crd, p, v)
+
+    try:
+        head(0, kind == "reference")
+    except Exception as exc:
+        if kind == "port":
+            raise
+        print(f"[bench] reference module unusable here ({exc}); timing the C restatements", file=sys.stderr)
+        kind = "port"
+        head(0, False)
+    t0 = time.perf_counter()
+    for h in range(heads):
+        head(h, kind == "reference")
+    per_head = (time.perf_counter() - t0) / heads
+    nnz = int(crd.size)
+    return {"value": round(4.0 * nnz * D / per_head / 1e12, 4), "unit": "TFLOP/s", "cores": O.num_threads(),
+            "kind": kind, "ms_per_step": round(per_head * H * 1e3, 1),
+            "sample": f"{heads} of {H} heads after 1 warm-up head (nnz per head {nnz}); ms_per_step is the per-head "
+                      f"time x {H}; SDDMM -> row softmax -> SpMM per head in fp32, the softmax leg is the "
+                      "oracle's C restatement of the benchmark's torch ops"}
+
+
+# ---- device timing ----------------------------------------------------------------------------
+_blocker = None
+
+
+def _time_steps(fn, steps, warmup, rounds=3):
+    """GPU time per step of `fn`, HIP events on torch's current stream (the
+    stream the kernels are launched on).  A few large device fills are queued
+    first, so that the step launches are all enqueued before the GPU reaches the
+    first of them: the interval is then the GPU's time for the steps, not the
+    host's time to issue them.  Median of `rounds` such measurements."""
     import torch
+    global _blocker
+    if _blocker is None:
+        _blocker = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
     for _ in range(warmup):
         fn()
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
+    results = []
+    for _ in range(rounds):
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(3):
+            _blocker.fill_(1.0)
+        start.record()
+        for _ in range(steps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        results.append(start.elapsed_time(stop) / steps)
+    return statistics.median(results)
+
+
+def _kernel_times(fn, samples):
+    """Average duration (ms) of each kernel `fn` launches, in launch order."""
+    from scorch_amd import native
+    rows = [native.kernel_times(fn) for _ in range(samples)]
+    width = min(len(r) for r in rows)
+    return [sum(r[i] for r in rows) / len(rows) for i in range(width)]
+
+
+def _warmup_calls(fn, warmup):
+    """The warm-up calls one by one with their wall time (ms): the first builds
+    whatever is computed once per operand."""
+    import torch
+    out = []
+    for _ in range(warmup):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
         fn()
-    stop.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(stop) / steps
+        torch.cuda.synchronize()
+        out.append(round((time.perf_counter() - t0) * 1e3, 3))
+    return out
 
 
 def _vendor_time(call_name, fn, steps, warmup):
     """Times a torch routine on the same operands; an error becomes a field."""
     try:
-        return {"call": call_name, "ms_per_step": round(_time_steps(fn, steps, warmup), 4)}
+        return {"call": call_name, "ms_per_step": round(_time_steps(fn, steps, warmup, rounds=1), 4)}
     except RuntimeError as err:
         return {"call": call_name, "error": str(err).splitlines()[0]}
 
 
-def vendor_spmm(pos, crd, val, B2d, steps, warmup):
-    """torch.sparse.mm on the same CSR operands (torch routes it to the ROCm
-    sparse library): a second GPU implementation timed beside ours.  Returns a
-    JSON-ready dict; never part of `value`."""
-    import torch
-    M = pos.numel() - 1
-    A = torch.sparse_csr_tensor(pos, crd, val, size=(M, B2d.shape[0]))
-    try:
-        ms = _time_steps(lambda: torch.sparse.mm(A, B2d), steps, warmup)
-    except RuntimeError as err:                       # e.g. unsupported size
-        return {"call": "torch.sparse.mm(csr, dense)", "error": str(err).splitlines()[0]}
-    return {"call": "torch.sparse.mm(csr, dense)", "ms_per_step": round(ms, 4)}
+def _hbm_roofline(kernel, kernel_ms, algo, traffic, provenance, extra=None):
+    achieved = algo / (kernel_ms * 1e-3) / 1e9
+    out = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+           "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "algorithmic_bytes": algo,
+           "kernel_ms_avg": round(kernel_ms, 5)}
+    if provenance:
+        out["traffic_measured_at"] = provenance
+    if extra:
+        out.update(extra)
+    return out
 
 
-def side_workload(args, dev) -> int:
-    """Times one of the other workloads (not the headline metric): same JSON
-    shape, HIP-event time per step, algorithmic and gather-model bandwidth."""
+def _t(a):
+    import numpy as np
     import torch
-    from scorch_amd import workloads
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+# ---- the benchmark configurations ----------------------------------------------------------------
+def run_spmm(name, args, headline=False):
+    """CSR SpMM fp32: gcn_powerlaw (the headline), spmm_uniform, sae_decoder."""
+    import torch
     from scorch_amd import scorch_ops_hip as H
-    t = lambda a: torch.from_numpy(a).to(dev)
-    if args.workload == "attention_blocksparse":
-        w = workloads.attention_blocksparse()
-        Hh, S, D = w["H"], w["S"], w["D"]
-        q, k, v = (t(w[n]).to(torch.bfloat16) for n in ("q", "k", "v"))
-        brp, bci = t(w["block_row_ptr"]), t(w["block_col_idx"])
-        nnz = int(w["block_col_idx"].size) * w["block"] ** 2
-        fn = lambda: H.attn_blocksparse_bf16(q, k, v, brp, bci, float(w["scale"]))
-        ms = _time_steps(fn, args.steps, args.warmup)
-        flops = 4.0 * nnz * D * Hh
-        algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
-        extra = {}
-        if args.vendor:
-            # (a) the composition the reference's benchmark uses, per head and in fp32, on this
-            # package's own kernels: SDDMM -> row softmax -> SpMM (bench_sparse_transformer.py:354-372)
-            import numpy as np
-            blk = w["block"]
-            rows_b = np.repeat(np.arange(brp.numel() - 1), np.diff(w["block_row_ptr"]))
-            dense_blocks = np.zeros((S // blk, S // blk), bool)
-            dense_blocks[rows_b, w["block_col_idx"]] = True
-            mask = torch.from_numpy(np.kron(dense_blocks, np.ones((blk, blk), bool))).to(dev)
-            csr = mask.to(torch.float32).to_sparse_csr()
-            pos, crd = csr.crow_indices().to(torch.int32), csr.col_indices().to(torch.int32)
-            ones = torch.ones(crd.numel(), device=dev)
-            qf, kf, vf = q.float(), k.float(), v.float()
+    from scorch_amd import workloads
+    t0 = time.time()
+    if name == "gcn_powerlaw":
+        w = workloads.gcn_powerlaw(M=args.rows, N=args.features, window=args.window)
+        default_size = (args.rows, args.features, args.window) == (1 << 20, 128, 0)
+    elif name == "spmm_uniform":
+        w, default_size = workloads.spmm_uniform(), True
+    else:
+        w, default_size = workloads.sae_decoder(), True
+    M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
+    print(f"[bench] generated {name}: M={M} K={K} nnz={nnz} N={N} in {time.time() - t0:.1f}s", file=sys.stderr)
+    pos, crd, val, B = _t(w["row_ptr"]), _t(w["col_idx"]), _t(w["vals"]), _t(w["B"]).reshape(-1)
+    call = ([M, N], [M, K], [[], [pos, crd]], val, [K, N], [[], []], B)
+    fn = lambda: H.spmm_csr_float_v2(*call)
 
-            def unfused():
-                outs = []
-                for h in range(Hh):
-                    sc = H.sddmm_csr_float([S, S], [S, S], [[], [pos, crd]], ones, [S, D], [[], []],
-                                           qf[h].reshape(-1), [S, D], [[], []], kf[h].reshape(-1))
-                    p = H.softmax_csr_float(pos, sc.storage.value, float(w["scale"]))
-                    outs.append(H.spmm_csr_float_v2([S, D], [S, S], [[], [pos, crd]], p, [S, D], [[], []],
-                                                    vf[h].reshape(-1)).storage.value)
-                return outs
+    warm = _warmup_calls(fn, args.warmup)
+    if headline:
+        # the contract's timed region: exactly K steps between two synchronisations, wall clock
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t_begin = time.perf_counter()
+        start.record()
+        for _ in range(args.steps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t_begin) * 1e3 / args.steps
+        event_ms = start.elapsed_time(stop) / args.steps
+    else:
+        ms_per_step = event_ms = _time_steps(fn, args.steps, 0)
 
-            extra["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM per head (this package, fp32)",
-                                                          unfused, max(args.steps // 4, 2), 1)
-            # (b) torch's dense attention with the same mask
-            import torch.nn.functional as F
-            extra["vendor_library"] = _vendor_time(
-                "F.scaled_dot_product_attention(bf16, dense boolean mask)",
-                lambda: F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask[None, None],
-                                                       scale=float(w["scale"])), max(args.steps // 4, 2), 1)
-        print(json.dumps({**extra,
-                          "metric": "fused block-sparse attention TFLOP/s", "value": round(flops / ms / 1e9, 2),
-                          "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
-                          "warmup": args.warmup, "dtype": "bf16", "data": "synthetic",
-                          "higher_is_better": True,
-                          "config": {"workload": "attention_blocksparse_bf16", "S": S, "H": Hh, "D": D,
-                                     "block": w["block"], "active_blocks": int(bci.numel()),
-                                     "nnz_per_head": nnz},
-                          "mfma_frac_of_2.5PFLOPs": round(flops / ms / 1e9 / 2500.0, 4),
-                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1)}))
-        return 0
+    tiled = getattr(B, "_scorch_tiled", None) is not None
+    plan = getattr(pos, "_scorch_plan", None)
+    kernels = _kernel_times(fn, min(args.steps, 10))
+    if tiled:
+        path, names = "tiled", ["spmm_tiled_clear_kernel", "spmm_tiled_kernel<float,0>", "spmm_fixup_kernel<float,1,0>"]
+    elif len(kernels) == 1:
+        lanes = 64 if N % 4 else max(8, min(64, 1 << (max(N // 4, 1) - 1).bit_length()))
+        path, names = "rows", [f"spmm_rows_kernel<float,{4 if N % 4 == 0 else 1},{lanes}>"]
+    else:
+        vec = 4 if N % 256 == 0 else 2 if N % 128 == 0 else 1
+        path = "merge"
+        names = [f"spmm_merge_kernel<float,{vec},0>" if N * 4 > 256 else "spmm_grouped_kernel<float,...>",
+                 "spmm_fixup_kernel<float,...>"]
+    dominant = max(range(len(kernels)), key=lambda i: kernels[i])
+    # a single-launch step: the queued per-step time is the kernel's duration without the events'
+    # own overhead, which matters for kernels of a few microseconds
+    kernel_ms = event_ms if len(kernels) == 1 and not headline else kernels[dominant]
+
+    flops = 2.0 * nnz * N
+    algo, gather = spmm_algorithmic_bytes(M, K, N, nnz), spmm_gather_bytes(M, N, nnz)
+    traffic, provenance = measured_traffic(name, default_size)
+    rec = {
+        "metric": "CSR SpMM GFLOP/s + HBM GB/s (% peak), power-law 1M rows, N=128 fp32" if headline
+                  else "CSR SpMM GFLOP/s",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2), "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name + "_spmm_fp32" if name == "gcn_powerlaw" else name + "_fp32",
+                   "rows": M, "cols": K, "nnz": nnz, "features": N,
+                   "seed": workloads.SEEDS[name]},
+        "warmup_ms": warm,
+        "path": path,
+        "longest_row": plan.max_row if plan is not None else None,
+        "kernels_ms": {n: round(k, 5) for n, k in zip(names, kernels)},
+        "event_ms_per_step": round(event_ms, 5),
+        "hbm_gbps_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
+        "roofline": _hbm_roofline(names[dominant], kernel_ms, algo, traffic, provenance,
+                                  {"gather_model_bytes": gather,
+                                   "gather_model_gbps": round(gather / (kernel_ms * 1e-3) / 1e9, 1)}),
+    }
+    if name == "gcn_powerlaw":
+        rec["config"].update({"degree": "zipf(2.1), mean 16 after the cap of 50000, distinct neighbours, + self-loops",
+                              "values": "D^-1/2 (A+I) D^-1/2"})
+        if args.window:
+            rec["config"]["neighbour_window"] = args.window
+    if args.graph and not headline:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        rec["ms_per_step_graph_replay"] = round(_time_steps(graph.replay, args.steps, 2), 5)
+    if args.vendor:
+        A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, K))
+        B2 = B.reshape(K, N)
+        rec["vendor_library"] = _vendor_time("torch.sparse.mm(csr, dense)", lambda: torch.sparse.mm(A_t, B2),
+                                             max(args.steps // 2, 2), 1)
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline_spmm(w)
+    return rec
+
+
+def run_sddmm(args):
+    import torch
+    from scorch_amd import scorch_ops_hip as H
+    from scorch_amd import workloads
+    w = workloads.sddmm_uniform()
+    M, n_cols, K, nnz = w["M"], w["n_cols"], w["K"], int(w["col_idx"].size)
+    pos, crd, val, A, B = _t(w["row_ptr"]), _t(w["col_idx"]), _t(w["vals"]), _t(w["A"]), _t(w["B"])
+    rows = _t(w["row_idx"])
+    Af, Bf = A.reshape(-1), B.reshape(-1)
+    csr = lambda: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [pos, crd]], val, [M, K], [[], []], Af,
+                                    [n_cols, K], [[], []], Bf)
+    coo = lambda: H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows], [crd]], val, [M, K], [[], []], Af,
+                                             [n_cols, K], [[], []], Bf)
+    warm = _warmup_calls(csr, args.warmup)
+    ms = _time_steps(csr, args.steps, 0)
+    ms_coo = _time_steps(coo, args.steps, 2)
+    flops = 2.0 * nnz * K + nnz
+    # every array once: row_ptr, col_idx, mask values, A, B, result values; the CSR-mask kernel
+    # also writes the result's row coordinates, 4 more bytes per entry (not counted)
+    algo = 4 * (M + 1) + 4 * nnz * 3 + 4 * M * K + 4 * n_cols * K
+    gather = algo - 4 * n_cols * K + 4 * nnz * K
+    traffic, provenance = measured_traffic("sddmm_uniform", True)
+    rec = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+           "ms_per_step_coo_mask": round(ms_coo, 5), "higher_is_better": True, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K,
+                      "seed": workloads.SEEDS["sddmm_uniform"]},
+           "warmup_ms": warm,
+           "roofline": _hbm_roofline("sddmm_kernel<16,4,false,false>", ms, algo, traffic, provenance,
+                                     {"row_coordinate_output_bytes": 4 * nnz, "gather_model_bytes": gather,
+                                      "gather_model_gbps": round(gather / ms / 1e6, 1)})}
+    if args.vendor:
+        mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
+        Bt = B.t().contiguous()
+        rec["vendor_library"] = _vendor_time("torch.sparse.sampled_addmm(mask, A, B^T, beta=0)",
+                                             lambda: torch.sparse.sampled_addmm(mask, A, Bt, beta=0.0),
+                                             max(args.steps // 2, 2), 1)
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline_sddmm(w)
+    return rec
+
+
+def run_attention(args):
+    import numpy as np
+    import torch
+    from scorch_amd import scorch_ops_hip as H
+    from scorch_amd import workloads
+    w = workloads.attention_blocksparse()
+    Hh, S, D = w["H"], w["S"], w["D"]
+    q, k, v = (_t(w[n]).to(torch.bfloat16) for n in ("q", "k", "v"))
+    brp, bci = _t(w["block_row_ptr"]), _t(w["block_col_idx"])
+    nnz = int(w["block_col_idx"].size) * w["block"] ** 2
+    fn = lambda: H.attn_blocksparse_bf16(q, k, v, brp, bci, float(w["scale"]))
+    warm = _warmup_calls(fn, args.warmup)
+    ms = _time_steps(fn, args.steps, 0)
+    flops = 4.0 * nnz * D * Hh
+    algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
+    achieved = flops / ms / 1e9
+    traffic, provenance = measured_traffic("attention_blocksparse", True)
+    rec = {"metric": "fused block-sparse attention TFLOP/s", "value": round(achieved, 2), "unit": "TFLOP/s",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+           "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "attention_blocksparse_bf16", "S": S, "H": Hh, "D": D, "block": w["block"],
+                      "active_blocks": int(bci.numel()), "nnz_per_head": nnz,
+                      "seed": workloads.SEEDS["attention_blocksparse"]},
+           "warmup_ms": warm,
+           "roofline": {"bound": "mfma", "kernel": "attn_blocksparse_kernel<false>", "achieved": round(achieved, 1),
+                        "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
+                        "flops": flops, "algorithmic_bytes": algo, "kernel_ms_avg": round(ms, 5),
+                        "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                        **({"traffic_measured_at": provenance} if provenance else {})}}
+    if args.vendor:
+        # (a) the composition the reference's benchmark uses, per head and in fp32, on this
+        # package's own kernels: SDDMM -> row softmax -> SpMM (bench_sparse_transformer.py:354-372)
+        pos_np, crd_np = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], w["block"])
+        pos, crd = _t(pos_np), _t(crd_np)
+        ones = torch.ones(crd.numel(), device="cuda")
+        qf, kf, vf = q.float(), k.float(), v.float()
+
+        def unfused():
+            outs = []
+            for h in range(Hh):
+                sc = H.sddmm_csr_float([S, S], [S, S], [[], [pos, crd]], ones, [S, D], [[], []],
+                                       qf[h].reshape(-1), [S, D], [[], []], kf[h].reshape(-1))
+                p = H.softmax_csr_float(pos, sc.storage.value, float(w["scale"]))
+                outs.append(H.spmm_csr_float_v2([S, D], [S, S], [[], [pos, crd]], p, [S, D], [[], []],
+                                                vf[h].reshape(-1)).storage.value)
+            return outs
+
+        rec["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM per head (this package, fp32)",
+                                                    unfused, max(args.steps // 4, 2), 1)
+        # (b) torch's dense attention with the same mask
+        import torch.nn.functional as F
+        blk = w["block"]
+        rows_b = np.repeat(np.arange(brp.numel() - 1), np.diff(w["block_row_ptr"]))
+        dense_blocks = np.zeros((S // blk, S // blk), bool)
+        dense_blocks[rows_b, w["block_col_idx"]] = True
+        mask = torch.from_numpy(np.kron(dense_blocks, np.ones((blk, blk), bool))).cuda()
+        rec["vendor_library"] = _vendor_time(
+            "F.scaled_dot_product_attention(bf16, dense boolean mask)",
+            lambda: F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=mask[None, None],
+                                                   scale=float(w["scale"])), max(args.steps // 4, 2), 1)
+    if not args.no_cpu:
+        rec["cpu_baseline"] = cpu_baseline_attention(w)
+    return rec
+
+
+# ---- workloads beside the five configurations -------------------------------------------------------
+def run_extra(args):
+    import numpy as np
+    import torch
+    from scorch_amd import scorch_ops_hip as H
+    from scorch_amd import workloads
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32", "data": "synthetic",
+            "higher_is_better": True}
     if args.workload == "gcn_forward":
         # The two-layer GCN forward pass of the reference's graph benchmark
         # (bench/bench_gcn.py:320-357) on the headline graph: linear -> A_hat x -> + bias
@@ -226,8 +489,8 @@ def side_workload(args, dev) -> int:
         w = workloads.gcn_powerlaw(M=args.rows, N=args.features)
         M, nnz = w["M"], int(w["col_idx"].size)
         hidden, classes = 128, 64
-        adj = scorch.STensor.from_csr_arrays(t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), (M, M))
-        x0 = t(w["B"])
+        adj = scorch.STensor.from_csr_arrays(_t(w["row_ptr"]), _t(w["col_idx"]), _t(w["vals"]), (M, M))
+        x0 = _t(w["B"])
         gen = torch.Generator(device="cuda").manual_seed(5)
         weights = {"w1": torch.randn(hidden, args.features, device="cuda", generator=gen) * 0.1,
                    "b1": torch.randn(hidden, device="cuda", generator=gen) * 0.1,
@@ -264,39 +527,33 @@ def side_workload(args, dev) -> int:
         ms_unfused = _time_steps(unfused, args.steps, args.warmup)
         out = {"metric": "two-layer GCN forward passes per second", "value": round(1e3 / ms_fused, 2),
                "unit": "1/s", "ms_per_step": round(ms_fused, 4), "ms_per_step_unfused": round(ms_unfused, 4),
-               "max_abs_difference_fused_unfused": err, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-               "dtype": "f32", "data": "synthetic", "higher_is_better": True,
+               "max_abs_difference_fused_unfused": err, **base,
                "config": {"workload": "gcn_forward_fp32", "rows": M, "nnz": nnz, "features": args.features,
                           "hidden": hidden, "classes": classes}}
         if args.vendor:
-            out["vendor_library"] = _vendor_time("torch.sparse.mm in the same forward pass", vendor, args.steps,
-                                                 args.warmup)
-        print(json.dumps(out))
-        return 0
+            out["vendor_library"] = _vendor_time("torch.sparse.mm in the same forward pass", vendor,
+                                                 max(args.steps // 2, 2), 1)
+        return out
     if args.workload == "softmax_rows":
         # every row --row-length entries long, or a causal mask (row i has i + 1) with --row-length 0
-        import numpy as np
         M = args.rows if args.rows != 1 << 20 else 8192
         lens = np.full(M, args.row_length, np.int64) if args.row_length > 0 else np.arange(1, M + 1, dtype=np.int64)
-        pos = t(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
+        pos = _t(np.concatenate([[0], np.cumsum(lens)]).astype(np.int32))
         nnz = int(lens.sum())
         val = torch.randn(nnz, device="cuda")
         ms = _time_steps(lambda: H.softmax_csr_float(pos, val, 1.0), args.steps, args.warmup)
         algo = 8 * nnz + 4 * (M + 1)
-        print(json.dumps({"metric": "CSR row softmax GFLOP/s (4 flops per entry)",
-                          "value": round(4.0 * nnz / ms / 1e6, 2), "unit": "GFLOP/s", "ms_per_step": round(ms, 4),
-                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
-                          "data": "synthetic", "higher_is_better": True,
-                          "config": {"workload": "softmax_rows_fp32", "rows": M, "nnz": nnz,
-                                     "row_length": args.row_length if args.row_length > 0 else "causal"},
-                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
-                          "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}))
-        return 0
+        return {"metric": "CSR row softmax GFLOP/s (4 flops per entry)", "value": round(4.0 * nnz / ms / 1e6, 2),
+                "unit": "GFLOP/s", "ms_per_step": round(ms, 4), **base,
+                "config": {"workload": "softmax_rows_fp32", "rows": M, "nnz": nnz,
+                           "row_length": args.row_length if args.row_length > 0 else "causal"},
+                "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     if args.workload in ("spmv_powerlaw", "softmax_powerlaw"):
         w = workloads.gcn_powerlaw(M=args.rows, N=1)
         M, nnz = w["M"], int(w["col_idx"].size)
-        pos, crd, val = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"])
-        x = t(w["B"]).reshape(-1)
+        pos, crd, val = _t(w["row_ptr"]), _t(w["col_idx"]), _t(w["vals"])
+        x = _t(w["B"]).reshape(-1)
         if args.workload == "spmv_powerlaw":
             fn = lambda: H.prebuilt_spmv_csr_f32([M], [M, M], [[], [pos, crd]], val, [M], [[]], x)
             algo, flops, name = 8 * nnz + 4 * (M + 1) + 8 * M, 2.0 * nnz, "CSR SpMV GFLOP/s"
@@ -304,107 +561,47 @@ def side_workload(args, dev) -> int:
             fn = lambda: H.softmax_csr_float(pos, val, 1.0)
             algo, flops, name = 8 * nnz + 4 * (M + 1), 4.0 * nnz, "CSR row softmax GFLOP/s (4 flops per entry)"
         ms = _time_steps(fn, args.steps, args.warmup)
-        vendor = None
+        out = {"metric": name, "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s", "ms_per_step": round(ms, 4),
+               **base, "config": {"workload": args.workload + "_fp32", "rows": M, "nnz": nnz},
+               "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+               "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}
         if args.vendor and args.workload == "spmv_powerlaw":
             A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, M))
-            vendor = _vendor_time("torch.mv(csr, x)", lambda: torch.mv(A_t, x), args.steps, args.warmup)
-        print(json.dumps({**({"vendor_library": vendor} if vendor else {}),
-                          "metric": name, "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
-                          "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-                          "dtype": "f32", "data": "synthetic", "higher_is_better": True,
-                          "config": {"workload": args.workload + "_fp32", "rows": M, "nnz": nnz},
-                          "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
-                          "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}))
-        return 0
+            out["vendor_library"] = _vendor_time("torch.mv(csr, x)", lambda: torch.mv(A_t, x), args.steps, 1)
+        return out
     if args.workload == "spgemm_powerlaw":
         # A @ A for the power-law graph at 1/8 of the headline size (the square of the
         # full graph has billions of products)
         rows = args.rows if args.rows != 1 << 20 else 1 << 17
         w = workloads.gcn_powerlaw(M=rows, N=4, max_degree=5000)
         M = w["M"]
-        pos, crd, val = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"])
-        fn = lambda: H.prebuilt_spmspm_csr_f32([M, M], [M, M], [[], [pos, crd]], val, [M, M],
-                                               [[], [pos, crd]], val)
-        out = fn()
-        nnz_c = int(out.storage.value.numel())
+        pos, crd, val = _t(w["row_ptr"]), _t(w["col_idx"]), _t(w["vals"])
+        fn = lambda: H.prebuilt_spmspm_csr_f32([M, M], [M, M], [[], [pos, crd]], val, [M, M], [[], [pos, crd]], val)
+        nnz_c = int(fn().storage.value.numel())
         deg = (pos[1:] - pos[:-1]).long()
         products = int(deg[crd.long()].sum().item())
-        ms = _time_steps(fn, args.steps, args.warmup)
-        vendor = None
+        ms = _time_steps(fn, args.steps, args.warmup, rounds=1)
+        out = {"metric": "CSR SpGEMM GFLOP/s (2 flops per product)", "value": round(2.0 * products / ms / 1e6, 2),
+               "unit": "GFLOP/s", "ms_per_step": round(ms, 4), **base,
+               "config": {"workload": "spgemm_powerlaw_fp32", "rows": M, "nnz_a": int(crd.numel()),
+                          "products": products, "nnz_c": nnz_c},
+               "note": "symbolic + numeric passes and the host read of nnz(C) between them"}
         if args.vendor:
             A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, M))
-            vendor = _vendor_time("torch.sparse.mm(csr, csr)", lambda: torch.sparse.mm(A_t, A_t),
-                                  max(2, args.steps // 4), 1)
-        print(json.dumps({"metric": "CSR SpGEMM GFLOP/s (2 flops per product)",
-                          "value": round(2.0 * products / ms / 1e6, 2), "unit": "GFLOP/s",
-                          "ms_per_step": round(ms, 4), "n_gpus": 1, "steps": args.steps,
-                          "warmup": args.warmup, "dtype": "f32", "data": "synthetic",
-                          "higher_is_better": True,
-                          "config": {"workload": "spgemm_powerlaw_fp32", "rows": M, "nnz_a": int(crd.numel()),
-                                     "products": products, "nnz_c": nnz_c},
-                          "note": "symbolic + numeric passes and the host read of nnz(C) between them",
-                          **({"vendor_library": vendor} if vendor else {})}))
-        return 0
-    if args.workload == "sddmm_uniform":
-        w = workloads.sddmm_uniform()
-        M, n_cols, K, nnz = w["M"], w["n_cols"], w["K"], int(w["col_idx"].size)
-        pos, crd, val, A, B = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), t(w["A"]), t(w["B"])
-        rows = t(w["row_idx"])
-        csr = lambda: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [pos, crd]], val, [M, K], [[], []],
-                                        A.reshape(-1), [n_cols, K], [[], []], B.reshape(-1))
-        coo = lambda: H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows], [crd]], val, [M, K],
-                                                 [[], []], A.reshape(-1), [n_cols, K], [[], []],
-                                                 B.reshape(-1))
-        ms = _time_steps(csr, args.steps, args.warmup)
-        ms_coo = _time_steps(coo, args.steps, args.warmup)
-        flops = 2.0 * nnz * K + nnz
-        algo = 4 * (M + 1) + 4 * nnz * 3 + 4 * M * K + 4 * n_cols * K + 4 * nnz   # + row output
-        gather = algo - 4 * n_cols * K + 4 * nnz * K
-        out = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
-               "ms_per_step": round(ms, 4), "ms_per_step_coo_mask": round(ms_coo, 4),
-               "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K}}
-        if not args.no_cpu:
-            out["cpu_baseline"] = cpu_baseline_sddmm(w)
-        if args.vendor:
-            mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
-            Bt = B.t().contiguous()
-            out["vendor_library"] = _vendor_time(
-                "torch.sparse.sampled_addmm(mask, A, B^T, beta=0)",
-                lambda: torch.sparse.sampled_addmm(mask, A, Bt, beta=0.0), args.steps, args.warmup)
-    else:
-        w = workloads.spmm_uniform() if args.workload == "spmm_uniform" else workloads.sae_decoder()
-        M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
-        pos, crd, val, B = t(w["row_ptr"]), t(w["col_idx"]), t(w["vals"]), t(w["B"]).reshape(-1)
-        fn = lambda: H.spmm_csr_float_v2([M, N], [M, K], [[], [pos, crd]], val, [K, N], [[], []], B)
-        ms = _time_steps(fn, args.steps, args.warmup)
-        flops = 2.0 * nnz * N
-        algo, gather = algorithmic_bytes(M, K, N, nnz), gather_bytes(M, N, nnz)
-        out = {"metric": "CSR SpMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
-               "ms_per_step": round(ms, 4),
-               "config": {"workload": args.workload + "_fp32", "rows": M, "cols": K, "nnz": nnz,
-                          "features": N}}
-        if args.graph:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                fn()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                fn()
-            out["ms_per_step_graph_replay"] = round(_time_steps(graph.replay, args.steps, args.warmup), 4)
-        if args.vendor:
-            out["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
-        if not args.no_cpu:
-            out["cpu_baseline"] = cpu_baseline(w)
-    out.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "f32",
-                "data": "synthetic", "higher_is_better": True,
-                "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
-                "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                "gather_model_bytes": gather, "gather_model_gbps": round(gather / ms / 1e6, 1)})
-    print(json.dumps(out))
-    return 0
+            out["vendor_library"] = _vendor_time("torch.sparse.mm(csr, csr)", lambda: torch.sparse.mm(A_t, A_t),
+                                                 max(2, args.steps // 4), 1)
+        return out
+    raise ValueError(args.workload)
+
+
+def run_workload(name, args, headline=False):
+    if name in ("gcn_powerlaw", "spmm_uniform", "sae_decoder"):
+        return run_spmm(name, args, headline)
+    if name == "sddmm_uniform":
+        return run_sddmm(args)
+    if name == "attention_blocksparse":
+        return run_attention(args)
+    return run_extra(args)
 
 
 def main() -> int:
@@ -419,14 +616,14 @@ def main() -> int:
                          "all nodes (same degrees; shows what the kernel does when rows share neighbours)")
     ap.add_argument("--row-length", type=int, default=0,
                     help="softmax_rows: entries per row (0: a causal mask, row i has i + 1 entries)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="gcn_powerlaw",
-                    choices=["gcn_powerlaw", "spmm_uniform", "sae_decoder", "sddmm_uniform",
-                             "attention_blocksparse", "spgemm_powerlaw", "spmv_powerlaw",
-                             "softmax_powerlaw", "softmax_rows", "gcn_forward"],
-                    help="gcn_powerlaw is the headline line; the others time the parity workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--headline-only", action="store_true", help="skip the records of the other four configurations")
+    ap.add_argument("--workload", default=None,
+                    choices=[HEADLINE, *CONFIG_WORKLOADS, "spgemm_powerlaw", "spmv_powerlaw", "softmax_powerlaw",
+                             "softmax_rows", "gcn_forward"],
+                    help="print this workload's record alone (default: the headline line with all configurations)")
     ap.add_argument("--vendor", action="store_true",
-                    help="also time torch's own sparse routine on the same operands (SpMM, SDDMM, SpGEMM, SpMV)")
+                    help="also time torch's own sparse routine on the same operands")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replay (SpMM side workloads)")
     args = ap.parse_args()
@@ -436,8 +633,7 @@ def main() -> int:
         return 2
 
     import torch
-    from scorch_amd import native, workloads
-    from scorch_amd import scorch_ops_hip as H
+    from scorch_amd import native
 
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)
@@ -445,86 +641,20 @@ def main() -> int:
     if not os.path.exists(native.library_path()):
         print("libscorch_hip.so is not built (python __graft_entry__.py)", file=sys.stderr)
         return 1
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
+    torch.cuda.set_device(0)
 
-    if args.workload != "gcn_powerlaw":
-        return side_workload(args, dev)
-
-    t0 = time.time()
-    w = workloads.gcn_powerlaw(M=args.rows, N=args.features, window=args.window)
-    M, K, N, nnz = w["M"], w["K"], w["N"], int(w["col_idx"].size)
-    print(f"[bench] generated {WORKLOAD}: M={M} nnz={nnz} N={N} in {time.time() - t0:.1f}s", file=sys.stderr)
-
-    pos = torch.from_numpy(w["row_ptr"]).to(dev)
-    crd = torch.from_numpy(w["col_idx"]).to(dev)
-    val = torch.from_numpy(w["vals"]).to(dev)
-    B = torch.from_numpy(w["B"]).to(dev).reshape(-1)
-    call = ([M, N], [M, K], [[], [pos, crd]], val, [K, N], [[], []], B)
-
-    for _ in range(args.warmup):
-        out = H.spmm_csr_float_v2(*call)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_begin = time.perf_counter()
-    start.record()
-    for _ in range(args.steps):
-        out = H.spmm_csr_float_v2(*call)
-    stop.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t_begin
-    ms_per_step = wall * 1e3 / args.steps
-    event_ms_per_step = start.elapsed_time(stop) / args.steps
-
-    # per-kernel durations: events around each kernel, on the launch stream
-    L = native.lib()
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    ws_bytes = L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, 4)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    C = out.storage.value
-    kernel_ms = (ctypes.c_float * 2)()
-    merge_ms, fixup_ms = [], []
-    for _ in range(args.steps):
-        native.check(L.scorch_hip_spmm_csr_f32_timed(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
-                                                     val.data_ptr(), B.data_ptr(), C.data_ptr(),
-                                                     ws.data_ptr(), ws.numel(), stream, kernel_ms))
-        merge_ms.append(kernel_ms[0])
-        fixup_ms.append(kernel_ms[1])
-    merge_avg = sum(merge_ms) / len(merge_ms)
-    fixup_avg = sum(fixup_ms) / len(fixup_ms)
-
-    flops = 2.0 * nnz * N
-    algo = algorithmic_bytes(M, K, N, nnz)
-    achieved = algo / (merge_avg * 1e-3) / 1e9
-    result = {
-        "metric": "CSR SpMM GFLOP/s + HBM GB/s (% peak), power-law 1M rows, N=128 fp32",
-        "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2),
-        "unit": "GFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": WORKLOAD, "rows": M, "cols": K, "nnz": nnz, "features": N,
-                   "degree": "zipf(2.1) scaled to mean 16, cap 50000, + self-loops",
-                   "values": "D^-1/2 (A+I) D^-1/2", "seed": workloads.SEEDS["gcn_powerlaw"],
-                   **({"neighbour_window": args.window} if args.window else {})},
-        "hbm_gbps_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
-        "hbm_frac_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-        "event_ms_per_step": round(event_ms_per_step, 4),
-        "roofline": {
-            "bound": "hbm", "kernel": "spmm_merge_kernel<float,2,0>" if N == 128 else "spmm_merge_kernel",
-            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES if (M, N) == (1 << 20, 128) else None,
-            "algorithmic_bytes": algo, "gather_model_bytes": gather_bytes(M, N, nnz),
-            "gather_model_gbps": round(gather_bytes(M, N, nnz) / (merge_avg * 1e-3) / 1e9, 1),
-            "kernel_ms_avg": round(merge_avg, 4), "fixup_kernel_ms_avg": round(fixup_avg, 4),
-        },
-    }
-    if args.vendor:
-        result["vendor_library"] = vendor_spmm(pos, crd, val, B.reshape(K, N), args.steps, args.warmup)
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(w)
+    if args.workload is not None:
+        print(json.dumps(run_workload(args.workload, args, headline=args.workload == HEADLINE)))
+        return 0
+    result = run_workload(HEADLINE, args, headline=True)
+    if not args.headline_only:
+        result["configs"] = []
+        for name in CONFIG_WORKLOADS:
+            torch.cuda.empty_cache()
+            try:
+                result["configs"].append(run_workload(name, args))
+            except Exception as exc:  # one configuration failing must not lose the headline line
+                result["configs"].append({"config": {"workload": name}, "error": f"{type(exc).__name__}: {exc}"})
     print(json.dumps(result))
     return 0
 

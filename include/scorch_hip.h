@@ -69,6 +69,19 @@ SCORCH_HIP_API int scorch_hip_abi_version(void);
 /* Message of the calling thread's most recent failed call ("" if none). */
 SCORCH_HIP_API const char *scorch_hip_last_error(void);
 
+/* Benchmarking aid: per-kernel durations of the calls made in between, on the
+ * calling host thread.  After scorch_hip_timing_begin() the SpMM, SDDMM and
+ * attention entry points record a HIP event on their stream before their first
+ * kernel, between their kernels and after their last (16 events at most; later
+ * ones are dropped).  scorch_hip_timing_end() waits for the last event and
+ * writes the time between consecutive events, in milliseconds, to
+ * interval_ms[0 .. min(*count, capacity)); *count is the number of intervals.
+ * One call per bracket gives one interval per kernel, in launch order.  The
+ * reference's only timing is wall-clock around a whole call
+ * (src/scorch/prebuilt_kernels.py:217-222). */
+SCORCH_HIP_API int scorch_hip_timing_begin(void);
+SCORCH_HIP_API int scorch_hip_timing_end(float *interval_ms /* host */, int capacity, int *count /* host */);
+
 /* ------------------------------------------------------------------------
  * SpMM: C[M,N] = A_csr[M,K] * B[K,N], all of one dtype.
  *
@@ -137,6 +150,110 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_f32_timed(int64_t M, int64_t K, int64_t N
                                   const float *B, float *C,
                                   void *workspace, size_t workspace_bytes, void *stream,
                                   float *kernel_ms /* host, [2] */);
+
+/* ------------------------------------------------------------------------
+ * What a caller can compute once per sparse operand and reuse in every later
+ * product with it.  The reference has no such step: its dispatch is stateless
+ * (src/scorch/prebuilt_kernels.py:198-224), but its callers multiply by one
+ * matrix many times (a graph's normalised adjacency in every layer and
+ * iteration, bench/bench_gcn.py:314-329; weights converted once outside the
+ * loop, bench/README_sparse_autoencoder.md:86).  All of it lives in memory the
+ * caller owns; the library keeps no state.
+ *
+ * scorch_hip_csr_inspect writes four int32 to `report` (device):
+ *   [0] 1 if row_ptr is malformed (row_ptr[0] != 0, row_ptr[M] != nnz, or a
+ *       pointer below its predecessor), else 0
+ *   [1] 1 if a column index lies outside [0, K), else 0
+ *   [2] the longest row
+ *   [3] the number of empty rows
+ * It reads row_ptr[0..M] and col_idx[0..nnz) only, so it is safe on malformed
+ * input; a caller that reads the report back (one synchronisation) can refuse
+ * the operand before any kernel dereferences it, and knows whether all rows
+ * are short.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_csr_inspect(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
+                           const int32_t *col_idx, int32_t *report /* device, [4] */, void *stream);
+
+/* Row-split SpMM for matrices whose rows are all short: C = act(A * B + bias)
+ * in one launch, without workspace (a team of lanes per row; no rows are cut,
+ * so there are no carries to fold).  Same contraction as
+ * scorch_hip_spmm_csr_<T> / _bias_act_f32 (csrc/spmm.h:28-150,2007-2089); bias
+ * may be NULL (then act must be SCORCH_HIP_ACT_NONE).  Correct for rows of any
+ * length but slow when one is long (a row is walked by one team): meant for
+ * operands whose longest row, as scorch_hip_csr_inspect reports it, is a few
+ * hundred entries at most.  Bit-reproducible. */
+SCORCH_HIP_API int scorch_hip_spmm_csr_rows_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                 const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                 const float *B, const float *bias, int act, float *C, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_rows_f64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                 const int32_t *row_ptr, const int32_t *col_idx, const double *vals,
+                                 const double *B, const double *bias, int act, double *C, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_rows_i32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                 const int32_t *row_ptr, const int32_t *col_idx, const int32_t *vals,
+                                 const int32_t *B, const int32_t *bias, int act, int32_t *C, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_rows_i64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                 const int32_t *row_ptr, const int32_t *col_idx, const int64_t *vals,
+                                 const int64_t *B, const int64_t *bias, int act, int64_t *C, void *stream);
+
+/* Merge-path SpMM with its chunk boundaries computed beforehand.
+ * scorch_hip_spmm_csr_bounds fills `bounds` (device, 8-byte aligned,
+ * scorch_hip_spmm_csr_bounds_bytes(M, nnz, N, sizeof(T)) bytes) from row_ptr;
+ * the boundaries depend on row_ptr, N and the element size only.
+ * scorch_hip_spmm_csr_planned_<T> is scorch_hip_spmm_csr_<T> (with the
+ * optional bias / activation of _bias_act_f32) whose wavefronts read their two
+ * boundaries from `bounds` instead of searching row_ptr; bounds may be NULL,
+ * and the call is then the unplanned one.  Same results bit for bit.  The
+ * caller vouches that `bounds` was built from this row_ptr with these M, nnz,
+ * N and element size. */
+SCORCH_HIP_API size_t scorch_hip_spmm_csr_bounds_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem_size);
+SCORCH_HIP_API int scorch_hip_spmm_csr_bounds(int64_t M, int64_t nnz, int64_t N, size_t elem_size,
+                               const int32_t *row_ptr, void *bounds, size_t bounds_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_planned_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                    const float *B, const float *bias, int act, float *C,
+                                    const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_planned_f64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx, const double *vals,
+                                    const double *B, const double *bias, int act, double *C,
+                                    const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_planned_i32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx, const int32_t *vals,
+                                    const int32_t *B, const int32_t *bias, int act, int32_t *C,
+                                    const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_planned_i64(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx, const int64_t *vals,
+                                    const int64_t *B, const int64_t *bias, int act, int64_t *C,
+                                    const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* SpMM against a wide dense operand that is reused (a weight matrix), stored
+ * once by column tiles.  The reference's weight-sparse autoencoder multiplies
+ * every batch by the same dense decoder weight (bench/bench_sparse_autoencoder.py:
+ * 250-276); with B row-major each stored entry of A gathers a whole row of B
+ * from memory, although every row of B is gathered several times.
+ *   Bt[tile][k][c]: tile t holds columns [32 t, 32 t + 32) of B (fp32; 128-byte
+ *   tile rows), K rows contiguous, zero padded past N;
+ *   scorch_hip_dense_tiled_bytes(K, N, 4) bytes, 128-byte aligned.
+ * scorch_hip_dense_to_tiled_f32 builds Bt from a row-major B (one read and one
+ * write of B).  scorch_hip_spmm_csr_tiled_f32 is scorch_hip_spmm_csr_planned_f32
+ * with Bt in place of B: every XCD keeps one tile of Bt in its L2 while all rows
+ * of A gather from it, so B comes from memory about once.  Results agree with
+ * the other SpMM entry points to rounding (rows of more than 64 entries are
+ * summed in another grouping) and are bit-reproducible from run to run.
+ * scorch_hip_dense_tiled_recommended is 1 when the layout pays: rows of B of
+ * 2 KiB and more, K * 128 bytes within an L2's reach (3 MiB), and nnz >= 2 K. */
+SCORCH_HIP_API size_t scorch_hip_dense_tiled_bytes(int64_t K, int64_t N, size_t elem_size);
+SCORCH_HIP_API int scorch_hip_dense_tiled_recommended(int64_t K, int64_t N, int64_t nnz, size_t elem_size);
+SCORCH_HIP_API int scorch_hip_dense_to_tiled_f32(int64_t K, int64_t N, const float *B, float *Bt,
+                                  size_t bt_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_tiled_f32(int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                  const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                  const float *Bt, size_t bt_bytes, const float *bias, int act, float *C,
+                                  const void *bounds, size_t bounds_bytes,
+                                  void *workspace, size_t workspace_bytes, void *stream);
 
 /* Fused C = act(A * B + bias), bias is T[N] broadcast over rows.
  * Replaces spmm_csr_bias_act<float, relu> (csrc/spmm.h:28-89), bound as

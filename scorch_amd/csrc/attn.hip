@@ -266,6 +266,7 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
   hipStream_t s = static_cast<hipStream_t>(stream);
   const __bf16 *q = static_cast<const __bf16 *>(Q), *k = static_cast<const __bf16 *>(K),
                *v = static_cast<const __bf16 *>(V);
+  mark_launch(s);
   if (scale < 0.0f)
     attn_blocksparse_kernel<true><<<grid, kBlockThreads, 0, s>>>(
         (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
@@ -275,5 +276,6 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
         (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
         static_cast<__bf16 *>(O));
   SCORCH_HIP_CHECK(hipGetLastError());
+  mark_launch(s);
   return SCORCH_HIP_OK;
 }

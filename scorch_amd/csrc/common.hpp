@@ -66,6 +66,24 @@ inline int check_csr_args(const char *fn, int64_t M, int64_t K, int64_t nnz, con
   return SCORCH_HIP_OK;
 }
 
+// ---- per-kernel timing for benchmarks ---------------------------------------
+// Between scorch_hip_timing_begin() and scorch_hip_timing_end() on a host thread,
+// every entry point records a HIP event on its stream before its first launch,
+// between its launches and after its last (mark_launch); _end returns the
+// intervals.  Outside such a bracket mark_launch is one thread-local test.
+constexpr int kMaxLaunchMarks = 16;
+struct LaunchMarks {
+  hipEvent_t ev[kMaxLaunchMarks];
+  int count = 0;
+  bool created = false, active = false;
+};
+LaunchMarks *launch_marks();  // the calling thread's
+
+inline void mark_launch(hipStream_t stream) {
+  LaunchMarks *m = launch_marks();
+  if (m->active && m->count < kMaxLaunchMarks) (void)hipEventRecord(m->ev[m->count++], stream);
+}
+
 // ---- arithmetic traits --------------------------------------------------------
 // Integer kernels accumulate in the unsigned type of the same width so that
 // overflow wraps (the reference's signed overflow wraps in practice).

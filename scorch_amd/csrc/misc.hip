@@ -9,6 +9,11 @@ char *error_buffer() {
   return buf;
 }
 
+LaunchMarks *launch_marks() {
+  static thread_local LaunchMarks marks;
+  return &marks;
+}
+
 // ---- CSR row softmax ----------------------------------------------------------
 // p = exp(s - max_row) / sum_row over the stored entries of each row, in three
 // phases (maximum, sum of exponentials, normalised write) like the five torch
@@ -381,6 +386,31 @@ extern "C" {
 int scorch_hip_abi_version(void) { return SCORCH_HIP_ABI_VERSION; }
 
 const char *scorch_hip_last_error(void) { return scorch::error_buffer(); }
+
+int scorch_hip_timing_begin(void) {
+  scorch::LaunchMarks *m = scorch::launch_marks();
+  if (!m->created) {
+    for (int i = 0; i < scorch::kMaxLaunchMarks; ++i) SCORCH_HIP_CHECK(hipEventCreate(&m->ev[i]));
+    m->created = true;
+  }
+  m->count = 0;
+  m->active = true;
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_timing_end(float *interval_ms, int capacity, int *count) {
+  const char *fn = "scorch_hip_timing_end";
+  scorch::LaunchMarks *m = scorch::launch_marks();
+  SCORCH_REQUIRE(m->active, "%s: no scorch_hip_timing_begin on this thread", fn);
+  m->active = false;
+  SCORCH_REQUIRE(count != nullptr && (capacity == 0 || interval_ms != nullptr), "%s: NULL output", fn);
+  const int intervals = m->count > 0 ? m->count - 1 : 0;
+  *count = intervals;
+  if (m->count > 0) SCORCH_HIP_CHECK(hipEventSynchronize(m->ev[m->count - 1]));
+  for (int i = 0; i < intervals && i < capacity; ++i)
+    SCORCH_HIP_CHECK(hipEventElapsedTime(&interval_ms[i], m->ev[i], m->ev[i + 1]));
+  return SCORCH_HIP_OK;
+}
 
 size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz) {
   if (M <= 0 || nnz <= 0) return 0;

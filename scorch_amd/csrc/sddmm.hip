@@ -128,6 +128,7 @@ int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
   const int per_lane = vec4 ? 4 : 1;
   const int64_t lanes_needed = (K + per_lane - 1) / per_lane;
 
+  mark_launch(stream);
 #define SCORCH_SDDMM_LAUNCH(GS, VEC, LONG)                                                         \
   sddmm_kernel<GS, VEC, COO, LONG><<<grid, kBlockThreads, 0, stream>>>(M, K, nnz, rows, col_idx,   \
                                                                       mask_vals, A, B, out_vals,  \
@@ -146,6 +147,7 @@ int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
 #undef SCORCH_SDDMM_PICK
 #undef SCORCH_SDDMM_LAUNCH
   SCORCH_HIP_CHECK(hipGetLastError());
+  mark_launch(stream);
   return SCORCH_HIP_OK;
 }
 

@@ -27,97 +27,19 @@
 // Columns beyond 64 * VEC are covered by column tiles (each tile walks the same
 // chunks again; A's indices are small next to the B rows gathered).  Tiles are
 // placed on XCDs so that a tile's slice of B stays in one L2 (map_workgroup).
-#include "common.hpp"
+#include "spmm.hpp"
 
 #include <mutex>
 
 namespace scorch {
-
-constexpr int kItemsPerWave = 256;  // most merge items (row ends + nonzeros) per wavefront
-constexpr int kMinItemsPerWave = 32;
-constexpr int kGather = 8;          // B-row loads in flight per wavefront
-
-enum Epilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasRelu = 2 };
-
-// Workgroup id -> (column tile, block of wavefront spans).  Workgroups are dealt
-// to the 8 XCDs round robin by their linear id, and every XCD has its own L2.
-// With a multiple of 8 column tiles, tile t is given to XCD t % 8 and each XCD
-// works through its tiles one after the other: the B rows a tile gathers
-// (K rows of 64 * VEC elements) are then fetched into one L2 only and stay
-// there while the tile is processed.
-struct TileMap {
-  int tile;
-  int64_t block;
-};
-
-__device__ __forceinline__ TileMap map_workgroup(int64_t id, int n_tiles, int64_t blocks_per_tile) {
-  TileMap m;
-  if (n_tiles > 1 && (n_tiles & 7) == 0) {
-    const int xcd = (int)(id & 7);
-    const int64_t slot = id >> 3;
-    m.tile = xcd + 8 * (int)(slot / blocks_per_tile);
-    m.block = slot % blocks_per_tile;
-  } else {
-    m.tile = (int)(id / blocks_per_tile);
-    const int64_t rem = id % blocks_per_tile;
-    // rem & 7 is the XCD when blocks_per_tile is a multiple of 8 (the SpMM launchers
-    // see to that): every XCD gets one contiguous eighth of the chunks, so that B
-    // rows shared by neighbouring rows of A are found in its L2
-    m.block = (blocks_per_tile & 7) == 0 ? xcd_contiguous(rem, blocks_per_tile) : rem;
-  }
-  return m;
-}
-
-template <typename T, int EPI>
-__device__ __forceinline__ T apply_epilogue(typename Acc<T>::type acc, T bias) {
-  T r = (T)acc;
-  if (EPI != kEpiNone) r = r + bias;
-  if (EPI == kEpiBiasRelu) r = r > (T)0 ? r : (T)0;
-  return r;
-}
-
-// Chunk boundaries.  Chunk c nominally covers the merged positions [c * items,
-// (c + 1) * items).  A boundary that falls inside a row moves forward to just
-// after the row's end marker when that is at most `snap` items away: the row
-// is then summed by one chunk and leaves no carry.  Most rows are short, so
-// most boundaries snap, and carries remain for rows that really span chunks.
-// The result depends on the nominal position only, so the two chunks on either
-// side of a boundary agree on it.  x: rows finished before the boundary, y:
-// nonzeros before it.
-constexpr int kSnapItems = 64;
-
-struct Boundary {
-  int x, y;
-};
-
-__device__ __forceinline__ Boundary chunk_boundary(int64_t d, int M, int64_t total_items,
-                                                   const int *__restrict__ row_ptr, int snap) {
-  Boundary b;
-  if (d >= total_items) {
-    b.x = M;
-    b.y = (int)(total_items - M);
-    return b;
-  }
-  auto row_end_key = [&](int i) { return (int64_t)row_ptr[i + 1] + i; };
-  b.x = wave_count_below(M, d, row_end_key);
-  b.y = uniform((int)(d - b.x));
-  if (b.x < M) {
-    const int begin = uniform(row_ptr[b.x]), end = uniform(row_ptr[b.x + 1]);
-    const int64_t after_marker = (int64_t)end + b.x + 1;
-    if (begin < b.y && after_marker - d <= snap) {  // the row is under way and nearly done
-      b.x += 1;
-      b.y = end;
-    }
-  }
-  return b;
-}
 
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
-    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
+    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val,
+    const Boundary *__restrict__ bounds) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int kSlots = kItemsPerWave + kSnapItems;
@@ -135,8 +57,9 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 
   const int64_t d0 = chunk * items_per_chunk;
   if (d0 >= total_items) return;  // only wave-level synchronisation below
-  const Boundary from = chunk_boundary(d0, M, total_items, row_ptr, snap);
-  const Boundary to = chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
+  const Boundary from = bounds ? load_boundary(bounds, chunk) : chunk_boundary(d0, M, total_items, row_ptr, snap);
+  const Boundary to = bounds ? load_boundary(bounds, chunk + 1)
+                             : chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
   const int x0 = from.x, y0 = from.y, x1 = to.x, y1 = to.y;
   const int n_nz = y1 - y0;
   const int n_rows = x1 - x0;
@@ -243,7 +166,8 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
-    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val) {
+    int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val,
+    const Boundary *__restrict__ bounds) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int G = kWaveSize / LPR;
@@ -264,8 +188,9 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
 
   const int64_t d0 = span * items_per_chunk;
   if (d0 >= total_items) return;  // only wave-level synchronisation below
-  const Boundary from = chunk_boundary(d0, M, total_items, row_ptr, snap);
-  const Boundary to = chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
+  const Boundary from = bounds ? load_boundary(bounds, span) : chunk_boundary(d0, M, total_items, row_ptr, snap);
+  const Boundary to = bounds ? load_boundary(bounds, span + 1)
+                             : chunk_boundary(d0 + items_per_chunk, M, total_items, row_ptr, snap);
   const int x0 = from.x, y0 = from.y, x1 = to.x, y1 = to.y;
   const int n_nz = y1 - y0;
   const int n_rows = x1 - x0;
@@ -366,133 +291,49 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
 }
 
 
-// End of the run of equal carry rows that starts at `start` (a member): a 64-way
-// search by the whole wavefront.  The members of a run are consecutive, so
-// "same row" holds up to the end and nowhere after.
-__device__ __forceinline__ int64_t carry_run_end(const int *__restrict__ carry_row, int64_t start,
-                                                 int64_t num_chunks, int row) {
-  const int lane = wave_lane();
-  int64_t last = start, stop = num_chunks;  // a known member; the first position known to lie beyond
-  while (stop - last > 1) {
-    const int64_t step = (stop - last + kWaveSize) / (kWaveSize + 1);
-    const int64_t probe = last + (int64_t)(lane + 1) * step;
-    const bool same = probe < stop && carry_row[probe] == row;
-    const int members = __popcll(__ballot(same));  // lanes 0 .. members - 1
-    const int64_t reached = last + (int64_t)members * step;
-    if (members < kWaveSize && reached + step < stop) stop = reached + step;  // lane `members` saw the end
-    last = reached;
-  }
-  return last + 1;
-}
-
-// Folds the carries into C.  A wavefront looks at kFixupChunks consecutive
-// chunks' carry rows (one lane each, one load); those that head a run of equal
-// rows are then taken one after the other by the whole wavefront, lanes on
-// columns: the run is summed in chunk order and added to the row of C, with
-// the epilogue.  Few chunks leave a carry (see chunk_boundary), so most
-// wavefronts only look: fewer, wider-looking wavefronts cost less to start,
-// while a matrix of long rows, where every chunk leaves a carry, still has
-// its heads spread over many wavefronts.
-constexpr int kFixupChunks = 8;
-template <typename T, int VEC, int EPI>
-__global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
-    int N, int64_t num_chunks, const int *__restrict__ carry_row, const T *__restrict__ carry_val,
-    T *__restrict__ C, const T *__restrict__ bias) {
-  using A = typename Acc<T>::type;
-  using VecT = Vec<T, VEC>;
-  const int lane = wave_lane();
-  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
-  const int64_t c = wave * kFixupChunks + lane;
-  int row = -1, after = -1;
-  if (lane < kFixupChunks && c < num_chunks) {
-    row = carry_row[c];
-    after = c + 1 < num_chunks ? carry_row[c + 1] : -1;
-    if (row >= 0 && c > 0 && carry_row[c - 1] == row) row = -1;  // not the head of its run
-  }
-  unsigned long long pending = __ballot(row >= 0);
-  while (pending) {  // uniform over the wavefront
-    const int owner = __ffsll(pending) - 1;
-    pending &= pending - 1;
-    const int r = __shfl(row, owner);
-    const int64_t start = c - lane + owner;
-    // a run of one, the usual case, needs no search
-    const int64_t end = __shfl(after, owner) != r ? start + 1 : carry_run_end(carry_row, start, num_chunks, r);
-    for (int col0 = lane * VEC; col0 < N; col0 += kWaveSize * VEC) {
-      VecT *dst = reinterpret_cast<VecT *>(C + (size_t)r * (size_t)N + col0);
-      VecT o = *dst;  // issued before the carries so that both are in flight together
-      A sum[VEC];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) sum[v] = (A)0;
-      int64_t e = start;
-      constexpr int kBatch = 32;  // loads in flight: a long row spans hundreds of chunks
-      for (; e + kBatch <= end; e += kBatch) {
-        VecT part[kBatch];
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-          part[u] = *reinterpret_cast<const VecT *>(carry_val + (size_t)(e + u) * (size_t)N + col0);
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) sum[v] += (A)part[u].v[v];
-      }
-      for (; e < end; ++e) {
-        const VecT part = *reinterpret_cast<const VecT *>(carry_val + (size_t)e * (size_t)N + col0);
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) sum[v] += (A)part.v[v];
-      }
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        const T b = EPI != kEpiNone ? bias[col0 + v] : (T)0;
-        o.v[v] = apply_epilogue<T, EPI>(sum[v] + (A)o.v[v], b);
-      }
-      *dst = o;
-    }
-  }
-}
-
 // ---- host side ----------------------------------------------------------------
 
-// Shape of the work split.  A chunk holds nominally up to 256 merge items, one
-// chunk per wavefront; small problems use smaller chunks, so that they are
-// spread over more, shorter wavefronts.  (A wavefront that walked two or more
-// consecutive chunks with one carry for all of them was measured: the same
-// time on a graph with uniform neighbours, slower -- 0.81 against 0.69 ms on the
-// 4,096-neighbour graph -- where neighbouring rows share columns, because an XCD
-// then has a wider stretch of rows in flight than its L2 covers.)
-struct SpmmSplit {
-  int items_per_chunk;
-  int snap;        // see chunk_boundary
-  int64_t spans;   // chunks = wavefronts with work = carry records
-};
-
-inline SpmmSplit spmm_split(int64_t M, int64_t nnz, int64_t N, size_t elem) {
-  const int64_t total = M + nnz;
-  SpmmSplit sp;
-  // every column tile (up to 1 KiB of a row) walks all chunks again
-  const int64_t tiles = (N * (int64_t)elem + 1023) / 1024;
-  const int64_t per_wave = total * (tiles > 0 ? tiles : 1) / 8192;  // 256 CUs x 32 wavefronts
-  sp.items_per_chunk = kMinItemsPerWave;
-  while (sp.items_per_chunk < kItemsPerWave && sp.items_per_chunk * 2 <= per_wave)
-    sp.items_per_chunk *= 2;
-  sp.snap = sp.items_per_chunk < kSnapItems ? sp.items_per_chunk : kSnapItems;
-  sp.spans = (total + sp.items_per_chunk - 1) / sp.items_per_chunk;
-  return sp;
+// ---- chunk boundaries computed once -----------------------------------------------------------
+// The boundaries depend on row_ptr and on the split only, not on the values or
+// the dense operand: a caller that multiplies by the same sparse matrix again
+// and again (a graph's adjacency in every layer and iteration) computes them once
+// with spmm_bounds_kernel, one thread per boundary, and hands them to the
+// kernels, whose wavefronts then read two records instead of searching row_ptr
+// twice.  bounds[c] is what chunk_boundary returns for position c * items.
+__global__ __launch_bounds__(kBlockThreads) void spmm_bounds_kernel(int M, int64_t total_items,
+                                                                    int items_per_chunk, int snap,
+                                                                    int64_t num_bounds,
+                                                                    const int *__restrict__ row_ptr,
+                                                                    Boundary *__restrict__ bounds) {
+  const int64_t c = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  if (c >= num_bounds) return;
+  const int64_t d = c * items_per_chunk;
+  Boundary b;
+  if (d >= total_items) {
+    b.x = M;
+    b.y = (int)(total_items - M);
+  } else {
+    // rows whose end marker (position row_ptr[i + 1] + i) lies before d
+    int lo = 0, hi = M;
+    while (lo < hi) {
+      const int mid = lo + (hi - lo) / 2;
+      if ((int64_t)row_ptr[mid + 1] + mid < d) lo = mid + 1; else hi = mid;
+    }
+    b.x = lo;
+    b.y = (int)(d - lo);
+    if (b.x < M) {
+      const int begin = row_ptr[b.x], end = row_ptr[b.x + 1];
+      if (begin < b.y && (int64_t)end + b.x + 1 - d <= snap) {  // as in chunk_boundary
+        b.x += 1;
+        b.y = end;
+      }
+    }
+  }
+  bounds[c] = b;
 }
 
-// Carry records the workspace must hold: the most any kernel variant produces
-// for this shape (one record per chunk of the wide-tile split).
-inline int64_t spmm_num_chunks(int64_t M, int64_t nnz, int64_t N, size_t elem) {
-  const SpmmSplit sp = spmm_split(M, nnz, N, elem);
-  return (M + nnz + sp.items_per_chunk - 1) / sp.items_per_chunk;
-}
-
-inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
-
-// Workspace layout: carry_row int32[num_chunks] padded to 256 bytes, then
-// carry_val T[num_chunks * N].
-inline size_t spmm_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
-  const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
-  return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256);
+inline size_t spmm_bounds_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
+  return (size_t)(spmm_split(M, nnz, N, elem).spans + 1) * sizeof(Boundary);
 }
 
 // Optional per-kernel timing: events recorded on the launch stream around each
@@ -512,7 +353,7 @@ struct KernelTimer {
 template <typename T, int VEC, int EPI>
 int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
                 const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
-                KernelTimer *timer) {
+                KernelTimer *timer, const Boundary *bounds) {
   const SpmmSplit split = spmm_split(M, nnz, N, sizeof(T));
   const int64_t chunks = split.spans;
   int *carry_row = static_cast<int *>(workspace);
@@ -528,16 +369,19 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
                 (long long)(blocks_per_tile * n_tiles));
   const dim3 grid((unsigned)(blocks_per_tile * n_tiles));
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
+  mark_launch(stream);
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
-      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val);
+      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val, bounds);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
+  mark_launch(stream);
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
   spmm_fixup_kernel<T, VEC, EPI><<<dim3((unsigned)((chunks + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
                                    stream>>>(N, chunks, carry_row, carry_val, C, bias);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
+  mark_launch(stream);
   return SCORCH_HIP_OK;
 }
 
@@ -547,7 +391,7 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
 template <typename T, int VEC, int LPR, int EPI>
 int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx,
                         const T *vals, const T *B, const T *bias, T *C, void *workspace,
-                        hipStream_t stream) {
+                        hipStream_t stream, const Boundary *bounds) {
   const int64_t total = (int64_t)M + nnz;
   const int tile = LPR * VEC;
   const int n_tiles = (N + tile - 1) / tile;
@@ -557,6 +401,9 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
   while (ipc < kItemsPerWave && ipc * 2 <= per_wave) ipc *= 2;
   const int wide_ipc = spmm_split(M, nnz, N, sizeof(T)).items_per_chunk;
   if (ipc < wide_ipc) ipc = wide_ipc;  // never more carry records than the workspace holds
+  if (bounds && ipc != wide_ipc)
+    return fail(SCORCH_HIP_ERUNTIME, "SpMM: the chunk boundaries were built for %d items per chunk, not %d",
+                wide_ipc, ipc);
   const int64_t spans = (total + ipc - 1) / ipc;
   if (spans > spmm_num_chunks(M, nnz, N, sizeof(T)))
     return fail(SCORCH_HIP_ERUNTIME, "SpMM: %lld carry records exceed the workspace's %lld",
@@ -569,14 +416,17 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
   if (blocks_per_tile * n_tiles > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
+  mark_launch(stream);
   spmm_grouped_kernel<T, VEC, LPR, EPI><<<dim3((unsigned)(blocks_per_tile * n_tiles)), kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, total, ipc, ipc < kSnapItems ? ipc : kSnapItems, n_tiles,
-      blocks_per_tile, carry_row, carry_val);
+      blocks_per_tile, carry_row, carry_val, bounds);
   SCORCH_HIP_CHECK(hipGetLastError());
+  mark_launch(stream);
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
   spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((spans + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
                                  stream>>>(N, spans, carry_row, carry_val, C, bias);
   SCORCH_HIP_CHECK(hipGetLastError());
+  mark_launch(stream);
   return SCORCH_HIP_OK;
 }
 
@@ -591,28 +441,11 @@ inline int narrow_tile_bytes(int64_t K, int64_t N, int64_t nnz, size_t elem) {
   return row_bytes <= 256 ? (int)row_bytes : 0;
 }
 
-// Elements per lane.  Preferred: the widest vector (at most 16 bytes) that
-// divides N, is aligned and still keeps all 64 lanes busy (64 * VEC <= N).
-// Narrow N: the narrowest vector that covers N with one column tile.
-template <typename T>
-int pick_vec(int64_t N, const void *B, const void *C, const void *ws) {
-  constexpr int kMaxVec = (int)(16 / sizeof(T));
-  auto usable = [&](int vec) {
-    const size_t bytes = sizeof(T) * vec;
-    return N % vec == 0 && aligned_to(B, bytes) && aligned_to(C, bytes) && aligned_to(ws, bytes);
-  };
-  for (int vec = kMaxVec; vec > 1; vec /= 2)
-    if (usable(vec) && (int64_t)kWaveSize * vec <= N) return vec;
-  for (int vec = 2; vec <= kMaxVec; vec *= 2)
-    if (usable(vec) && (int64_t)kWaveSize * vec >= N && (int64_t)kWaveSize * (vec / 2) < N) return vec;
-  return 1;
-}
-
 template <typename T, int EPI>
 int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
                const int32_t *col_idx, const T *vals, const T *B, const T *bias, T *C,
                void *workspace, size_t workspace_bytes, void *stream,
-               KernelTimer *timer = nullptr) {
+               KernelTimer *timer = nullptr, const void *bounds_buffer = nullptr, size_t bounds_bytes = 0) {
   if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
   SCORCH_REQUIRE(N >= 0, "%s: negative N=%lld", fn, (long long)N);
   if (N > INT32_MAX - kWaveSize * 4)
@@ -629,6 +462,15 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
                 workspace ? workspace_bytes : (size_t)0);
   SCORCH_REQUIRE(aligned_to(workspace, 256), "%s: workspace must be 256-byte aligned", fn);
 
+  const Boundary *bounds = static_cast<const Boundary *>(bounds_buffer);
+  if (bounds) {
+    const size_t have = spmm_bounds_bytes(M, nnz, N, sizeof(T));
+    if (bounds_bytes < have)
+      return fail(SCORCH_HIP_EWORKSPACE, "%s: chunk boundaries of %zu bytes needed, %zu given", fn, have,
+                  bounds_bytes);
+    SCORCH_REQUIRE(aligned_to(bounds, 8), "%s: the chunk boundaries must be 8-byte aligned", fn);
+  }
+
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int m = (int)M, n = (int)N;
   if (const int tile_bytes = timer ? 0 : narrow_tile_bytes(K, N, nnz, sizeof(T))) {
@@ -640,7 +482,7 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
     const int64_t tile_elems = tile_bytes / (int)sizeof(T) < N ? tile_bytes / (int)sizeof(T) : N;
     const int64_t lanes = (tile_elems + vec - 1) / vec;
 #define SCORCH_GROUPED(VEC, LPR) \
-  return launch_spmm_grouped<T, VEC, LPR, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s)
+  return launch_spmm_grouped<T, VEC, LPR, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, bounds)
 #define SCORCH_GROUPED_LANES(VEC)                      \
   do {                                                 \
     if (lanes <= 8) SCORCH_GROUPED(VEC, 8);            \
@@ -659,11 +501,11 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
   const int vec = pick_vec<T>(N, B, C, workspace);
   if constexpr (sizeof(T) == 4) {
     if (vec == 4)
-      return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
+      return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
   }
   if (vec == 2)
-    return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
-  return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer);
+    return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
+  return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
 }
 
 
@@ -988,6 +830,64 @@ int scorch_hip_spmm_csr_bias_act_f32(int64_t M, int64_t K, int64_t N, int64_t nn
                                                            stream);
   return scorch::fail(SCORCH_HIP_EINVAL, "%s: unknown activation %d", fn, act);
 }
+
+size_t scorch_hip_spmm_csr_bounds_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem_size) {
+  if (M < 0 || nnz < 0 || N < 0 || elem_size == 0) return 0;
+  return scorch::spmm_bounds_bytes(M, nnz, N, elem_size);
+}
+
+int scorch_hip_spmm_csr_bounds(int64_t M, int64_t nnz, int64_t N, size_t elem_size, const int32_t *row_ptr,
+                               void *bounds, size_t bounds_bytes, void *stream) {
+  const char *fn = "scorch_hip_spmm_csr_bounds";
+  if (M < 0 || nnz < 0 || N < 0 || elem_size == 0)
+    return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld nnz=%lld N=%lld)", fn, (long long)M,
+                        (long long)nnz, (long long)N);
+  if (M >= INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: M and nnz must fit the int32 index arrays", fn);
+  SCORCH_REQUIRE(row_ptr != nullptr && bounds != nullptr, "%s: row_ptr or bounds is NULL", fn);
+  SCORCH_REQUIRE(scorch::aligned_to(row_ptr, 4) && scorch::aligned_to(bounds, 8),
+                 "%s: row_ptr must be 4-byte and bounds 8-byte aligned", fn);
+  const size_t need = scorch::spmm_bounds_bytes(M, nnz, N, elem_size);
+  if (bounds_bytes < need)
+    return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: %zu bytes needed for the boundaries, %zu given", fn, need,
+                        bounds_bytes);
+  const scorch::SpmmSplit split = scorch::spmm_split(M, nnz, N, elem_size);
+  const int64_t num_bounds = split.spans + 1;
+  scorch::spmm_bounds_kernel<<<dim3((unsigned)((num_bounds + scorch::kBlockThreads - 1) / scorch::kBlockThreads)),
+                               scorch::kBlockThreads, 0, static_cast<hipStream_t>(stream)>>>(
+      (int)M, M + nnz, split.items_per_chunk, split.snap, num_bounds, row_ptr,
+      static_cast<scorch::Boundary *>(bounds));
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+#define SCORCH_DEFINE_SPMM_PLANNED(SUFFIX, T)                                                              \
+  int scorch_hip_spmm_csr_planned_##SUFFIX(int64_t M, int64_t K, int64_t N, int64_t nnz,                    \
+                                           const int32_t *row_ptr, const int32_t *col_idx, const T *vals,   \
+                                           const T *B, const T *bias, int act, T *C, const void *bounds,    \
+                                           size_t bounds_bytes, void *workspace, size_t workspace_bytes,    \
+                                           void *stream) {                                                  \
+    const char *fn = "scorch_hip_spmm_csr_planned_" #SUFFIX;                                                \
+    if (!bias && act == SCORCH_HIP_ACT_NONE)                                                                \
+      return scorch::spmm_entry<T, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, nullptr,  \
+                                                     C, workspace, workspace_bytes, stream, nullptr,        \
+                                                     bounds, bounds_bytes);                                 \
+    if (bias && act == SCORCH_HIP_ACT_NONE)                                                                 \
+      return scorch::spmm_entry<T, scorch::kEpiBias>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, bias, C,  \
+                                                     workspace, workspace_bytes, stream, nullptr, bounds,   \
+                                                     bounds_bytes);                                         \
+    if (bias && act == SCORCH_HIP_ACT_RELU)                                                                 \
+      return scorch::spmm_entry<T, scorch::kEpiBiasRelu>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, bias, \
+                                                         C, workspace, workspace_bytes, stream, nullptr,    \
+                                                         bounds, bounds_bytes);                             \
+    return scorch::fail(SCORCH_HIP_EINVAL, "%s: activation %d (with%s bias) is not supported", fn, act,     \
+                        bias ? "" : "out");                                                                 \
+  }
+
+SCORCH_DEFINE_SPMM_PLANNED(f32, float)
+SCORCH_DEFINE_SPMM_PLANNED(f64, double)
+SCORCH_DEFINE_SPMM_PLANNED(i32, int32_t)
+SCORCH_DEFINE_SPMM_PLANNED(i64, int64_t)
 
 int scorch_hip_spmm_csr_f32_static(int64_t M, int64_t K, int64_t N, int64_t nnz,
                                    const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

@@ -20,6 +20,9 @@ _size = ctypes.c_size_t
 OK, EINVAL, EWORKSPACE, ERUNTIME, EUNSUPPORTED = 0, 1, 2, 3, 4
 
 _SPMM = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
+_SPMM_ROWS = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, ctypes.c_int, _ptr, _ptr]
+_SPMM_PLANNED = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr, _size,
+                 _ptr]
 _SPGEMM = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 _SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 
@@ -27,12 +30,31 @@ _SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 SIGNATURES = {
     "scorch_hip_abi_version": (ctypes.c_int, []),
     "scorch_hip_last_error": (ctypes.c_char_p, []),
+    "scorch_hip_timing_begin": (ctypes.c_int, []),
+    "scorch_hip_timing_end": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), ctypes.c_int,
+                                             ctypes.POINTER(ctypes.c_int)]),
     "scorch_hip_spmm_csr_workspace_bytes": (_size, [_i64, _i64, _i64, _size]),
     "scorch_hip_spmm_csr_f32": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_f64": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_i32": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_i64": (ctypes.c_int, _SPMM),
     "scorch_hip_spmm_csr_f32_static": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_csr_inspect": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_spmm_csr_rows_f32": (ctypes.c_int, _SPMM_ROWS),
+    "scorch_hip_spmm_csr_rows_f64": (ctypes.c_int, _SPMM_ROWS),
+    "scorch_hip_spmm_csr_rows_i32": (ctypes.c_int, _SPMM_ROWS),
+    "scorch_hip_spmm_csr_rows_i64": (ctypes.c_int, _SPMM_ROWS),
+    "scorch_hip_spmm_csr_bounds_bytes": (_size, [_i64, _i64, _i64, _size]),
+    "scorch_hip_spmm_csr_bounds": (ctypes.c_int, [_i64, _i64, _i64, _size, _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_spmm_csr_planned_f32": (ctypes.c_int, _SPMM_PLANNED),
+    "scorch_hip_spmm_csr_planned_f64": (ctypes.c_int, _SPMM_PLANNED),
+    "scorch_hip_spmm_csr_planned_i32": (ctypes.c_int, _SPMM_PLANNED),
+    "scorch_hip_spmm_csr_planned_i64": (ctypes.c_int, _SPMM_PLANNED),
+    "scorch_hip_dense_tiled_bytes": (_size, [_i64, _i64, _size]),
+    "scorch_hip_dense_tiled_recommended": (ctypes.c_int, [_i64, _i64, _i64, _size]),
+    "scorch_hip_dense_to_tiled_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_spmm_csr_tiled_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr,
+                                                     ctypes.c_int, _ptr, _ptr, _size, _ptr, _size, _ptr]),
     "scorch_hip_spmm_csr_f32_timed": (ctypes.c_int, _SPMM + [ctypes.POINTER(ctypes.c_float)]),
     "scorch_hip_spmm_csr_bias_act_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr]),
@@ -92,6 +114,22 @@ def lib() -> ctypes.CDLL:
                     fn.argtypes = argtypes
                 _lib = handle
     return _lib
+
+
+def kernel_times(call):
+    """Run ``call()`` (one library call, or several) and return the duration of each
+    kernel it launched, in milliseconds, in launch order (scorch_hip_timing_begin /
+    _end).  Synchronises."""
+    L = lib()
+    check(L.scorch_hip_timing_begin())
+    try:
+        call()
+    finally:
+        ms = (ctypes.c_float * 16)()
+        n = ctypes.c_int(0)
+        rc = L.scorch_hip_timing_end(ms, 16, ctypes.byref(n))
+    check(rc)
+    return [ms[i] for i in range(min(n.value, 16))]
 
 
 def last_error() -> str:

@@ -9,38 +9,52 @@ src/scorch/trace.py:288-299) can call either module.  The tensors must live on
 a HIP device; the work is done by libscorch_hip.so on the current stream of
 the operands' device and the call returns without synchronising.
 
-Only the symbols of the SpMM / SDDMM / SpMV path exist here.  A symbol the
-reference resolves first but this module lacks simply is not found, and the
-reference's resolver moves on (prebuilt_kernels.py:96-101).
+Every symbol of the reference's matmul registry has a counterpart here (CSR x
+dense, CSR x vector, CSR x CSR and the two coordinate-form products) beside
+the SDDMM and fused-epilogue symbols.
+
+What the reference's stateless dispatch does not have: a sparse operand is
+inspected the first time it is seen (index validation, longest row) and the
+result, with the chunk boundaries of the merge-path kernels, is kept on the
+operand's row-pointer tensor; a wide dense operand that comes back unchanged
+is re-stored once by column tiles (see CsrPlan and _tiled_operand below).
 """
 from __future__ import annotations
 
-from typing import Optional
+import os
+from typing import Dict, Optional, Tuple
 
 import torch
 
 from . import native
-from .utils import check_csr_indices, index_checks_enabled
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
 
 class TensorIndex:
+    __slots__ = ("mode_indices",)
+
     def __init__(self, mode_indices=None):
         self.mode_indices = mode_indices if mode_indices is not None else []
 
 
 class TensorStorage:
+    __slots__ = ("value", "index")
+
     def __init__(self, value=None, index=None):
         self.value = value
         self.index = index if index is not None else TensorIndex()
 
 
 class Tensor:
-    """Result carrier with the fields of the reference's csrc/header.h:4-16."""
+    """Result carrier with the fields of the reference's csrc/header.h:4-16
+    (``workspace``: scratch memory that must live as long as the result, see
+    _workspace)."""
+    __slots__ = ("storage", "workspace")
 
     def __init__(self, value=None, mode_indices=None):
         self.storage = TensorStorage(value, TensorIndex(mode_indices))
+        self.workspace = None
 
 
 # ---- helpers -----------------------------------------------------------------
@@ -49,7 +63,14 @@ _workspaces = {}
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     """Scratch buffer for (device, stream), grown on demand.  Kernels on one
-    stream run in order, so they can share it."""
+    stream run in order, so they can share it; host threads that launch on
+    different streams get different buffers.  While the stream is being
+    captured into a HIP graph the buffer comes fresh from the graph's own memory
+    pool instead: a replay must not write into a block that eager calls on the
+    same stream use, or that was replaced by a larger one and returned to the
+    allocator since the capture."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
     key = (device.index, stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
@@ -84,8 +105,6 @@ def _csr_parts(mode_indices, what: str, n_cols: Optional[int] = None):
     if len(mode_indices) != 2 or len(mode_indices[1]) != 2:
         raise ValueError(f"scorch_ops_hip: {what} is not a CSR (\"d,s\") operand")
     pos, crd = _index(mode_indices[1][0], what + " pos"), _index(mode_indices[1][1], what + " crd")
-    if n_cols is not None and index_checks_enabled():
-        check_csr_indices(pos, crd, n_cols, "scorch_ops_hip: " + what)
     return pos, crd
 
 
@@ -122,41 +141,208 @@ class _on_device:
         return False
 
 
+# ---- what is computed once per operand ---------------------------------------------
+def plans_enabled() -> bool:
+    """Sparse operands are inspected and planned unless SCORCH_HIP_PLAN=0."""
+    return os.environ.get("SCORCH_HIP_PLAN", "1") not in ("", "0")
+
+
+ROWS_KERNEL_MAX_ROW = 256   # longest row for which the row-split kernel is chosen
+
+# Which SpMM kernel serves a product.  "auto" (the default; SCORCH_HIP_SPMM_PATH
+# overrides it at import) decides from the operand's plan; the other values pin one
+# path whatever the operand looks like, for tests and measurements:
+#   "rows"             the row-split kernel
+#   "merge"            the merge-path kernels, with precomputed chunk boundaries
+#   "merge_unplanned"  the merge-path kernels searching row_ptr in every wavefront
+#   "tiled"            fp32 only: the dense operand re-stored by column tiles (built
+#                      at once), merge-path split; other dtypes as "merge"
+SPMM_PATHS = ("auto", "rows", "merge", "merge_unplanned", "tiled")
+SPMM_PATH = os.environ.get("SCORCH_HIP_SPMM_PATH", "auto")
+
+
+class CsrPlan:
+    """Facts about one CSR index that do not change from call to call: it is well
+    formed, its longest row, and (filled in on demand, per dense width) the
+    chunk boundaries of the merge-path kernels.  Lives as an attribute of the
+    row-pointer tensor, so it is dropped with the operand, and is rebuilt when
+    either index tensor has been written to since."""
+    __slots__ = ("key", "max_row", "empty_rows", "bounds")
+
+    def __init__(self, key, max_row: int, empty_rows: int):
+        self.key = key
+        self.max_row = max_row
+        self.empty_rows = empty_rows
+        self.bounds: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, what: str = "operand") -> Optional[CsrPlan]:
+    """The plan of (pos, crd), built on first sight: one inspection kernel and
+    one read of its four-integer report (a synchronisation).  Raises ValueError
+    for a malformed index -- row pointers that do not start at 0, end at
+    len(crd) or decrease, column indices outside [0, n_cols) -- before any
+    kernel dereferences it.  None when planning is switched off or the stream
+    is being captured (no synchronisation is possible there)."""
+    key = (pos._version, crd.data_ptr(), crd._version, crd.numel(), n_rows, n_cols)
+    plan = getattr(pos, "_scorch_plan", None)
+    if plan is not None and plan.key == key:
+        return plan
+    if not plans_enabled():
+        return None
+    if pos.numel() != n_rows + 1:
+        raise ValueError(f"scorch_ops_hip: {what}: row pointer has {pos.numel()} entries, expected {n_rows + 1}")
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    dev = pos.device
+    report = torch.empty(4, dtype=torch.int32, device=dev)
+    with _on_device(dev):
+        native.check(native.lib().scorch_hip_csr_inspect(n_rows, n_cols, crd.numel(), pos.data_ptr(),
+                                                         crd.data_ptr(), report.data_ptr(), _stream(dev)))
+    bad_rows, bad_cols, max_row, empty_rows = report.tolist()
+    if bad_rows or bad_cols:
+        problems = []
+        if bad_rows:
+            problems.append(f"row_ptr must start at 0, never decrease and end at {crd.numel()}")
+        if bad_cols:
+            problems.append(f"a column index lies outside [0, {n_cols})")
+        raise ValueError(f"scorch_ops_hip: {what}: malformed CSR index: " + "; ".join(problems))
+    plan = CsrPlan(key, max_row, empty_rows)
+    try:
+        pos._scorch_plan = plan
+    except (AttributeError, RuntimeError):      # an object that takes no attributes: plan per call
+        pass
+    return plan
+
+
+def _chunk_bounds(plan: CsrPlan, pos: torch.Tensor, M: int, nnz: int, N: int, elem: int, L, stream) -> torch.Tensor:
+    """Chunk boundaries of the merge-path split for dense width N, computed once."""
+    bounds = plan.bounds.get((N, elem))
+    if bounds is None:
+        bounds = torch.empty(L.scorch_hip_spmm_csr_bounds_bytes(M, nnz, N, elem), dtype=torch.uint8,
+                             device=pos.device)
+        native.check(L.scorch_hip_spmm_csr_bounds(M, nnz, N, elem, pos.data_ptr(), bounds.data_ptr(),
+                                                  bounds.numel(), stream))
+        plan.bounds[(N, elem)] = bounds
+    return bounds
+
+
+def tiled_operands_enabled() -> bool:
+    """A wide dense operand that is multiplied again unchanged is re-stored by
+    column tiles unless SCORCH_HIP_TILED=0."""
+    return os.environ.get("SCORCH_HIP_TILED", "1") not in ("", "0")
+
+
+def _dense_owner(values: torch.Tensor) -> torch.Tensor:
+    """The tensor object that carries a dense operand's cached layouts: the user's
+    own tensor when `values` is the flat view STensor.from_torch made of it."""
+    return getattr(values, "_scorch_origin", values)
+
+
+def prepare_dense_operand(values: torch.Tensor, K: int, N: int) -> Optional[torch.Tensor]:
+    """Store a dense fp32 operand (K x N, row-major, on a HIP device) by column
+    tiles now, for the products that follow (what a second product with the same
+    unchanged tensor would trigger by itself).  Returns the tiled copy, which
+    stays attached to the tensor until the tensor is written to or dropped; None
+    if the layout does not apply (other dtypes)."""
+    if values.dtype != torch.float32:
+        return None
+    owner = _dense_owner(values)
+    dev = values.device
+    L = native.lib()
+    flat = values if values.is_contiguous() else values.contiguous()
+    bt = torch.empty(L.scorch_hip_dense_tiled_bytes(K, N, 4) // 4, dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        native.check(L.scorch_hip_dense_to_tiled_f32(K, N, flat.data_ptr(), bt.data_ptr(), bt.numel() * 4,
+                                                     _stream(dev)))
+    owner._scorch_tiled = (owner._version, values.data_ptr(), K, N, bt)
+    return bt
+
+
+def _tiled_operand(values: torch.Tensor, K: int, N: int, nnz: int, L) -> Optional[torch.Tensor]:
+    """The column-tile copy of a dense operand if it has one that is still valid,
+    or if this is the second product in a row with the same unchanged tensor
+    (then it is built now); else None.  Only for shapes where the layout pays."""
+    if N < 512 or values.dtype != torch.float32:      # (rows of 2 KiB and more: the library's own first test)
+        return None
+    if not tiled_operands_enabled() or not L.scorch_hip_dense_tiled_recommended(K, N, nnz, 4):
+        return None
+    owner = _dense_owner(values)
+    stamp = (owner._version, values.data_ptr(), K, N)
+    cached = getattr(owner, "_scorch_tiled", None)
+    if cached is not None and cached[:4] == stamp:
+        return cached[4]
+    if getattr(owner, "_scorch_seen", None) == stamp and not torch.cuda.is_current_stream_capturing():
+        return prepare_dense_operand(values, K, N)
+    try:
+        owner._scorch_seen = stamp
+    except (AttributeError, RuntimeError):
+        pass
+    return None
+
+
 # ---- SpMM ----------------------------------------------------------------------
 def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values,
           bias=None, act=0):
     M, K = int(A_shape[0]), int(A_shape[1])
     N = int(B_shape[1])
-    if int(B_shape[0]) != K or tuple(int(s) for s in result_shape) != (M, N):
+    if int(B_shape[0]) != K or len(result_shape) != 2 or int(result_shape[0]) != M or int(result_shape[1]) != N:
         raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)} "
                          f"result{tuple(result_shape)}")
-    pos, crd = _csr_parts(A_mode_indices, "A", K)
+    pos, crd = _csr_parts(A_mode_indices, "A")
     a_val = _flat(A_values, dtype, "A values")
     b_val = _flat(B_values, dtype, "B values")
     if pos.numel() != M + 1 or b_val.numel() != K * N or crd.numel() != a_val.numel():
         raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
     dev = _device_of(pos, crd, a_val, b_val)
     nnz = a_val.numel()
+    bias_ptr = None
+    if bias is not None:
+        if dtype != torch.float32:
+            raise TypeError("scorch_ops_hip: the fused bias / activation kernels are fp32")
+        bias = _flat(bias, dtype, "bias")
+        if bias.numel() != N or bias.device != dev:
+            raise ValueError("scorch_ops_hip: bias must have N elements on the operands' device")
+        bias_ptr = bias.data_ptr()
+    if SPMM_PATH not in SPMM_PATHS:
+        raise ValueError(f"scorch_ops_hip: SPMM_PATH is {SPMM_PATH!r}, expected one of {SPMM_PATHS}")
+    plan = csr_plan(pos, crd, M, K, "A")
     out = torch.empty(M * N, dtype=dtype, device=dev)
     L = native.lib()
+    suffix = _SUFFIX[dtype]
+    elem = a_val.element_size()
+    path = SPMM_PATH if M > 0 and N > 0 else "merge_unplanned"
     with _on_device(dev):
         stream = _stream(dev)
-        need = L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, a_val.element_size())
-        ws = _workspace(dev, stream, need)
-        if bias is None:
-            fn = getattr(L, "scorch_hip_spmm_csr_" + _SUFFIX[dtype])
-            rc = fn(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(),
-                    out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+        # a wide dense operand that keeps coming back is served from its column-tile copy
+        tiled = None
+        if path == "auto":
+            tiled = _tiled_operand(B_values, K, N, nnz, L)
+        elif path == "tiled" and dtype == torch.float32:
+            tiled = prepare_dense_operand(B_values, K, N)
+        if tiled is None and (path == "rows" or (path == "auto" and plan is not None
+                                                 and plan.max_row <= ROWS_KERNEL_MAX_ROW)):
+            # every row is short: one launch of the row-split kernel, no workspace
+            rc = getattr(L, "scorch_hip_spmm_csr_rows_" + suffix)(
+                M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(), bias_ptr, act,
+                out.data_ptr(), stream)
+            native.check(rc)
+            return Tensor(out, [[], []])
+        ws = _workspace(dev, stream, L.scorch_hip_spmm_csr_workspace_bytes(M, nnz, N, elem))
+        bounds = _chunk_bounds(plan, pos, M, nnz, N, elem, L, stream) \
+            if plan is not None and path != "merge_unplanned" else None
+        bounds_ptr, bounds_bytes = (bounds.data_ptr(), bounds.numel()) if bounds is not None else (None, 0)
+        if tiled is not None:
+            rc = L.scorch_hip_spmm_csr_tiled_f32(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(),
+                                                 tiled.data_ptr(), tiled.numel() * 4, bias_ptr, act, out.data_ptr(),
+                                                 bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
         else:
-            bias = _flat(bias, dtype, "bias")
-            if bias.numel() != N or bias.device != dev:
-                raise ValueError("scorch_ops_hip: bias must have N elements on the operands' device")
-            rc = L.scorch_hip_spmm_csr_bias_act_f32(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
-                                                    a_val.data_ptr(), b_val.data_ptr(), bias.data_ptr(),
-                                                    act, out.data_ptr(), ws.data_ptr(), ws.numel(),
-                                                    stream)
+            rc = getattr(L, "scorch_hip_spmm_csr_planned_" + suffix)(
+                M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(), bias_ptr, act,
+                out.data_ptr(), bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
     native.check(rc)
-    return Tensor(out, [[], []])
+    result = Tensor(out, [[], []])
+    result.workspace = ws      # a buffer handed out during a graph capture lives as long as the result
+    return result
 
 
 def _make_spmm(dtype):
@@ -216,14 +402,16 @@ def _make_spgemm(dtype):
         M, K, N = int(A_shape[0]), int(A_shape[1]), int(B_shape[1])
         if int(B_shape[0]) != K:
             raise ValueError(f"scorch_ops_hip: shape mismatch A{tuple(A_shape)} B{tuple(B_shape)}")
-        a_pos, a_crd = _csr_parts(A_mode_indices, "A", K)
-        b_pos, b_crd = _csr_parts(B_mode_indices, "B", N)
+        a_pos, a_crd = _csr_parts(A_mode_indices, "A")
+        b_pos, b_crd = _csr_parts(B_mode_indices, "B")
         a_val = _flat(A_values, dtype, "A values")
         b_val = _flat(B_values, dtype, "B values")
         if a_pos.numel() != M + 1 or b_pos.numel() != K + 1 or a_crd.numel() != a_val.numel() \
                 or b_crd.numel() != b_val.numel():
             raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
         dev = _device_of(a_pos, a_crd, a_val, b_pos, b_crd, b_val)
+        csr_plan(a_pos, a_crd, M, K, "A")      # validates the indices (once per operand)
+        csr_plan(b_pos, b_crd, K, N, "B")
         L = native.lib()
         with _on_device(dev):
             stream = _stream(dev)
@@ -256,12 +444,13 @@ prebuilt_spmspm_csr_i64 = _make_spgemm(torch.int64)
 def _make_spmv(dtype):
     def kernel(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
         M, K = int(A_shape[0]), int(A_shape[1])
-        pos, crd = _csr_parts(A_mode_indices, "A", K)
+        pos, crd = _csr_parts(A_mode_indices, "A")
         a_val = _flat(A_values, dtype, "A values")
         x = _flat(B_values, dtype, "x values")
         if pos.numel() != M + 1 or x.numel() != K or crd.numel() != a_val.numel():
             raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
         dev = _device_of(pos, crd, a_val, x)
+        csr_plan(pos, crd, M, K, "A")
         y = torch.empty(M, dtype=dtype, device=dev)
         L = native.lib()
         with _on_device(dev):
@@ -324,11 +513,12 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     mask entry in mask order: what the reference's generated kernel returns for
     this case (src/scorch/ops.py:638-666).  mode_indices = [[rows], [S's crd]]."""
     M, n_cols, K, a, b = _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values)
-    pos, crd = _csr_parts(S_mode_indices, "S", n_cols)
+    pos, crd = _csr_parts(S_mode_indices, "S")
     s_val = _flat(S_values, torch.float32, "S values")
     if pos.numel() != M + 1 or crd.numel() != s_val.numel():
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
     dev = _device_of(pos, crd, s_val, a, b)
+    csr_plan(pos, crd, M, n_cols, "S")
     out = torch.empty_like(s_val)
     rows = torch.empty_like(crd)
     with _on_device(dev):

@@ -188,9 +188,14 @@ class STensor(torch.nn.Module):
             return STensor._csr(tensor.shape, tensor.crow_indices(), tensor.col_indices(),
                                 tensor.values(), name, mode_order)
         fmt = TensorFormat([LevelFormat(LevelType.DENSE) for _ in tensor.shape])
+        value = tensor.flatten()
+        if value is not tensor and value.is_cuda and value.data_ptr() == tensor.data_ptr():
+            # a view of the caller's tensor: layouts the device kernels cache for this
+            # operand are kept on the caller's object, which outlives the view
+            value._scorch_origin = tensor
         return STensor(name=name, shape=tuple(tensor.shape), storage=TensorStorage(
             index=TensorIndex(fmt, [[] for _ in tensor.shape], mode_order=mode_order),
-            value=tensor.flatten()))
+            value=value))
 
     # ---- conversion ------------------------------------------------------------------
     def _as_torch_sparse(self) -> torch.Tensor:

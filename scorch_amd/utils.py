@@ -2,8 +2,6 @@
 from .format import parse_format  # noqa: F401  (same import path as the reference's utils.parse_format)
 
 
-import os
-
 import torch
 
 
@@ -14,8 +12,10 @@ def check_csr_indices(row_ptr: torch.Tensor, col_idx: torch.Tensor, n_cols: int,
 
     Neither the reference's kernels nor the HIP kernels look at index contents: an
     out-of-range column is undefined behaviour on the host and a memory fault on a
-    GPU.  The check runs with torch operations on whatever device holds the
-    arrays and costs one pass over them plus a synchronisation."""
+    GPU.  This check runs with torch operations on whatever device holds the
+    arrays (one pass over them plus a synchronisation) and names what is wrong;
+    the device wrappers make the same checks with one kernel the first time they
+    see an operand (scorch_ops_hip.csr_plan)."""
     if row_ptr.numel() == 0:
         raise ValueError(f"{what}: empty row pointer")
     problems = []
@@ -31,9 +31,3 @@ def check_csr_indices(row_ptr: torch.Tensor, col_idx: torch.Tensor, n_cols: int,
             problems.append(f"column indices span [{lo}, {hi}], outside [0, {n_cols})")
     if problems:
         raise ValueError(f"{what}: malformed CSR index: " + "; ".join(problems))
-
-
-def index_checks_enabled() -> bool:
-    """True when SCORCH_HIP_CHECK_INDICES is set to something other than 0/empty:
-    the device wrappers then validate every sparse operand before launching."""
-    return os.environ.get("SCORCH_HIP_CHECK_INDICES", "0") not in ("", "0")

@@ -19,7 +19,26 @@ def host(t):
     return t.detach().cpu().numpy()
 
 
-def hip_spmm(row_ptr, col_idx, vals, B, bias=None, relu=False, K=None):
+class spmm_path:
+    """``with spmm_path("rows"):`` pins the SpMM kernel the wrappers choose."""
+
+    def __init__(self, path):
+        self.path = path
+
+    def __enter__(self):
+        self.previous, H.SPMM_PATH = H.SPMM_PATH, self.path or H.SPMM_PATH
+
+    def __exit__(self, *exc):
+        H.SPMM_PATH = self.previous
+        return False
+
+
+def hip_spmm(row_ptr, col_idx, vals, B, bias=None, relu=False, K=None, path=None):
+    with spmm_path(path):
+        return _hip_spmm(row_ptr, col_idx, vals, B, bias, relu, K)
+
+
+def _hip_spmm(row_ptr, col_idx, vals, B, bias, relu, K):
     M, N = len(row_ptr) - 1, B.shape[1]
     K = B.shape[0] if K is None else K
     args = ([M, N], [M, K], [[], [dev(row_ptr), dev(col_idx)]], dev(vals), [K, N], [[], []],

@@ -18,6 +18,8 @@ from scorch_amd import workloads
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-5
+# every kernel that can serve a product is pinned in turn (scorch_ops_hip.SPMM_PATH)
+PATHS = ["rows", "merge", "merge_unplanned", "tiled"]
 SPMM_F32_CASES = ["spmm_square95", "spmm_dispatch32", "spmm_rect", "spmm_wide300", "spmm_emptyrows",
                   "spmm_n1", "spmm_longrow", "spmm_allzero", "spmm_diag_literal"]
 
@@ -62,12 +64,13 @@ def test_golden_bias_act(golden, oracle, relu):
 
 # N chosen to hit every vector width and tile count: 1 lane, odd, < 64, = 64,
 # between tiles, 2-wide vectors (128), partial second tile (192), 4-wide (256+), many tiles
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("N", [1, 3, 17, 48, 64, 70, 96, 100, 128, 130, 192, 256, 300, 512, 1028])
-def test_widths_against_oracle(oracle, N):
+def test_widths_against_oracle(oracle, N, path):
     rng = np.random.default_rng(N)
     rp, ci, v = random_csr(rng, 333, 217, 0.06, empty_rows=(0, 100, 332))
     B = rng.standard_normal((217, N)).astype(np.float32)
-    got = hip_spmm(rp, ci, v, B)
+    got = hip_spmm(rp, ci, v, B, path=path)
     assert oracle.rel_fro(got, oracle.spmm_fp64(rp, ci, v, B)) <= TOL
     np.testing.assert_allclose(got, oracle.spmm_csr_f32_v2(rp, ci, v, B), rtol=1e-4, atol=1e-5)
 
@@ -101,28 +104,30 @@ def row_length_cases():
 ROW_CASES = row_length_cases()
 
 
+@pytest.mark.parametrize("path", PATHS + ["auto"])
 @pytest.mark.parametrize("name", sorted(ROW_CASES))
 @pytest.mark.parametrize("N", [32, 128, 260])
-def test_row_length_distributions(oracle, name, N):
+def test_row_length_distributions(oracle, name, N, path):
     rp, ci = ROW_CASES[name]          # columns unsorted and repeating: allowed
     rng = np.random.default_rng(len(name) + N)
     v = rng.uniform(-1, 1, ci.size).astype(np.float32)
     B = rng.standard_normal((500, N)).astype(np.float32)
-    got = hip_spmm(rp, ci, v, B)
+    got = hip_spmm(rp, ci, v, B, path=path)
     ref64 = oracle.spmm_fp64(rp, ci, v, B)
     assert oracle.rel_fro(got, ref64) <= TOL
     assert not got[np.diff(rp) == 0].any()
 
 
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("name", ["power_law", "long_ends", "mostly_empty"])
 @pytest.mark.parametrize("relu", [False, True])
-def test_bias_act_on_split_rows(oracle, name, relu):
+def test_bias_act_on_split_rows(oracle, name, relu, path):
     rp, ci = ROW_CASES[name]
     rng = np.random.default_rng(7)
     v = rng.uniform(-1, 1, ci.size).astype(np.float32)
     B = rng.standard_normal((500, 128)).astype(np.float32)
     bias = rng.standard_normal(128).astype(np.float32)
-    got = hip_spmm(rp, ci, v, B, bias=bias, relu=relu)
+    got = hip_spmm(rp, ci, v, B, bias=bias, relu=relu, path=path)
     ref = oracle.spmm_fp64(rp, ci, v, B) + bias.astype(np.float64)
     if relu:
         ref = np.maximum(ref, 0)
@@ -132,9 +137,10 @@ def test_bias_act_on_split_rows(oracle, name, relu):
                                atol=2e-5)
 
 
+@pytest.mark.parametrize("path", ["rows", "merge", "merge_unplanned"])
 @pytest.mark.parametrize("dtype", [np.float64, np.int32, np.int64])
 @pytest.mark.parametrize("N", [5, 64, 128, 200])
-def test_other_dtypes_against_oracle(oracle, dtype, N):
+def test_other_dtypes_against_oracle(oracle, dtype, N, path):
     rp, ci = ROW_CASES["power_law"]
     rng = np.random.default_rng(N)
     if np.issubdtype(dtype, np.integer):
@@ -143,7 +149,7 @@ def test_other_dtypes_against_oracle(oracle, dtype, N):
     else:
         v = rng.uniform(-1, 1, ci.size).astype(dtype)
         B = rng.standard_normal((500, N)).astype(dtype)
-    got = hip_spmm(rp, ci, v, B)
+    got = hip_spmm(rp, ci, v, B, path=path)
     want = oracle.spmm_csr_typed(rp, ci, v, B)
     if np.issubdtype(dtype, np.integer):
         assert np.array_equal(got, want)        # wraps identically (int32 products overflow here)
@@ -255,14 +261,15 @@ def test_uniform_workload_reference_size(oracle):
                                rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("path", ["merge", "tiled", "rows"])
 @pytest.mark.parametrize("M", [1024, 4096])
-def test_sae_decoder_workload(oracle, M):
+def test_sae_decoder_workload(oracle, M, path):
     """Sparse-autoencoder decoder shape (32 entries per row, K = 16,384, N = 4096): at a quarter of the
     rows, and at the full 4096 rows that `bench.py --workload sae_decoder` times (the work split
     depends on the size, so the two take different chunk sizes)."""
     w = workloads.sae_decoder(M=M)
     assert w["K"] == 16_384 and w["N"] == 4096 and w["col_idx"].size == 32 * M
-    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"])
+    got = hip_spmm(w["row_ptr"], w["col_idx"], w["vals"], w["B"], path=path)
     assert oracle.rel_fro(got, oracle.spmm_fp64(w["row_ptr"], w["col_idx"], w["vals"], w["B"])) <= TOL
 
 

@@ -276,7 +276,8 @@ def test_change_mode_order_rejects_what_it_cannot_do():
 
 
 def test_check_csr_indices_names_what_is_wrong(monkeypatch):
-    from scorch_amd.utils import check_csr_indices, index_checks_enabled
+    from scorch_amd.scorch_ops_hip import plans_enabled, tiled_operands_enabled
+    from scorch_amd.utils import check_csr_indices
     pos = torch.tensor([0, 2, 2, 5], dtype=torch.int32)
     crd = torch.tensor([0, 3, 1, 2, 3], dtype=torch.int32)
     check_csr_indices(pos, crd, 4)                                   # well-formed: no exception
@@ -288,7 +289,10 @@ def test_check_csr_indices_names_what_is_wrong(monkeypatch):
         check_csr_indices(torch.tensor([0, 2, 2, 4], dtype=torch.int32), crd, 4)
     with pytest.raises(ValueError, match=r"row_ptr\[0\] = 1"):
         check_csr_indices(torch.tensor([1, 2, 2, 5], dtype=torch.int32), crd, 4)
-    monkeypatch.delenv("SCORCH_HIP_CHECK_INDICES", raising=False)
-    assert not index_checks_enabled()
-    monkeypatch.setenv("SCORCH_HIP_CHECK_INDICES", "1")
-    assert index_checks_enabled()
+    # operands are inspected (and planned) by default; both switches are opt-outs
+    monkeypatch.delenv("SCORCH_HIP_PLAN", raising=False)
+    monkeypatch.delenv("SCORCH_HIP_TILED", raising=False)
+    assert plans_enabled() and tiled_operands_enabled()
+    monkeypatch.setenv("SCORCH_HIP_PLAN", "0")
+    monkeypatch.setenv("SCORCH_HIP_TILED", "0")
+    assert not plans_enabled() and not tiled_operands_enabled()
