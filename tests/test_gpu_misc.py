@@ -357,15 +357,14 @@ def test_sparse_to_sparse_conversion_does_not_densify():
     assert torch.allclose(scorch.matmul(C, x), want, atol=1e-4)
 
 
-def test_index_check_stops_a_bad_operand_before_the_launch(monkeypatch):
-    """With SCORCH_HIP_CHECK_INDICES=1 an out-of-range column raises ValueError in
-    the Python layer; nothing is launched."""
-    monkeypatch.setenv("SCORCH_HIP_CHECK_INDICES", "1")
+def test_index_check_stops_a_bad_operand_before_the_launch():
+    """An out-of-range column raises ValueError from the inspection every operand gets when
+    it is first seen; the product's kernel is not launched."""
     pos = torch.tensor([0, 1, 2], dtype=torch.int32, device="cuda")
     crd = torch.tensor([0, 7], dtype=torch.int32, device="cuda")      # 7 >= K = 4
     val = torch.ones(2, device="cuda")
     B = torch.ones(4 * 8, device="cuda")
-    with pytest.raises(ValueError, match="column indices span"):
+    with pytest.raises(ValueError, match="column index lies outside"):
         H.spmm_csr_float_v2([2, 8], [2, 4], [[], [pos, crd]], val, [4, 8], [[], []], B)
     good = torch.tensor([0, 3], dtype=torch.int32, device="cuda")
     out = H.spmm_csr_float_v2([2, 8], [2, 4], [[], [pos, good]], val, [4, 8], [[], []], B)
