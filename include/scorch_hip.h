@@ -322,7 +322,9 @@ SCORCH_HIP_API int scorch_hip_spmv_csr_i64(int64_t M, int64_t K, int64_t nnz, co
  * known:
  *   1. _symbolic writes c_row_ptr[M + 1] (device).  The caller reads
  *      c_row_ptr[M] back (that read synchronises) and allocates c_col_idx
- *      and c_vals of that length.
+ *      and c_vals of that length.  c_row_ptr[M] == -1 means that the result
+ *      has 2^31 entries or more, which its int32 row pointer cannot hold: the
+ *      rest of c_row_ptr is then meaningless and _numeric must not be called.
  *   2. _numeric_<T> fills c_col_idx and c_vals.
  * As in the reference, column indices are ascending within each row and every
  * structurally reachable entry is stored, also when its value sums to zero.

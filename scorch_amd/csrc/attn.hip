@@ -33,6 +33,7 @@ namespace scorch {
 
 constexpr int kAttnBlock = 64;  // mask block edge: queries per workgroup, keys per step
 constexpr int kAttnDim = 64;    // head dimension
+constexpr float kRescaleSlack = 8.0f;  // see the online softmax in the kernel
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -77,8 +78,14 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O) {
-  __shared__ __attribute__((aligned(1024))) unsigned char s_k[2][kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_v[2][kTileBytes];
+  // Two buffers each for K and V, as four separate arrays: the compiler then sees that the
+  // loads which fill one buffer (they write LDS asynchronously) cannot touch the buffer being
+  // read, and does not make the reads wait for them.  (As halves of one array, every second key
+  // block waited for its own prefetch before its first LDS read.)
+  __shared__ __attribute__((aligned(1024))) unsigned char s_k0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_k1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_v0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_v1[kTileBytes];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
@@ -118,6 +125,9 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) o_acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -3.0e38f;
+  // (scale 0: every score counts as 0, nothing ever needs rescaling beyond the first block)
+  const float inv_scale_log2e = scale_log2e != 0.0f ? 1.0f / scale_log2e : 0.0f;
+  float raise_at = NEGATIVE_SCALE ? 3.0e38f : -3.0e38f;  // the first key block always sets m_run
   floatx4 l_acc = floatx4{0.f, 0.f, 0.f, 0.f};  // row sums of P, taken by the matrix core (ones row)
   bf16x8 ones;
 #pragma unroll
@@ -126,21 +136,24 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   const int kb_begin = block_row_ptr[qb];
   const int kb_end = block_row_ptr[qb + 1];
 
+
   // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with two instructions
   // of eight rows each.  Lane L of instruction u lands at row 16w + 8u + L / 8,
   // position L % 8, which holds chunk (L % 8) ^ (row & 7) = (L % 8) ^ (L / 8).
   const int src_in_tile = (16 * w + (lane >> 3)) * 128 + (((lane & 7) ^ (lane >> 3)) * 16);
   auto load_tile = [&](auto buf_tag, int it) {
     constexpr int kBuf = decltype(buf_tag)::value;
+    unsigned char *k_dst = kBuf ? s_k1 : s_k0;
+    unsigned char *v_dst = kBuf ? s_v1 : s_v0;
     const size_t tile = (size_t)uniform(block_col_idx[it]) * kTileBytes;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void *)(Kb + tile + src_in_tile + u * 1024),
-          (__attribute__((address_space(3))) void *)(&s_k[kBuf][(16 * w + 8 * u) * 128]), 16, 0, 0);
+          (__attribute__((address_space(3))) void *)(&k_dst[(16 * w + 8 * u) * 128]), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void *)(Vb + tile + src_in_tile + u * 1024),
-          (__attribute__((address_space(3))) void *)(&s_v[kBuf][(16 * w + 8 * u) * 128]), 16, 0, 0);
+          (__attribute__((address_space(3))) void *)(&v_dst[(16 * w + 8 * u) * 128]), 16, 0, 0);
     }
   };
   using Even = std::integral_constant<int, 0>;
@@ -156,18 +169,21 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   const int v_chunk = (n & 3) >> 1;
 
   if (kb_begin < kb_end) load_tile(Even{}, kb_begin);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   auto key_block = [&](auto tag, int it) {
     constexpr int buf = decltype(tag)::value;
     using Other = std::integral_constant<int, buf ^ 1>;
+    const unsigned char *k_src = buf ? s_k1 : s_k0;
+    const unsigned char *v_src = buf ? s_v1 : s_v0;
     if (it + 1 < kb_end) load_tile(Other{}, it + 1);  // its last readers passed the previous barrier
 
     floatx4 st[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&s_k[buf][2048 * t + k_off]);
-      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&s_k[buf][2048 * t + (k_off ^ 64)]);
+      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&k_src[2048 * t + k_off]);
+      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&k_src[2048 * t + (k_off ^ 64)]);
       st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_lo, q_op[0], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
       st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_hi, q_op[1], st[t], 0, 0, 0);
     }
@@ -177,25 +193,34 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) mx = NEGATIVE_SCALE ? fminf(mx, st[t][r]) : fmaxf(mx, st[t][r]);
-    mx *= scale_log2e;
-    mx = combine_query_lanes(mx, [](float a, float b) { return fmaxf(a, b); });
-    const float m_new = fmaxf(m_run, mx);
-    if (__any(m_new > m_run)) {
+    // The running maximum only has to keep the exponentials in range, so it is raised (and the
+    // accumulators rescaled) only when a score exceeds it by more than kRescaleSlack in the
+    // base-2 exponent: probabilities then reach 2^kRescaleSlack at most, which fp32 sums and bf16
+    // operands hold with the same relative precision, and the final division by the row sum
+    // cancels the common factor.  Whether that is the case is decided on each lane's own 16 raw
+    // scores against `raise_at` = (m_run + kRescaleSlack) / scale: a query's four lanes share its
+    // m_run, so one of them sees any score that matters, and the exchange between lanes that the
+    // true maximum needs is paid only when the branch is taken -- after a row's first key blocks
+    // hardly ever.
+    if (__any(NEGATIVE_SCALE ? mx < raise_at : mx > raise_at)) {
+      mx = combine_query_lanes(mx * scale_log2e, [](float a, float b) { return fmaxf(a, b); });
+      const float m_new = fmaxf(m_run, mx);
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_acc[0] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
+      m_run = m_new;
+      raise_at = (m_run + kRescaleSlack) * inv_scale_log2e;
     }
-    m_run = m_new;
 
     bf16x8 p_op[2];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_new));
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_run));
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
 
@@ -204,8 +229,8 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const int at = 4096 * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
-        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&s_v[buf][at]);
-        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&s_v[buf][at + 2048]);
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 2048]);
         const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         const bf16x8 v_op = __builtin_bit_cast(bf16x8, packed);
         o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
@@ -213,7 +238,10 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 #pragma unroll
     for (int s = 0; s < 2; ++s) l_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, p_op[s], l_acc, 0, 0, 0);
 
-    __syncthreads();  // waits for the loads issued above, and lets the next block overwrite this buffer
+    // the tile requested above must have landed in LDS before any wavefront reads it: the wait
+    // is stated here and not left to the compiler's bookkeeping of asynchronous LDS writes
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // ... and lets the next block overwrite this buffer
   };
 
   for (int it = kb_begin; it < kb_end; it += 2) {

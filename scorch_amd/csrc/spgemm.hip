@@ -284,16 +284,27 @@ __device__ __forceinline__ void for_each_product(int a_lo, int a_hi, int t, cons
 constexpr int kScanPerThread = 16;
 constexpr int kScanTile = kBlockThreads * kScanPerThread;
 
+// (*grand_total also receives the sum of all counts in 64 bits: the row pointer is int32,
+// and a result of 2^31 entries or more must be reported, not wrapped)
 __global__ __launch_bounds__(kBlockThreads) void scan_tile_totals_kernel(const int *__restrict__ data,
                                                                          int64_t n,
-                                                                         int *__restrict__ totals) {
+                                                                         int *__restrict__ totals,
+                                                                         unsigned long long *__restrict__ grand_total) {
   __shared__ int s_scan[kWavesPerBlock + 1];
   const int64_t first = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
   int mine = 0;
-  for (int e = 0; e < kScanPerThread; ++e) mine += first + e < n ? data[first + e] : 0;
+  long long wide = 0;
+  for (int e = 0; e < kScanPerThread; ++e) {
+    const int v = first + e < n ? data[first + e] : 0;
+    mine += v;
+    wide += v;
+  }
   int total = 0;
   (void)block_exclusive_scan(mine, s_scan, total);
   if (threadIdx.x == 0) totals[blockIdx.x] = total;
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) wide += __shfl_xor(wide, off);
+  if (wave_lane() == 0 && wide > 0) atomicAdd(grand_total, (unsigned long long)wide);
 }
 
 __global__ __launch_bounds__(kBlockThreads) void scan_spine_kernel(int *__restrict__ totals,
@@ -310,8 +321,10 @@ __global__ __launch_bounds__(kBlockThreads) void scan_spine_kernel(int *__restri
   }
 }
 
+// (the last element, the total, becomes -1 when the 64-bit total does not fit an int32)
 __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restrict__ data, int64_t n,
-                                                                   const int *__restrict__ totals) {
+                                                                   const int *__restrict__ totals,
+                                                                   const unsigned long long *__restrict__ grand_total) {
   __shared__ int s_scan[kWavesPerBlock + 1];
   const int64_t first = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanPerThread;
   int v[kScanPerThread];
@@ -323,7 +336,7 @@ __global__ __launch_bounds__(kBlockThreads) void scan_apply_kernel(int *__restri
   int total = 0;
   int running = totals[blockIdx.x] + block_exclusive_scan(mine, s_scan, total);
   for (int e = 0; e < kScanPerThread; ++e) {
-    if (first + e < n) data[first + e] = running;
+    if (first + e < n) data[first + e] = first + e == n - 1 && *grand_total > (unsigned long long)INT32_MAX ? -1 : running;
     running += v[e];
   }
 }
@@ -456,7 +469,8 @@ __device__ __forceinline__ int huge_row(const int *__restrict__ rows, int M, int
   return idx < n_giant ? rows[M - 1 - idx] : rows[idx - n_giant];
 }
 
-// counters: [0] medium rows, [1] huge rows, [2] small rows, [5] giant rows listed; [3], [4] next row to hand out
+// counters: [0] medium rows, [1] huge rows, [2] small rows, [5] giant rows listed; [3], [4] next row to hand out;
+// [6..7] one 64-bit sum: the number of entries of the result
 __global__ void spgemm_reset_kernel(int *counters, int *c_pos_last) {
   if (threadIdx.x < 8) counters[threadIdx.x] = 0;
   if (threadIdx.x == 0 && c_pos_last) *c_pos_last = 0;
@@ -1204,11 +1218,12 @@ int spgemm_run(int M, int N, const int *a_pos, const int *a_crd, const T *a_val,
   if (!NUMERIC) {
     const int64_t n = (int64_t)M + 1;
     const unsigned tiles = (unsigned)((n + kScanTile - 1) / kScanTile);
-    scan_tile_totals_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals);
+    unsigned long long *grand_total = reinterpret_cast<unsigned long long *>(ws.counters + 6);
+    scan_tile_totals_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals, grand_total);
     SCORCH_HIP_CHECK(hipGetLastError());
     scan_spine_kernel<<<1, kBlockThreads, 0, stream>>>(ws.scan_totals, tiles);
     SCORCH_HIP_CHECK(hipGetLastError());
-    scan_apply_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals);
+    scan_apply_kernel<<<tiles, kBlockThreads, 0, stream>>>(c_pos, n, ws.scan_totals, grand_total);
     SCORCH_HIP_CHECK(hipGetLastError());
   }
   return SCORCH_HIP_OK;

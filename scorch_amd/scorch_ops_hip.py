@@ -423,6 +423,9 @@ def _make_spgemm(dtype):
                                                           c_pos.data_ptr(), ws.data_ptr(), ws.numel(),
                                                           stream))
             nnz = int(c_pos[-1].item())
+            if nnz < 0:
+                raise native.ScorchHipError(native.EUNSUPPORTED,
+                                            "SpGEMM: the result has 2^31 entries or more, beyond its int32 row pointer")
             c_crd = torch.empty(nnz, dtype=torch.int32, device=dev)
             c_val = torch.empty(nnz, dtype=dtype, device=dev)
             fn = getattr(L, "scorch_hip_spgemm_csr_numeric_" + _SUFFIX[dtype])

@@ -9,6 +9,9 @@ product, the call is served by the fused SpMM kernel
 stores each row.  Any other chain runs as the plain ``matmul`` followed by the
 same torch operations, one after the other -- what the reference's non-prebuilt
 route amounts to (trace.py:304-358) -- so results are identical either way.
+Whatever the function does after the chain (a reduction, an indexing step, a
+second consumer of the product) is run from the traced graph on the chain's
+result, so the decorated function always returns what the plain function would.
 """
 from __future__ import annotations
 
@@ -47,6 +50,8 @@ class FusionSpec:
     post_ops: PostOps
     extra_arg_indices: List[int]        # arguments that are operands of the post-ops
     output_format: Optional[str] = None
+    chain_nodes: List[torch.fx.Node] = field(default_factory=list)   # matmul and the chain, in order
+    complete: bool = True               # the chain's last node is what the function returns
 
 
 _BINARY = {operator.add: "add", operator.mul: "mul", torch.add: "add", torch.mul: "mul"}
@@ -107,6 +112,7 @@ def analyze_fx_graph(graph: torch.fx.Graph, real_args: tuple) -> FusionSpec:
     chain = PostOps()
     extra: List[int] = []
     node = matmul_node
+    walked = [matmul_node]
     while len(node.users) == 1:
         (user,) = node.users
         if user.op != "call_function":
@@ -124,8 +130,31 @@ def analyze_fx_graph(graph: torch.fx.Graph, real_args: tuple) -> FusionSpec:
         else:
             break
         node = user
+        walked.append(node)
     kwargs = dict(matmul_node.kwargs)
-    return FusionSpec(matmul_node, matmul_args, kwargs, chain, extra, kwargs.get("format"))
+    # the runners return the chain's result: that is the function's result only if the
+    # chain's last node feeds the output node directly and nothing else
+    users = list(node.users)
+    complete = len(users) == 1 and users[0].op == "output" and users[0].args[0] is node
+    return FusionSpec(matmul_node, matmul_args, kwargs, chain, extra, kwargs.get("format"), walked, complete)
+
+
+class _Remainder(torch.fx.Interpreter):
+    """Runs the traced function with the value of the chain's last node given: the
+    nodes of the chain are not executed again, everything else is."""
+
+    def __init__(self, module: torch.fx.GraphModule, spec: FusionSpec, value: Any):
+        super().__init__(module)
+        self._skip = set(spec.chain_nodes[:-1])
+        self._tail = spec.chain_nodes[-1]
+        self._value = value
+
+    def run_node(self, n: torch.fx.Node) -> Any:
+        if n is self._tail:
+            return self._value
+        if n in self._skip:
+            return None     # consumed by the next node of the chain only
+        return super().run_node(n)
 
 
 def _as_stensor(x) -> STensor:
@@ -199,17 +228,22 @@ class compile:
     def __init__(self, fn: Callable):
         self.fn = fn
         self._fx_graph: Optional[torch.fx.GraphModule] = None
-        self._cache: Dict[tuple, Callable] = {}
+        self._cache: Dict[tuple, tuple] = {}
 
     def __call__(self, *args: Any) -> Any:
         if self._fx_graph is None:
             self._fx_graph = _symbolic_trace(self.fn)
         key = self._build_cache_key(args)
-        runner = self._cache.get(key)
-        if runner is None:
-            runner = compile_fused(analyze_fx_graph(self._fx_graph.graph, args), args)
-            self._cache[key] = runner
-        return runner(args)
+        cached = self._cache.get(key)
+        if cached is None:
+            spec = analyze_fx_graph(self._fx_graph.graph, args)
+            cached = (compile_fused(spec, args), spec)
+            self._cache[key] = cached
+        runner, spec = cached
+        result = runner(args)
+        if spec.complete:
+            return result
+        return _Remainder(self._fx_graph, spec, result).run(*args)
 
     @staticmethod
     def _build_cache_key(args: tuple) -> tuple:

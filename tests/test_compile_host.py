@@ -43,6 +43,38 @@ def test_fusion_analysis_stops_at_a_non_elementwise_consumer():
     adj, x = csr_and_dense()
     spec = analyze_fx_graph(_symbolic_trace(fn).graph, (adj, x, torch.rand(16)))
     assert [op.kind for op in spec.post_ops.ops] == ["add"]
+    assert not spec.complete and [n.op for n in spec.chain_nodes] == ["call_function"] * 2
+    whole = analyze_fx_graph(_symbolic_trace(bias_relu).graph, (adj, x, torch.rand(16)))
+    assert whole.complete and len(whole.chain_nodes) == 3
+
+
+def test_what_follows_the_chain_is_run_from_the_graph(monkeypatch):
+    """(matmul + c).sum(dim=1) * 2 returns a vector, not the product with its bias: the steps
+    after the chain run on the chain's result.  The product itself is stubbed (no device here)."""
+    from scorch_amd import trace
+    adj, x = csr_and_dense()
+    dense = adj.to_dense().to_torch()
+
+    def fake_matmul(a, b, **kwargs):
+        return dense @ (b.to_torch() if isinstance(b, STensor) else b)
+
+    monkeypatch.setattr(trace.ops, "matmul", fake_matmul)
+    monkeypatch.setattr(trace, "_try_prebuilt_fused", lambda spec, args: None)
+
+    @scorch_compile
+    def reduced(a, b, c):
+        return (scorch.matmul(a, b, format="dd") + c).sum(dim=1) * 2.0
+
+    @scorch_compile
+    def two_consumers(a, b, c):
+        h = scorch.matmul(a, b, format="dd")
+        return torch.relu(h + c) - h
+
+    c = torch.rand(16)
+    out = reduced(adj, x, c)
+    assert out.shape == (64,)
+    torch.testing.assert_close(out, (dense @ x + c).sum(dim=1) * 2.0)
+    torch.testing.assert_close(two_consumers(adj, x, c), torch.relu(dense @ x + c) - dense @ x)
 
 
 def test_runner_choice():

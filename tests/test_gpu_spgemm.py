@@ -336,3 +336,27 @@ def test_coordinate_stensors_multiply_on_the_device():
     assert torch.allclose(out.to_torch().cpu(), a_t @ b_t, atol=1e-5)
     dense = scorch.matmul(a, STensor.from_torch(b_t, "B").to("cuda"))
     assert isinstance(dense, torch.Tensor) and torch.allclose(dense.cpu(), a_t @ b_t, atol=1e-5)
+
+
+def test_result_beyond_the_int32_row_pointer_is_reported():
+    """32,769 rows that each select one dense row of 65,536 entries: 2^31 + 65,536 result entries.
+    The symbolic pass counts them in 64 bits and says so instead of wrapping the row pointer."""
+    from scorch_amd import native
+    M, N = (1 << 15) + 1, 1 << 16
+    a_pos = torch.arange(M + 1, dtype=torch.int32, device="cuda")
+    a_crd = torch.zeros(M, dtype=torch.int32, device="cuda")
+    b_pos = torch.tensor([0, N], dtype=torch.int32, device="cuda")
+    b_crd = torch.arange(N, dtype=torch.int32, device="cuda")
+    with pytest.raises(native.ScorchHipError, match="2\\^31") as err:
+        H.prebuilt_spmspm_csr_f32([M, N], [M, 1], [[], [a_pos, a_crd]], torch.ones(M, device="cuda"), [1, N],
+                                  [[], [b_pos, b_crd]], torch.ones(N, device="cuda"))
+    assert err.value.code == native.EUNSUPPORTED
+    # one row fewer fits: the symbolic pass alone (the result itself would take 17 GB)
+    M -= 2
+    L = native.lib()
+    c_pos = torch.empty(M + 1, dtype=torch.int32, device="cuda")
+    ws = torch.empty(L.scorch_hip_spgemm_csr_workspace_bytes(M, N, 1), dtype=torch.uint8, device="cuda")
+    native.check(L.scorch_hip_spgemm_csr_symbolic(M, 1, N, a_pos.data_ptr(), a_crd.data_ptr(), b_pos.data_ptr(),
+                                                  b_crd.data_ptr(), c_pos.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                  torch.cuda.current_stream().cuda_stream))
+    assert int(c_pos[-1]) == M * N and int(c_pos[1]) == N
