@@ -137,7 +137,7 @@ def cpu_baseline_sddmm(w, repeats=5):
                       "incl. wrapping the operands"}
 
 
-def cpu_baseline_attention(w, heads=2):
+def cpu_baseline_attention(w, heads=2, pattern=None):
     """The per-head composition of the reference's attention benchmark
     (bench/bench_sparse_transformer.py:354-372) on the host cores, fp32, for a
     sample of the heads: its SDDMM and SpMM kernels (oracle/_ref, or the C
@@ -147,7 +147,8 @@ def cpu_baseline_attention(w, heads=2):
     from oracle import oracle as O
     from scorch_amd import workloads
     S, D, H = w["S"], w["D"], w["H"]
-    pos, crd = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], w["block"])
+    pos, crd = pattern if pattern is not None else workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"],
+                                                                          w["block"])
     rows = np.repeat(np.arange(S, dtype=np.int32), np.diff(pos))
     ones = np.ones(crd.size, np.float32)
     kind = "reference" if O.have_ref() else "port"
@@ -444,6 +445,9 @@ def run_attention(args):
         qf, kf, vf = q.float(), k.float(), v.float()
 
         def unfused():
+            return H.sparse_attention_csr(pos, crd, qf, kf, vf, float(w["scale"]))
+
+        def unfused_per_head():
             outs = []
             for h in range(Hh):
                 sc = H.sddmm_csr_float([S, S], [S, S], [[], [pos, crd]], ones, [S, D], [[], []],
@@ -453,8 +457,11 @@ def run_attention(args):
                                                 vf[h].reshape(-1)).storage.value)
             return outs
 
-        rec["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM per head (this package, fp32)",
-                                                    unfused, max(args.steps // 4, 2), 1)
+        rec["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM, one launch each for all heads "
+                                                    "(this package, fp32)", unfused, max(args.steps // 4, 2), 1)
+        rec["unfused_fp32_pipeline_per_head"] = _vendor_time(
+            "SDDMM -> softmax -> SpMM per head from a Python loop, as the reference's benchmark runs it "
+            "(this package, fp32)", unfused_per_head, max(args.steps // 4, 2), 1)
         # (b) torch's dense attention with the same mask
         import torch.nn.functional as F
         blk = w["block"]
@@ -533,6 +540,37 @@ def run_extra(args):
         if args.vendor:
             out["vendor_library"] = _vendor_time("torch.sparse.mm in the same forward pass", vendor,
                                                  max(args.steps // 2, 2), 1)
+        return out
+    if args.workload == "attention_longformer":
+        # The reference's sparse-transformer benchmark shape (bench/bench_sparse_transformer.py:49-60,
+        # 194-209): embedding 256 in 8 heads (head dimension 32), Longformer mask with a window of 64 on
+        # either side and one global token, fp32; SDDMM -> row softmax -> SpMM, one launch each for all heads.
+        S, heads, D = (args.rows if args.rows != 1 << 20 else 4096), 8, 32
+        rp_np, ci_np = workloads.longformer_mask(S)
+        rp, ci = _t(rp_np), _t(ci_np)
+        gen = torch.Generator(device="cuda").manual_seed(7)
+        q, k, v = (torch.randn(heads, S, D, device="cuda", generator=gen) for _ in range(3))
+        scale = D ** -0.5
+        fn = lambda: H.sparse_attention_csr(rp, ci, q, k, v, scale)
+        ms = _time_steps(fn, args.steps, args.warmup)
+        nnz = int(ci_np.size)
+        out = {"metric": "sparse attention (SDDMM -> softmax -> SpMM) GFLOP/s", "unit": "GFLOP/s",
+               "value": round(heads * (4.0 * nnz * D + 5.0 * nnz) / ms / 1e6, 2), "ms_per_step": round(ms, 5), **base,
+               "config": {"workload": "attention_longformer_fp32", "S": S, "H": heads, "D": D, "window": 64,
+                          "global_tokens": 1, "nnz_per_head": nnz}}
+        if args.vendor:
+            import torch.nn.functional as F
+            rows = torch.repeat_interleave(torch.arange(S, device="cuda"), (rp[1:] - rp[:-1]).long())
+            live = torch.zeros(S, S, dtype=torch.bool, device="cuda")
+            live[rows, ci.long()] = True
+            out["vendor_library"] = _vendor_time(
+                "F.scaled_dot_product_attention(fp32, dense boolean mask)",
+                lambda: F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=live[None, None],
+                                                       scale=scale), max(args.steps // 4, 2), 1)
+        if not args.no_cpu:
+            w = {"S": S, "H": heads, "D": D, "q": q.cpu().numpy(), "k": k.cpu().numpy(), "v": v.cpu().numpy(),
+                 "scale": scale}
+            out["cpu_baseline"] = cpu_baseline_attention(w, heads=2, pattern=(rp_np, ci_np))
         return out
     if args.workload == "softmax_rows":
         # every row --row-length entries long, or a causal mask (row i has i + 1) with --row-length 0
@@ -620,7 +658,7 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true", help="skip the records of the other four configurations")
     ap.add_argument("--workload", default=None,
                     choices=[HEADLINE, *CONFIG_WORKLOADS, "spgemm_powerlaw", "spmv_powerlaw", "softmax_powerlaw",
-                             "softmax_rows", "gcn_forward"],
+                             "softmax_rows", "gcn_forward", "attention_longformer"],
                     help="print this workload's record alone (default: the headline line with all configurations)")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch's own sparse routine on the same operands")

@@ -398,6 +398,43 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_
                                      const void *Q, const void *K, const void *V, float scale,
                                      void *O, void *stream);
 
+/* ------------------------------------------------------------------------
+ * One sparsity pattern, `batch` value arrays: the three steps of the reference's
+ * sparse attention -- SDDMM, row softmax, SpMM, which its benchmark runs head by
+ * head from a Python loop (bench/bench_sparse_transformer.py:325,354-372) -- each
+ * as one launch over all heads (grid.y = head).  For any CSR mask and any head
+ * dimension; the fused kernel above covers block masks at D = 64 only.
+ * Problem h uses A + h M K, B + h n_cols K (resp. vals + h nnz, B + h K N) and
+ * writes out + h nnz (resp. C + h M N); the pattern and, for SDDMM, the mask's
+ * values are shared.  batch <= 65535.  Results are those of `batch` separate
+ * calls, bit for bit.
+ *   _sddmm_csr_batched: out_row_idx (may be NULL) is written once, nnz entries.
+ *   _softmax_csr_batched: workspace as for scorch_hip_softmax_csr_f32.
+ *   _spmm_csr_rows_batched: the row-split kernel (short rows), no workspace.
+ *   _spmm_csr_batched: the merge-path kernels; workspace of
+ *     scorch_hip_spmm_csr_batched_workspace_bytes(batch, M, nnz, N) bytes;
+ *     `bounds` as for scorch_hip_spmm_csr_planned_f32 (may be NULL).
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_sddmm_csr_batched_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                                     const int32_t *row_ptr, const int32_t *col_idx,
+                                     const float *mask_vals /* [nnz] */, const float *A /* [batch, M, K] */,
+                                     const float *B /* [batch, n_cols, K] */, float *out_vals /* [batch, nnz] */,
+                                     int32_t *out_row_idx /* [nnz] or NULL */, void *stream);
+SCORCH_HIP_API int scorch_hip_softmax_csr_batched_f32(int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
+                                       const float *vals /* [batch, nnz] */, float scale,
+                                       float *out /* [batch, nnz] */, void *workspace, size_t workspace_bytes,
+                                       void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_rows_batched_f32(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                         const int32_t *row_ptr, const int32_t *col_idx,
+                                         const float *vals /* [batch, nnz] */, const float *B /* [batch, K, N] */,
+                                         float *C /* [batch, M, N] */, void *stream);
+SCORCH_HIP_API size_t scorch_hip_spmm_csr_batched_workspace_bytes(int64_t batch, int64_t M, int64_t nnz, int64_t N);
+SCORCH_HIP_API int scorch_hip_spmm_csr_batched_f32(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx,
+                                    const float *vals /* [batch, nnz] */, const float *B /* [batch, K, N] */,
+                                    float *C /* [batch, M, N] */, const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
 /* Rows of a CSR matrix's entries: row_idx[p] = i for row_ptr[i] <= p < row_ptr[i+1].
  * The device-side counterpart of the "d,s" -> "o,o" index conversion the
  * reference performs on the host (STensor.from_coo / to_sparse,

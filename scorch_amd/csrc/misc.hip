@@ -165,7 +165,12 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
                                                                     const int *__restrict__ row_ptr,
                                                                     const float *vals, float scale,
                                                                     float *out, int *giant_count,
-                                                                    int *__restrict__ giant_rows) {
+                                                                    int *__restrict__ giant_rows, int64_t nnz) {
+  // grid.y > 1: several value arrays over one pattern; problem h reads and writes nnz entries
+  // further on, and only problem 0 lists the pattern's giant rows (they are the same for all)
+  vals += blockIdx.y * nnz;
+  out += blockIdx.y * nnz;
+  const bool list_giants = blockIdx.y == 0;
   // A lane group takes kTeamRows rows, one from each block of 256 / G consecutive rows
   // the workgroup owns, and requests the entries of all of them before it works on the
   // first: these rows are short, and with one row in flight per group the kernel waits on
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   const int w = threadIdx.x / kWaveSize;
   const int n_quarter = s_count[0], n_wave = s_count[1], n_long_wave = s_count[2], n_block = s_count[3],
             n_giant = s_count[4];
-  if (n_giant > 0) {  // uniform over the workgroup; rows are independent, so the list's order is free
+  if (n_giant > 0 && list_giants) {  // uniform over the workgroup; rows are independent, so the list's order is free
     if (threadIdx.x == 0) s_giant_base = atomicAdd(giant_count, n_giant);
     __syncthreads();
     for (int i = threadIdx.x; i < n_giant; i += kBlockThreads) giant_rows[s_giant_base + i] = s_list[4][i];
@@ -274,9 +279,11 @@ __global__ void softmax_reset_kernel(int *giant_count) {
 
 __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel(
     const int *__restrict__ row_ptr, const float *vals, float scale, float *out,
-    const int *__restrict__ giant_count, const int *__restrict__ giant_rows) {
+    const int *__restrict__ giant_count, const int *__restrict__ giant_rows, int64_t nnz) {
   constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
   __shared__ float s_red[kWaves];
+  vals += blockIdx.y * nnz;  // problem blockIdx.y of a batch over one pattern
+  out += blockIdx.y * nnz;
   const int n = *giant_count;
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
@@ -417,15 +424,16 @@ size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz) {
   return scorch::softmax_workspace_bytes(M, nnz);
 }
 
-int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, const float *vals,
-                               float scale, float *out, void *workspace, size_t workspace_bytes,
-                               void *stream) {
-  const char *fn = "scorch_hip_softmax_csr_f32";
+static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
+                             const float *vals, float scale, float *out, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  if (batch < 0 || batch > 65535)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
   if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
   if (M >= INT32_MAX || nnz > INT32_MAX)
     return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
   SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
-  if (M == 0 || nnz == 0) return SCORCH_HIP_OK;
+  if (batch == 0 || M == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
   const size_t need = scorch::softmax_workspace_bytes(M, nnz);
   if (need > 0 && (!workspace || workspace_bytes < need))
@@ -442,11 +450,11 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
   }
   const int g = scorch::softmax_group_width(M, nnz);
   const int64_t rows_per_block = scorch::kBlockThreads / g * scorch::softmax_team_rows(g);
-  const dim3 grid((unsigned)((M + rows_per_block - 1) / rows_per_block));
+  const dim3 grid((unsigned)((M + rows_per_block - 1) / rows_per_block), (unsigned)batch);
   const int m = (int)M;
 #define SCORCH_SOFTMAX(G)                                                                               \
   scorch::softmax_csr_kernel<G><<<grid, scorch::kBlockThreads, 0, s>>>(m, row_ptr, vals, scale, out, \
-                                                                       giant_count, giant_rows)
+                                                                       giant_count, giant_rows, nnz)
   switch (g) {
     case 2: SCORCH_SOFTMAX(2); break;
     case 4: SCORCH_SOFTMAX(4); break;
@@ -458,13 +466,29 @@ int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, c
 #undef SCORCH_SOFTMAX
   SCORCH_HIP_CHECK(hipGetLastError());
   if (need > 0) {  // else no row can be that long
-    const int64_t most = scorch::softmax_giant_capacity(M, nnz);
-    const dim3 giant_grid((unsigned)(most < scorch::kSoftmaxGiantBlocks ? most : scorch::kSoftmaxGiantBlocks));
+    int64_t most = scorch::softmax_giant_capacity(M, nnz);
+    if (most > scorch::kSoftmaxGiantBlocks) most = scorch::kSoftmaxGiantBlocks;
+    if (batch > 1 && most > 128) most = 128;  // every problem brings its own workgroups
+    const dim3 giant_grid((unsigned)most, (unsigned)batch);
     scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(
-        row_ptr, vals, scale, out, giant_count, giant_rows);
+        row_ptr, vals, scale, out, giant_count, giant_rows, nnz);
     SCORCH_HIP_CHECK(hipGetLastError());
   }
   return SCORCH_HIP_OK;
+}
+
+int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int32_t *row_ptr, const float *vals,
+                               float scale, float *out, void *workspace, size_t workspace_bytes,
+                               void *stream) {
+  return softmax_csr_entry("scorch_hip_softmax_csr_f32", 1, M, nnz, row_ptr, vals, scale, out, workspace,
+                           workspace_bytes, stream);
+}
+
+int scorch_hip_softmax_csr_batched_f32(int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
+                                       const float *vals, float scale, float *out, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
+  return softmax_csr_entry("scorch_hip_softmax_csr_batched_f32", batch, M, nnz, row_ptr, vals, scale, out,
+                           workspace, workspace_bytes, stream);
 }
 
 int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr, int32_t *row_idx,

@@ -29,9 +29,17 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
     int M, int K, int64_t nnz, const int *__restrict__ rows /* row_idx (COO) or row_ptr (CSR) */,
     const int *__restrict__ col_idx, const float *__restrict__ mask_vals,
     const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ out_vals,
-    int *__restrict__ out_row_idx) {
+    int *__restrict__ out_row_idx, int64_t batch_stride_a, int64_t batch_stride_b) {
   using VecT = Vec<float, VEC>;
   const int lane = wave_lane();
+  // grid.y > 1: several products over one mask (one per attention head); problem h has its own A,
+  // B and result values, the mask's values are shared and the row coordinates are written once
+  if (blockIdx.y > 0) {
+    A += blockIdx.y * batch_stride_a;
+    B += blockIdx.y * batch_stride_b;
+    out_vals += blockIdx.y * nnz;
+    out_row_idx = nullptr;
+  }
   // the grid is a multiple of 8 workgroups; every XCD takes a contiguous eighth of the entries
   const int64_t wave = xcd_contiguous(blockIdx.x, gridDim.x) * kWavesPerBlock + threadIdx.x / kWaveSize;
   const int64_t first = wave * kEntriesPerWave;
@@ -121,9 +129,10 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
 template <bool COO>
 int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
                  const float *mask_vals, const float *A, const float *B, float *out_vals,
-                 int *out_row_idx, hipStream_t stream) {
+                 int *out_row_idx, hipStream_t stream, int batch = 1, int64_t batch_stride_a = 0,
+                 int64_t batch_stride_b = 0) {
   const int64_t waves = (nnz + kEntriesPerWave - 1) / kEntriesPerWave;
-  const dim3 grid((unsigned)round_up_8((waves + kWavesPerBlock - 1) / kWavesPerBlock));
+  const dim3 grid((unsigned)round_up_8((waves + kWavesPerBlock - 1) / kWavesPerBlock), (unsigned)batch);
   const bool vec4 = K % 4 == 0 && aligned_to(A, 16) && aligned_to(B, 16);
   const int per_lane = vec4 ? 4 : 1;
   const int64_t lanes_needed = (K + per_lane - 1) / per_lane;
@@ -132,7 +141,8 @@ int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
 #define SCORCH_SDDMM_LAUNCH(GS, VEC, LONG)                                                         \
   sddmm_kernel<GS, VEC, COO, LONG><<<grid, kBlockThreads, 0, stream>>>(M, K, nnz, rows, col_idx,   \
                                                                       mask_vals, A, B, out_vals,  \
-                                                                      out_row_idx)
+                                                                      out_row_idx, batch_stride_a,  \
+                                                                      batch_stride_b)
 #define SCORCH_SDDMM_PICK(VEC)                                              \
   do {                                                                      \
     if (lanes_needed <= 4) SCORCH_SDDMM_LAUNCH(4, VEC, false);              \
@@ -155,7 +165,10 @@ template <bool COO>
 int sddmm_entry(const char *fn, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
                 const int32_t *rows, const int32_t *col_idx, const float *mask_vals,
                 const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
-                void *stream) {
+                void *stream, int64_t batch = 1) {
+  if (batch < 0 || batch > 65535)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
+  if (batch == 0) return SCORCH_HIP_OK;
   if (M < 0 || n_cols < 0 || K < 0 || nnz < 0)
     return fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld n_cols=%lld K=%lld nnz=%lld)", fn,
                 (long long)M, (long long)n_cols, (long long)K, (long long)nnz);
@@ -171,7 +184,7 @@ int sddmm_entry(const char *fn, int64_t M, int64_t n_cols, int64_t K, int64_t nn
                      aligned_to(out_row_idx, 4),
                  "%s: arrays must be 4-byte aligned", fn);
   return launch_sddmm<COO>((int)M, (int)K, nnz, rows, col_idx, mask_vals, A, B, out_vals,
-                           out_row_idx, static_cast<hipStream_t>(stream));
+                           out_row_idx, static_cast<hipStream_t>(stream), (int)batch, M * K, n_cols * K);
 }
 
 }  // namespace scorch
@@ -192,6 +205,14 @@ int scorch_hip_sddmm_csr_f32(int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
                              float *out_vals, int32_t *out_row_idx, void *stream) {
   return scorch::sddmm_entry<false>("scorch_hip_sddmm_csr_f32", M, n_cols, K, nnz, row_ptr,
                                     col_idx, mask_vals, A, B, out_vals, out_row_idx, stream);
+}
+
+int scorch_hip_sddmm_csr_batched_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                                     const int32_t *row_ptr, const int32_t *col_idx, const float *mask_vals,
+                                     const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
+                                     void *stream) {
+  return scorch::sddmm_entry<false>("scorch_hip_sddmm_csr_batched_f32", M, n_cols, K, nnz, row_ptr, col_idx,
+                                    mask_vals, A, B, out_vals, out_row_idx, stream, batch);
 }
 
 }  // extern "C"

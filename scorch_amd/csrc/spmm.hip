@@ -39,10 +39,14 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
     int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val,
-    const Boundary *__restrict__ bounds) {
+    const Boundary *__restrict__ bounds, SpmmBatch batch) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int kSlots = kItemsPerWave + kSnapItems;
+  vals += blockIdx.y * batch.vals;  // problem blockIdx.y of a batch over one pattern
+  B += blockIdx.y * batch.b;
+  C += blockIdx.y * batch.c;
+  carry_val += blockIdx.y * batch.carry;
 
   __shared__ int s_col[kWavesPerBlock][kSlots];
   __shared__ T s_val[kWavesPerBlock][kSlots];
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
   // Whatever is left belongs to row x1, whose marker lies in a later chunk.
   const int row_start = uniform(s_rp[w][n_rows]);  // row_ptr[x1]
   const int tail = y1 - (row_start > y0 ? row_start : y0);
-  if (where.tile == 0 && lane == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
+  if (where.tile == 0 && lane == 0 && blockIdx.y == 0) carry_row[chunk] = tail > 0 ? x1 : -1;
   if (tail > 0 && active) {
     VecT o;
 #pragma unroll
@@ -167,11 +171,15 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
     int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val,
-    const Boundary *__restrict__ bounds) {
+    const Boundary *__restrict__ bounds, SpmmBatch batch) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int G = kWaveSize / LPR;
   constexpr int kSlots = kItemsPerWave + kSnapItems;
+  vals += blockIdx.y * batch.vals;  // problem blockIdx.y of a batch over one pattern
+  B += blockIdx.y * batch.b;
+  C += blockIdx.y * batch.c;
+  carry_val += blockIdx.y * batch.carry;
 
   __shared__ int s_col[kWavesPerBlock][kSlots];
   __shared__ T s_val[kWavesPerBlock][kSlots];
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
         *reinterpret_cast<VecT *>(carry_val + (size_t)span * (size_t)N + col0) = o;
       }
     }
-    if (live && slot == n_rows && where.tile == 0 && t == 0) carry_row[span] = len > 0 ? x1 : -1;
+    if (live && slot == n_rows && where.tile == 0 && t == 0 && blockIdx.y == 0) carry_row[span] = len > 0 ? x1 : -1;
   }
 }
 
@@ -353,9 +361,10 @@ struct KernelTimer {
 template <typename T, int VEC, int EPI>
 int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
                 const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
-                KernelTimer *timer, const Boundary *bounds) {
+                KernelTimer *timer, const Boundary *bounds, int batch, int64_t K) {
   const SpmmSplit split = spmm_split(M, nnz, N, sizeof(T));
   const int64_t chunks = split.spans;
+  const SpmmBatch strides = {nnz, K * N, (int64_t)M * N, chunks * N};
   int *carry_row = static_cast<int *>(workspace);
   T *carry_val = reinterpret_cast<T *>(
       static_cast<char *>(workspace) +
@@ -367,18 +376,18 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
   if (blocks_per_tile * n_tiles > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
-  const dim3 grid((unsigned)(blocks_per_tile * n_tiles));
+  const dim3 grid((unsigned)(blocks_per_tile * n_tiles), (unsigned)batch);
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   mark_launch(stream);
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
-      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val, bounds);
+      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val, bounds, strides);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
   mark_launch(stream);
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
-  spmm_fixup_kernel<T, VEC, EPI><<<dim3((unsigned)((chunks + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
-                                   stream>>>(N, chunks, carry_row, carry_val, C, bias);
+  spmm_fixup_kernel<T, VEC, EPI><<<dim3((unsigned)((chunks + fix_per_block - 1) / fix_per_block), (unsigned)batch),
+                                   kBlockThreads, 0, stream>>>(N, chunks, carry_row, carry_val, C, bias, strides);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[2], stream));
   mark_launch(stream);
@@ -391,7 +400,7 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
 template <typename T, int VEC, int LPR, int EPI>
 int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx,
                         const T *vals, const T *B, const T *bias, T *C, void *workspace,
-                        hipStream_t stream, const Boundary *bounds) {
+                        hipStream_t stream, const Boundary *bounds, int batch, int64_t K) {
   const int64_t total = (int64_t)M + nnz;
   const int tile = LPR * VEC;
   const int n_tiles = (N + tile - 1) / tile;
@@ -417,14 +426,16 @@ int launch_spmm_grouped(int M, int N, int64_t nnz, const int *row_ptr, const int
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM: %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
   mark_launch(stream);
-  spmm_grouped_kernel<T, VEC, LPR, EPI><<<dim3((unsigned)(blocks_per_tile * n_tiles)), kBlockThreads, 0, stream>>>(
+  const SpmmBatch strides = {nnz, K * N, (int64_t)M * N, spans * N};
+  spmm_grouped_kernel<T, VEC, LPR, EPI><<<dim3((unsigned)(blocks_per_tile * n_tiles), (unsigned)batch), kBlockThreads,
+                                          0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, total, ipc, ipc < kSnapItems ? ipc : kSnapItems, n_tiles,
-      blocks_per_tile, carry_row, carry_val, bounds);
+      blocks_per_tile, carry_row, carry_val, bounds, strides);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(stream);
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
-  spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((spans + fix_per_block - 1) / fix_per_block)), kBlockThreads, 0,
-                                 stream>>>(N, spans, carry_row, carry_val, C, bias);
+  spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((spans + fix_per_block - 1) / fix_per_block), (unsigned)batch),
+                                 kBlockThreads, 0, stream>>>(N, spans, carry_row, carry_val, C, bias, strides);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(stream);
   return SCORCH_HIP_OK;
@@ -445,7 +456,11 @@ template <typename T, int EPI>
 int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
                const int32_t *col_idx, const T *vals, const T *B, const T *bias, T *C,
                void *workspace, size_t workspace_bytes, void *stream,
-               KernelTimer *timer = nullptr, const void *bounds_buffer = nullptr, size_t bounds_bytes = 0) {
+               KernelTimer *timer = nullptr, const void *bounds_buffer = nullptr, size_t bounds_bytes = 0,
+               int64_t batch = 1) {
+  if (batch < 0 || batch > 65535)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
+  if (batch == 0) return SCORCH_HIP_OK;
   if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
   SCORCH_REQUIRE(N >= 0, "%s: negative N=%lld", fn, (long long)N);
   if (N > INT32_MAX - kWaveSize * 4)
@@ -482,7 +497,8 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
     const int64_t tile_elems = tile_bytes / (int)sizeof(T) < N ? tile_bytes / (int)sizeof(T) : N;
     const int64_t lanes = (tile_elems + vec - 1) / vec;
 #define SCORCH_GROUPED(VEC, LPR) \
-  return launch_spmm_grouped<T, VEC, LPR, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, bounds)
+  return launch_spmm_grouped<T, VEC, LPR, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, bounds, \
+                                               (int)batch, K)
 #define SCORCH_GROUPED_LANES(VEC)                      \
   do {                                                 \
     if (lanes <= 8) SCORCH_GROUPED(VEC, 8);            \
@@ -501,11 +517,14 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
   const int vec = pick_vec<T>(N, B, C, workspace);
   if constexpr (sizeof(T) == 4) {
     if (vec == 4)
-      return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
+      return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
+                                  (int)batch, K);
   }
   if (vec == 2)
-    return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
-  return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds);
+    return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
+                                  (int)batch, K);
+  return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
+                                  (int)batch, K);
 }
 
 
@@ -888,6 +907,20 @@ SCORCH_DEFINE_SPMM_PLANNED(f32, float)
 SCORCH_DEFINE_SPMM_PLANNED(f64, double)
 SCORCH_DEFINE_SPMM_PLANNED(i32, int32_t)
 SCORCH_DEFINE_SPMM_PLANNED(i64, int64_t)
+
+size_t scorch_hip_spmm_csr_batched_workspace_bytes(int64_t batch, int64_t M, int64_t nnz, int64_t N) {
+  if (batch <= 0 || M < 0 || nnz < 0 || N < 0) return 0;
+  return scorch::spmm_batched_workspace_bytes(batch, M, nnz, N, sizeof(float));
+}
+
+int scorch_hip_spmm_csr_batched_f32(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                    const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                    const float *B, float *C, const void *bounds, size_t bounds_bytes,
+                                    void *workspace, size_t workspace_bytes, void *stream) {
+  return scorch::spmm_entry<float, scorch::kEpiNone>("scorch_hip_spmm_csr_batched_f32", M, K, N, nnz, row_ptr,
+                                                     col_idx, vals, B, nullptr, C, workspace, workspace_bytes,
+                                                     stream, nullptr, bounds, bounds_bytes, batch);
+}
 
 int scorch_hip_spmm_csr_f32_static(int64_t M, int64_t K, int64_t N, int64_t nnz,
                                    const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

@@ -95,6 +95,13 @@ __device__ __forceinline__ Boundary load_boundary(const Boundary *__restrict__ b
   return b;
 }
 
+// Several products over one sparsity pattern in one launch (grid.y = problem; one per
+// attention head): how far apart, in elements, the problems' value arrays, dense operands,
+// results and carry rows lie.  All zero for a single product.
+struct SpmmBatch {
+  int64_t vals, b, c, carry;
+};
+
 // Shape of the work split.  A chunk holds nominally up to 256 merge items, one
 // chunk per wavefront; small problems use smaller chunks, so that they are
 // spread over more, shorter wavefronts.  (A wavefront that walked two or more
@@ -139,6 +146,12 @@ constexpr size_t kPaceBytes = 8 * kPaceStride * sizeof(int);
 inline size_t spmm_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
   return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256) + kPaceBytes;
+}
+
+// A batch of products over one pattern: one carry_row array, then carry_val for every problem.
+inline size_t spmm_batched_workspace_bytes(int64_t batch, int64_t M, int64_t nnz, int64_t N, size_t elem) {
+  const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
+  return align_up(chunks * sizeof(int), 256) + align_up((size_t)batch * chunks * (size_t)N * elem, 256) + kPaceBytes;
 }
 
 // Elements per lane.  Preferred: the widest vector (at most 16 bytes) that
@@ -189,9 +202,11 @@ constexpr int kFixupChunks = 8;
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_fixup_kernel(
     int N, int64_t num_chunks, const int *__restrict__ carry_row, const T *__restrict__ carry_val,
-    T *__restrict__ C, const T *__restrict__ bias) {
+    T *__restrict__ C, const T *__restrict__ bias, SpmmBatch batch) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
+  carry_val += blockIdx.y * batch.carry;
+  C += blockIdx.y * batch.c;
   const int lane = wave_lane();
   const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
   const int64_t c = wave * kFixupChunks + lane;

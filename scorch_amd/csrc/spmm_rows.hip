@@ -34,8 +34,13 @@ template <typename T, int VEC, int LPR>
 __global__ __launch_bounds__(kBlockThreads) void spmm_rows_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
-    const T *__restrict__ bias, int relu, int team_shift, int n_tiles, int64_t blocks_per_tile) {
+    const T *__restrict__ bias, int relu, int team_shift, int n_tiles, int64_t blocks_per_tile,
+    int64_t batch_nnz, int64_t batch_b, int64_t batch_c) {
   using A = typename Acc<T>::type;
+  // grid.y > 1: several products over one pattern, each with its own values, B and C
+  vals += blockIdx.y * batch_nnz;
+  B += blockIdx.y * batch_b;
+  C += blockIdx.y * batch_c;
   using VecT = Vec<T, VEC>;
   constexpr int G = kWaveSize / LPR;
 
@@ -120,7 +125,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_rows_kernel(
 
 template <typename T, int VEC, int LPR>
 int launch_spmm_rows(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
-                     const T *B, const T *bias, int relu, T *C, hipStream_t stream) {
+                     const T *B, const T *bias, int relu, T *C, hipStream_t stream, int batch, int64_t K) {
   constexpr int G = kWaveSize / LPR;
   const int tile = LPR * VEC;
   const int n_tiles = (N + tile - 1) / tile;
@@ -139,8 +144,9 @@ int launch_spmm_rows(int M, int N, int64_t nnz, const int *row_ptr, const int *c
     return fail(SCORCH_HIP_EUNSUPPORTED, "SpMM (row split): %lld workgroups exceed the launch limit",
                 (long long)(blocks_per_tile * n_tiles));
   mark_launch(stream);
-  spmm_rows_kernel<T, VEC, LPR><<<dim3((unsigned)(blocks_per_tile * n_tiles)), kBlockThreads, 0, stream>>>(
-      M, N, row_ptr, col_idx, vals, B, C, bias, relu, team_shift, n_tiles, blocks_per_tile);
+  spmm_rows_kernel<T, VEC, LPR><<<dim3((unsigned)(blocks_per_tile * n_tiles), (unsigned)batch), kBlockThreads, 0,
+                                 stream>>>(M, N, row_ptr, col_idx, vals, B, C, bias, relu, team_shift, n_tiles,
+                                           blocks_per_tile, nnz, K * N, (int64_t)M * N);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(stream);
   return SCORCH_HIP_OK;
@@ -149,7 +155,10 @@ int launch_spmm_rows(int M, int N, int64_t nnz, const int *row_ptr, const int *c
 template <typename T>
 int spmm_rows_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
                     const int32_t *col_idx, const T *vals, const T *B, const T *bias, int act, T *C,
-                    void *stream) {
+                    void *stream, int64_t batch = 1) {
+  if (batch < 0 || batch > 65535)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
+  if (batch == 0) return SCORCH_HIP_OK;
   if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
   SCORCH_REQUIRE(N >= 0, "%s: negative N=%lld", fn, (long long)N);
   if (N > INT32_MAX - kWaveSize * 4)
@@ -174,7 +183,7 @@ int spmm_rows_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz
   // lanes that cover a row of B (at most a wavefront: wider rows take several column tiles)
   const int64_t lanes = (N + vec - 1) / vec;
 #define SCORCH_ROWS(VEC, LPR) \
-  return launch_spmm_rows<T, VEC, LPR>(m, n, nnz, row_ptr, col_idx, vals, B, bias, relu, C, s)
+  return launch_spmm_rows<T, VEC, LPR>(m, n, nnz, row_ptr, col_idx, vals, B, bias, relu, C, s, (int)batch, K)
 #define SCORCH_ROWS_LANES(VEC)              \
   do {                                      \
     if (lanes <= 8) SCORCH_ROWS(VEC, 8);    \
@@ -244,6 +253,13 @@ extern "C" {
     return scorch::spmm_rows_entry<T>("scorch_hip_spmm_csr_rows_" #SUFFIX, M, K, N, nnz, row_ptr,        \
                                       col_idx, vals, B, bias, act, C, stream);                           \
   }
+
+int scorch_hip_spmm_csr_rows_batched_f32(int64_t batch, int64_t M, int64_t K, int64_t N, int64_t nnz,
+                                         const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                                         const float *B, float *C, void *stream) {
+  return scorch::spmm_rows_entry<float>("scorch_hip_spmm_csr_rows_batched_f32", M, K, N, nnz, row_ptr, col_idx,
+                                        vals, B, nullptr, SCORCH_HIP_ACT_NONE, C, stream, batch);
+}
 
 SCORCH_DEFINE_SPMM_ROWS(f32, float)
 SCORCH_DEFINE_SPMM_ROWS(f64, double)

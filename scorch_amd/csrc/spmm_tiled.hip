@@ -337,7 +337,8 @@ int spmm_tiled_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nn
   mark_launch(s);
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
   spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((split.spans + fix_per_block - 1) / fix_per_block)),
-                                 kBlockThreads, 0, s>>>((int)N, split.spans, carry_row, carry_val, C, bias);
+                                 kBlockThreads, 0, s>>>((int)N, split.spans, carry_row, carry_val, C, bias,
+                                                        SpmmBatch{0, 0, 0, 0});
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
   return SCORCH_HIP_OK;

@@ -626,6 +626,113 @@ def spmspm_coo_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B
     return Tensor(out.storage.value, [[rows], [c_crd]])
 
 
+# ---- one pattern, several value arrays (one per attention head) ------------------------
+def _batched_dense(t: torch.Tensor, batch: int, rows: int, cols: int, what: str) -> torch.Tensor:
+    if t.dtype != torch.float32 or t.dim() != 3 or tuple(t.shape) != (batch, rows, cols):
+        raise ValueError(f"scorch_ops_hip: {what} must be a float32 tensor of shape ({batch}, {rows}, {cols}), "
+                         f"got {t.dtype} {tuple(t.shape)}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, B: torch.Tensor):
+    """out[h, p] = S.val[p] * <A[h, i_p, :], B[h, j_p, :]> for every head h and stored entry p of
+    the CSR mask S: the SDDMM step of the reference's sparse attention for all heads in one launch
+    (bench/bench_sparse_transformer.py:354-361 runs it per head).  A is (H, M, K), B is (H, n_cols, K).
+    Returns (values of shape (H, nnz), row coordinates int32[nnz])."""
+    M, n_cols = int(S_shape[0]), int(S_shape[1])
+    pos, crd = _csr_parts(S_mode_indices, "S")
+    s_val = _flat(S_values, torch.float32, "S values")
+    H, K = int(A.shape[0]), int(A.shape[2])
+    a, b = _batched_dense(A, H, M, K, "A"), _batched_dense(B, H, n_cols, K, "B")
+    if pos.numel() != M + 1 or crd.numel() != s_val.numel():
+        raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
+    dev = _device_of(pos, crd, s_val, a, b)
+    csr_plan(pos, crd, M, n_cols, "S")
+    nnz = s_val.numel()
+    out = torch.empty((H, nnz), dtype=torch.float32, device=dev)
+    rows = torch.empty_like(crd)
+    with _on_device(dev):
+        rc = native.lib().scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                           s_val.data_ptr(), a.data_ptr(), b.data_ptr(),
+                                                           out.data_ptr(), rows.data_ptr(), _stream(dev))
+    native.check(rc)
+    return out, rows
+
+
+def softmax_csr_float_batched(row_ptr: torch.Tensor, values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Row softmax of ``scale * values[h]`` over one CSR pattern for every head h;
+    values is (H, nnz)."""
+    pos = _index(row_ptr, "row_ptr")
+    if values.dtype != torch.float32 or values.dim() != 2:
+        raise ValueError("scorch_ops_hip: values must be a float32 tensor of shape (H, nnz)")
+    v = values if values.is_contiguous() else values.contiguous()
+    dev = _device_of(pos, v)
+    H, nnz = int(v.shape[0]), int(v.shape[1])
+    out = torch.empty_like(v)
+    L = native.lib()
+    with _on_device(dev):
+        stream = _stream(dev)
+        need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, nnz)
+        ws = _workspace(dev, stream, need) if need else None
+        rc = L.scorch_hip_softmax_csr_batched_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(), float(scale),
+                                                  out.data_ptr(), ws.data_ptr() if need else None,
+                                                  ws.numel() if need else 0, stream)
+    native.check(rc)
+    return out
+
+
+def spmm_csr_float_batched(A_shape, A_mode_indices, A_values: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """C[h] = A_h @ B[h] where every A_h has the CSR pattern given and the values A_values[h]:
+    the last step of the reference's sparse attention (bench/bench_sparse_transformer.py:370-372) for
+    all heads in one launch.  A_values is (H, nnz), B is (H, K, N); returns (H, M, N)."""
+    M, K = int(A_shape[0]), int(A_shape[1])
+    pos, crd = _csr_parts(A_mode_indices, "A")
+    if A_values.dtype != torch.float32 or A_values.dim() != 2:
+        raise ValueError("scorch_ops_hip: A values must be a float32 tensor of shape (H, nnz)")
+    a_val = A_values if A_values.is_contiguous() else A_values.contiguous()
+    H, nnz = int(a_val.shape[0]), int(a_val.shape[1])
+    N = int(B.shape[2])
+    b = _batched_dense(B, H, K, N, "B")
+    if pos.numel() != M + 1 or crd.numel() != nnz:
+        raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
+    dev = _device_of(pos, crd, a_val, b)
+    plan = csr_plan(pos, crd, M, K, "A")
+    out = torch.empty((H, M, N), dtype=torch.float32, device=dev)
+    if H == 0 or M == 0 or N == 0:
+        return out
+    L = native.lib()
+    with _on_device(dev):
+        stream = _stream(dev)
+        if SPMM_PATH == "rows" or (SPMM_PATH == "auto" and plan is not None and plan.max_row <= ROWS_KERNEL_MAX_ROW):
+            rc = L.scorch_hip_spmm_csr_rows_batched_f32(H, M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                        a_val.data_ptr(), b.data_ptr(), out.data_ptr(), stream)
+        else:
+            ws = _workspace(dev, stream, L.scorch_hip_spmm_csr_batched_workspace_bytes(H, M, nnz, N))
+            bounds = _chunk_bounds(plan, pos, M, nnz, N, 4, L, stream) \
+                if plan is not None and SPMM_PATH != "merge_unplanned" else None
+            rc = L.scorch_hip_spmm_csr_batched_f32(H, M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(),
+                                                   b.data_ptr(), out.data_ptr(),
+                                                   bounds.data_ptr() if bounds is not None else None,
+                                                   bounds.numel() if bounds is not None else 0, ws.data_ptr(),
+                                                   ws.numel(), stream)
+    native.check(rc)
+    return out
+
+
+def sparse_attention_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
+                         v: torch.Tensor, scale: float) -> torch.Tensor:
+    """softmax(scale * q k^T restricted to a CSR mask) v for q, k, v of shape (H, S, D), fp32: the
+    reference's sparse attention (bench/bench_sparse_transformer.py:354-372: SDDMM, row softmax and
+    SpMM per head) as three launches for all heads.  Any mask, any head dimension; rows of the mask
+    without entries give zero rows."""
+    H, S, D = (int(x) for x in q.shape)
+    ones = torch.ones(col_idx.numel(), dtype=torch.float32, device=q.device)
+    mask = [[], [row_ptr, col_idx]]
+    scores, _ = sddmm_csr_float_batched([S, S], mask, ones, q, k)
+    probs = softmax_csr_float_batched(row_ptr, scores, scale)
+    return spmm_csr_float_batched([S, S], mask, probs, v)
+
+
 def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,
                           block_col_idx: torch.Tensor, scale: float, block: int = 64) -> torch.Tensor:
     """softmax(scale * q k^T over a block mask) v for q, k, v of shape (H, S, D),

@@ -212,6 +212,33 @@ def blocks_to_csr(block_row_ptr: np.ndarray, block_col_idx: np.ndarray, block: i
     return row_ptr.astype(np.int32), col_idx.astype(np.int32)
 
 
+def longformer_mask(S: int, window: int = 64, n_global: int = 1):
+    """CSR pattern (row_ptr, col_idx; int32) of the Longformer-style attention mask of the
+    reference's sparse-transformer benchmark (bench/bench_sparse_transformer.py:194-209): token
+    i attends to the tokens within ``window`` positions on either side, and the first
+    ``n_global`` tokens attend to and are attended by every token.  With the benchmark's
+    settings (window 64, one global token) the mask has 62,782 entries at S = 512 and 532,286
+    at S = 4096 (bench/README_sparse_transformer.md:78-81)."""
+    i = np.arange(S, dtype=np.int64)
+    lo = np.maximum(i - window, 0)
+    hi = np.minimum(i + window, S - 1) + 1                  # the window, [lo, hi)
+    n_global = min(n_global, S)
+    extra = np.minimum(lo, n_global)                         # global columns left of the window
+    lens = (hi - lo) + extra
+    lens[:n_global] = S
+    row_ptr = np.zeros(S + 1, dtype=np.int64)
+    np.cumsum(lens, out=row_ptr[1:])
+    cols = np.empty(int(row_ptr[-1]), dtype=np.int32)
+    for r in range(S):
+        seg = cols[row_ptr[r]:row_ptr[r + 1]]
+        if r < n_global:
+            seg[:] = np.arange(S, dtype=np.int32)
+        else:
+            seg[:extra[r]] = np.arange(extra[r], dtype=np.int32)
+            seg[extra[r]:] = np.arange(lo[r], hi[r], dtype=np.int32)
+    return row_ptr.astype(np.int32), cols
+
+
 def sae_decoder(M: int = 4096, K: int = 16_384, N: int = 4096, k: int = 32,
                 seed: int = SEEDS["sae_decoder"]) -> Dict[str, np.ndarray]:
     """Sparse-autoencoder decoder input: per row the top ``k`` of ReLU(N(0, 1))

@@ -257,7 +257,7 @@ def test_compile_spmm_bias_relu_csr():
     result = fused(adj, x.cuda(), bias.cuda())
     assert isinstance(result, torch.Tensor) and result.is_cuda
     assert torch.allclose(result.cpu(), torch.relu(dense_a @ x + bias), atol=1e-4)
-    assert list(fused._cache.values())[0].fused_symbol == "spmm_csr_bias_relu_float"
+    assert list(fused._cache.values())[0][0].fused_symbol == "spmm_csr_bias_relu_float"
     # second call reuses the trace and the runner
     again = fused(adj, x.cuda(), bias.cuda())
     assert torch.equal(result, again) and len(fused._cache) == 1
@@ -278,7 +278,7 @@ def test_compile_spmm_bias_csr_and_unfused_chain():
     out = bias_only(adj, x.cuda(), bias.cuda())
     assert torch.allclose(out.cpu(), dense_a @ x + bias, atol=1e-4)
     chained = tanh_chain(adj, x.cuda(), bias.cuda())
-    assert list(tanh_chain._cache.values())[0].fused_symbol is None      # runs matmul + torch ops
+    assert list(tanh_chain._cache.values())[0][0].fused_symbol is None      # runs matmul + torch ops
     assert torch.allclose(chained.cpu(), torch.tanh((dense_a @ x) * bias), atol=1e-4)
 
 

@@ -85,3 +85,18 @@ def test_gcn_powerlaw_neighbour_window():
     np.testing.assert_allclose(w["vals"], 1 / np.sqrt(d[rows] * d[w["col_idx"]]), rtol=1e-6)
     plain = workloads.gcn_powerlaw(M=M, N=4, seed=3, max_degree=400)
     assert np.abs(plain["col_idx"].astype(np.int64) - np.repeat(np.arange(M), np.diff(plain["row_ptr"]))).max() > M // 4
+
+
+def test_longformer_mask_matches_the_reference_benchmarks_counts():
+    """reference: bench/README_sparse_transformer.md:78-81 (window 64 on either side, one global
+    token): 62,782 entries at S = 512, 532,286 at S = 4096; and the definition itself
+    (bench/bench_sparse_transformer.py:194-209) on a small dense mask."""
+    for S, nnz in ((512, 62_782), (4096, 532_286)):
+        rp, ci = workloads.longformer_mask(S)
+        assert rp[-1] == ci.size == nnz and rows_sorted_unique(rp, ci)
+    S, w, g = 40, 3, 2
+    rp, ci = workloads.longformer_mask(S, window=w, n_global=g)
+    dense = np.zeros((S, S), bool)
+    dense[np.repeat(np.arange(S), np.diff(rp)), ci] = True
+    i, j = np.indices((S, S))
+    assert np.array_equal(dense, (np.abs(i - j) <= w) | (i < g) | (j < g))
