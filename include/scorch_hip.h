@@ -290,6 +290,23 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_f32(int64_t M, int64_t n_cols, int64_t K
                              const float *mask_vals, const float *A, const float *B,
                              float *out_vals, int32_t *out_row_idx, void *stream);
 
+/* SDDMM for a CSR mask whose pattern is used again and again (an attention mask
+ * serves every head, layer and step), with B larger than one of the GPU's eight
+ * L2 caches but not than all of them together.  The reference has no such step.
+ * scorch_hip_sddmm_csr_lists sorts the mask's entries once into eight lists by
+ * the eighth of the column range they fall in (`lists`: device, 256-byte aligned,
+ * scorch_hip_sddmm_csr_lists_bytes(nnz) bytes; it depends on row_ptr, col_idx and
+ * n_cols only).  scorch_hip_sddmm_csr_listed_f32 is scorch_hip_sddmm_csr_batched_f32
+ * computed list by list, each list on one XCD, whose L2 then keeps that eighth of
+ * B: the same products, the same results bit for bit.  K <= 256. */
+SCORCH_HIP_API size_t scorch_hip_sddmm_csr_lists_bytes(int64_t nnz);
+SCORCH_HIP_API int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
+                               const int32_t *col_idx, void *lists, size_t lists_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                                    const void *lists, size_t lists_bytes, const float *mask_vals,
+                                    const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
+                                    void *stream);
+
 /* ------------------------------------------------------------------------
  * SpMV: y[M] = A_csr[M,K] * x[K].
  * Replaces spmv_csr<T> (csrc/kernels.h:13-49), bound as

@@ -126,6 +126,232 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
   }
 }
 
+// ---- a mask that is used again and again: its entries listed per XCD ------------------------
+// With B larger than one L2 (4 MB per XCD) most of the gathered B rows come over
+// the fabric, although all of B would fit the eight L2s together.  For a mask
+// whose pattern stays (an attention mask serves every head, layer and step) the
+// entries are therefore listed once by the column range they fall in, one range
+// per XCD: XCD x then only ever gathers rows of B from its eighth of B, which
+// stays in its L2, at the price of every XCD streaming all of A once.
+//
+// sddmm_bucket_count_kernel / sddmm_bucket_fill_kernel build the lists: each
+// wavefront takes kEntriesPerWave consecutive entries (so that a row's entries
+// stay together in the lists and its row of A is reused from the vector cache),
+// counts them per range, reserves that many slots in every range's list with one
+// atomic each, and writes (entry number, row, column) there.  The order of the
+// wavefronts' pieces inside a list varies from build to build; the products do
+// not depend on it.
+constexpr int kBuckets = 8;  // one per XCD
+// Workgroups per XCD of the kernel that walks the lists.  All of them must be resident at once:
+// the id & 7 = XCD rule holds for workgroups dispatched in order, and once the chip is full later
+// ones go wherever a slot frees up (65,536^2 mask, 64 per row, K = 64: with 256 per XCD the fetch
+// traffic was the plain kernel's 0.86 GB; with 192, 0.44 GB and 0.124 ms against the plain
+// kernel's 0.130; with 128, 0.43 GB and 0.165 ms: fewer wavefronts hide less latency).
+constexpr int kListedWorkgroupsPerXcd = 192;
+
+__device__ __forceinline__ int sddmm_entry_row(const int *__restrict__ row_ptr, int row_lo, int row_hi, int64_t p) {
+  int lo = row_lo, hi = row_hi;  // answer in [lo, hi]
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)row_ptr[mid + 1] <= p) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+// counts[b] += entries whose column lies in range b; columns outside [0, n_cols) count for no range
+__global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_count_kernel(int64_t nnz, int cols_per_bucket,
+                                                                           const int *__restrict__ col_idx,
+                                                                           int *__restrict__ counts) {
+  const int lane = wave_lane();
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  const int64_t first = wave * kEntriesPerWave;
+  if (first >= nnz) return;
+  const int64_t last = first + kEntriesPerWave < nnz ? first + kEntriesPerWave : nnz;
+  int mine[kBuckets] = {0};
+  for (int64_t p = first + lane; p < last; p += kWaveSize) {
+    const unsigned b = (unsigned)col_idx[p] / (unsigned)cols_per_bucket;
+#pragma unroll
+    for (int k = 0; k < kBuckets; ++k) mine[k] += b == (unsigned)k;
+  }
+#pragma unroll
+  for (int k = 0; k < kBuckets; ++k) {
+    int total = mine[k];
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    if (lane == 0 && total > 0) atomicAdd(&counts[k], total);
+  }
+}
+
+// counts[0 .. 7]: entries per range (from the kernel above); counts[8 .. 15]: slots handed out so far.
+// list_ptr[b] = start of range b's list; entries go to entry_pos / entry_row / entry_col.
+__global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_fill_kernel(
+    int M, int64_t nnz, int cols_per_bucket, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
+    int *__restrict__ counts, int *__restrict__ list_ptr, int *__restrict__ entry_pos,
+    int *__restrict__ entry_row, int *__restrict__ entry_col) {
+  const int lane = wave_lane();
+  int start[kBuckets];
+  {
+    int run = 0;
+#pragma unroll
+    for (int k = 0; k < kBuckets; ++k) {
+      start[k] = run;
+      run += counts[k];
+    }
+    if (blockIdx.x == 0 && threadIdx.x <= kBuckets) {
+      int at = 0;
+      for (int k = 0; k < (int)threadIdx.x; ++k) at += counts[k];
+      list_ptr[threadIdx.x] = at;
+    }
+  }
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
+  const int64_t first = wave * kEntriesPerWave;
+  if (first >= nnz) return;
+  const int64_t last = first + kEntriesPerWave < nnz ? first + kEntriesPerWave : nnz;
+  auto end_key = [&](int i) { return (int64_t)row_ptr[i + 1]; };
+  const int row_lo = wave_count_below(M, first + 1, end_key);
+  const int row_hi = wave_count_below(M, last, end_key);
+
+  constexpr int kRounds = kEntriesPerWave / kWaveSize;
+  int col[kRounds], row[kRounds];
+  unsigned bucket[kRounds];
+  int mine[kBuckets] = {0};
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int64_t p = first + r * kWaveSize + lane;
+    bucket[r] = ~0u;
+    col[r] = row[r] = 0;
+    if (p < last) {
+      col[r] = col_idx[p];
+      row[r] = sddmm_entry_row(row_ptr, row_lo, row_hi, p);
+      bucket[r] = (unsigned)col[r] / (unsigned)cols_per_bucket;
+    }
+#pragma unroll
+    for (int k = 0; k < kBuckets; ++k) mine[k] += bucket[r] == (unsigned)k;
+  }
+  // slots of this wavefront in every list (one atomic per list), then every entry's slot: the
+  // wavefront's entries keep their order inside a list, so that a row's entries stay next to each
+  // other there (its row of A is then reused from the vector cache, and the entry's mask value
+  // and result lie next to its neighbours')
+  int base[kBuckets];
+#pragma unroll
+  for (int k = 0; k < kBuckets; ++k) {
+    int total = mine[k];
+#pragma unroll
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    int reserved = 0;
+    if (lane == 0 && total > 0) reserved = atomicAdd(&counts[kBuckets + k], total);
+    base[k] = start[k] + __shfl(reserved, 0);
+  }
+  const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (kWaveSize - lane));
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+#pragma unroll
+    for (int k = 0; k < kBuckets; ++k) {
+      const unsigned long long members = __ballot(bucket[r] == (unsigned)k);
+      if (bucket[r] == (unsigned)k) {
+        const int at = base[k] + __popcll(members & below);
+        entry_pos[at] = (int)(first + r * kWaveSize + lane);
+        entry_row[at] = row[r];
+        entry_col[at] = col[r];
+      }
+      base[k] += __popcll(members);
+    }
+  }
+}
+
+// The SDDMM proper over such lists.  Workgroup ids are dealt to the XCDs round robin, so
+// workgroup id & 7 is the XCD and the range; the XCD's workgroups share out its list in
+// pieces of kEntriesPerWave entries.  Everything else as in sddmm_kernel.
+template <int GS, int VEC>
+__global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
+    int K, const int *__restrict__ list_ptr, const int *__restrict__ entry_pos,
+    const int *__restrict__ entry_row, const int *__restrict__ entry_col,
+    const float *__restrict__ mask_vals, const float *__restrict__ A, const float *__restrict__ B,
+    float *__restrict__ out_vals, int *__restrict__ out_row_idx, int64_t nnz, int64_t batch_stride_a,
+    int64_t batch_stride_b) {
+  using VecT = Vec<float, VEC>;
+  if (blockIdx.y > 0) {  // problem blockIdx.y of a batch over one mask
+    A += blockIdx.y * batch_stride_a;
+    B += blockIdx.y * batch_stride_b;
+    out_vals += blockIdx.y * nnz;
+    out_row_idx = nullptr;
+  }
+  const int lane = wave_lane();
+  const int xcd = blockIdx.x & 7;
+  const int64_t begin = list_ptr[xcd], end = list_ptr[xcd + 1];
+  const int64_t waves_per_xcd = (int64_t)(gridDim.x >> 3) * kWavesPerBlock;
+  const int t = lane % GS;
+  const int g = lane / GS;
+  for (int64_t first = begin + ((int64_t)(blockIdx.x >> 3) * kWavesPerBlock + threadIdx.x / kWaveSize) * kEntriesPerWave;
+       first < end; first += waves_per_xcd * kEntriesPerWave) {
+    const int64_t last = first + kEntriesPerWave < end ? first + kEntriesPerWave : end;
+    for (int64_t base = first; base < last; base += kWaveSize) {
+      const int64_t e = base + lane;
+      const bool valid = e < last;
+      int row = 0, col = 0, pos = 0;
+      float scale = 0.0f;
+      if (valid) {
+        pos = entry_pos[e];
+        row = entry_row[e];
+        col = entry_col[e];
+        scale = mask_vals[pos];
+      }
+      float mine = 0.0f;
+      if (K <= GS * VEC) {
+        // One load per lane covers a row.  Consecutive entries of a list mostly share their row
+        // of A (a row's entries of one column range lie together): the group keeps that row in
+        // registers and reloads it only when the row changes.
+        const int k = t * VEC;
+        const bool in_row = k < K;
+        VecT av;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) av.v[v] = 0.0f;
+        int held = -1;
+#pragma unroll 4
+        for (int s = 0; s < GS; ++s) {
+          const int src = g * GS + s;
+          const int r = __shfl(row, src);
+          const int c = __shfl(col, src);
+          if (r != held && in_row) av = *reinterpret_cast<const VecT *>(A + (size_t)r * (size_t)K + k);
+          held = r;
+          float dot = 0.0f;
+          if (in_row) {
+            const VecT bv = *reinterpret_cast<const VecT *>(B + (size_t)c * (size_t)K + k);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
+          }
+#pragma unroll
+          for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+          if (t == s) mine = dot;
+        }
+      } else {
+#pragma unroll 4
+        for (int s = 0; s < GS; ++s) {
+          const int src = g * GS + s;
+          const int r = __shfl(row, src);
+          const int c = __shfl(col, src);
+          const float *a = A + (size_t)r * (size_t)K;
+          const float *b = B + (size_t)c * (size_t)K;
+          float dot = 0.0f;
+          for (int k = t * VEC; k < K; k += GS * VEC) {
+            const VecT av = *reinterpret_cast<const VecT *>(a + k);
+            const VecT bv = *reinterpret_cast<const VecT *>(b + k);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
+          }
+#pragma unroll
+          for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+          if (t == s) mine = dot;
+        }
+      }
+      if (valid) {
+        out_vals[pos] = scale * mine;
+        if (out_row_idx) out_row_idx[pos] = row;
+      }
+    }
+  }
+}
+
 template <bool COO>
 int launch_sddmm(int M, int K, int64_t nnz, const int *rows, const int *col_idx,
                  const float *mask_vals, const float *A, const float *B, float *out_vals,
@@ -187,6 +413,31 @@ int sddmm_entry(const char *fn, int64_t M, int64_t n_cols, int64_t K, int64_t nn
                            out_row_idx, static_cast<hipStream_t>(stream), (int)batch, M * K, n_cols * K);
 }
 
+inline size_t align_up_256(size_t v) { return (v + 255) / 256 * 256; }
+
+// Layout of the per-XCD entry lists inside the caller's buffer.
+struct SddmmLists {
+  int *counts;     // [16]
+  int *list_ptr;   // [9]
+  int *entry_pos, *entry_row, *entry_col;  // [nnz] each
+};
+
+inline SddmmLists sddmm_lists(void *buffer, int64_t nnz) {
+  char *base = static_cast<char *>(buffer);
+  const size_t array = align_up_256((size_t)nnz * sizeof(int32_t));
+  SddmmLists l;
+  l.counts = reinterpret_cast<int *>(base);
+  l.list_ptr = l.counts + 16;
+  l.entry_pos = reinterpret_cast<int *>(base + 256);
+  l.entry_row = reinterpret_cast<int *>(base + 256 + array);
+  l.entry_col = reinterpret_cast<int *>(base + 256 + 2 * array);
+  return l;
+}
+
+__global__ void sddmm_lists_clear_kernel(int *counts) {
+  if (threadIdx.x < 32) counts[threadIdx.x] = 0;
+}
+
 }  // namespace scorch
 
 extern "C" {
@@ -213,6 +464,98 @@ int scorch_hip_sddmm_csr_batched_f32(int64_t batch, int64_t M, int64_t n_cols, i
                                      void *stream) {
   return scorch::sddmm_entry<false>("scorch_hip_sddmm_csr_batched_f32", M, n_cols, K, nnz, row_ptr, col_idx,
                                     mask_vals, A, B, out_vals, out_row_idx, stream, batch);
+}
+
+size_t scorch_hip_sddmm_csr_lists_bytes(int64_t nnz) {
+  if (nnz < 0) return 0;
+  // 16 counters and 9 list starts (256 bytes), then entry numbers, rows and columns
+  return 256 + 3 * scorch::align_up_256((size_t)nnz * sizeof(int32_t));
+}
+
+int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
+                               const int32_t *col_idx, void *lists, size_t lists_bytes, void *stream) {
+  const char *fn = "scorch_hip_sddmm_csr_lists";
+  if (M < 0 || n_cols < 0 || nnz < 0)
+    return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld n_cols=%lld nnz=%lld)", fn, (long long)M,
+                        (long long)n_cols, (long long)nnz);
+  if (M >= INT32_MAX || n_cols > INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  SCORCH_REQUIRE(row_ptr != nullptr && lists != nullptr, "%s: row_ptr or lists is NULL", fn);
+  SCORCH_REQUIRE(nnz == 0 || col_idx != nullptr, "%s: col_idx is NULL", fn);
+  SCORCH_REQUIRE(scorch::aligned_to(row_ptr, 4) && scorch::aligned_to(col_idx, 4) && scorch::aligned_to(lists, 256),
+                 "%s: index arrays must be 4-byte and lists 256-byte aligned", fn);
+  if (lists_bytes < scorch_hip_sddmm_csr_lists_bytes(nnz))
+    return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: %zu bytes needed for the lists, %zu given", fn,
+                        scorch_hip_sddmm_csr_lists_bytes(nnz), lists_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  scorch::SddmmLists l = scorch::sddmm_lists(lists, nnz);
+  scorch::sddmm_lists_clear_kernel<<<1, 64, 0, s>>>(l.counts);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  if (nnz == 0 || n_cols == 0) return SCORCH_HIP_OK;
+  const int cols_per_bucket = (int)((n_cols + scorch::kBuckets - 1) / scorch::kBuckets);
+  const int64_t waves = (nnz + scorch::kEntriesPerWave - 1) / scorch::kEntriesPerWave;
+  const dim3 grid((unsigned)((waves + scorch::kWavesPerBlock - 1) / scorch::kWavesPerBlock));
+  scorch::sddmm_bucket_count_kernel<<<grid, scorch::kBlockThreads, 0, s>>>(nnz, cols_per_bucket, col_idx, l.counts);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  scorch::sddmm_bucket_fill_kernel<<<grid, scorch::kBlockThreads, 0, s>>>((int)M, nnz, cols_per_bucket, row_ptr,
+                                                                         col_idx, l.counts, l.list_ptr, l.entry_pos,
+                                                                         l.entry_row, l.entry_col);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                                    const void *lists, size_t lists_bytes, const float *mask_vals,
+                                    const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
+                                    void *stream) {
+  const char *fn = "scorch_hip_sddmm_csr_listed_f32";
+  if (batch < 0 || batch > 65535)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
+  if (M < 0 || n_cols < 0 || K < 0 || nnz < 0)
+    return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size (M=%lld n_cols=%lld K=%lld nnz=%lld)", fn,
+                        (long long)M, (long long)n_cols, (long long)K, (long long)nnz);
+  if (M >= INT32_MAX || n_cols > INT32_MAX || K > INT32_MAX || nnz > INT32_MAX)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  if (batch == 0 || nnz == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(lists && mask_vals && out_vals, "%s: NULL lists or value array", fn);
+  SCORCH_REQUIRE(K == 0 || (A && B), "%s: NULL dense operand", fn);
+  SCORCH_REQUIRE(scorch::aligned_to(lists, 256) && scorch::aligned_to(mask_vals, 4) && scorch::aligned_to(out_vals, 4) &&
+                     scorch::aligned_to(A, 4) && scorch::aligned_to(B, 4) && scorch::aligned_to(out_row_idx, 4),
+                 "%s: lists must be 256-byte aligned, the other arrays 4-byte", fn);
+  if (lists_bytes < scorch_hip_sddmm_csr_lists_bytes(nnz))
+    return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: lists of %zu bytes expected, %zu given", fn,
+                        scorch_hip_sddmm_csr_lists_bytes(nnz), lists_bytes);
+  if (K > 256)
+    return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: K=%lld beyond 256 is served by scorch_hip_sddmm_csr_f32 only", fn,
+                        (long long)K);
+  const scorch::SddmmLists l = scorch::sddmm_lists(const_cast<void *>(lists), nnz);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // a resident grid: every XCD's workgroups walk that XCD's list
+  const int64_t waves = (nnz / scorch::kBuckets + scorch::kEntriesPerWave - 1) / scorch::kEntriesPerWave + 1;
+  int64_t wgs = (waves + scorch::kWavesPerBlock - 1) / scorch::kWavesPerBlock;
+  if (wgs > scorch::kListedWorkgroupsPerXcd) wgs = scorch::kListedWorkgroupsPerXcd;
+  const dim3 grid((unsigned)(wgs * 8), (unsigned)batch);
+  const bool vec4 = K % 4 == 0 && scorch::aligned_to(A, 16) && scorch::aligned_to(B, 16);
+  const int64_t lanes_needed = (K + (vec4 ? 4 : 1) - 1) / (vec4 ? 4 : 1);
+  scorch::mark_launch(s);
+#define SCORCH_LISTED(GS, VEC)                                                                                   \
+  scorch::sddmm_listed_kernel<GS, VEC><<<grid, scorch::kBlockThreads, 0, s>>>(                                   \
+      (int)K, l.list_ptr, l.entry_pos, l.entry_row, l.entry_col, mask_vals, A, B, out_vals, out_row_idx, nnz,   \
+      M * K, n_cols * K)
+#define SCORCH_LISTED_PICK(VEC)                          \
+  do {                                                   \
+    if (lanes_needed <= 4) SCORCH_LISTED(4, VEC);        \
+    else if (lanes_needed <= 8) SCORCH_LISTED(8, VEC);   \
+    else if (lanes_needed <= 16) SCORCH_LISTED(16, VEC); \
+    else if (lanes_needed <= 32) SCORCH_LISTED(32, VEC); \
+    else SCORCH_LISTED(64, VEC);                         \
+  } while (0)
+  if (vec4) SCORCH_LISTED_PICK(4); else SCORCH_LISTED_PICK(1);
+#undef SCORCH_LISTED_PICK
+#undef SCORCH_LISTED
+  SCORCH_HIP_CHECK(hipGetLastError());
+  scorch::mark_launch(s);
+  return SCORCH_HIP_OK;
 }
 
 }  // extern "C"

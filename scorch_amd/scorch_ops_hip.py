@@ -167,13 +167,15 @@ class CsrPlan:
     chunk boundaries of the merge-path kernels.  Lives as an attribute of the
     row-pointer tensor, so it is dropped with the operand, and is rebuilt when
     either index tensor has been written to since."""
-    __slots__ = ("key", "max_row", "empty_rows", "bounds")
+    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses")
 
     def __init__(self, key, max_row: int, empty_rows: int):
         self.key = key
         self.max_row = max_row
         self.empty_rows = empty_rows
         self.bounds: Dict[Tuple[int, int], torch.Tensor] = {}
+        self.sddmm_lists: Optional[torch.Tensor] = None   # the mask's entries listed per XCD (SDDMM)
+        self.sddmm_uses = 0                                # SDDMM calls that could have used them
 
 
 def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, what: str = "operand") -> Optional[CsrPlan]:
@@ -474,6 +476,35 @@ prebuilt_spmv_csr_i32 = _make_spmv(torch.int32)
 prebuilt_spmv_csr_i64 = _make_spmv(torch.int64)
 
 
+SDDMM_PATHS = ("auto", "plain", "listed")
+# "auto": a CSR mask seen for the second time, with a dense right operand between 8 and 20 MB
+# (beyond one L2, within the eight together), is served from per-XCD entry lists; "plain" /
+# "listed" pin one path (SCORCH_HIP_SDDMM_PATH sets the default).
+SDDMM_PATH = os.environ.get("SCORCH_HIP_SDDMM_PATH", "auto")
+
+
+def _sddmm_lists(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, K: int, L, stream) -> Optional[torch.Tensor]:
+    """The mask's per-XCD entry lists if this product should use them (built on the
+    second such product with the mask), else None."""
+    if SDDMM_PATH not in SDDMM_PATHS:
+        raise ValueError(f"scorch_ops_hip: SDDMM_PATH is {SDDMM_PATH!r}, expected one of {SDDMM_PATHS}")
+    if SDDMM_PATH == "plain" or plan is None or K > 256 or K == 0 or crd.numel() == 0:
+        return None
+    if SDDMM_PATH == "auto":
+        b_bytes = n_cols * K * 4
+        if not (8 << 20) <= b_bytes <= (20 << 20) or crd.numel() < 4 * n_cols:
+            return None
+        plan.sddmm_uses += 1
+        if plan.sddmm_lists is None and (plan.sddmm_uses < 2 or torch.cuda.is_current_stream_capturing()):
+            return None
+    if plan.sddmm_lists is None:
+        lists = torch.empty(L.scorch_hip_sddmm_csr_lists_bytes(crd.numel()), dtype=torch.uint8, device=pos.device)
+        native.check(L.scorch_hip_sddmm_csr_lists(M, n_cols, crd.numel(), pos.data_ptr(), crd.data_ptr(),
+                                                  lists.data_ptr(), lists.numel(), stream))
+        plan.sddmm_lists = lists
+    return plan.sddmm_lists
+
+
 # ---- SDDMM ---------------------------------------------------------------------
 def _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values):
     M, n_cols = int(S_shape[0]), int(S_shape[1])
@@ -521,14 +552,21 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     if pos.numel() != M + 1 or crd.numel() != s_val.numel():
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
     dev = _device_of(pos, crd, s_val, a, b)
-    csr_plan(pos, crd, M, n_cols, "S")
+    plan = csr_plan(pos, crd, M, n_cols, "S")
     out = torch.empty_like(s_val)
     rows = torch.empty_like(crd)
+    L = native.lib()
     with _on_device(dev):
-        rc = native.lib().scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(),
-                                                   crd.data_ptr(), s_val.data_ptr(), a.data_ptr(),
-                                                   b.data_ptr(), out.data_ptr(), rows.data_ptr(),
-                                                   _stream(dev))
+        stream = _stream(dev)
+        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream)
+        if lists is not None:
+            rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
+                                                   s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                   rows.data_ptr(), stream)
+        else:
+            rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(), crd.data_ptr(),
+                                            s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                            rows.data_ptr(), stream)
     native.check(rc)
     return Tensor(out, [[rows], [crd]])
 
@@ -647,14 +685,22 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     if pos.numel() != M + 1 or crd.numel() != s_val.numel():
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
     dev = _device_of(pos, crd, s_val, a, b)
-    csr_plan(pos, crd, M, n_cols, "S")
+    plan = csr_plan(pos, crd, M, n_cols, "S")
     nnz = s_val.numel()
     out = torch.empty((H, nnz), dtype=torch.float32, device=dev)
     rows = torch.empty_like(crd)
+    L = native.lib()
     with _on_device(dev):
-        rc = native.lib().scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),
-                                                           s_val.data_ptr(), a.data_ptr(), b.data_ptr(),
-                                                           out.data_ptr(), rows.data_ptr(), _stream(dev))
+        stream = _stream(dev)
+        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream)
+        if lists is not None:
+            rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
+                                                   s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                   rows.data_ptr(), stream)
+        else:
+            rc = L.scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                    rows.data_ptr(), stream)
     native.check(rc)
     return out, rows
 

@@ -142,3 +142,63 @@ def test_full_size_workload():
     coo = H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows_ref], [ci]], s, [M, K], [[], []],
                                      A.reshape(-1), [n_cols, K], [[], []], B.reshape(-1))
     assert torch.equal(coo.storage.value, out.storage.value)
+
+
+# ---- a reused mask: its entries listed per XCD ---------------------------------------------------
+@pytest.mark.parametrize("K", [8, 32, 64, 100, 256])
+def test_listed_path_equals_the_plain_one(K, monkeypatch):
+    """The same products computed list by list (one list per XCD, by column range): bit for bit
+    the plain kernel's values and row coordinates, for one product and for a batch over the mask."""
+    from scorch_amd import scorch_ops_hip as H
+    w = workloads.sddmm_uniform(M=3000, n_cols=2500, per_row=40, K=K, seed=K, unit_mask=False)
+    rp, ci, sv = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    A, B = dev(w["A"]), dev(w["B"])
+    call = lambda: H.sddmm_csr_float([3000, 2500], [3000, 2500], [[], [rp, ci]], sv, [3000, K], [[], []],
+                                     A.reshape(-1), [2500, K], [[], []], B.reshape(-1))
+    monkeypatch.setattr(H, "SDDMM_PATH", "plain")
+    plain = call()
+    monkeypatch.setattr(H, "SDDMM_PATH", "listed")
+    listed = call()
+    assert rp._scorch_plan.sddmm_lists is not None
+    assert torch.equal(plain.storage.value, listed.storage.value)
+    assert torch.equal(plain.storage.index.mode_indices[0][0], listed.storage.index.mode_indices[0][0])
+    A3 = torch.stack([A, A * 2, A - 1])
+    B3 = torch.stack([B, B + 1, B * 0.5])
+    got, rows = H.sddmm_csr_float_batched([3000, 2500], [[], [rp, ci]], sv, A3, B3)
+    monkeypatch.setattr(H, "SDDMM_PATH", "plain")
+    want, rows_plain = H.sddmm_csr_float_batched([3000, 2500], [[], [rp, ci]], sv, A3, B3)
+    assert torch.equal(got, want) and torch.equal(rows, rows_plain)
+
+
+def test_listed_path_with_ragged_rows_and_empty_column_ranges(oracle, monkeypatch):
+    """Rows of very different lengths, empty rows, and all columns in the first eighth but one."""
+    from scorch_amd import scorch_ops_hip as H
+    rng = np.random.default_rng(31)
+    lens = rng.integers(0, 50, 700); lens[[0, 350]] = [3000, 0]
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = rng.integers(0, 500, int(rp[-1])).astype(np.int32)
+    ci[-1] = 3999
+    sv = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    A = rng.standard_normal((700, 48)).astype(np.float32)
+    B = rng.standard_normal((4000, 48)).astype(np.float32)
+    monkeypatch.setattr(H, "SDDMM_PATH", "listed")
+    rows, cols, vals = hip_sddmm_csr(rp, ci, sv, A, B, (700, 4000))
+    want_rows = np.repeat(np.arange(700, dtype=np.int32), lens)
+    assert np.array_equal(rows, want_rows) and np.array_equal(cols, ci)
+    assert oracle.rel_fro(vals, oracle.sddmm_fp64(want_rows, ci, sv, A, B)) <= 1e-5
+
+
+def test_auto_builds_the_lists_on_the_second_product_at_full_size(oracle):
+    """65,536^2, 64 per row, K = 64: B is 16 MB, beyond one L2 and within the eight together."""
+    from scorch_amd import scorch_ops_hip as H
+    w = workloads.sddmm_uniform()
+    M, n_cols, K = w["M"], w["n_cols"], w["K"]
+    rp, ci, sv = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    A, B = dev(w["A"]).reshape(-1), dev(w["B"]).reshape(-1)
+    call = lambda: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [rp, ci]], sv, [M, K], [[], []], A, [n_cols, K],
+                                     [[], []], B).storage.value
+    first = call()
+    assert rp._scorch_plan.sddmm_lists is None
+    second = call()
+    assert rp._scorch_plan.sddmm_lists is not None
+    assert torch.equal(first, second) and torch.equal(second, call())
