@@ -21,6 +21,7 @@ is re-stored once by column tiles (see CsrPlan and _tiled_operand below).
 """
 from __future__ import annotations
 
+import math
 import os
 from typing import Dict, Optional, Tuple
 
@@ -438,8 +439,73 @@ def _make_spgemm(dtype):
     return kernel
 
 
-prebuilt_spmspm_csr_f32 = _make_spgemm(torch.float32)
-spmspm_csr_float = _make_spgemm(torch.float32)
+_spgemm_f32_atomic = _make_spgemm(torch.float32)
+
+# fp32 CSR x CSR sums are accumulated with floating-point atomics, so their last bits depend
+# on the order in which the hardware happens to serve them.  With SPGEMM_REPRODUCIBLE (default:
+# SCORCH_HIP_SPGEMM_REPRODUCIBLE) the fp32 product is computed in 64-bit fixed point instead,
+# where addition is associative: the same bits on every run, whatever the order.
+SPGEMM_REPRODUCIBLE = os.environ.get("SCORCH_HIP_SPGEMM_REPRODUCIBLE", "0") not in ("", "0")
+
+
+def spmspm_csr_f32_reproducible(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+    """C = A @ B, all CSR, fp32 values, with sums that do not depend on the order of the
+    additions: both operands are rounded to fixed point (A to multiples of 2^-sa, B of 2^-sb),
+    multiplied with the exact int64 kernel, and the sums scaled back.  sa and sb are the largest
+    shifts for which no row's sum can overflow: with P the largest number of products in a row,
+    each operand keeps (62 - ceil(log2 P)) / 2 bits below its largest magnitude -- 23 bits, fp32's
+    own, for P up to 65,536.  An entry's error is at most P * 2^-(bits) * max|A| * max|B|; small
+    entries of operands with a wide range of magnitudes lose relative precision.  Same structure
+    as the default mode (reference: csrc/kernels.h:52-202)."""
+    M, K, N = int(A_shape[0]), int(A_shape[1]), int(B_shape[1])
+    a_pos, a_crd = _csr_parts(A_mode_indices, "A")
+    b_pos, b_crd = _csr_parts(B_mode_indices, "B")
+    a_val, b_val = _flat(A_values, torch.float32, "A values"), _flat(B_values, torch.float32, "B values")
+    if a_pos.numel() != M + 1 or b_pos.numel() != K + 1 or a_crd.numel() != a_val.numel() \
+            or b_crd.numel() != b_val.numel():
+        raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
+    dev = _device_of(a_pos, a_crd, a_val, b_pos, b_crd, b_val)
+    csr_plan(a_pos, a_crd, M, K, "A")
+    if a_val.numel() == 0 or b_val.numel() == 0:
+        return _spgemm_f32_atomic(result_shape, A_shape, A_mode_indices, a_val, B_shape, B_mode_indices, b_val)
+    if not (bool(torch.isfinite(a_val).all()) and bool(torch.isfinite(b_val).all())):
+        raise ValueError("scorch_ops_hip: the reproducible SpGEMM needs finite values")
+    # most products in one row of C: sum over the row's entries of the lengths of the B rows they select
+    b_len = (b_pos[1:] - b_pos[:-1]).to(torch.int64)
+    per_entry = b_len[a_crd.long()]
+    rows = csr_row_indices(a_pos, int(a_crd.numel())).long()
+    most = int(torch.zeros(M, dtype=torch.int64, device=dev).index_add_(0, rows, per_entry).max())
+    bits = (62 - max(most, 1).bit_length()) // 2
+    a_max, b_max = float(a_val.abs().max()), float(b_val.abs().max())
+
+    def fixed(values, largest):
+        if largest == 0.0:
+            return torch.zeros(values.shape, dtype=torch.int64, device=dev), 0
+        shift = bits - (math.frexp(largest)[1])        # |values| * 2^shift < 2^bits
+        return torch.round(torch.ldexp(values.double(), torch.tensor(shift, device=dev))).to(torch.int64), shift
+
+    a_fix, sa = fixed(a_val, a_max)
+    b_fix, sb = fixed(b_val, b_max)
+    out = prebuilt_spmspm_csr_i64(result_shape, A_shape, A_mode_indices, a_fix, B_shape, B_mode_indices, b_fix)
+    c_fix = out.storage.value
+    c_val = torch.ldexp(c_fix.double(), torch.tensor(-(sa + sb), device=dev)).to(torch.float32)
+    return Tensor(c_val, out.storage.index.mode_indices)
+
+
+def _spgemm_f32(*args):
+    return spmspm_csr_f32_reproducible(*args) if SPGEMM_REPRODUCIBLE else _spgemm_f32_atomic(*args)
+
+
+def prebuilt_spmspm_csr_f32(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+    """C = A @ B, all CSR, fp32 (reference: csrc/kernels.h:52-202).  Sums by floating-point
+    atomics unless SPGEMM_REPRODUCIBLE is set (see spmspm_csr_f32_reproducible)."""
+    return _spgemm_f32(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values)
+
+
+def spmspm_csr_float(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values):
+    return _spgemm_f32(result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mode_indices, B_values)
+
+
 prebuilt_spmspm_csr_f64 = _make_spgemm(torch.float64)
 prebuilt_spmspm_csr_i32 = _make_spgemm(torch.int32)
 prebuilt_spmspm_csr_i64 = _make_spgemm(torch.int64)

@@ -14,6 +14,7 @@ from conftest import random_csr
 from gpu_util import dev, host
 from scorch_amd import STensor
 from scorch_amd import scorch_ops_hip as H
+from scorch_amd import workloads
 
 pytestmark = pytest.mark.gpu
 SYMBOL = {np.dtype(np.float32): "prebuilt_spmspm_csr_f32", np.dtype(np.float64): "prebuilt_spmspm_csr_f64",
@@ -360,3 +361,31 @@ def test_result_beyond_the_int32_row_pointer_is_reported():
                                                   b_crd.data_ptr(), c_pos.data_ptr(), ws.data_ptr(), ws.numel(),
                                                   torch.cuda.current_stream().cuda_stream))
     assert int(c_pos[-1]) == M * N and int(c_pos[1]) == N
+
+
+def test_reproducible_mode_gives_the_same_bits_on_every_run(oracle, monkeypatch):
+    """fp32 sums in 64-bit fixed point: identical values from run to run (the default mode's
+    atomics only promise that to rounding), the same structure, and within the fp32 bar of fp64."""
+    w = workloads.gcn_powerlaw(M=30_000, N=1, seed=13, max_degree=4000)
+    rp, ci, v = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"])
+    shape = [30_000, 30_000]
+    call = lambda: H.prebuilt_spmspm_csr_f32(shape, shape, [[], [rp, ci]], v, shape, [[], [rp, ci]], v)
+    plain = call()
+    monkeypatch.setattr(H, "SPGEMM_REPRODUCIBLE", True)
+    runs = [call() for _ in range(3)]
+    for r in runs[1:]:
+        assert torch.equal(r.storage.value, runs[0].storage.value)
+    for mine, theirs in zip(runs[0].storage.index.mode_indices[1], plain.storage.index.mode_indices[1]):
+        assert torch.equal(mine, theirs)
+    A = sp.csr_matrix((w["vals"].astype(np.float64), w["col_idx"], w["row_ptr"]), shape=(30_000, 30_000))
+    ref = (A @ A).tocsr()
+    ref.sort_indices()
+    assert np.array_equal(host(runs[0].storage.index.mode_indices[1][1]), ref.indices)
+    assert oracle.rel_fro(host(runs[0].storage.value), ref.data) <= 1e-5
+    assert oracle.rel_fro(host(plain.storage.value), ref.data) <= 1e-5
+    # the COO x COO symbol and matmul go the same way
+    small = H.spmspm_csr_float([3, 3], [3, 3], [[], [dev(np.array([0, 1, 2, 3], np.int32)),
+                                                      dev(np.array([2, 0, 1], np.int32))]], dev(np.array([0.5, -2.0, 3.0], np.float32)),
+                               [3, 3], [[], [dev(np.array([0, 1, 2, 3], np.int32)), dev(np.array([1, 2, 0], np.int32))]],
+                               dev(np.array([4.0, 0.25, -1.0], np.float32)))
+    assert host(small.storage.value).tolist() == [-0.5, -8.0, 0.75]
