@@ -430,7 +430,7 @@ def run_attention(args):
                       "active_blocks": int(bci.numel()), "nnz_per_head": nnz,
                       "seed": workloads.SEEDS["attention_blocksparse"]},
            "warmup_ms": warm,
-           "roofline": {"bound": "mfma", "kernel": "attn_blocksparse_kernel<false>", "achieved": round(achieved, 1),
+           "roofline": {"bound": "mfma", "kernel": "attn_blocksparse_kernel<64, false, false>", "achieved": round(achieved, 1),
                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
                         "flops": flops, "algorithmic_bytes": algo, "kernel_ms_avg": round(ms, 5),
@@ -558,6 +558,15 @@ def run_extra(args):
                "value": round(heads * (4.0 * nnz * D + 5.0 * nnz) / ms / 1e6, 2), "ms_per_step": round(ms, 5), **base,
                "config": {"workload": "attention_longformer_fp32", "S": S, "H": heads, "D": D, "window": 64,
                           "global_tokens": 1, "nnz_per_head": nnz}}
+        # the same mask through the fused bf16 kernel: 64 x 64 blocks with per-block bit masks
+        qb, kb, vb = (t.to(torch.bfloat16) for t in (q, k, v))
+        bm = H.attention_block_mask(rp, ci, S)
+        ms_fused = _time_steps(lambda: H.sparse_attention_bf16(qb, kb, vb, rp, ci, scale), args.steps, args.warmup)
+        diff = (H.sparse_attention_bf16(qb, kb, vb, rp, ci, scale).float() - fn()).norm() / fn().norm()
+        out["fused_bf16"] = {"ms_per_step": round(ms_fused, 5), "active_blocks": bm.n_active_blocks,
+                             "distinct_block_masks": bm.n_masks,
+                             "live_share_of_active_blocks": round(bm.density_in_blocks, 4),
+                             "rel_fro_vs_fp32_pipeline": float(diff)}
         if args.vendor:
             import torch.nn.functional as F
             rows = torch.repeat_interleave(torch.arange(S, device="cuda"), (rp[1:] - rp[:-1]).long())

@@ -404,23 +404,38 @@ SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int3
  * entries: block_row_ptr int32[S / block + 1], block_col_idx
  * int32[n_active_blocks]; every entry of an active block is live.  Query rows
  * whose block row has no active block give zeros.
- * Built for D = 64 and block = 64 (other values: SCORCH_HIP_EUNSUPPORTED).
+ * Built for D = 32, 64 and 128 and block = 64 (other values:
+ * SCORCH_HIP_EUNSUPPORTED).
  * One kernel does what the reference's attention benchmark composes per head
  * from SDDMM, a row softmax and SpMM (bench/bench_sparse_transformer.py:354-372);
  * the reference has no fused or bf16 counterpart.
+ *
+ * The _masked form serves masks that are not unions of whole blocks (the
+ * reference's Longformer pattern, a sliding window plus global tokens,
+ * bench/bench_sparse_transformer.py:117-141; a causal diagonal): active block i
+ * is fully live when block_mask_index[i] < 0, and otherwise restricted to the
+ * 64 x 64 bit mask block_masks[64 * block_mask_index[i] .. + 63], where bit j
+ * of word r says that query r of the block row attends to key j of the block.
+ * block_mask_index is int32[n_active_blocks], block_masks uint64[64 * n_masks]
+ * (several blocks may share one mask).  Queries without any live key give zeros.
  * ---------------------------------------------------------------------- */
 SCORCH_HIP_API int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D, int64_t block,
                                      int64_t n_active_blocks,
                                      const int32_t *block_row_ptr, const int32_t *block_col_idx,
                                      const void *Q, const void *K, const void *V, float scale,
                                      void *O, void *stream);
+SCORCH_HIP_API int scorch_hip_attn_blocksparse_masked_bf16(
+    int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks,
+    const int32_t *block_row_ptr, const int32_t *block_col_idx, const int32_t *block_mask_index,
+    int64_t n_masks, const uint64_t *block_masks, const void *Q, const void *K, const void *V,
+    float scale, void *O, void *stream);
 
 /* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's
  * sparse attention -- SDDMM, row softmax, SpMM, which its benchmark runs head by
  * head from a Python loop (bench/bench_sparse_transformer.py:325,354-372) -- each
  * as one launch over all heads (grid.y = head).  For any CSR mask and any head
- * dimension; the fused kernel above covers block masks at D = 64 only.
+ * dimension and in fp32; the fused kernel above is bf16, for D = 32, 64 or 128.
  * Problem h uses A + h M K, B + h n_cols K (resp. vals + h nnz, B + h K N) and
  * writes out + h nnz (resp. C + h M N); the pattern and, for SDDMM, the mask's
  * values are shared.  batch <= 65535.  Results are those of `batch` separate

@@ -32,7 +32,6 @@
 namespace scorch {
 
 constexpr int kAttnBlock = 64;  // mask block edge: queries per workgroup, keys per step
-constexpr int kAttnDim = 64;    // head dimension
 constexpr float kRescaleSlack = 8.0f;  // see the online softmax in the kernel
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -61,23 +60,42 @@ __device__ __forceinline__ float combine_query_lanes(float x, Op op) {
 }
 
 // K and V tiles are written to LDS by the load itself (global_load_lds_dwordx4):
-// no staging registers, no LDS store instructions; with 90 VGPRs and 32 KB of
-// LDS per workgroup five workgroups share a CU.  Such a load puts lane L's 16
+// no staging registers, no LDS store instructions; at D = 64, with 124 VGPRs and
+// 32 KB of LDS per workgroup, four workgroups share a CU.  Such a load puts lane L's 16
 // bytes at (wave-uniform base) + 16 L, so a wavefront instruction fills eight
 // whole 128-byte rows and rows cannot be padded against bank conflicts.  Instead
 // the 16-byte chunks of a row are permuted: chunk c of row r lies at position
 // c ^ (r & 7).  The permutation is applied on the way in (each lane fetches the
 // chunk that belongs at its LDS position) and undone by the readers' address
-// arithmetic.  (Staging through registers with padded rows: 118 VGPRs, 36 KB,
-// four workgroups per CU, 12 % slower.)
-constexpr int kTileBytes = kAttnBlock * kAttnDim * 2;  // 8 KB, rows of 128 bytes
+// arithmetic.  (Staging through registers with padded rows measured 12 % slower.)
+//
+// Head dimension D is 32, 64 or 128: a tile row is RB = 2 D bytes, i.e. CPR = D / 8 chunks of 16
+// bytes, a tile 64 RB bytes.  The permutation is chunk c of row r at position c ^ swizzle(r) with
+// swizzle(r) = r & 7 (for D = 32, where a row has only four chunks, (r >> 1) & 3): what matters
+// is that the eight lanes the LDS serves together, which read the same chunk of eight
+// consecutive rows, fall into eight different 16-byte bank groups.
+template <int D>
+struct AttnTile {
+  static constexpr int kRowBytes = 2 * D;
+  static constexpr int kChunksPerRow = D / 8;
+  static constexpr int kBytes = kAttnBlock * kRowBytes;
+  static constexpr int kRowsPerLoad = 1024 / kRowBytes;     // rows one wavefront load instruction fills
+  static constexpr int kLoadsPerWave = 16 / kRowsPerLoad;   // a wavefront fills 16 rows of a tile
+  __device__ static __forceinline__ int swizzle(int row) { return D == 32 ? (row >> 1) & 3 : row & 7; }
+};
 
-template <bool NEGATIVE_SCALE>
+template <int D, bool NEGATIVE_SCALE, bool MASKED>
 __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
-    const int *__restrict__ block_col_idx, const __bf16 *__restrict__ Q,
+    const int *__restrict__ block_col_idx, const int *__restrict__ block_mask_index,
+    const unsigned long long *__restrict__ block_masks, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O) {
+  using Tile = AttnTile<D>;
+  constexpr int kTileBytes = Tile::kBytes;
+  constexpr int kRowBytes = Tile::kRowBytes;
+  constexpr int kSteps = D / 32;   // MFMA steps of the first product (contraction over D)
+  constexpr int kFeat = D / 16;    // 16-feature tiles of the second product
   // Two buffers each for K and V, as four separate arrays: the compiler then sees that the
   // loads which fill one buffer (they write LDS asynchronously) cannot touch the buffer being
   // read, and does not make the reads wait for them.  (As halves of one array, every second key
@@ -110,20 +128,20 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     }
   }
   const int qb = n_blocks - 1 - rank;  // longest block rows first
-  const size_t head_off = (size_t)head * (size_t)S * kAttnDim;
+  const size_t head_off = (size_t)head * (size_t)S * D;
   const __bf16 *Qh = Q + head_off;
   const unsigned char *Kb = reinterpret_cast<const unsigned char *>(K + head_off);
   const unsigned char *Vb = reinterpret_cast<const unsigned char *>(V + head_off);
 
   const int query = qb * kAttnBlock + w * 16 + n;
-  bf16x8 q_op[2];
+  bf16x8 q_op[kSteps];
 #pragma unroll
-  for (int s = 0; s < 2; ++s)
-    q_op[s] = *reinterpret_cast<const bf16x8 *>(Qh + (size_t)query * kAttnDim + 8 * g + 32 * s);
+  for (int s = 0; s < kSteps; ++s)
+    q_op[s] = *reinterpret_cast<const bf16x8 *>(Qh + (size_t)query * D + 8 * g + 32 * s);
 
-  floatx4 o_acc[4];
+  floatx4 o_acc[kFeat];
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt) o_acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int dt = 0; dt < kFeat; ++dt) o_acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -3.0e38f;
   // (scale 0: every score counts as 0, nothing ever needs rescaling beyond the first block)
   const float inv_scale_log2e = scale_log2e != 0.0f ? 1.0f / scale_log2e : 0.0f;
@@ -137,36 +155,43 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
   const int kb_end = block_row_ptr[qb + 1];
 
 
-  // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with two instructions
-  // of eight rows each.  Lane L of instruction u lands at row 16w + 8u + L / 8,
-  // position L % 8, which holds chunk (L % 8) ^ (row & 7) = (L % 8) ^ (L / 8).
-  const int src_in_tile = (16 * w + (lane >> 3)) * 128 + (((lane & 7) ^ (lane >> 3)) * 16);
+  // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with kLoadsPerWave instructions of
+  // kRowsPerLoad rows each.  Lane L of instruction u lands at row 16w + u kRowsPerLoad + L / CPR,
+  // position L % CPR, which holds chunk (L % CPR) ^ swizzle(row).
+  int src_in_tile[Tile::kLoadsPerWave];
+#pragma unroll
+  for (int u = 0; u < Tile::kLoadsPerWave; ++u) {
+    const int row = 16 * w + u * Tile::kRowsPerLoad + lane / Tile::kChunksPerRow;
+    src_in_tile[u] = row * kRowBytes + (((lane % Tile::kChunksPerRow) ^ Tile::swizzle(row)) * 16);
+  }
   auto load_tile = [&](auto buf_tag, int it) {
     constexpr int kBuf = decltype(buf_tag)::value;
     unsigned char *k_dst = kBuf ? s_k1 : s_k0;
     unsigned char *v_dst = kBuf ? s_v1 : s_v0;
     const size_t tile = (size_t)uniform(block_col_idx[it]) * kTileBytes;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < Tile::kLoadsPerWave; ++u) {
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(Kb + tile + src_in_tile + u * 1024),
-          (__attribute__((address_space(3))) void *)(&k_dst[(16 * w + 8 * u) * 128]), 16, 0, 0);
+          (const __attribute__((address_space(1))) void *)(Kb + tile + src_in_tile[u]),
+          (__attribute__((address_space(3))) void *)(&k_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(Vb + tile + src_in_tile + u * 1024),
-          (__attribute__((address_space(3))) void *)(&v_dst[(16 * w + 8 * u) * 128]), 16, 0, 0);
+          (const __attribute__((address_space(1))) void *)(Vb + tile + src_in_tile[u]),
+          (__attribute__((address_space(3))) void *)(&v_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]), 16, 0, 0);
     }
   };
   using Even = std::integral_constant<int, 0>;
   using Odd = std::integral_constant<int, 1>;
 
-  // Readers' offsets inside a tile.  K: row 16t + n, chunks g and g + 4 (positions
-  // g ^ (n & 7) and that ^ 4).  V^T: row 32s + 16h + 4g + n / 4, 8 bytes at feature
-  // 16dt + 4 (n % 4), i.e. chunk 2dt + (n % 4) / 2, half (n % 4) % 2.
-  const int k_off = n * 128 + ((g ^ (n & 7)) * 16);
+  // Readers' offsets inside a tile.  K: row 16t + n, chunk 4s + g for contraction step s (its
+  // swizzle depends on n only).  V^T: row 32s + 16h + 4g + n / 4, 8 bytes at feature
+  // 16dt + 4 (n % 4), i.e. chunk 2dt + (n % 4) / 2, half (n % 4) % 2 (swizzle: on 4g + n / 4).
+  const int k_swz = Tile::swizzle(n);
+  const int k_row = n * kRowBytes;
   const int v_row = 4 * g + (n >> 2);
-  const int v_swz = v_row & 7;
-  const int v_off = v_row * 128 + (n & 1) * 8;
+  const int v_swz = Tile::swizzle(v_row);
+  const int v_off = v_row * kRowBytes + (n & 1) * 8;
   const int v_chunk = (n & 3) >> 1;
+  const int my_query_in_block = w * 16 + n;
 
   if (kb_begin < kb_end) load_tile(Even{}, kb_begin);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -182,10 +207,31 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     floatx4 st[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const bf16x8 k_lo = *reinterpret_cast<const bf16x8 *>(&k_src[2048 * t + k_off]);
-      const bf16x8 k_hi = *reinterpret_cast<const bf16x8 *>(&k_src[2048 * t + (k_off ^ 64)]);
-      st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_lo, q_op[0], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-      st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_hi, q_op[1], st[t], 0, 0, 0);
+      st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        const bf16x8 k_op = *reinterpret_cast<const bf16x8 *>(
+            &k_src[16 * kRowBytes * t + k_row + (((4 * s + g) ^ k_swz) * 16)]);
+        st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_op, q_op[s], st[t], 0, 0, 0);
+      }
+    }
+
+    // A block that is only partly live brings a 64 x 64 bit mask: bit j of word i says whether
+    // query i of the block row attends to key j of the block.  A lane holds the scores of its
+    // query against keys 16t + 4g + r (bit 16t + r of the word shifted down by 4g); dead ones are
+    // kept out of the maximum here and get probability zero below.
+    int mask_at = -1;
+    unsigned long long live = ~0ull;
+    if constexpr (MASKED) {
+      mask_at = uniform(block_mask_index[it]);
+      if (mask_at >= 0) {
+        live = block_masks[(size_t)mask_at * kAttnBlock + my_query_in_block] >> (4 * g);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (!((live >> (16 * t + r)) & 1ull)) st[t][r] = NEGATIVE_SCALE ? 3.0e38f : -3.0e38f;
+      }
     }
 
     float mx = st[0][0];
@@ -208,7 +254,7 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       l_acc[0] *= alpha;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
       m_run = m_new;
@@ -220,17 +266,20 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_run));
+        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_run));
+        if constexpr (MASKED) {
+          if (!((live >> (16 * t + r)) & 1ull)) p = 0.0f;
+        }
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
 
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const int at = 4096 * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
+        const int at = 32 * kRowBytes * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
         const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
-        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 2048]);
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 16 * kRowBytes]);
         const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         const bf16x8 v_op = __builtin_bit_cast(bf16x8, packed);
         o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
@@ -251,9 +300,9 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 
   const float l = l_acc[0];
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // block rows without key blocks give zeros
-  __bf16 *out = O + head_off + (size_t)query * kAttnDim;
+  __bf16 *out = O + head_off + (size_t)query * D;
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt) {
+  for (int dt = 0; dt < kFeat; ++dt) {
     bf16x4 o;
 #pragma unroll
     for (int r = 0; r < 4; ++r) o[r] = (__bf16)(o_acc[dt][r] * inv);
@@ -263,20 +312,40 @@ __global__ __launch_bounds__(kBlockThreads) void attn_blocksparse_kernel(
 
 }  // namespace scorch
 
-extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D, int64_t block,
-                                                int64_t n_active_blocks,
-                                                const int32_t *block_row_ptr,
-                                                const int32_t *block_col_idx, const void *Q,
-                                                const void *K, const void *V, float scale, void *O,
-                                                void *stream) {
-  using namespace scorch;
-  const char *fn = "scorch_hip_attn_blocksparse_bf16";
+namespace scorch {
+
+template <int D>
+static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int n_blocks, int H,
+                            const int32_t *block_row_ptr, const int32_t *block_col_idx,
+                            const int32_t *block_mask_index, const unsigned long long *block_masks,
+                            const __bf16 *q, const __bf16 *k, const __bf16 *v, float scale_log2e,
+                            __bf16 *o) {
+#define SCORCH_ATTN_LAUNCH(NEG, MASKED)                                                          \
+  attn_blocksparse_kernel<D, NEG, MASKED><<<grid, kBlockThreads, 0, s>>>(                        \
+      S, n_blocks, H, block_row_ptr, block_col_idx, block_mask_index, block_masks, q, k, v,      \
+      scale_log2e, o)
+  const bool masked = block_mask_index != nullptr;
+  if (negative) {
+    if (masked) SCORCH_ATTN_LAUNCH(true, true); else SCORCH_ATTN_LAUNCH(true, false);
+  } else {
+    if (masked) SCORCH_ATTN_LAUNCH(false, true); else SCORCH_ATTN_LAUNCH(false, false);
+  }
+#undef SCORCH_ATTN_LAUNCH
+}
+
+// Shared by the two entry points; block_mask_index == nullptr means every listed block is
+// fully live.
+static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t block,
+                      int64_t n_active_blocks, const int32_t *block_row_ptr,
+                      const int32_t *block_col_idx, const int32_t *block_mask_index,
+                      const uint64_t *block_masks, const void *Q, const void *K, const void *V,
+                      float scale, void *O, void *stream) {
   if (H < 0 || S < 0 || D < 0 || block <= 0 || n_active_blocks < 0)
     return fail(SCORCH_HIP_EINVAL, "%s: negative size (H=%lld S=%lld D=%lld block=%lld)", fn,
                 (long long)H, (long long)S, (long long)D, (long long)block);
-  if (D != kAttnDim || block != kAttnBlock)
-    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: only head dimension %d and %d x %d mask blocks are built "
-                "(got D=%lld block=%lld)", fn, kAttnDim, kAttnBlock, kAttnBlock, (long long)D,
+  if ((D != 32 && D != 64 && D != 128) || block != kAttnBlock)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: only head dimensions 32, 64 and 128 and %d x %d mask "
+                "blocks are built (got D=%lld block=%lld)", fn, kAttnBlock, kAttnBlock, (long long)D,
                 (long long)block);
   if (S % kAttnBlock != 0)
     return fail(SCORCH_HIP_EINVAL, "%s: S=%lld is not a multiple of the block size", fn, (long long)S);
@@ -294,16 +363,50 @@ extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D,
   hipStream_t s = static_cast<hipStream_t>(stream);
   const __bf16 *q = static_cast<const __bf16 *>(Q), *k = static_cast<const __bf16 *>(K),
                *v = static_cast<const __bf16 *>(V);
+  __bf16 *o = static_cast<__bf16 *>(O);
+  const unsigned long long *masks = reinterpret_cast<const unsigned long long *>(block_masks);
   mark_launch(s);
-  if (scale < 0.0f)
-    attn_blocksparse_kernel<true><<<grid, kBlockThreads, 0, s>>>(
-        (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
-        static_cast<__bf16 *>(O));
+  if (D == 32)
+    attn_launch_dim<32>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
+                        block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
+  else if (D == 64)
+    attn_launch_dim<64>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
+                        block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
   else
-    attn_blocksparse_kernel<false><<<grid, kBlockThreads, 0, s>>>(
-        (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx, q, k, v, scale_log2e,
-        static_cast<__bf16 *>(O));
+    attn_launch_dim<128>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
+                         block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
   return SCORCH_HIP_OK;
+}
+
+}  // namespace scorch
+
+extern "C" int scorch_hip_attn_blocksparse_bf16(int64_t H, int64_t S, int64_t D, int64_t block,
+                                                int64_t n_active_blocks,
+                                                const int32_t *block_row_ptr,
+                                                const int32_t *block_col_idx, const void *Q,
+                                                const void *K, const void *V, float scale, void *O,
+                                                void *stream) {
+  return scorch::attn_entry("scorch_hip_attn_blocksparse_bf16", H, S, D, block, n_active_blocks,
+                            block_row_ptr, block_col_idx, nullptr, nullptr, Q, K, V, scale, O,
+                            stream);
+}
+
+extern "C" int scorch_hip_attn_blocksparse_masked_bf16(
+    int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks,
+    const int32_t *block_row_ptr, const int32_t *block_col_idx, const int32_t *block_mask_index,
+    int64_t n_masks, const uint64_t *block_masks, const void *Q, const void *K, const void *V,
+    float scale, void *O, void *stream) {
+  using namespace scorch;
+  const char *fn = "scorch_hip_attn_blocksparse_masked_bf16";
+  if (n_masks < 0) return fail(SCORCH_HIP_EINVAL, "%s: n_masks=%lld", fn, (long long)n_masks);
+  if (n_active_blocks > 0 && H > 0 && S > 0) {
+    SCORCH_REQUIRE(block_mask_index != nullptr, "%s: block_mask_index is NULL", fn);
+    SCORCH_REQUIRE(n_masks == 0 || block_masks != nullptr, "%s: block_masks is NULL", fn);
+    SCORCH_REQUIRE(aligned_to(block_masks, 8), "%s: block_masks must be 8-byte aligned", fn);
+  }
+  return attn_entry(fn, H, S, D, block, n_active_blocks, block_row_ptr, block_col_idx,
+                    n_active_blocks > 0 ? block_mask_index : nullptr, block_masks, Q, K, V, scale,
+                    O, stream);
 }

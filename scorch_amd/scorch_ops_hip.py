@@ -845,12 +845,111 @@ def sparse_attention_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, q: torch.
     return spmm_csr_float_batched([S, S], mask, probs, v)
 
 
+class BlockMask:
+    """A CSR attention mask regrouped into 64 x 64 blocks for the fused attention kernel: the block
+    pattern in CSR form, and for every active block either -1 (all 4096 entries live) or the index
+    of its 64-word bit mask (bit j of word r: query r of the block row attends to key j of the
+    block).  Blocks with equal masks share one."""
+    __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz")
+
+    def __init__(self, S, block, block_row_ptr, block_col_idx, block_mask_index, block_masks, nnz):
+        self.S, self.block, self.nnz = S, block, nnz
+        self.block_row_ptr, self.block_col_idx = block_row_ptr, block_col_idx
+        self.block_mask_index, self.block_masks = block_mask_index, block_masks
+
+    @property
+    def n_active_blocks(self) -> int:
+        return int(self.block_col_idx.numel())
+
+    @property
+    def n_masks(self) -> int:
+        return int(self.block_masks.numel()) // self.block
+
+    @property
+    def density_in_blocks(self) -> float:
+        """Share of the entries of the active blocks that are live: the fused kernel computes whole
+        blocks, so 1 / this is its overhead over the mask's own entry count."""
+        return self.nnz / max(1, self.n_active_blocks * self.block * self.block)
+
+
+def block_mask_from_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -> BlockMask:
+    """Regroup an S x S CSR mask (S a multiple of 64) into a BlockMask, with torch operations on
+    the device the mask lives on.  Done once per mask (see attention_block_mask for the cached
+    form); duplicate entries are tolerated."""
+    block = 64
+    if S % block:
+        raise ValueError("scorch_ops_hip: S must be a multiple of 64")
+    dev = row_ptr.device
+    nb = S // block
+    rp = row_ptr.to(torch.int64)
+    if rp.numel() != S + 1:
+        raise ValueError("scorch_ops_hip: row_ptr length does not match S")
+    cols = col_idx.to(torch.int64)
+    rows = torch.repeat_interleave(torch.arange(S, device=dev, dtype=torch.int64), rp[1:] - rp[:-1])
+    if rows.numel() != cols.numel():
+        raise ValueError("scorch_ops_hip: row_ptr does not describe col_idx")
+    if cols.numel() and (int(cols.min()) < 0 or int(cols.max()) >= S):
+        raise ValueError("scorch_ops_hip: column index out of range")
+    entry = torch.unique((rows // block * nb + cols // block) * (block * block) + rows % block * block + cols % block)
+    nnz = int(entry.numel())
+    blocks, block_of = torch.unique(entry // (block * block), return_inverse=True)  # sorted: block row major
+    n_active = int(blocks.numel())
+    words = torch.zeros(n_active * block, dtype=torch.int64, device=dev)
+    within = entry % (block * block)
+    # distinct bits: the sum is the union (1 << 63 wraps to the sign bit, as it should)
+    words.index_add_(0, block_of * block + within // block, torch.ones_like(within) << (within % block))
+    words = words.view(n_active, block)
+    full = (words == -1).all(dim=1)
+    mask_index = torch.full((n_active,), -1, dtype=torch.int32, device=dev)
+    partial = torch.nonzero(~full).flatten()
+    if partial.numel():
+        masks, which = torch.unique(words[partial], dim=0, return_inverse=True)
+        mask_index[partial] = which.to(torch.int32)
+    else:
+        masks = torch.zeros((0, block), dtype=torch.int64, device=dev)
+    block_row_ptr = torch.zeros(nb + 1, dtype=torch.int64, device=dev)
+    block_row_ptr[1:] = torch.cumsum(torch.bincount(blocks // nb, minlength=nb), 0)
+    return BlockMask(S, block, block_row_ptr.to(torch.int32), (blocks % nb).to(torch.int32), mask_index,
+                     masks.contiguous().view(-1), nnz)
+
+
+def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -> BlockMask:
+    """block_mask_from_csr, kept with the mask's row_ptr tensor and rebuilt when either index
+    array is replaced or written to."""
+    key = (row_ptr.data_ptr(), row_ptr._version, col_idx.data_ptr(), col_idx._version, int(col_idx.numel()), S)
+    cached = getattr(row_ptr, "_scorch_block_mask", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    bm = block_mask_from_csr(row_ptr, col_idx, S)
+    try:
+        row_ptr._scorch_block_mask = (key, bm)
+    except AttributeError:
+        pass
+    return bm
+
+
+def sparse_attention_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_ptr: torch.Tensor,
+                          col_idx: torch.Tensor, scale: float) -> torch.Tensor:
+    """softmax(scale * q k^T restricted to a CSR mask) v for bf16 q, k, v of shape (H, S, D), D in
+    {32, 64, 128}, S a multiple of 64, in one fused kernel: the mask is regrouped into 64 x 64
+    blocks with bit masks once (attention_block_mask) and the kernel computes every block that
+    holds an entry.  Same result as sparse_attention_csr up to bf16 rounding of the operands, the
+    probabilities and the result."""
+    bm = attention_block_mask(row_ptr, col_idx, int(q.shape[1]))
+    return attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, scale, block=bm.block,
+                                 block_mask_index=bm.block_mask_index, block_masks=bm.block_masks)
+
+
 def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,
-                          block_col_idx: torch.Tensor, scale: float, block: int = 64) -> torch.Tensor:
+                          block_col_idx: torch.Tensor, scale: float, block: int = 64,
+                          block_mask_index: Optional[torch.Tensor] = None,
+                          block_masks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """softmax(scale * q k^T over a block mask) v for q, k, v of shape (H, S, D),
     bf16, in one kernel; fp32 accumulation, bf16 result.  The fused form of the
     per-head SDDMM -> softmax -> SpMM pipeline of
-    bench/bench_sparse_transformer.py:354-372."""
+    bench/bench_sparse_transformer.py:354-372.  With block_mask_index (int32 per active block, -1
+    = fully live) and block_masks (int64, 64 words per mask) a block is restricted to the entries
+    its bit mask names."""
     for name, t in (("q", q), ("k", k), ("v", v)):
         if t.dtype != torch.bfloat16 or t.dim() != 3:
             raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
@@ -863,10 +962,35 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     if brp.numel() != S // block + 1:
         raise ValueError("scorch_ops_hip: block_row_ptr length does not match S / block")
     out = torch.empty_like(q)
+    if block_mask_index is None:
+        with _on_device(dev):
+            rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),
+                                                               bci.data_ptr(), q.data_ptr(), k.data_ptr(),
+                                                               v.data_ptr(), float(scale), out.data_ptr(),
+                                                               _stream(dev))
+        native.check(rc)
+        return out
+    bmi = _index(block_mask_index, "block_mask_index")
+    if block_masks is None or block_masks.dtype != torch.int64 or not block_masks.is_contiguous():
+        raise TypeError("scorch_ops_hip: block_masks must be a contiguous int64 tensor")
+    if bmi.numel() != bci.numel():
+        raise ValueError("scorch_ops_hip: block_mask_index must have one entry per active block")
+    if block_masks.numel() % block or block_masks.device != q.device or bmi.device != q.device:
+        raise ValueError("scorch_ops_hip: block_masks must hold 64 words per mask on the operands' device")
+    n_masks = block_masks.numel() // block
+    # the kernel trusts the mask indices as it trusts block_col_idx; a caller that built them by
+    # hand gets them checked here, once per index tensor
+    if getattr(bmi, "_scorch_mask_checked", None) != (bmi._version, n_masks):
+        if bmi.numel() and int(bmi.max()) >= n_masks:
+            raise ValueError("scorch_ops_hip: block_mask_index names a mask beyond block_masks")
+        try:
+            bmi._scorch_mask_checked = (bmi._version, n_masks)
+        except AttributeError:
+            pass
     with _on_device(dev):
-        rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),
-                                                           bci.data_ptr(), q.data_ptr(), k.data_ptr(),
-                                                           v.data_ptr(), float(scale), out.data_ptr(),
-                                                           _stream(dev))
+        rc = native.lib().scorch_hip_attn_blocksparse_masked_bf16(
+            H, S, D, block, bci.numel(), brp.data_ptr(), bci.data_ptr(), bmi.data_ptr(), n_masks,
+            block_masks.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), out.data_ptr(),
+            _stream(dev))
     native.check(rc)
     return out

@@ -154,7 +154,7 @@ def test_attention_rejects_unsupported_shapes(L):
     def call(H=2, S=128, D=64, block=64, nblk=3, brp=FAKE, bci=FAKE, q=FAKE, k=FAKE, v=FAKE, o=FAKE):
         return f(H, S, D, block, nblk, brp, bci, q, k, v, 0.125, o, NULL)
 
-    assert call(D=128) == native.EUNSUPPORTED
+    assert call(D=96) == native.EUNSUPPORTED
     assert b"head dimension" in L.scorch_hip_last_error()
     assert call(block=32) == native.EUNSUPPORTED
     assert call(S=100) == native.EINVAL
@@ -163,6 +163,18 @@ def test_attention_rejects_unsupported_shapes(L):
     assert call(q=NULL) == native.EINVAL
     assert call(o=ctypes.c_void_p(0x1008)) == native.EINVAL      # not 16-byte aligned
     assert call(H=0, q=NULL, k=NULL, v=NULL, o=NULL) == native.OK
+
+    g = L.scorch_hip_attn_blocksparse_masked_bf16
+
+    def masked(D=32, nblk=3, bmi=FAKE, n_masks=1, masks=FAKE, q=FAKE):
+        return g(2, 128, D, 64, nblk, FAKE, FAKE, bmi, n_masks, masks, q, FAKE, FAKE, 0.125, FAKE, NULL)
+
+    assert masked(D=48) == native.EUNSUPPORTED
+    assert masked(bmi=NULL) == native.EINVAL
+    assert masked(masks=NULL) == native.EINVAL
+    assert masked(masks=ctypes.c_void_p(0x1004)) == native.EINVAL  # not 8-byte aligned
+    assert masked(n_masks=-1) == native.EINVAL
+    assert masked(q=NULL) == native.EINVAL
 
 
 def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):

@@ -141,3 +141,120 @@ def test_short_and_odd_block_rows(oracle, blocks_per_row):
     ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
                                             brp, bci, 64, 0.125)
     assert oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+# ---- other head dimensions, and masks that are not unions of whole blocks ----
+
+@pytest.mark.parametrize("D", [32, 128])
+@pytest.mark.parametrize("S,heads,seed", [(64, 1, 10), (512, 3, 11)])
+def test_other_head_dimensions(oracle, D, S, heads, seed):
+    w, q, k, v = bf16_inputs(S, heads, D, seed)
+    out = run_fused(w, q, k, v).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            w["block_row_ptr"], w["block_col_idx"], 64, float(w["scale"]))
+    assert oracle.rel_fro(out, ref) <= 5e-3
+
+
+def csr_of(mask_bool):
+    rp = np.concatenate([[0], np.cumsum(mask_bool.sum(1))]).astype(np.int32)
+    return rp, np.nonzero(mask_bool)[1].astype(np.int32)
+
+
+def masked_case(oracle, mask_bool, heads, D, seed, scale=None):
+    S = mask_bool.shape[0]
+    rng = np.random.default_rng(seed)
+    q, k, v = (torch.from_numpy(rng.standard_normal((heads, S, D)).astype(np.float32)).to(torch.bfloat16)
+               for _ in range(3))
+    scale = D ** -0.5 if scale is None else scale
+    rp, ci = csr_of(mask_bool)
+    out = H.sparse_attention_bf16(q.cuda(), k.cuda(), v.cuda(), dev(rp), dev(ci), scale).float().cpu().numpy()
+    ref = np.stack([oracle.attention_dense_fp64(q[h].float().numpy(), k[h].float().numpy(),
+                                                v[h].float().numpy(), mask_bool, scale) for h in range(heads)])
+    return out, ref
+
+
+def test_block_mask_regrouping_of_a_csr_mask():
+    """The block structure built from a CSR mask: every entry in exactly its block's bit mask,
+    full blocks marked -1, equal masks shared."""
+    S = 256
+    rng = np.random.default_rng(20)
+    mask = rng.random((S, S)) < 0.02
+    mask[64:128, 128:192] = True                       # a full block
+    mask[192:256, :] = False                           # an empty block row
+    mask[0:64, 0:64] = np.tri(64, dtype=bool)          # two equal partial blocks
+    mask[128:192, 64:128] = np.tri(64, dtype=bool)
+    rp, ci = csr_of(mask)
+    bm = H.block_mask_from_csr(dev(rp), dev(ci), S)
+    brp, bci, bmi = (t.cpu().numpy() for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index))
+    words = bm.block_masks.cpu().numpy().view(np.uint64).reshape(-1, 64)
+    assert bm.nnz == int(mask.sum()) and brp[-1] == bci.size and brp[4] == brp[3]
+    rebuilt = np.zeros_like(mask)
+    for br in range(4):
+        for i in range(brp[br], brp[br + 1]):
+            bits = (np.full((64, 64), True) if bmi[i] < 0 else
+                    ((words[bmi[i]][:, None] >> np.arange(64, dtype=np.uint64)[None, :]) & np.uint64(1)).astype(bool))
+            rebuilt[64 * br:64 * br + 64, 64 * bci[i]:64 * bci[i] + 64] = bits
+    assert np.array_equal(rebuilt, mask)
+    at = {(br, int(bci[i])): int(bmi[i]) for br in range(4) for i in range(brp[br], brp[br + 1])}
+    assert at[(1, 2)] == -1 and at[(0, 0)] == at[(2, 1)] >= 0
+    assert bm.n_masks < bci.size
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_random_entry_mask(oracle, D):
+    S = 256
+    rng = np.random.default_rng(21 + D)
+    mask = rng.random((S, S)) < 0.1
+    mask[7, :] = False                                 # a query without keys inside active blocks
+    mask[64:128, :] = False                            # an empty block row
+    mask[130, :] = False
+    mask[130, 255] = True                              # one key only (bit 63 of its word)
+    out, ref = masked_case(oracle, mask, 2, D, 22)
+    assert not out[:, 7].any() and not out[:, 64:128].any()
+    assert oracle.rel_fro(out, ref) <= 5e-3
+
+
+@pytest.mark.parametrize("D", [32, 64])
+def test_causal_mask(oracle, D):
+    S = 512
+    out, ref = masked_case(oracle, np.tri(S, dtype=bool), 2, D, 23)
+    assert oracle.rel_fro(out, ref) <= 5e-3
+
+
+def test_masked_negative_scale_and_large_scores(oracle):
+    S = 256
+    rng = np.random.default_rng(24)
+    mask = rng.random((S, S)) < 0.3
+    out, ref = masked_case(oracle, mask, 1, 32, 25, scale=-3.0)
+    assert np.isfinite(out).all() and oracle.rel_fro(out, ref) <= TOL_BF16
+    out, ref = masked_case(oracle, mask, 1, 32, 26, scale=4.0)
+    assert np.isfinite(out).all() and oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+def test_longformer_mask_reference_shape(oracle):
+    """The reference's attention benchmark at its own shape (bench/bench_sparse_transformer.py:117-141,
+    README: S = 4096, 8 heads, D = 32, window 64 + one global token, 532,286 entries): every head
+    against the dense masked softmax in fp64 on the device, and against the fp32 three-launch form."""
+    S, heads, D = 4096, 8, 32
+    rp, ci = workloads.longformer_mask(S)
+    assert ci.size == 532286
+    rng = np.random.default_rng(27)
+    q, k, v = (torch.from_numpy(rng.standard_normal((heads, S, D)).astype(np.float32)).to(torch.bfloat16).cuda()
+               for _ in range(3))
+    scale = D ** -0.5
+    drp, dci = dev(rp), dev(ci)
+    out = H.sparse_attention_bf16(q, k, v, drp, dci, scale)
+    assert torch.equal(out, H.sparse_attention_bf16(q, k, v, drp, dci, scale))      # cached plan, same bits
+    dense = torch.zeros(S, S, dtype=torch.bool)
+    dense[torch.from_numpy(np.repeat(np.arange(S), np.diff(rp))), torch.from_numpy(ci).long()] = True
+    dense = dense.cuda()
+    worst = 0.0
+    for h in range(heads):
+        s = (q[h].double() @ k[h].double().T) * scale
+        s.masked_fill_(~dense, float("-inf"))
+        ref = torch.softmax(s, dim=-1) @ v[h].double()
+        worst = max(worst, (torch.linalg.norm(out[h].double() - ref) / torch.linalg.norm(ref)).item())
+    assert worst <= TOL_BF16, worst
+    unfused = H.sparse_attention_csr(drp, dci, q.float(), k.float(), v.float(), scale)
+    err = (torch.linalg.norm(out.float() - unfused) / torch.linalg.norm(unfused)).item()
+    assert err <= TOL_BF16
