@@ -46,13 +46,28 @@ CONFIG_WORKLOADS = ("spmm_uniform", "sddmm_uniform", "attention_blocksparse", "s
 # Measured constants: valid for the default sizes and for the kernels as they
 # stood at the named commit only (null for anything else); the summaries with
 # the commands are the named files.
+# bytes = FETCH_SIZE [KiB] x 1024 x 2.0 + WRITE_SIZE [KiB] x 1024 of the dominant kernel, the factors
+# being what the same counters read for a copy of known size (profiles/copy_calibration.md).
 MEASURED_TRAFFIC = {
-    # filled in from the profiles named; see profiles/*.md
+    ("gcn_powerlaw", "merge"): {"bytes": 9_795_510_000, "commit": "4fe4dfe",
+                                "profile": "profiles/spmm_merge_kernel_gcn_powerlaw.md"},
+    ("spmm_uniform", "rows"): {"bytes": 10_820_000, "commit": "4fe4dfe",
+                               "profile": "profiles/spmm_rows_kernel_uniform_4096.md"},
+    ("sae_decoder", "tiled"): {"bytes": 696_340_000, "commit": "4fe4dfe",
+                               "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
+    ("sae_decoder", "merge"): {"bytes": 1_779_270_000, "commit": "4fe4dfe",
+                               "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
+    ("sddmm_uniform", "listed"): {"bytes": 515_470_000, "commit": "4fe4dfe",
+                                  "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("sddmm_uniform", "plain"): {"bytes": 897_790_000, "commit": "4fe4dfe",
+                                 "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "commit": "4fe4dfe",
+                                         "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
 }
 
 
-def measured_traffic(name, default_size):
-    rec = MEASURED_TRAFFIC.get(name)
+def measured_traffic(name, path, default_size):
+    rec = MEASURED_TRAFFIC.get((name, path))
     if rec is None or not default_size:
         return None, None
     return rec["bytes"], {"commit": rec["commit"], "profile": rec["profile"]}
@@ -251,6 +266,9 @@ def _hbm_roofline(kernel, kernel_ms, algo, traffic, provenance, extra=None):
            "kernel_ms_avg": round(kernel_ms, 5)}
     if provenance:
         out["traffic_measured_at"] = provenance
+        # what the memory system moved per second for this kernel: the distance to the HBM peak that
+        # remains once the re-reads the access pattern forces are counted
+        out["traffic_gbps"] = round(traffic / (kernel_ms * 1e-3) / 1e9, 1)
     if extra:
         out.update(extra)
     return out
@@ -318,7 +336,7 @@ def run_spmm(name, args, headline=False):
 
     flops = 2.0 * nnz * N
     algo, gather = spmm_algorithmic_bytes(M, K, N, nnz), spmm_gather_bytes(M, N, nnz)
-    traffic, provenance = measured_traffic(name, default_size)
+    traffic, provenance = measured_traffic(name, path, default_size)
     rec = {
         "metric": "CSR SpMM GFLOP/s + HBM GB/s (% peak), power-law 1M rows, N=128 fp32" if headline
                   else "CSR SpMM GFLOP/s",
@@ -385,14 +403,17 @@ def run_sddmm(args):
     # also writes the result's row coordinates, 4 more bytes per entry (not counted)
     algo = 4 * (M + 1) + 4 * nnz * 3 + 4 * M * K + 4 * n_cols * K
     gather = algo - 4 * n_cols * K + 4 * nnz * K
-    traffic, provenance = measured_traffic("sddmm_uniform", True)
+    plan = getattr(pos, "_scorch_plan", None)
+    listed = plan is not None and plan.sddmm_lists is not None
+    traffic, provenance = measured_traffic("sddmm_uniform", "listed" if listed else "plain", True)
     rec = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
            "ms_per_step_coo_mask": round(ms_coo, 5), "higher_is_better": True, "dtype": "f32", "data": "synthetic",
            "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K,
                       "seed": workloads.SEEDS["sddmm_uniform"]},
            "warmup_ms": warm,
-           "roofline": _hbm_roofline("sddmm_kernel<16,4,false,false>", ms, algo, traffic, provenance,
+           "path": "listed" if listed else "plain",
+           "roofline": _hbm_roofline("sddmm_listed_kernel<16,4>" if listed else "sddmm_kernel<16,4,false,false>", ms, algo, traffic, provenance,
                                      {"row_coordinate_output_bytes": 4 * nnz, "gather_model_bytes": gather,
                                       "gather_model_gbps": round(gather / ms / 1e6, 1)})}
     if args.vendor:
@@ -422,7 +443,7 @@ def run_attention(args):
     flops = 4.0 * nnz * D * Hh
     algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
     achieved = flops / ms / 1e9
-    traffic, provenance = measured_traffic("attention_blocksparse", True)
+    traffic, provenance = measured_traffic("attention_blocksparse", "fused", True)
     rec = {"metric": "fused block-sparse attention TFLOP/s", "value": round(achieved, 2), "unit": "TFLOP/s",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
            "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
@@ -541,6 +562,17 @@ def run_extra(args):
             out["vendor_library"] = _vendor_time("torch.sparse.mm in the same forward pass", vendor,
                                                  max(args.steps // 2, 2), 1)
         return out
+    if args.workload == "copy_calibration":
+        # 1 GiB read and 1 GiB written by a plain elementwise kernel: what the memory counters
+        # (FETCH_SIZE, WRITE_SIZE) read for a known amount of traffic gives the factor by which the
+        # counters of the other workloads are scaled.
+        n = 1 << 28
+        x = torch.ones(n, device="cuda")
+        y = torch.empty_like(x)
+        ms = _time_steps(lambda: torch.mul(x, 2.0, out=y), args.steps, args.warmup)
+        return {"metric": "copy GB/s (read + write)", "value": round(8.0 * n / ms / 1e6, 1), "unit": "GB/s",
+                "ms_per_step": round(ms, 4), **base,
+                "config": {"workload": "copy_calibration", "bytes_read": 4 * n, "bytes_written": 4 * n}}
     if args.workload == "attention_longformer":
         # The reference's sparse-transformer benchmark shape (bench/bench_sparse_transformer.py:49-60,
         # 194-209): embedding 256 in 8 heads (head dimension 32), Longformer mask with a window of 64 on
@@ -667,7 +699,7 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true", help="skip the records of the other four configurations")
     ap.add_argument("--workload", default=None,
                     choices=[HEADLINE, *CONFIG_WORKLOADS, "spgemm_powerlaw", "spmv_powerlaw", "softmax_powerlaw",
-                             "softmax_rows", "gcn_forward", "attention_longformer"],
+                             "softmax_rows", "gcn_forward", "attention_longformer", "copy_calibration"],
                     help="print this workload's record alone (default: the headline line with all configurations)")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch's own sparse routine on the same operands")
