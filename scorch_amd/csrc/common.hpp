@@ -94,6 +94,18 @@ template <> struct Acc<int64_t> { using type = uint64_t; };
 // ---- device helpers ---------------------------------------------------------
 template <typename T, int V> struct alignas(sizeof(T) * V) Vec { T v[V]; };
 
+// A store marked as streaming: data that nothing reads again, which should not push out of the
+// L2 what other accesses of the same kernel come back to.
+template <typename T>
+__device__ __forceinline__ void store_streaming(T *p, T x) {
+  __builtin_nontemporal_store(x, p);
+}
+template <typename T, int V>
+__device__ __forceinline__ void store_streaming(T *p, const Vec<T, V> &x) {
+  typedef T Native __attribute__((ext_vector_type(V)));
+  __builtin_nontemporal_store(__builtin_bit_cast(Native, x), reinterpret_cast<Native *>(p));
+}
+
 __device__ __forceinline__ int wave_lane() { return threadIdx.x & (kWaveSize - 1); }
 
 // Value of lane 0's copy in a scalar register: tells the compiler a value is

@@ -345,8 +345,11 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
         }
       }
       if (valid) {
-        out_vals[pos] = scale * mine;
-        if (out_row_idx) out_row_idx[pos] = row;
+        // The results are scattered 4-byte writes that nothing reads again: marked as streaming
+        // they do not take L2 lines from the XCD's part of B (8 % faster at 65,536^2; the same
+        // mark on the loads of the lists or of A made the kernel slower).
+        store_streaming(out_vals + pos, scale * mine);
+        if (out_row_idx) store_streaming(out_row_idx + pos, row);
       }
     }
   }

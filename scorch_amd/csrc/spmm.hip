@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 #pragma unroll
       for (int v = 0; v < VEC; ++v)
         o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
-      *reinterpret_cast<VecT *>(C + (size_t)x * (size_t)N + col0) = o;
+      store_streaming(C + (size_t)x * (size_t)N + col0, o);
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_grouped_kernel(
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
           o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
-        *reinterpret_cast<VecT *>(C + (size_t)(x0 + slot) * (size_t)N + col0) = o;
+        store_streaming(C + (size_t)(x0 + slot) * (size_t)N + col0, o);
       } else if (len > 0) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) o.v[v] = (T)acc[v];

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_rows_kernel(
       if (relu) r = r > (T)0 ? r : (T)0;
       o.v[v] = r;
     }
-    *reinterpret_cast<VecT *>(C + (size_t)row * (size_t)N + col0) = o;
+    store_streaming(C + (size_t)row * (size_t)N + col0, o);
   }
 }
 

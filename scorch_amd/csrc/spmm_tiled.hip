@@ -40,9 +40,10 @@ constexpr int kTiledBatch = 8;                 // tile-row loads in flight per l
 constexpr int kTiledMaxWorkgroupsPerXcd = 256; // 32 CUs x 8 workgroups
 constexpr int kPacePolls = 400;                // polls after which a wavefront stops waiting for the others
 // Share of an XCD's workgroups that must have finished a tile before the next is begun.  On the
-// decoder shape (4096 x 16384, 32 per row, N = 4096): no pacing 0.158 ms and 0.93 GB fetched; 75 %
-// 0.155 ms, 0.65 GB; 90 % 0.165 ms, 0.45 GB; 100 % 0.258 ms, 0.28 GB (the slice comes in once, but
-// every tile waits for its slowest workgroup).
+// decoder shape (4096 x 16384, 32 per row, N = 4096), with C written by streaming stores: no
+// pacing 0.146 ms; 50 to 80 % 0.135 - 0.137 ms; 90 % 0.141 ms; 95 % 0.150 ms (the slice comes in
+// fewer times, but every tile waits for its slowest workgroups).  Of the flat range the upper end
+// fetches least.
 constexpr int kPacePercent = 80;
 constexpr int kTiledPacedWorkgroupsPerXcd = 160;  // 32 CUs x 5 workgroups surely resident together
 
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
             for (int v = 0; v < VEC; ++v)
               o.v[v] = partial ? (T)acc[v] : apply_epilogue<T, EPI>(acc[v], bias_v[v]);
             if (vector_stores) {
-              *reinterpret_cast<VecT *>(dst) = o;
+              store_streaming(dst, o);  // C passes through once; the L2 is for the slice of B
             } else {
 #pragma unroll
               for (int v = 0; v < VEC; ++v)
