@@ -94,6 +94,32 @@ template <> struct Acc<int64_t> { using type = uint64_t; };
 // ---- device helpers ---------------------------------------------------------
 template <typename T, int V> struct alignas(sizeof(T) * V) Vec { T v[V]; };
 
+// Sum over the GS lanes of a group (GS a power of two, groups aligned), every lane receiving the
+// total, with the pairing x(i) + x(i ^ off) for off = GS / 2 down to 1.  Within a row of 16 lanes
+// the exchanges are row rotations carried by the add itself (DPP): once the steps above have made
+// the values periodic with period 2 off, lane (i + off) mod 16 holds what lane i ^ off holds.  A
+// shuffle instead goes through the LDS pipe and has to be waited for.  Groups below 16 lanes share
+// a row with other groups and keep the shuffles.
+template <int N>
+__device__ __forceinline__ float row_rotated(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + N, 0xf, 0xf, false));
+}
+template <int GS>
+__device__ __forceinline__ float group_sum(float x) {
+  if constexpr (GS >= 16) {
+#pragma unroll
+    for (int off = GS / 2; off >= 16; off >>= 1) x += __shfl_xor(x, off);
+    x += row_rotated<8>(x);
+    x += row_rotated<4>(x);
+    x += row_rotated<2>(x);
+    x += row_rotated<1>(x);
+  } else {
+#pragma unroll
+    for (int off = GS / 2; off > 0; off >>= 1) x += __shfl_xor(x, off);
+  }
+  return x;
+}
+
 // A store marked as streaming: data that nothing reads again, which should not push out of the
 // L2 what other accesses of the same kernel come back to.
 template <typename T>

@@ -114,8 +114,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
             for (int v = 0; v < VEC; ++v) dot += av[u].v[v] * bv[u].v[v];
         }
       }
-#pragma unroll
-      for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+      dot = group_sum<GS>(dot);
       if (t == s) mine = dot;
     }
 
@@ -320,8 +319,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
 #pragma unroll
             for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
           }
-#pragma unroll
-          for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+          dot = group_sum<GS>(dot);
           if (t == s) mine = dot;
         }
       } else {
@@ -339,8 +337,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
 #pragma unroll
             for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
           }
-#pragma unroll
-          for (int off = GS / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+          dot = group_sum<GS>(dot);
           if (t == s) mine = dot;
         }
       }
