@@ -82,10 +82,7 @@ struct AttnTile {
   static constexpr int kRowsPerLoad = 1024 / kRowBytes;     // rows one wavefront load instruction fills
   static constexpr int kLoadsPerWave = 16 / kRowsPerLoad;   // a wavefront fills 16 rows of a tile
   __device__ static __forceinline__ int swizzle(int row) { return D == 32 ? (row >> 1) & 3 : row & 7; }
-  // Wavefronts per SIMD the kernel is compiled for.  Stating it bounds the register budget at
-  // 512 / this, and with a budget of 256 or fewer the compiler keeps MFMA accumulators in ordinary
-  // vector registers; left to assume 512 registers it puts them in accumulation registers and
-  // copies all of them out and back around the softmax of every key block.
+  // Wavefronts per SIMD the kernel is compiled for: the register budget is 512 / this.
   static constexpr int kWavesPerSimd = D == 128 ? 2 : 4;
 };
 
