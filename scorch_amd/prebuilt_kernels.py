@@ -5,9 +5,10 @@ The table below is the reference's (:37-93): (lhs rank, rhs rank, lhs format,
 rhs format, output format) -> candidate symbol names per dtype, tried in
 order.  What differs is the module the symbols are looked up in: the
 reference looks in its pybind module ``scorch_ops``; here operands live on a
-HIP device and the symbols come from ``scorch_ops_hip``.  Families that module
-does not provide (CSR x CSR, COO x COO, COO x dense) resolve to ``None``, as
-they would in a reference build that lacked those symbols.
+HIP device and the symbols come from ``scorch_ops_hip``, which provides every
+family of the table (CSR x dense, CSR x CSR, COO x dense, COO x COO and the
+matrix-vector products); a symbol that a module lacks resolves to ``None``,
+as it does in the reference.
 """
 from __future__ import annotations
 
