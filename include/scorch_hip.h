@@ -430,6 +430,25 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_masked_bf16(
     int64_t n_masks, const uint64_t *block_masks, const void *Q, const void *K, const void *V,
     float scale, void *O, void *stream);
 
+/* The same with long block rows shared out among workgroups (a mask with a global token has a
+ * block row that holds every key block: as one workgroup's work it sets the time of the whole
+ * launch).  The work is a list of items, longest first, 4 int32 each (16-byte aligned): block row,
+ * begin and end of its stretch within block_col_idx, and the slot its partial result goes to, or
+ * -1 for a whole block row, which writes O itself.  The stretches of a shared-out row have
+ * consecutive slots; split_rows lists those rows, 4 int32 each: block row, first slot, number of
+ * stretches, 0.  Partial results (unnormalised sums, reference maximum, row sum per query) go
+ * through `workspace` (256-byte aligned, scorch_hip_attn_blocksparse_split_workspace_bytes(H,
+ * n_slots, D) bytes; not to be shared by calls that may overlap in time) and a second kernel
+ * combines them.  block_mask_index may be NULL (every block fully live).  No counterpart in the
+ * reference, like the two entry points above. */
+SCORCH_HIP_API size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, int64_t n_slots, int64_t D);
+SCORCH_HIP_API int scorch_hip_attn_blocksparse_split_bf16(
+    int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
+    const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
+    const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
+    const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
+    void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's
  * sparse attention -- SDDMM, row softmax, SpMM, which its benchmark runs head by

@@ -93,7 +93,8 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     const int *__restrict__ block_col_idx, const int *__restrict__ block_mask_index,
     const unsigned long long *__restrict__ block_masks, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
-    __bf16 *__restrict__ O) {
+    __bf16 *__restrict__ O, int n_items, const int4 *__restrict__ items, int n_slots,
+    float *__restrict__ partials) {
   using Tile = AttnTile<D>;
   constexpr int kTileBytes = Tile::kBytes;
   constexpr int kRowBytes = Tile::kRowBytes;
@@ -123,14 +124,28 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     const int id = blockIdx.x;
     if (n_heads % 8 == 0) {
       const int xcd = id & 7, slot = id >> 3;
-      head = xcd + 8 * (slot / n_blocks);
-      rank = slot % n_blocks;
+      head = xcd + 8 * (slot / n_items);
+      rank = slot % n_items;
     } else {
-      head = id / n_blocks;
-      rank = id % n_blocks;
+      head = id / n_items;
+      rank = id % n_items;
     }
   }
-  const int qb = n_blocks - 1 - rank;  // longest block rows first
+  // A workgroup's work item is a block row, or -- when `items` is given -- a stretch of a block
+  // row's key blocks (x: block row, y and z: the stretch within block_col_idx, w: where its
+  // partial result goes, or -1 for a whole row that writes O itself).  Items come longest first.
+  int qb, kb_begin, kb_end, part_slot = -1;
+  if (items) {
+    const int4 item = items[rank];
+    qb = uniform(item.x);
+    kb_begin = uniform(item.y);
+    kb_end = uniform(item.z);
+    part_slot = uniform(item.w);
+  } else {
+    qb = n_blocks - 1 - rank;  // (masks with longer block rows further down: longest first)
+    kb_begin = block_row_ptr[qb];
+    kb_end = block_row_ptr[qb + 1];
+  }
   const size_t head_off = (size_t)head * (size_t)S * D;
   const __bf16 *Qh = Q + head_off;
   const unsigned char *Kb = reinterpret_cast<const unsigned char *>(K + head_off);
@@ -154,8 +169,6 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
 #pragma unroll
   for (int j = 0; j < 8; ++j) ones[j] = (__bf16)1.0f;
 
-  const int kb_begin = block_row_ptr[qb];
-  const int kb_end = block_row_ptr[qb + 1];
 
 
   // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with kLoadsPerWave instructions of
@@ -302,7 +315,19 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
   }
 
   const float l = l_acc[0];
-  const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // block rows without key blocks give zeros
+  if (part_slot >= 0) {
+    // a stretch of a block row: the unnormalised sums, the reference maximum they are relative to
+    // and the row sum go to the workspace; attn_merge_kernel combines the row's stretches
+    float *part = partials + (((size_t)head * n_slots + part_slot) * kAttnBlock + (w * 16 + n)) * (D + 4);
+#pragma unroll
+    for (int dt = 0; dt < kFeat; ++dt) *reinterpret_cast<floatx4 *>(part + 16 * dt + 4 * g) = o_acc[dt];
+    if (g == 0) {
+      part[D] = m_run;
+      part[D + 1] = l;
+    }
+    return;
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // queries without a live key give zeros
   __bf16 *out = O + head_off + (size_t)query * D;
 #pragma unroll
   for (int dt = 0; dt < kFeat; ++dt) {
@@ -310,6 +335,48 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
 #pragma unroll
     for (int r = 0; r < 4; ++r) o[r] = (__bf16)(o_acc[dt][r] * inv);
     *reinterpret_cast<bf16x4 *>(out + 16 * dt + 4 * g) = o;
+  }
+}
+
+// Combines the stretches of a block row that was shared out: with m* the largest of the
+// stretches' reference maxima (base-2 exponents), O = sum_p 2^(m_p - m*) O_p / sum_p 2^(m_p - m*) l_p.
+// One workgroup per (split row, head); thread t takes query t / 4 and a quarter of the features.
+template <int D>
+__global__ __launch_bounds__(kBlockThreads) void attn_merge_kernel(int S, int n_slots,
+                                                                   const int4 *__restrict__ split_rows,
+                                                                   const float *__restrict__ partials,
+                                                                   __bf16 *__restrict__ O) {
+  const int4 row = split_rows[blockIdx.x];  // x: block row, y: first slot, z: number of stretches
+  const int head = blockIdx.y;
+  const int q = threadIdx.x >> 2, quarter = threadIdx.x & 3;
+  constexpr int kMine = D / 4;  // features per thread
+  const float *base = partials + (((size_t)head * n_slots + row.y) * kAttnBlock + q) * (D + 4);
+  const size_t part_stride = (size_t)kAttnBlock * (D + 4);
+  float m_star = -3.0e38f;
+  for (int p = 0; p < row.z; ++p) m_star = fmaxf(m_star, base[p * part_stride + D]);
+  float acc[kMine];
+#pragma unroll
+  for (int j = 0; j < kMine; ++j) acc[j] = 0.0f;
+  float l = 0.0f;
+  for (int p = 0; p < row.z; ++p) {
+    const float *part = base + p * part_stride;
+    const float weight = __builtin_amdgcn_exp2f(part[D] - m_star);
+    l += weight * part[D + 1];
+#pragma unroll
+    for (int j = 0; j < kMine; j += 4) {
+      const floatx4 o = *reinterpret_cast<const floatx4 *>(part + quarter * kMine + j);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[j + r] += weight * o[r];
+    }
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  __bf16 *out = O + ((size_t)head * S + (size_t)row.x * kAttnBlock + q) * D + quarter * kMine;
+#pragma unroll
+  for (int j = 0; j < kMine; j += 4) {
+    bf16x4 o;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = (__bf16)(acc[j + r] * inv);
+    *reinterpret_cast<bf16x4 *>(out + j) = o;
   }
 }
 
@@ -322,11 +389,11 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
                             const int32_t *block_row_ptr, const int32_t *block_col_idx,
                             const int32_t *block_mask_index, const unsigned long long *block_masks,
                             const __bf16 *q, const __bf16 *k, const __bf16 *v, float scale_log2e,
-                            __bf16 *o) {
+                            __bf16 *o, int n_items, const int4 *items, int n_slots, float *partials) {
 #define SCORCH_ATTN_LAUNCH(NEG, MASKED)                                                          \
   attn_blocksparse_kernel<D, NEG, MASKED><<<grid, kBlockThreads, 0, s>>>(                        \
       S, n_blocks, H, block_row_ptr, block_col_idx, block_mask_index, block_masks, q, k, v,      \
-      scale_log2e, o)
+      scale_log2e, o, n_items, items, n_slots, partials)
   const bool masked = block_mask_index != nullptr;
   if (negative) {
     if (masked) SCORCH_ATTN_LAUNCH(true, true); else SCORCH_ATTN_LAUNCH(true, false);
@@ -336,13 +403,26 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
 #undef SCORCH_ATTN_LAUNCH
 }
 
-// Shared by the two entry points; block_mask_index == nullptr means every listed block is
-// fully live.
+// Block rows shared out among several workgroups (scorch_hip_attn_blocksparse_split_bf16).
+struct AttnSplit {
+  int64_t n_items = 0, n_split_rows = 0, n_slots = 0;
+  const int32_t *items = nullptr;       // 4 per item: block row, begin, end, slot (-1: writes O itself)
+  const int32_t *split_rows = nullptr;  // 4 per split row: block row, first slot, stretches, 0
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
+};
+
+inline size_t attn_split_workspace_bytes(int64_t H, int64_t n_slots, int64_t D) {
+  return (size_t)H * (size_t)n_slots * kAttnBlock * (size_t)(D + 4) * sizeof(float);
+}
+
+// Shared by the entry points; block_mask_index == nullptr means every listed block is fully
+// live, split == nullptr that every block row is one workgroup's.
 static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t block,
                       int64_t n_active_blocks, const int32_t *block_row_ptr,
                       const int32_t *block_col_idx, const int32_t *block_mask_index,
                       const uint64_t *block_masks, const void *Q, const void *K, const void *V,
-                      float scale, void *O, void *stream) {
+                      float scale, void *O, void *stream, const AttnSplit *split = nullptr) {
   if (H < 0 || S < 0 || D < 0 || block <= 0 || n_active_blocks < 0)
     return fail(SCORCH_HIP_EINVAL, "%s: negative size (H=%lld S=%lld D=%lld block=%lld)", fn,
                 (long long)H, (long long)S, (long long)D, (long long)block);
@@ -354,14 +434,35 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
     return fail(SCORCH_HIP_EINVAL, "%s: S=%lld is not a multiple of the block size", fn, (long long)S);
   if (H * (S / kAttnBlock) > INT32_MAX || S * D > INT32_MAX)
     return fail(SCORCH_HIP_EUNSUPPORTED, "%s: H=%lld or S=%lld too large", fn, (long long)H, (long long)S);
-  SCORCH_REQUIRE(block_row_ptr != nullptr, "%s: block_row_ptr is NULL", fn);
+  SCORCH_REQUIRE(split || block_row_ptr != nullptr, "%s: block_row_ptr is NULL", fn);
   if (H == 0 || S == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(n_active_blocks == 0 || block_col_idx != nullptr, "%s: block_col_idx is NULL", fn);
   SCORCH_REQUIRE(Q && K && V && O, "%s: NULL Q/K/V/O", fn);
   SCORCH_REQUIRE(aligned_to(Q, 16) && aligned_to(K, 16) && aligned_to(V, 16) && aligned_to(O, 16),
                  "%s: Q, K, V and O must be 16-byte aligned", fn);
   const int n_blocks = (int)(S / kAttnBlock);
-  const dim3 grid((unsigned)(n_blocks * H));
+  int n_items = n_blocks, n_slots = 0;
+  const int4 *items = nullptr;
+  float *partials = nullptr;
+  if (split) {
+    if (split->n_items < 0 || split->n_split_rows < 0 || split->n_slots < 0 || split->n_items * H > INT32_MAX ||
+        split->n_slots > INT32_MAX)
+      return fail(SCORCH_HIP_EINVAL, "%s: n_items=%lld n_split_rows=%lld n_slots=%lld", fn,
+                  (long long)split->n_items, (long long)split->n_split_rows, (long long)split->n_slots);
+    if (split->n_items == 0) return SCORCH_HIP_OK;
+    SCORCH_REQUIRE(split->items != nullptr && aligned_to(split->items, 16), "%s: items must be 16-byte aligned", fn);
+    SCORCH_REQUIRE(split->n_split_rows == 0 || (split->split_rows != nullptr && aligned_to(split->split_rows, 16)),
+                   "%s: split_rows must be 16-byte aligned", fn);
+    const size_t need = attn_split_workspace_bytes(H, split->n_slots, D);
+    if (need > 0 && (!split->workspace || split->workspace_bytes < need || !aligned_to(split->workspace, 256)))
+      return fail(SCORCH_HIP_EWORKSPACE, "%s: a 256-byte aligned workspace of %zu bytes is needed, %zu given", fn,
+                  need, split->workspace ? split->workspace_bytes : (size_t)0);
+    n_items = (int)split->n_items;
+    n_slots = (int)split->n_slots;
+    items = reinterpret_cast<const int4 *>(split->items);
+    partials = static_cast<float *>(split->workspace);
+  }
+  const dim3 grid((unsigned)(n_items * H));
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const __bf16 *q = static_cast<const __bf16 *>(Q), *k = static_cast<const __bf16 *>(K),
@@ -370,16 +471,25 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
   const unsigned long long *masks = reinterpret_cast<const unsigned long long *>(block_masks);
   mark_launch(s);
   if (D == 32)
-    attn_launch_dim<32>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
-                        block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
+    attn_launch_dim<32>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
   else if (D == 64)
-    attn_launch_dim<64>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
-                        block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
+    attn_launch_dim<64>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
   else
-    attn_launch_dim<128>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr,
-                         block_col_idx, block_mask_index, masks, q, k, v, scale_log2e, o);
+    attn_launch_dim<128>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
+                         block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
+  if (split && split->n_split_rows > 0) {
+    const dim3 merge_grid((unsigned)split->n_split_rows, (unsigned)H);
+    const int4 *rows = reinterpret_cast<const int4 *>(split->split_rows);
+    if (D == 32) attn_merge_kernel<32><<<merge_grid, kBlockThreads, 0, s>>>((int)S, n_slots, rows, partials, o);
+    else if (D == 64) attn_merge_kernel<64><<<merge_grid, kBlockThreads, 0, s>>>((int)S, n_slots, rows, partials, o);
+    else attn_merge_kernel<128><<<merge_grid, kBlockThreads, 0, s>>>((int)S, n_slots, rows, partials, o);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    mark_launch(s);
+  }
   return SCORCH_HIP_OK;
 }
 
@@ -412,4 +522,34 @@ extern "C" int scorch_hip_attn_blocksparse_masked_bf16(
   return attn_entry(fn, H, S, D, block, n_active_blocks, block_row_ptr, block_col_idx,
                     n_active_blocks > 0 ? block_mask_index : nullptr, block_masks, Q, K, V, scale,
                     O, stream);
+}
+
+extern "C" size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, int64_t n_slots, int64_t D) {
+  if (H <= 0 || n_slots <= 0 || D <= 0) return 0;
+  return scorch::attn_split_workspace_bytes(H, n_slots, D);
+}
+
+extern "C" int scorch_hip_attn_blocksparse_split_bf16(
+    int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
+    const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
+    const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
+    const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
+    void *workspace, size_t workspace_bytes, void *stream) {
+  using namespace scorch;
+  const char *fn = "scorch_hip_attn_blocksparse_split_bf16";
+  if (n_masks < 0) return fail(SCORCH_HIP_EINVAL, "%s: n_masks=%lld", fn, (long long)n_masks);
+  if (block_mask_index != nullptr) {
+    SCORCH_REQUIRE(n_masks == 0 || block_masks != nullptr, "%s: block_masks is NULL", fn);
+    SCORCH_REQUIRE(aligned_to(block_masks, 8), "%s: block_masks must be 8-byte aligned", fn);
+  }
+  AttnSplit split;
+  split.n_items = n_items;
+  split.n_split_rows = n_split_rows;
+  split.n_slots = n_slots;
+  split.items = items;
+  split.split_rows = split_rows;
+  split.workspace = workspace;
+  split.workspace_bytes = workspace_bytes;
+  return attn_entry(fn, H, S, D, block, n_active_blocks, nullptr, block_col_idx, block_mask_index, block_masks,
+                    Q, K, V, scale, O, stream, &split);
 }

@@ -850,12 +850,16 @@ class BlockMask:
     pattern in CSR form, and for every active block either -1 (all 4096 entries live) or the index
     of its 64-word bit mask (bit j of word r: query r of the block row attends to key j of the
     block).  Blocks with equal masks share one."""
-    __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz")
+    __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz",
+                 "items", "split_rows", "n_slots")
 
     def __init__(self, S, block, block_row_ptr, block_col_idx, block_mask_index, block_masks, nnz):
         self.S, self.block, self.nnz = S, block, nnz
         self.block_row_ptr, self.block_col_idx = block_row_ptr, block_col_idx
         self.block_mask_index, self.block_masks = block_mask_index, block_masks
+        # set by split_long_block_rows when some block row is shared out among workgroups
+        self.items = self.split_rows = None
+        self.n_slots = 0
 
     @property
     def n_active_blocks(self) -> int:
@@ -913,6 +917,41 @@ def block_mask_from_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) ->
                      masks.contiguous().view(-1), nnz)
 
 
+def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None) -> BlockMask:
+    """Share block rows with more than `longest` key blocks out among several workgroups (in
+    stretches of equal length up to `longest`); by default `longest` is twice the mean number of
+    key blocks per block row, at least 8, so that masks whose rows are of similar length are left
+    alone and a row that attends to everything (a global token) is not the one workgroup the whole
+    launch waits for.  Fills bm.items / bm.split_rows / bm.n_slots (None / None / 0 when no row is
+    long enough)."""
+    brp = bm.block_row_ptr.cpu().tolist()
+    nb = len(brp) - 1
+    lens = [brp[i + 1] - brp[i] for i in range(nb)]
+    if longest is None:
+        longest = max(8, 2 * -(-sum(lens) // max(nb, 1)))
+    bm.items = bm.split_rows = None
+    bm.n_slots = 0
+    if longest < 1 or max(lens, default=0) <= longest:
+        return bm
+    items, split_rows, slot = [], [], 0
+    for row, n in enumerate(lens):
+        if n <= longest:
+            items.append((n, row, brp[row], brp[row + 1], -1))
+            continue
+        parts = -(-n // longest)
+        split_rows.append((row, slot, parts, 0))
+        for part in range(parts):
+            lo, hi = brp[row] + n * part // parts, brp[row] + n * (part + 1) // parts
+            items.append((hi - lo, row, lo, hi, slot))
+            slot += 1
+    items.sort(key=lambda it: -it[0])                     # longest first
+    dev = bm.block_row_ptr.device
+    bm.items = torch.tensor([it[1:] for it in items], dtype=torch.int32, device=dev).reshape(-1)
+    bm.split_rows = torch.tensor(split_rows, dtype=torch.int32, device=dev).reshape(-1)
+    bm.n_slots = slot
+    return bm
+
+
 def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -> BlockMask:
     """block_mask_from_csr, kept with the mask's row_ptr tensor and rebuilt when either index
     array is replaced or written to."""
@@ -920,7 +959,7 @@ def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -
     cached = getattr(row_ptr, "_scorch_block_mask", None)
     if cached is not None and cached[0] == key:
         return cached[1]
-    bm = block_mask_from_csr(row_ptr, col_idx, S)
+    bm = split_long_block_rows(block_mask_from_csr(row_ptr, col_idx, S))
     try:
         row_ptr._scorch_block_mask = (key, bm)
     except AttributeError:
@@ -936,8 +975,42 @@ def sparse_attention_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row
     holds an entry.  Same result as sparse_attention_csr up to bf16 rounding of the operands, the
     probabilities and the result."""
     bm = attention_block_mask(row_ptr, col_idx, int(q.shape[1]))
-    return attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, scale, block=bm.block,
-                                 block_mask_index=bm.block_mask_index, block_masks=bm.block_masks)
+    if bm.items is None:
+        return attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, scale, block=bm.block,
+                                     block_mask_index=bm.block_mask_index, block_masks=bm.block_masks)
+    return attn_blocksparse_split_bf16(q, k, v, bm, scale)
+
+
+def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: BlockMask,
+                                scale: float) -> torch.Tensor:
+    """attn_blocksparse_bf16 over a BlockMask whose long block rows split_long_block_rows has
+    shared out among workgroups: their partial results go through a workspace and a second kernel
+    combines them.  Same result up to the rounding of the partial sums' combination."""
+    if bm.items is None:
+        raise ValueError("scorch_ops_hip: this BlockMask has no shared-out rows (split_long_block_rows)")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dtype != torch.bfloat16 or t.dim() != 3:
+            raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
+    if q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
+    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+    dev = _device_of(q, k, v, bm.block_col_idx, bm.block_mask_index, bm.block_masks, bm.items)
+    H, S, D = q.shape
+    if S != bm.S:
+        raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
+    out = torch.empty_like(q)
+    L = native.lib()
+    with _on_device(dev):
+        stream = _stream(dev)
+        need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(H, bm.n_slots, D)
+        ws = _workspace(dev, stream, need)
+        rc = L.scorch_hip_attn_blocksparse_split_bf16(
+            H, S, D, bm.block, bm.n_active_blocks, bm.items.numel() // 4, bm.items.data_ptr(),
+            bm.split_rows.numel() // 4, bm.split_rows.data_ptr(), bm.n_slots, bm.block_col_idx.data_ptr(),
+            bm.block_mask_index.data_ptr(), bm.n_masks, bm.block_masks.data_ptr(), q.data_ptr(), k.data_ptr(),
+            v.data_ptr(), float(scale), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+    native.check(rc)
+    return out
 
 
 def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,

@@ -176,6 +176,24 @@ def test_attention_rejects_unsupported_shapes(L):
     assert masked(n_masks=-1) == native.EINVAL
     assert masked(q=NULL) == native.EINVAL
 
+    h = L.scorch_hip_attn_blocksparse_split_bf16
+    need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(2, 3, 32)
+    assert need == 2 * 3 * 64 * 36 * 4 and L.scorch_hip_attn_blocksparse_split_workspace_bytes(2, 0, 32) == 0
+
+    def split(D=32, n_items=5, items=FAKE, n_split=1, rows=FAKE, n_slots=3, ws=FAKE, ws_bytes=need, q=FAKE):
+        return h(2, 128, D, 64, 4, n_items, items, n_split, rows, n_slots, FAKE, NULL, 0, NULL, q, FAKE, FAKE,
+                 0.125, FAKE, ws, ws_bytes, NULL)
+
+    assert split(D=48) == native.EUNSUPPORTED
+    assert split(items=NULL) == native.EINVAL
+    assert split(items=ctypes.c_void_p(0x1004)) == native.EINVAL   # not 16-byte aligned
+    assert split(rows=NULL) == native.EINVAL
+    assert split(ws=NULL) == native.EWORKSPACE
+    assert split(ws_bytes=need - 1) == native.EWORKSPACE
+    assert split(n_items=-1) == native.EINVAL
+    assert split(q=NULL) == native.EINVAL
+    assert split(n_items=0, items=NULL) == native.OK
+
 
 def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):
     """The boundary is a C ABI: the header compiles as C99 and as C++11, and a C program linked

@@ -258,3 +258,64 @@ def test_longformer_mask_reference_shape(oracle):
     unfused = H.sparse_attention_csr(drp, dci, q.float(), k.float(), v.float(), scale)
     err = (torch.linalg.norm(out.float() - unfused) / torch.linalg.norm(unfused)).item()
     assert err <= TOL_BF16
+
+
+# ---- long block rows shared out among workgroups ----
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("longest", [1, 3, 4])
+def test_shared_out_block_rows(oracle, D, longest):
+    """A mask with a global token and a few long rows: every stretch length, stretches in which a
+    query has no live key, against the fp64 dense masked softmax and against the unsplit kernel."""
+    S = 512
+    rng = np.random.default_rng(30 + D + longest)
+    mask = np.abs(np.arange(S)[:, None] - np.arange(S)[None, :]) <= 40
+    mask[0, :] = True                                  # a global token: block row 0 holds all 8 blocks
+    mask[:, 0] = True
+    mask[300:310, ::7] = True                          # a few more long rows, sparse within their blocks
+    mask[65, :] = False                                # a query without keys
+    rp, ci = csr_of(mask)
+    q, k, v = (torch.from_numpy(rng.standard_normal((3, S, D)).astype(np.float32)).to(torch.bfloat16).cuda()
+               for _ in range(3))
+    scale = D ** -0.5
+    bm = H.block_mask_from_csr(dev(rp), dev(ci), S)
+    whole = H.attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, scale,
+                                    block_mask_index=bm.block_mask_index, block_masks=bm.block_masks)
+    H.split_long_block_rows(bm, longest)
+    assert bm.items is not None and bm.n_slots >= 2
+    # every key block is in exactly one item, and a shared-out row's stretches have consecutive slots
+    items = bm.items.cpu().numpy().reshape(-1, 4)
+    covered = np.zeros(bm.n_active_blocks, int)
+    for row, lo, hi, slot in items:
+        covered[lo:hi] += 1
+    assert (covered == 1).all() and (np.diff(items[:, 2] - items[:, 1]) <= 0).all()
+    out = H.attn_blocksparse_split_bf16(q, k, v, bm, scale)
+    assert torch.equal(out, H.attn_blocksparse_split_bf16(q, k, v, bm, scale))
+    ref = np.stack([oracle.attention_dense_fp64(q[h].float().cpu().numpy(), k[h].float().cpu().numpy(),
+                                                v[h].float().cpu().numpy(), mask, scale) for h in range(3)])
+    assert not out[:, 65].any()
+    assert oracle.rel_fro(out.float().cpu().numpy(), ref) <= 5e-3
+    err = ((out.float() - whole.float()).norm() / whole.float().norm()).item()
+    assert err <= 5e-3
+
+
+def test_shared_out_rows_with_negative_scale_and_unmasked_blocks(oracle):
+    """Whole blocks only (no bit masks in use), negative scale."""
+    w, q, k, v = bf16_inputs(1024, 2, 64, 31)
+    rp, ci = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], 64)
+    bm = H.split_long_block_rows(H.block_mask_from_csr(dev(rp), dev(ci), 1024), 2)
+    assert bm.items is not None and int((bm.block_mask_index >= 0).sum()) == 0
+    out = H.attn_blocksparse_split_bf16(q.cuda(), k.cuda(), v.cuda(), bm, -0.25).float().cpu().numpy()
+    ref = oracle.attention_blocksparse_fp64(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                            w["block_row_ptr"], w["block_col_idx"], 64, -0.25)
+    assert oracle.rel_fro(out, ref) <= TOL_BF16
+
+
+def test_masks_with_rows_of_similar_length_are_not_shared_out():
+    w = workloads.attention_blocksparse(S=1024, H=1, D=64)
+    rp, ci = workloads.blocks_to_csr(w["block_row_ptr"], w["block_col_idx"], 64)
+    bm = H.attention_block_mask(dev(rp), dev(ci), 1024)
+    assert bm.items is None and bm.n_slots == 0
+    rp, ci = workloads.longformer_mask(4096)
+    bm = H.attention_block_mask(dev(rp), dev(ci), 4096)
+    assert bm.items is not None and bm.split_rows.cpu().tolist()[:3] == [0, 0, 7]
