@@ -959,6 +959,9 @@ def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -
     cached = getattr(row_ptr, "_scorch_block_mask", None)
     if cached is not None and cached[0] == key:
         return cached[1]
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("scorch_ops_hip: the block form of an attention mask is built with host reads; call "
+                           "attention_block_mask(row_ptr, col_idx, S) once before capturing")
     bm = split_long_block_rows(block_mask_from_csr(row_ptr, col_idx, S))
     try:
         row_ptr._scorch_block_mask = (key, bm)
