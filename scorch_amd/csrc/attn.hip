@@ -232,6 +232,22 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
       }
     }
 
+    // The V^T operands of the second product are requested now, all of them, so that they arrive
+    // while the vector ALU does the softmax; requested one by one just before their MFMAs, every
+    // MFMA of the second product waits an LDS round trip.
+    bf16x8 v_ops[kFeat][2];
+#pragma unroll
+    for (int dt = 0; dt < kFeat; ++dt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int at = 32 * kRowBytes * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 16 * kRowBytes]);
+        const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        v_ops[dt][s] = __builtin_bit_cast(bf16x8, packed);
+      }
+    __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move the reads back down to their uses)
+
     // A block that is only partly live brings a 64 x 64 bit mask: bit j of word i says whether
     // query i of the block row attends to key j of the block.  A lane holds the scores of its
     // query against keys 16t + 4g + r (bit 16t + r of the word shifted down by 4g); dead ones are
@@ -292,14 +308,8 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
 #pragma unroll
     for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const int at = 32 * kRowBytes * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
-        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
-        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 16 * kRowBytes]);
-        const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const bf16x8 v_op = __builtin_bit_cast(bf16x8, packed);
-        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_op, p_op[s], o_acc[dt], 0, 0, 0);
-      }
+      for (int s = 0; s < 2; ++s)
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_ops[dt][s], p_op[s], o_acc[dt], 0, 0, 0);
 #pragma unroll
     for (int s = 0; s < 2; ++s) l_acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, p_op[s], l_acc, 0, 0, 0);
 
