@@ -59,8 +59,19 @@ __device__ __forceinline__ float combine_query_lanes(float x, Op op) {
   return op(__builtin_bit_cast(float, (unsigned)q[0]), __builtin_bit_cast(float, (unsigned)q[1]));
 }
 
-// K and V tiles are written to LDS by the load itself (global_load_lds_dwordx4):
-// no staging registers, no LDS store instructions; at D = 64, with 124 VGPRs and
+// One 16-byte-per-lane load from a buffer straight into LDS: the address is the buffer's base
+// (scalar) + a scalar byte offset + the lane's byte offset, the LDS target a scalar base + 16 x
+// lane.  (The buffer descriptor is built here, inside a device function: its type does not exist
+// in the host pass, which still has to instantiate the kernel templates' launch stubs.)
+__device__ __forceinline__ void load_to_lds_16(const void *buffer, int buffer_bytes, unsigned lane_offset,
+                                               int scalar_offset, __attribute__((address_space(3))) void *lds) {
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(buffer), 0, buffer_bytes, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds, 16, lane_offset, scalar_offset, 0, 0);
+}
+
+// K and V tiles are written to LDS by the load itself (buffer_load_dwordx4 ... lds):
+// no staging registers, no LDS store instructions; at D = 64, with 127 VGPRs and
 // 32 KB of LDS per workgroup, four workgroups share a CU.  Such a load puts lane L's 16
 // bytes at (wave-uniform base) + 16 L, so a wavefront instruction fills eight
 // whole 128-byte rows and rows cannot be padded against bank conflicts.  Instead
@@ -111,7 +122,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWaveSize - 1);
-  const int w = tid / kWaveSize;
+  const int w = uniform(tid / kWaveSize);  // a scalar: the LDS targets of the tile loads are then scalar too
   const int g = lane >> 4;
   const int n = lane & 15;
   int head, rank;
@@ -174,25 +185,27 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
   // Loading: wavefront w fills rows 16w .. 16w + 15 of a tile with kLoadsPerWave instructions of
   // kRowsPerLoad rows each.  Lane L of instruction u lands at row 16w + u kRowsPerLoad + L / CPR,
   // position L % CPR, which holds chunk (L % CPR) ^ swizzle(row).
-  int src_in_tile[Tile::kLoadsPerWave];
+  // The loads go through buffer descriptors of the head's K and V: the tile's byte offset is the
+  // instruction's scalar offset, the lane's place in the tile its vector offset, the LDS target
+  // comes from M0 -- a tile request costs no vector instructions at all.
+  unsigned src_in_tile[Tile::kLoadsPerWave];
 #pragma unroll
   for (int u = 0; u < Tile::kLoadsPerWave; ++u) {
     const int row = 16 * w + u * Tile::kRowsPerLoad + lane / Tile::kChunksPerRow;
-    src_in_tile[u] = row * kRowBytes + (((lane % Tile::kChunksPerRow) ^ Tile::swizzle(row)) * 16);
+    src_in_tile[u] = (unsigned)(row * kRowBytes + (((lane % Tile::kChunksPerRow) ^ Tile::swizzle(row)) * 16));
   }
+  const int head_bytes = (int)(unsigned)((size_t)S * D * 2);  // (the host has checked that it fits 32 bits)
   auto load_tile = [&](auto buf_tag, int it) {
     constexpr int kBuf = decltype(buf_tag)::value;
     unsigned char *k_dst = kBuf ? s_k1 : s_k0;
     unsigned char *v_dst = kBuf ? s_v1 : s_v0;
-    const size_t tile = (size_t)uniform(block_col_idx[it]) * kTileBytes;
+    const int tile = (int)((unsigned)uniform(block_col_idx[it]) * (unsigned)kTileBytes);
 #pragma unroll
     for (int u = 0; u < Tile::kLoadsPerWave; ++u) {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(Kb + tile + src_in_tile[u]),
-          (__attribute__((address_space(3))) void *)(&k_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void *)(Vb + tile + src_in_tile[u]),
-          (__attribute__((address_space(3))) void *)(&v_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]), 16, 0, 0);
+      load_to_lds_16(Kb, head_bytes, src_in_tile[u], tile,
+                     (__attribute__((address_space(3))) void *)(&k_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]));
+      load_to_lds_16(Vb, head_bytes, src_in_tile[u], tile,
+                     (__attribute__((address_space(3))) void *)(&v_dst[(16 * w + u * Tile::kRowsPerLoad) * kRowBytes]));
     }
   };
   using Even = std::integral_constant<int, 0>;
