@@ -247,18 +247,23 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
 
     // The V^T operands of the second product are requested now, all of them, so that they arrive
     // while the vector ALU does the softmax; requested one by one just before their MFMAs, every
-    // MFMA of the second product waits an LDS round trip.
+    // MFMA of the second product waits an LDS round trip.  (The masked kernel at D = 64 has no
+    // registers left for that and requests them after the softmax.)
+    constexpr bool kEarlyV = !(MASKED && D == 64);
     bf16x8 v_ops[kFeat][2];
+    auto request_v_operands = [&]() {
 #pragma unroll
-    for (int dt = 0; dt < kFeat; ++dt)
+      for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const int at = 32 * kRowBytes * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
-        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
-        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 16 * kRowBytes]);
-        const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        v_ops[dt][s] = __builtin_bit_cast(bf16x8, packed);
-      }
+        for (int s = 0; s < 2; ++s) {
+          const int at = 32 * kRowBytes * s + v_off + (((2 * dt + v_chunk) ^ v_swz) * 16);
+          const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at]);
+          const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v *)&v_src[at + 16 * kRowBytes]);
+          const short8v packed = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          v_ops[dt][s] = __builtin_bit_cast(bf16x8, packed);
+        }
+    };
+    if constexpr (kEarlyV) request_v_operands();
     __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move the reads back down to their uses)
 
     // A block that is only partly live brings a 64 x 64 bit mask: bit j of word i says whether
@@ -318,6 +323,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
         p_op[t >> 1][(t & 1) * 4 + r] = (__bf16)p;
       }
 
+    if constexpr (!kEarlyV) request_v_operands();
 #pragma unroll
     for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
