@@ -49,19 +49,19 @@ CONFIG_WORKLOADS = ("spmm_uniform", "sddmm_uniform", "attention_blocksparse", "s
 # bytes = FETCH_SIZE [KiB] x 1024 x 2.0 + WRITE_SIZE [KiB] x 1024 of the dominant kernel, the factors
 # being what the same counters read for a copy of known size (profiles/copy_calibration.md).
 MEASURED_TRAFFIC = {
-    ("gcn_powerlaw", "merge"): {"bytes": 9_790_600_000, "commit": "3014070",
+    ("gcn_powerlaw", "merge"): {"bytes": 9_790_600_000, "commit": "ea89918",
                                 "profile": "profiles/spmm_merge_kernel_gcn_powerlaw.md"},
-    ("spmm_uniform", "rows"): {"bytes": 10_820_000, "commit": "3014070",
+    ("spmm_uniform", "rows"): {"bytes": 10_820_000, "commit": "ea89918",
                                "profile": "profiles/spmm_rows_kernel_uniform_4096.md"},
-    ("sae_decoder", "tiled"): {"bytes": 666_300_000, "commit": "3014070",
+    ("sae_decoder", "tiled"): {"bytes": 666_300_000, "commit": "ea89918",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "commit": "3014070",
+    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "commit": "ea89918",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sddmm_uniform", "listed"): {"bytes": 453_300_000, "commit": "3014070",
+    ("sddmm_uniform", "listed"): {"bytes": 453_300_000, "commit": "ea89918",
                                   "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("sddmm_uniform", "plain"): {"bytes": 900_500_000, "commit": "3014070",
+    ("sddmm_uniform", "plain"): {"bytes": 900_500_000, "commit": "ea89918",
                                  "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "commit": "3014070",
+    ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "commit": "ea89918",
                                          "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
 }
 
