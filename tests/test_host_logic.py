@@ -2,6 +2,7 @@
 tensor model, the prebuilt-kernel registry and the routing decisions of
 matmul / einsum.  Mirrors tests/test_scorch/test_prebuilt_kernel_registry.py
 and the format checks of the reference; runs without a GPU."""
+import numpy as np
 import pytest
 import torch
 
@@ -296,3 +297,95 @@ def test_check_csr_indices_names_what_is_wrong(monkeypatch):
     monkeypatch.setenv("SCORCH_HIP_PLAN", "0")
     monkeypatch.setenv("SCORCH_HIP_TILED", "0")
     assert not plans_enabled() and not tiled_operands_enabled()
+
+
+# ---- the block form of an attention mask (torch ops, any device) ----
+
+def _csr_of(mask):
+    rp = np.concatenate([[0], np.cumsum(mask.sum(1))]).astype(np.int32)
+    return torch.from_numpy(rp), torch.from_numpy(np.nonzero(mask)[1].astype(np.int32))
+
+
+def _mask_of(bm):
+    """The dense mask a BlockMask stands for."""
+    brp, bci, bmi = (t.numpy() for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index))
+    words = bm.block_masks.numpy().view(np.uint64).reshape(-1, 64)
+    out = np.zeros((bm.S, bm.S), bool)
+    for br in range(bm.S // 64):
+        for i in range(brp[br], brp[br + 1]):
+            bits = (np.ones((64, 64), bool) if bmi[i] < 0 else
+                    ((words[bmi[i]][:, None] >> np.arange(64, dtype=np.uint64)[None, :]) & np.uint64(1)).astype(bool))
+            out[64 * br:64 * br + 64, 64 * bci[i]:64 * bci[i] + 64] = bits
+    return out
+
+
+def test_block_mask_from_csr_round_trips_and_shares_equal_masks():
+    rng = np.random.default_rng(40)
+    S = 320
+    mask = rng.random((S, S)) < 0.03
+    mask[0:64, 64:128] = True                      # a full block
+    mask[128:192, :] = False                       # an empty block row
+    mask[64:128, 0:64] = np.tri(64, dtype=bool)    # two equal partial blocks
+    mask[256:320, 192:256] = np.tri(64, dtype=bool)
+    mask[100, 319] = True                          # bit 63 of a word
+    rp, ci = _csr_of(mask)
+    bm = scorch_ops_hip.block_mask_from_csr(rp, ci, S)
+    assert np.array_equal(_mask_of(bm), mask) and bm.nnz == int(mask.sum())
+    brp, bci, bmi = (t.numpy() for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index))
+    at = {(br, int(bci[i])): int(bmi[i]) for br in range(5) for i in range(brp[br], brp[br + 1])}
+    assert at[(0, 1)] == -1 and at[(1, 0)] == at[(4, 3)] >= 0 and brp[3] == brp[2]
+    assert bm.n_masks < bm.n_active_blocks
+    # duplicate entries are tolerated
+    rp2 = torch.tensor([0, 3] + [3] * 63, dtype=torch.int32)
+    bm2 = scorch_ops_hip.block_mask_from_csr(rp2, torch.tensor([5, 5, 7], dtype=torch.int32), 64)
+    assert bm2.nnz == 2 and int(bm2.block_masks[0]) == (1 << 5) | (1 << 7)
+    with pytest.raises(ValueError):
+        scorch_ops_hip.block_mask_from_csr(rp2, torch.tensor([5, 64, 7], dtype=torch.int32), 64)
+    with pytest.raises(ValueError):
+        scorch_ops_hip.block_mask_from_csr(rp, ci, 100)
+
+
+def test_longformer_mask_in_block_form():
+    """The reference's Longformer pattern (window 64, one global token) at S = 4096: 314 active
+    blocks, 6 distinct masks, and only the global token's block row is shared out."""
+    from scorch_amd import workloads
+    rp, ci = workloads.longformer_mask(4096)
+    bm = scorch_ops_hip.split_long_block_rows(
+        scorch_ops_hip.block_mask_from_csr(torch.from_numpy(rp), torch.from_numpy(ci), 4096))
+    assert (bm.n_active_blocks, bm.n_masks, bm.nnz) == (314, 6, 532286)
+    assert bm.split_rows.tolist() == [0, 0, 7, 0] and bm.n_slots == 7
+    items = bm.items.view(-1, 4).numpy()
+    lengths = items[:, 2] - items[:, 1]
+    assert (np.diff(lengths) <= 0).all() and lengths.max() <= 10          # longest first, none long
+    covered = np.zeros(314, int)
+    for _, lo, hi, _ in items:
+        covered[lo:hi] += 1
+    assert (covered == 1).all()
+    assert sorted(items[items[:, 3] >= 0, 3].tolist()) == list(range(7))
+
+
+@pytest.mark.parametrize("longest", [1, 2, 5])
+def test_split_long_block_rows_covers_every_block_once(longest):
+    rng = np.random.default_rng(41 + longest)
+    nb = 12
+    active = rng.random((nb, nb)) < 0.5
+    active[3, :] = True
+    active[7, :] = False
+    mask = np.kron(active, np.ones((64, 64), bool))
+    rp, ci = _csr_of(mask)
+    bm = scorch_ops_hip.split_long_block_rows(scorch_ops_hip.block_mask_from_csr(rp, ci, 64 * nb), longest)
+    items = bm.items.view(-1, 4).numpy()
+    brp = bm.block_row_ptr.numpy()
+    covered = np.zeros(bm.n_active_blocks, int)
+    for row, lo, hi, slot in items:
+        assert brp[row] <= lo <= hi <= brp[row + 1] and hi - lo <= longest
+        assert lo < hi or brp[row] == brp[row + 1]       # only an empty block row has an empty item (it writes zeros)
+        covered[lo:hi] += 1
+        assert (slot >= 0) == (brp[row + 1] - brp[row] > longest)
+    assert (covered == 1).all()
+    for row, first, parts, _ in bm.split_rows.view(-1, 4).numpy():
+        mine = items[items[:, 0] == row]
+        assert sorted(mine[:, 3].tolist()) == list(range(first, first + parts))
+    # a mask whose rows are all short enough is left alone
+    bm = scorch_ops_hip.split_long_block_rows(scorch_ops_hip.block_mask_from_csr(rp, ci, 64 * nb), nb)
+    assert bm.items is None and bm.n_slots == 0
