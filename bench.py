@@ -202,30 +202,42 @@ def cpu_baseline_attention(w, heads=2, pattern=None):
 _blocker = None
 
 
-def _time_steps(fn, steps, warmup, rounds=3):
+def _time_steps(fn, steps, warmup, rounds=3, min_round_ms=4.0):
     """GPU time per step of `fn`, HIP events on torch's current stream (the
     stream the kernels are launched on).  A few large device fills are queued
     first, so that the step launches are all enqueued before the GPU reaches the
     first of them: the interval is then the GPU's time for the steps, not the
-    host's time to issue them.  Median of `rounds` such measurements."""
+    host's time to issue them.  Median of `rounds` such measurements.  A round of
+    `steps` steps that lasts less than `min_round_ms` is a pilot only: the rounds
+    that count then repeat the step until they last that long (a burst of a
+    millisecond is over before the GPU's clocks have settled), with as many fills
+    in front as the host needs to enqueue them."""
     import torch
     global _blocker
     if _blocker is None:
         _blocker = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
     for _ in range(warmup):
         fn()
-    results = []
-    for _ in range(rounds):
+
+    def one_round(n):
         torch.cuda.synchronize()
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for _ in range(3):
+        for _ in range(3 + int(n * 0.012 / 0.15)):  # ~12 us of host time per call, ~0.15 ms per fill
             _blocker.fill_(1.0)
         start.record()
-        for _ in range(steps):
+        for _ in range(n):
             fn()
         stop.record()
         torch.cuda.synchronize()
-        results.append(start.elapsed_time(stop) / steps)
+        return start.elapsed_time(stop) / n
+
+    results = [one_round(steps)]
+    n = steps
+    if results[0] * steps < min_round_ms:
+        n = min(int(min_round_ms / max(results[0], 1e-6)) + 1, 200 * steps)
+        results = []
+    while len(results) < rounds:
+        results.append(one_round(n))
     return statistics.median(results)
 
 
