@@ -426,7 +426,7 @@ size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz) {
 
 static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
                              const float *vals, float scale, float *out, void *workspace,
-                             size_t workspace_bytes, void *stream) {
+                             size_t workspace_bytes, void *stream, bool short_rows = false) {
   if (batch < 0 || batch > 65535)
     return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
   if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
@@ -435,7 +435,9 @@ static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t n
   SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
   if (batch == 0 || M == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
-  const size_t need = scorch::softmax_workspace_bytes(M, nnz);
+  // (short_rows: the caller vouches that no row has more than 4096 entries, so there is no list
+  // of giant rows to reset, fill or serve)
+  const size_t need = short_rows ? 0 : scorch::softmax_workspace_bytes(M, nnz);
   if (need > 0 && (!workspace || workspace_bytes < need))
     return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
                         workspace ? workspace_bytes : (size_t)0);
@@ -489,6 +491,12 @@ int scorch_hip_softmax_csr_batched_f32(int64_t batch, int64_t M, int64_t nnz, co
                                        size_t workspace_bytes, void *stream) {
   return softmax_csr_entry("scorch_hip_softmax_csr_batched_f32", batch, M, nnz, row_ptr, vals, scale, out,
                            workspace, workspace_bytes, stream);
+}
+
+int scorch_hip_softmax_csr_short_rows_f32(int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
+                                          const float *vals, float scale, float *out, void *stream) {
+  return softmax_csr_entry("scorch_hip_softmax_csr_short_rows_f32", batch, M, nnz, row_ptr, vals, scale, out,
+                           nullptr, 0, stream, true);
 }
 
 int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr, int32_t *row_idx,

@@ -638,6 +638,18 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
 
 
 # ---- neighbours of the path ---------------------------------------------------------
+SOFTMAX_SHORT_ROW = 4096     # rows up to this length never reach the row softmax's giant-row pass
+
+
+def _known_longest_row(pos: torch.Tensor, n_rows: int, nnz: int) -> Optional[int]:
+    """The longest row of the pattern if a plan made for this row pointer says so (a product with
+    the same pattern has inspected it), else None."""
+    plan = getattr(pos, "_scorch_plan", None)
+    if plan is not None and plan.key[0] == pos._version and plan.key[3] == nnz and plan.key[4] == n_rows:
+        return plan.max_row
+    return None
+
+
 def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """Row softmax of ``scale * values`` over a CSR pattern
     (reference: bench/bench_sparse_transformer.py:277-297)."""
@@ -646,13 +658,18 @@ def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float 
     dev = _device_of(pos, v)
     out = torch.empty_like(v)
     L = native.lib()
+    longest = _known_longest_row(pos, pos.numel() - 1, v.numel())
     with _on_device(dev):
         stream = _stream(dev)
-        need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, v.numel())
-        ws = _workspace(dev, stream, need) if need else None
-        rc = L.scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
-                                          float(scale), out.data_ptr(), ws.data_ptr() if need else None,
-                                          ws.numel() if need else 0, stream)
+        if longest is not None and longest <= SOFTMAX_SHORT_ROW:
+            rc = L.scorch_hip_softmax_csr_short_rows_f32(1, pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
+                                                         float(scale), out.data_ptr(), stream)
+        else:
+            need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, v.numel())
+            ws = _workspace(dev, stream, need) if need else None
+            rc = L.scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
+                                              float(scale), out.data_ptr(), ws.data_ptr() if need else None,
+                                              ws.numel() if need else 0, stream)
     native.check(rc)
     return out
 
@@ -782,13 +799,18 @@ def softmax_csr_float_batched(row_ptr: torch.Tensor, values: torch.Tensor, scale
     H, nnz = int(v.shape[0]), int(v.shape[1])
     out = torch.empty_like(v)
     L = native.lib()
+    longest = _known_longest_row(pos, pos.numel() - 1, nnz)
     with _on_device(dev):
         stream = _stream(dev)
-        need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, nnz)
-        ws = _workspace(dev, stream, need) if need else None
-        rc = L.scorch_hip_softmax_csr_batched_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(), float(scale),
-                                                  out.data_ptr(), ws.data_ptr() if need else None,
-                                                  ws.numel() if need else 0, stream)
+        if longest is not None and longest <= SOFTMAX_SHORT_ROW:
+            rc = L.scorch_hip_softmax_csr_short_rows_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(),
+                                                         float(scale), out.data_ptr(), stream)
+        else:
+            need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, nnz)
+            ws = _workspace(dev, stream, need) if need else None
+            rc = L.scorch_hip_softmax_csr_batched_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(),
+                                                      float(scale), out.data_ptr(), ws.data_ptr() if need else None,
+                                                      ws.numel() if need else 0, stream)
     native.check(rc)
     return out
 

@@ -85,3 +85,27 @@ def test_sparse_attention_at_the_reference_benchmarks_shape():
     assert worst <= 1e-5, worst          # fp32 throughout (the bf16 bar of the fused kernel is 1e-2)
     again = H.sparse_attention_csr(rp, ci, q, k, v, scale)
     assert torch.equal(out, again)
+
+
+def test_softmax_with_a_known_longest_row_skips_the_giant_row_pass():
+    """Once a product has inspected the pattern (so that its longest row is known and at most
+    4096), the row softmax runs as one launch; same bits as without that knowledge, and a pattern
+    with a longer row keeps the general form."""
+    rng = np.random.default_rng(9)
+    for longest in (4096, 4097):
+        lens = rng.integers(0, 40, 300)
+        lens[17] = longest
+        rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        ci = np.concatenate([np.sort(rng.choice(8192, n, replace=False)) for n in lens]).astype(np.int32)
+        vals = torch.from_numpy(rng.standard_normal((3, ci.size)).astype(np.float32)).cuda()
+        drp, dci = dev(rp), dev(ci)
+        before = H.softmax_csr_float_batched(drp, vals, 0.3)
+        assert H._known_longest_row(drp, 300, ci.size) is None
+        plan = H.csr_plan(drp, dci, 300, 8192)
+        assert plan.max_row == longest and H._known_longest_row(drp, 300, ci.size) == longest
+        after = H.softmax_csr_float_batched(drp, vals, 0.3)
+        assert torch.equal(before, after)
+        assert torch.equal(H.softmax_csr_float(drp, vals[1], 0.3), after[1])
+        sums = torch.zeros(3, 300, device="cuda").index_add_(
+            1, torch.repeat_interleave(torch.arange(300, device="cuda"), torch.from_numpy(lens).cuda()), after)
+        assert torch.allclose(sums[:, lens > 0], torch.ones_like(sums[:, lens > 0]), atol=1e-5)
