@@ -469,3 +469,29 @@ def test_spmv_matmul_wksp_and_precompile_follow_the_reference_signatures():
     d = scorch.matmul_wksp(a, STensor.from_torch(b_t, "B").to_sparse("ds").to("cuda"), output_format="dd")
     assert isinstance(d, STensor) and d.format.is_dense()
     assert torch.allclose(d.to_torch().cpu(), a_t @ b_t, atol=1e-5)
+
+
+def test_matmul_with_a_dense_torch_operand_takes_the_direct_route_and_agrees_with_the_general_one():
+    """scorch.matmul(CSR STensor, torch.Tensor) calls the resolved kernel without wrapping the dense
+    operand and the result; same bits as the general route, same keyword behaviour."""
+    rng = np.random.default_rng(77)
+    dense = (rng.random((96, 80)) < 0.1) * rng.standard_normal((96, 80))
+    A = STensor.from_torch(torch.from_numpy(dense.astype(np.float32)).to_sparse_csr()).to("cuda")
+    B = torch.from_numpy(rng.standard_normal((80, 24)).astype(np.float32)).cuda()
+    direct = scorch.matmul(A, B)
+    assert isinstance(direct, torch.Tensor) and direct.shape == (96, 24)
+    general = scorch.matmul(A, STensor.from_torch(B))
+    assert torch.equal(direct, general)
+    np.testing.assert_allclose(host(direct), dense.astype(np.float32) @ host(B), rtol=1e-4, atol=1e-5)
+    # a vector, a non-contiguous operand, the time dictionary, the other keyword routes
+    x = B[:, 3].contiguous()
+    assert torch.equal(scorch.matmul(A, x), scorch.matmul(A, STensor.from_torch(x)))
+    Bt = torch.from_numpy(rng.standard_normal((24, 80)).astype(np.float32)).cuda().t()
+    assert torch.equal(scorch.matmul(A, Bt), scorch.matmul(A, STensor.from_torch(Bt.contiguous())))
+    times = {}
+    assert torch.equal(scorch.matmul(A, B, time_dict=times), direct) and times["eval_time"] > 0
+    assert torch.equal(scorch.matmul(A, B, use_cache=False), direct)
+    as_csr = scorch.matmul(A, B, format="ds")
+    assert isinstance(as_csr, STensor) and torch.equal(as_csr.to_torch(), direct)
+    with pytest.raises(NotImplementedError):
+        scorch.matmul(A, B.double())
