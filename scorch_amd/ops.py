@@ -238,15 +238,50 @@ def _sddmm(mask: STensor, A: STensor, B: STensor, time_dict) -> Optional[STensor
     return _wrap(result_cpp, mask.shape, mask.format if mask_fmt == "o,o" else "oo")
 
 
+_canonical_cache: dict = {}
+
+
+def _sddmm_direct(mask, A, B, time_dict) -> Optional[STensor]:
+    """The SDDMM with a sparse STensor mask and two dense fp32 torch tensors on the device: the
+    kernel is called without wrapping the dense operands in STensors first."""
+    if not (isinstance(mask, STensor) and isinstance(A, torch.Tensor) and isinstance(B, torch.Tensor)):
+        return None
+    if A.layout != torch.strided or B.layout != torch.strided or A.dim() != 2 or B.dim() != 2:
+        return None
+    if not (A.is_cuda and B.is_cuda and mask.values.is_cuda):
+        return None
+    if mask.values.dtype != torch.float32 or A.dtype != torch.float32 or B.dtype != torch.float32:
+        return None
+    mask_fmt = str(mask.format)
+    if mask_fmt == "o,o":
+        fn = scorch_ops_hip.sddmm_coo_float_prebuilt
+    elif mask_fmt == "d,s" and mask.index.mode_order == [0, 1]:
+        fn = scorch_ops_hip.sddmm_csr_float
+    else:
+        return None
+    dense_index = [[], []]
+    result_cpp = _timed(lambda: fn(mask.shape, mask.shape, mask.index.mode_indices, mask.values,
+                                   tuple(A.shape), dense_index, A.reshape(-1),
+                                   tuple(B.shape), dense_index, B.reshape(-1)),
+                        mask.values.device, time_dict)
+    return _wrap(result_cpp, mask.shape, mask.format if mask_fmt == "o,o" else "oo")
+
+
 def einsum(expression: str, *tensors: Optional[Union[torch.Tensor, STensor]],
            compile_only: Optional[bool] = False, **kwargs: Any) -> Union[STensor, torch.Tensor]:
     """Einstein summation for the expressions that have a device kernel."""
     if compile_only:
         raise _not_prebuilt("einsum(compile_only=True)")
-    operands = tuple(STensor.from_torch(t) if isinstance(t, torch.Tensor) else t for t in tensors)
+    canon = _canonical_cache.get(expression)
+    if canon is None:
+        canon = _canonical_cache[expression] = _canonical(expression)
     time_dict = kwargs.get("time_dict", None)
     requested = kwargs.get("format", kwargs.get("output_format", None))
-    canon = _canonical(expression)
+    if canon == _SDDMM_EXPR and len(tensors) == 3 and requested is None:
+        direct = _sddmm_direct(*tensors, time_dict)
+        if direct is not None:
+            return direct
+    operands = tuple(STensor.from_torch(t) if isinstance(t, torch.Tensor) else t for t in tensors)
 
     if canon in (_SDDMM_EXPR, _SDDMM_EXPR_KJ) and len(operands) == 3:
         mask, A, B = operands

@@ -44,17 +44,20 @@ class STensor(torch.nn.Module):
                  storage: Optional[TensorStorage] = None, index: Optional[TensorIndex] = None,
                  value: Optional[torch.Tensor] = None, requires_grad: Optional[bool] = False) -> None:
         super().__init__()
-        self._storage = storage if storage is not None else TensorStorage(index=index, value=value,
-                                                                          shape=shape)
-        self._name = name
-        self._shape = tuple(shape) if shape is not None else None
+        # plain attributes (no parameter, buffer or sub-module among them): set past
+        # nn.Module.__setattr__, whose type checks cost more than everything else here
+        put = object.__setattr__
+        put(self, "_storage", storage if storage is not None else TensorStorage(index=index, value=value,
+                                                                                shape=shape))
+        put(self, "_name", name)
+        put(self, "_shape", tuple(shape) if shape is not None else None)
         if value is not None:
-            self._dtype = value.dtype
+            put(self, "_dtype", value.dtype)
         elif storage is not None and storage._value is not None:
-            self._dtype = storage._value.dtype
+            put(self, "_dtype", storage._value.dtype)
         else:
-            self._dtype = torch.float32
-        self.requires_grad = requires_grad
+            put(self, "_dtype", torch.float32)
+        put(self, "requires_grad", requires_grad)
 
     # ---- accessors the dispatch reads ------------------------------------------
     @property

@@ -202,3 +202,29 @@ def test_auto_builds_the_lists_on_the_second_product_at_full_size(oracle):
     second = call()
     assert rp._scorch_plan.sddmm_lists is not None
     assert torch.equal(first, second) and torch.equal(second, call())
+
+
+@pytest.mark.parametrize("mask_format", ["ds", "oo"])
+def test_einsum_with_dense_torch_operands_takes_the_direct_route(mask_format):
+    """scorch.einsum("ij,ik,jk->ij", mask, Q, K) with torch tensors for Q and K: same entries,
+    same order, same bits as with the operands wrapped in STensors first."""
+    import scorch_amd as scorch
+    from scorch_amd import STensor
+    rng = np.random.default_rng(12)
+    mask = ((rng.random((70, 90)) < 0.15) * rng.standard_normal((70, 90))).astype(np.float32)
+    S = STensor.from_torch(torch.from_numpy(mask).to_sparse_csr()).to("cuda")
+    if mask_format == "oo":
+        S = S.to_sparse("oo")
+    Q = torch.from_numpy(rng.standard_normal((70, 40)).astype(np.float32)).cuda()
+    K = torch.from_numpy(rng.standard_normal((90, 40)).astype(np.float32)).cuda()
+    direct = scorch.einsum("ij,ik,jk->ij", S, Q, K)
+    general = scorch.einsum("ij,ik,jk->ij", S, STensor.from_torch(Q), STensor.from_torch(K))
+    assert str(direct.format) == str(general.format) == "o,o"
+    for a, b in zip(direct.index.mode_indices, general.index.mode_indices):
+        assert torch.equal(a[0], b[0])
+    assert torch.equal(direct.values, general.values)
+    want = (Q.double() @ K.double().T).cpu().numpy() * mask
+    np.testing.assert_allclose(host(direct.to_torch()), want, rtol=1e-4, atol=1e-5)
+    times = {}
+    again = scorch.einsum("ab,ac,bc->ab", S, Q, K, time_dict=times)      # other index names, same expression
+    assert torch.equal(again.values, direct.values) and times["eval_time"] > 0
