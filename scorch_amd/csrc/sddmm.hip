@@ -8,8 +8,8 @@
 // (GS * VEC elements per load, so a K = 64 fp32 row is one dwordx4 access by
 // 16 lanes), multiply, and reduce with GS-wide butterfly shuffles.  After GS
 // steps lane L keeps the result of entry L and the batch is written with one
-// coalesced store.  Consecutive entries share their A row, which therefore
-// comes from the vector cache after its first use.
+// coalesced store.  Consecutive entries mostly share their A row, which a group
+// keeps in registers until the row changes (K up to GS * VEC).
 //
 // With a CSR mask the row of each entry is found by bisection of row_ptr; the
 // wavefront first narrows the range to the rows its entries span, so the
@@ -78,6 +78,11 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
     }
 
     float mine = 0.0f;
+    // !LONG: a group's piece of its current row of A stays in registers; a group's 16 or more
+    // consecutive entries mostly share a row, and a mask of long rows (an attention pattern)
+    // would otherwise ask the vector cache for the same line once per entry
+    int held_row = -1;
+    VecT held;
 #pragma unroll 4
     for (int s = 0; s < GS; ++s) {
       const int src = g * GS + s;
@@ -87,11 +92,15 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
       const float *b = B + (size_t)c * (size_t)K;
       float dot = 0.0f;
       if (!LONG) {
-        for (int k = t * VEC; k < K; k += GS * VEC) {
-          const VecT av = *reinterpret_cast<const VecT *>(a + k);
+        const int k = t * VEC;
+        if (k < K) {
           const VecT bv = *reinterpret_cast<const VecT *>(b + k);
+          if (r != held_row) {
+            held = *reinterpret_cast<const VecT *>(a + k);
+            held_row = r;
+          }
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) dot += av.v[v] * bv.v[v];
+          for (int v = 0; v < VEC; ++v) dot += held.v[v] * bv.v[v];
         }
       } else {
         constexpr int kPieces = 4;
