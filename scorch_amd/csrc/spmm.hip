@@ -576,23 +576,47 @@ __global__ __launch_bounds__(kBlockThreads) void spmv_merge_kernel(
   const int64_t nnz = total_items - M;
   int col[kNzLoads];
   T val[kNzLoads];
+  // (a chunk that lies inside the arrays reads them at constant offsets from a scalar base:
+  // no address arithmetic and no bounds checks per element)
+  const bool inside = (int64_t)y0 + ITEMS <= nnz;
+  if (inside) {
+    const int *c0 = col_idx + y0;
+    const T *v0 = vals + y0;
 #pragma unroll
-  for (int u = 0; u < kNzLoads; ++u) {
-    const int64_t p = (int64_t)y0 + lane + u * kWaveSize;
-    const bool ok = p < nnz;
-    col[u] = ok ? col_idx[p] : -1;
-    val[u] = ok ? vals[p] : (T)0;
+    for (int u = 0; u < kNzLoads; ++u) {
+      col[u] = c0[lane + u * kWaveSize];
+      val[u] = v0[lane + u * kWaveSize];
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < kNzLoads; ++u) {
+      const int64_t p = (int64_t)y0 + lane + u * kWaveSize;
+      const bool ok = p < nnz;
+      col[u] = ok ? col_idx[p] : -1;
+      val[u] = ok ? vals[p] : (T)0;
+    }
   }
   int rp[kRpLoads];
+  if ((int64_t)x0 + kRpLoads * kWaveSize <= M) {
+    const int *r0 = row_ptr + x0;
 #pragma unroll
-  for (int u = 0; u < kRpLoads; ++u) {
-    const int64_t r = (int64_t)x0 + lane + u * kWaveSize;
-    rp[u] = row_ptr[r < M ? r : M];
+    for (int u = 0; u < kRpLoads; ++u) rp[u] = r0[lane + u * kWaveSize];
+  } else {
+#pragma unroll
+    for (int u = 0; u < kRpLoads; ++u) {
+      const int64_t r = (int64_t)x0 + lane + u * kWaveSize;
+      rp[u] = row_ptr[r < M ? r : M];
+    }
   }
+  if (inside) {
 #pragma unroll
-  for (int u = 0; u < kNzLoads; ++u) {
-    const A xv = col[u] >= 0 ? (A)x[col[u]] : (A)0;
-    s_prod[w][lane + u * kWaveSize] = (A)val[u] * xv;
+    for (int u = 0; u < kNzLoads; ++u) s_prod[w][lane + u * kWaveSize] = (A)val[u] * (A)x[col[u]];
+  } else {
+#pragma unroll
+    for (int u = 0; u < kNzLoads; ++u) {
+      const A xv = col[u] >= 0 ? (A)x[col[u]] : (A)0;
+      s_prod[w][lane + u * kWaveSize] = (A)val[u] * xv;
+    }
   }
 #pragma unroll
   for (int u = 0; u < kRpLoads; ++u)
