@@ -17,6 +17,22 @@ from_torch = STensor.from_torch
 from_coo = STensor.from_coo
 from_csr = STensor.from_csr
 
+
+
+def __getattr__(name):
+    """Names this package does not define resolve to torch's, as in the reference
+    (src/scorch/__init__.py:14-18): ``scorch.float32``, ``scorch.rand(...)``."""
+    import importlib
+    import importlib.util
+    import torch
+    if not name.startswith("_") and importlib.util.find_spec(f"{__name__}.{name}") is not None:
+        return importlib.import_module(f"{__name__}.{name}")    # a submodule not imported yet
+    try:
+        return getattr(torch, name)
+    except AttributeError:
+        raise AttributeError(f"module {__name__!r} has no attribute {name!r}") from None
+
+
 __version__ = "0.1.0"
 
 __all__ = ["STensor", "TensorFormat", "TensorIndex", "TensorStorage", "LevelFormat", "LevelType",

@@ -389,3 +389,14 @@ def test_split_long_block_rows_covers_every_block_once(longest):
     # a mask whose rows are all short enough is left alone
     bm = scorch_ops_hip.split_long_block_rows(scorch_ops_hip.block_mask_from_csr(rp, ci, 64 * nb), nb)
     assert bm.items is None and bm.n_slots == 0
+
+
+def test_names_the_package_lacks_resolve_to_torch():
+    """reference: src/scorch/__init__.py:14-18"""
+    import scorch_amd as scorch
+    assert scorch.float32 is torch.float32
+    from scorch_amd import utils          # an own submodule wins over torch.utils
+    assert utils.__name__ == "scorch_amd.utils"
+    assert scorch.zeros(2, 3).shape == (2, 3)
+    with pytest.raises(AttributeError, match="no_such_name"):
+        scorch.no_such_name
