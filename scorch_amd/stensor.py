@@ -133,6 +133,43 @@ class STensor(torch.nn.Module):
 
     clone = copy
 
+    def validate(self) -> None:
+        """Raise ValueError unless the index arrays describe a tensor of this shape: row
+        pointers that start at 0, never decrease and end at the number of stored entries,
+        coordinates inside the shape (the reference leaves this method unimplemented,
+        stensor.py:142-145).  Reads the index arrays and synchronises."""
+        fmt = str(self.format)
+        count = self.values.numel()
+        if self.format.is_dense():
+            expected = 1
+            for extent in self.shape:
+                expected *= int(extent)
+            if count != expected:
+                raise ValueError(f"STensor: {count} values for a dense tensor of shape {tuple(self.shape)}")
+            return
+        if self.dim() != 2 or fmt not in ("d,s", "o,o"):
+            raise NotImplementedError(f"STensor.validate for format {fmt!r}")
+        order = self.index.mode_order
+        extents = [int(self.shape[order[0]]), int(self.shape[order[1]])]    # of the stored modes
+        levels = self.index.mode_indices
+        if fmt == "d,s":
+            pos, crd = levels[1]
+            if pos.numel() != extents[0] + 1 or crd.numel() != count:
+                raise ValueError("STensor: index array lengths do not match the shape and the values")
+            rows_ok = bool(pos[0] == 0) and bool(pos[-1] == count) and bool((pos[1:] >= pos[:-1]).all())
+            if not rows_ok:
+                raise ValueError(f"STensor: row pointers must start at 0, never decrease and end at {count}")
+            stored = [crd]
+            limits = [extents[1]]
+        else:
+            stored = [levels[0][0], levels[1][0]]
+            limits = extents
+            if any(c.numel() != count for c in stored):
+                raise ValueError("STensor: coordinate and value arrays differ in length")
+        for coordinates, limit in zip(stored, limits):
+            if count and (int(coordinates.min()) < 0 or int(coordinates.max()) >= limit):
+                raise ValueError(f"STensor: a coordinate lies outside [0, {limit})")
+
     # ---- construction --------------------------------------------------------------
     @staticmethod
     def _csr(shape, crow, col, values, name, mode_order=None) -> "STensor":

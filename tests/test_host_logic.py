@@ -400,3 +400,25 @@ def test_names_the_package_lacks_resolve_to_torch():
     assert scorch.zeros(2, 3).shape == (2, 3)
     with pytest.raises(AttributeError, match="no_such_name"):
         scorch.no_such_name
+
+
+def test_validate_accepts_well_formed_tensors_and_names_what_is_wrong():
+    from scorch_amd import STensor
+    dense = torch.tensor([[0.0, 2.0, 0.0], [1.0, 0.0, 3.0]])
+    for fmt in ("dd", "ds", "oo"):
+        t = STensor.from_torch(dense)
+        (t if fmt == "dd" else t.to_sparse(fmt)).validate()
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32)
+    vals = torch.ones(3)
+    STensor.from_csr_arrays(i32(0, 1, 3), i32(1, 0, 2), vals, (2, 3)).validate()
+    with pytest.raises(ValueError, match="row pointers"):
+        STensor.from_csr_arrays(i32(0, 2, 1), i32(1, 0, 2), vals, (2, 3)).validate()
+    with pytest.raises(ValueError, match="row pointers"):
+        STensor.from_csr_arrays(i32(0, 1, 2), i32(1, 0, 2), vals, (2, 3)).validate()
+    with pytest.raises(ValueError, match=r"outside \[0, 3\)"):
+        STensor.from_csr_arrays(i32(0, 1, 3), i32(1, 0, 3), vals, (2, 3)).validate()
+    with pytest.raises(ValueError, match="lengths"):
+        STensor.from_csr_arrays(i32(0, 1, 3, 3), i32(1, 0, 2), vals, (2, 3)).validate()
+    coo = STensor.from_coo(indices=torch.tensor([[0, 1, 2], [1, 0, 2]]), values=vals, shape=(2, 3))
+    with pytest.raises(ValueError, match=r"outside \[0, 2\)"):
+        coo.validate()
