@@ -150,11 +150,10 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
 // wavefronts' pieces inside a list varies from build to build; the products do
 // not depend on it.
 constexpr int kBuckets = 8;  // one per XCD
-// Workgroups per XCD of the kernel that walks the lists.  All of them must be resident at once:
-// the id & 7 = XCD rule holds for workgroups dispatched in order, and once the chip is full later
-// ones go wherever a slot frees up (65,536^2 mask, 64 per row, K = 64: with 256 per XCD the fetch
-// traffic was the plain kernel's 0.86 GB; with 192, 0.44 GB and 0.124 ms against the plain
-// kernel's 0.130; with 128, 0.43 GB and 0.165 ms: fewer wavefronts hide less latency).
+// Workgroups per XCD of the kernel that walks the lists: a grid that is resident as a whole,
+// workgroup id & 7 being the XCD it runs on (checked against the hardware's XCC_ID register: no
+// workgroup of 102,400 was elsewhere, also with 256 per XCD).  65,536^2 mask, 64 per row, K = 64:
+// 128 per XCD 0.165 ms (fewer wavefronts hide less latency), 192 and 256 the same 0.109 ms.
 constexpr int kListedWorkgroupsPerXcd = 192;
 
 __device__ __forceinline__ int sddmm_entry_row(const int *__restrict__ row_ptr, int row_lo, int row_hi, int64_t p) {
@@ -293,17 +292,27 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
   for (int64_t first = begin + ((int64_t)(blockIdx.x >> 3) * kWavesPerBlock + threadIdx.x / kWaveSize) * kEntriesPerWave;
        first < end; first += waves_per_xcd * kEntriesPerWave) {
     const int64_t last = first + kEntriesPerWave < end ? first + kEntriesPerWave : end;
-    for (int64_t base = first; base < last; base += kWaveSize) {
-      const int64_t e = base + lane;
+    // the piece's list entries and mask values are requested for all of its batches of 64 at
+    // once: two round trips to memory per piece instead of two per batch
+    constexpr int kBatches = kEntriesPerWave / kWaveSize;
+    int rows_of[kBatches], cols_of[kBatches], pos_of[kBatches];
+    float scale_of[kBatches];
+#pragma unroll
+    for (int b = 0; b < kBatches; ++b) {
+      const int64_t e = first + b * kWaveSize + lane;
       const bool valid = e < last;
-      int row = 0, col = 0, pos = 0;
-      float scale = 0.0f;
-      if (valid) {
-        pos = entry_pos[e];
-        row = entry_row[e];
-        col = entry_col[e];
-        scale = mask_vals[pos];
-      }
+      pos_of[b] = valid ? entry_pos[e] : -1;
+      rows_of[b] = valid ? entry_row[e] : 0;
+      cols_of[b] = valid ? entry_col[e] : 0;
+    }
+#pragma unroll
+    for (int b = 0; b < kBatches; ++b) scale_of[b] = pos_of[b] >= 0 ? mask_vals[pos_of[b]] : 0.0f;
+#pragma unroll
+    for (int b = 0; b < kBatches; ++b) {
+      if (first + b * kWaveSize >= last) break;
+      const int row = rows_of[b], col = cols_of[b], pos = pos_of[b];
+      const float scale = scale_of[b];
+      const bool valid = pos >= 0;
       float mine = 0.0f;
       if (K <= GS * VEC) {
         // One load per lane covers a row.  Consecutive entries of a list mostly share their row
