@@ -296,7 +296,8 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_f32(int64_t M, int64_t n_cols, int64_t K
  * scorch_hip_sddmm_csr_lists sorts the mask's entries once into eight lists by
  * the eighth of the column range they fall in (`lists`: device, 256-byte aligned,
  * scorch_hip_sddmm_csr_lists_bytes(nnz) bytes; it depends on row_ptr, col_idx and
- * n_cols only).  scorch_hip_sddmm_csr_listed_f32 is scorch_hip_sddmm_csr_batched_f32
+ * n_cols only, and a list holds its entries in the mask's order, the same on every
+ * build).  scorch_hip_sddmm_csr_listed_f32 is scorch_hip_sddmm_csr_batched_f32
  * computed list by list, each list on one XCD, whose L2 then keeps that eighth of
  * B: the same products, the same results bit for bit.  K <= 256. */
 SCORCH_HIP_API size_t scorch_hip_sddmm_csr_lists_bytes(int64_t nnz);

@@ -145,10 +145,11 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
 // sddmm_bucket_count_kernel / sddmm_bucket_fill_kernel build the lists: each
 // wavefront takes kEntriesPerWave consecutive entries (so that a row's entries
 // stay together in the lists and its row of A is reused from the vector cache),
-// counts them per range, reserves that many slots in every range's list with one
-// atomic each, and writes (entry number, row, column) there.  The order of the
-// wavefronts' pieces inside a list varies from build to build; the products do
-// not depend on it.
+// counts them per range (sddmm_bucket_count_kernel), a scan over the wavefronts'
+// counts gives every wavefront its place in every list (sddmm_bucket_scan_kernel),
+// and the wavefront writes (entry number, row, column) there
+// (sddmm_bucket_fill_kernel).  No atomics: the lists come out in entry order, the
+// same on every build.
 constexpr int kBuckets = 8;  // one per XCD
 // Workgroups per XCD of the kernel that walks the lists: a grid that is resident as a whole,
 // workgroup id & 7 being the XCD it runs on (checked against the hardware's XCC_ID register: no
@@ -165,10 +166,11 @@ __device__ __forceinline__ int sddmm_entry_row(const int *__restrict__ row_ptr, 
   return lo;
 }
 
-// counts[b] += entries whose column lies in range b; columns outside [0, n_cols) count for no range
+// wave_counts[wave][b] = entries of the wavefront's piece whose column lies in range b; columns
+// outside [0, n_cols) count for no range
 __global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_count_kernel(int64_t nnz, int cols_per_bucket,
                                                                            const int *__restrict__ col_idx,
-                                                                           int *__restrict__ counts) {
+                                                                           int *__restrict__ wave_counts) {
   const int lane = wave_lane();
   const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
   const int64_t first = wave * kEntriesPerWave;
@@ -180,36 +182,79 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_count_kernel(int64
 #pragma unroll
     for (int k = 0; k < kBuckets; ++k) mine[k] += b == (unsigned)k;
   }
+  int total = 0;  // lane k < kBuckets ends up with range k's count
 #pragma unroll
   for (int k = 0; k < kBuckets; ++k) {
-    int total = mine[k];
+    int sum = mine[k];
 #pragma unroll
-    for (int off = kWaveSize / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
-    if (lane == 0 && total > 0) atomicAdd(&counts[k], total);
+    for (int off = kWaveSize / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == k) total = sum;
+  }
+  if (lane < kBuckets) wave_counts[wave * kBuckets + lane] = total;
+}
+
+// One workgroup: wave_counts[wave][b] becomes the number of range-b entries in the pieces before
+// `wave`, and list_ptr[b] the start of range b's list (list_ptr[kBuckets] = entries listed).
+constexpr int kScanThreads = 1024;
+
+__global__ __launch_bounds__(kScanThreads) void sddmm_bucket_scan_kernel(int64_t n_waves, int *__restrict__ wave_counts,
+                                                                        int *__restrict__ list_ptr) {
+  constexpr int kScanWaves = kScanThreads / kWaveSize;
+  __shared__ int s_wave_total[kBuckets][kScanWaves];
+  __shared__ int s_running[kBuckets];
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  if (threadIdx.x < kBuckets) s_running[threadIdx.x] = 0;
+  __syncthreads();
+  for (int64_t base = 0; base < n_waves; base += kScanThreads) {
+    const int64_t i = base + threadIdx.x;
+    int count[kBuckets], upto[kBuckets];
+#pragma unroll
+    for (int k = 0; k < kBuckets; ++k) {
+      count[k] = i < n_waves ? wave_counts[i * kBuckets + k] : 0;
+      int v = count[k];
+#pragma unroll
+      for (int off = 1; off < kWaveSize; off <<= 1) {
+        const int from_below = __shfl_up(v, off);
+        if (lane >= off) v += from_below;
+      }
+      upto[k] = v;
+      if (lane == kWaveSize - 1) s_wave_total[k][w] = v;
+    }
+    __syncthreads();
+    if (i < n_waves) {
+#pragma unroll
+      for (int k = 0; k < kBuckets; ++k) {
+        int before = s_running[k];
+        for (int j = 0; j < w; ++j) before += s_wave_total[k][j];
+        wave_counts[i * kBuckets + k] = before + upto[k] - count[k];
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < kBuckets) {
+      int total = 0;
+      for (int j = 0; j < kScanWaves; ++j) total += s_wave_total[threadIdx.x][j];
+      s_running[threadIdx.x] += total;
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int k = 0; k < kBuckets; ++k) {
+      list_ptr[k] = at;
+      at += s_running[k];
+    }
+    list_ptr[kBuckets] = at;
   }
 }
 
-// counts[0 .. 7]: entries per range (from the kernel above); counts[8 .. 15]: slots handed out so far.
-// list_ptr[b] = start of range b's list; entries go to entry_pos / entry_row / entry_col.
+// The entries of every piece go to their places in the lists: range b's part of piece `wave`
+// starts at list_ptr[b] + wave_offsets[wave][b] (from the scan above).
 __global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_fill_kernel(
     int M, int64_t nnz, int cols_per_bucket, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
-    int *__restrict__ counts, int *__restrict__ list_ptr, int *__restrict__ entry_pos,
+    const int *__restrict__ wave_offsets, const int *__restrict__ list_ptr, int *__restrict__ entry_pos,
     int *__restrict__ entry_row, int *__restrict__ entry_col) {
   const int lane = wave_lane();
-  int start[kBuckets];
-  {
-    int run = 0;
-#pragma unroll
-    for (int k = 0; k < kBuckets; ++k) {
-      start[k] = run;
-      run += counts[k];
-    }
-    if (blockIdx.x == 0 && threadIdx.x <= kBuckets) {
-      int at = 0;
-      for (int k = 0; k < (int)threadIdx.x; ++k) at += counts[k];
-      list_ptr[threadIdx.x] = at;
-    }
-  }
   const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWaveSize;
   const int64_t first = wave * kEntriesPerWave;
   if (first >= nnz) return;
@@ -221,7 +266,6 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_fill_kernel(
   constexpr int kRounds = kEntriesPerWave / kWaveSize;
   int col[kRounds], row[kRounds];
   unsigned bucket[kRounds];
-  int mine[kBuckets] = {0};
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) {
     const int64_t p = first + r * kWaveSize + lane;
@@ -232,23 +276,13 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_bucket_fill_kernel(
       row[r] = sddmm_entry_row(row_ptr, row_lo, row_hi, p);
       bucket[r] = (unsigned)col[r] / (unsigned)cols_per_bucket;
     }
-#pragma unroll
-    for (int k = 0; k < kBuckets; ++k) mine[k] += bucket[r] == (unsigned)k;
   }
-  // slots of this wavefront in every list (one atomic per list), then every entry's slot: the
-  // wavefront's entries keep their order inside a list, so that a row's entries stay next to each
-  // other there (its row of A is then reused from the vector cache, and the entry's mask value
-  // and result lie next to its neighbours')
+  // every entry's slot: the wavefront's entries keep their order inside a list, so that a row's
+  // entries stay next to each other there (its row of A is then kept in registers, and the
+  // entry's mask value and result lie next to its neighbours')
   int base[kBuckets];
 #pragma unroll
-  for (int k = 0; k < kBuckets; ++k) {
-    int total = mine[k];
-#pragma unroll
-    for (int off = kWaveSize / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
-    int reserved = 0;
-    if (lane == 0 && total > 0) reserved = atomicAdd(&counts[kBuckets + k], total);
-    base[k] = start[k] + __shfl(reserved, 0);
-  }
+  for (int k = 0; k < kBuckets; ++k) base[k] = list_ptr[k] + wave_offsets[wave * kBuckets + k];
   const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (kWaveSize - lane));
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) {
@@ -435,25 +469,27 @@ inline size_t align_up_256(size_t v) { return (v + 255) / 256 * 256; }
 
 // Layout of the per-XCD entry lists inside the caller's buffer.
 struct SddmmLists {
-  int *counts;     // [16]
   int *list_ptr;   // [9]
   int *entry_pos, *entry_row, *entry_col;  // [nnz] each
+  int *wave_offsets;  // [pieces][kBuckets]: used while the lists are built
 };
+
+inline int64_t sddmm_pieces(int64_t nnz) { return (nnz + kEntriesPerWave - 1) / kEntriesPerWave; }
 
 inline SddmmLists sddmm_lists(void *buffer, int64_t nnz) {
   char *base = static_cast<char *>(buffer);
   const size_t array = align_up_256((size_t)nnz * sizeof(int32_t));
   SddmmLists l;
-  l.counts = reinterpret_cast<int *>(base);
-  l.list_ptr = l.counts + 16;
+  l.list_ptr = reinterpret_cast<int *>(base) + 16;
   l.entry_pos = reinterpret_cast<int *>(base + 256);
   l.entry_row = reinterpret_cast<int *>(base + 256 + array);
   l.entry_col = reinterpret_cast<int *>(base + 256 + 2 * array);
+  l.wave_offsets = reinterpret_cast<int *>(base + 256 + 3 * array);
   return l;
 }
 
-__global__ void sddmm_lists_clear_kernel(int *counts) {
-  if (threadIdx.x < 32) counts[threadIdx.x] = 0;
+__global__ void sddmm_lists_clear_kernel(int *list_ptr) {
+  if (threadIdx.x <= kBuckets) list_ptr[threadIdx.x] = 0;
 }
 
 }  // namespace scorch
@@ -486,8 +522,10 @@ int scorch_hip_sddmm_csr_batched_f32(int64_t batch, int64_t M, int64_t n_cols, i
 
 size_t scorch_hip_sddmm_csr_lists_bytes(int64_t nnz) {
   if (nnz < 0) return 0;
-  // 16 counters and 9 list starts (256 bytes), then entry numbers, rows and columns
-  return 256 + 3 * scorch::align_up_256((size_t)nnz * sizeof(int32_t));
+  // the 9 list starts (256 bytes), entry numbers, rows and columns, and the per-piece offsets the
+  // build works with
+  return 256 + 3 * scorch::align_up_256((size_t)nnz * sizeof(int32_t)) +
+         scorch::align_up_256((size_t)scorch::sddmm_pieces(nnz) * scorch::kBuckets * sizeof(int32_t));
 }
 
 int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
@@ -507,17 +545,22 @@ int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int
                         scorch_hip_sddmm_csr_lists_bytes(nnz), lists_bytes);
   hipStream_t s = static_cast<hipStream_t>(stream);
   scorch::SddmmLists l = scorch::sddmm_lists(lists, nnz);
-  scorch::sddmm_lists_clear_kernel<<<1, 64, 0, s>>>(l.counts);
-  SCORCH_HIP_CHECK(hipGetLastError());
-  if (nnz == 0 || n_cols == 0) return SCORCH_HIP_OK;
+  if (nnz == 0 || n_cols == 0) {
+    scorch::sddmm_lists_clear_kernel<<<1, 64, 0, s>>>(l.list_ptr);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    return SCORCH_HIP_OK;
+  }
   const int cols_per_bucket = (int)((n_cols + scorch::kBuckets - 1) / scorch::kBuckets);
-  const int64_t waves = (nnz + scorch::kEntriesPerWave - 1) / scorch::kEntriesPerWave;
+  const int64_t waves = scorch::sddmm_pieces(nnz);
   const dim3 grid((unsigned)((waves + scorch::kWavesPerBlock - 1) / scorch::kWavesPerBlock));
-  scorch::sddmm_bucket_count_kernel<<<grid, scorch::kBlockThreads, 0, s>>>(nnz, cols_per_bucket, col_idx, l.counts);
+  scorch::sddmm_bucket_count_kernel<<<grid, scorch::kBlockThreads, 0, s>>>(nnz, cols_per_bucket, col_idx,
+                                                                          l.wave_offsets);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  scorch::sddmm_bucket_scan_kernel<<<1, scorch::kScanThreads, 0, s>>>(waves, l.wave_offsets, l.list_ptr);
   SCORCH_HIP_CHECK(hipGetLastError());
   scorch::sddmm_bucket_fill_kernel<<<grid, scorch::kBlockThreads, 0, s>>>((int)M, nnz, cols_per_bucket, row_ptr,
-                                                                         col_idx, l.counts, l.list_ptr, l.entry_pos,
-                                                                         l.entry_row, l.entry_col);
+                                                                         col_idx, l.wave_offsets, l.list_ptr,
+                                                                         l.entry_pos, l.entry_row, l.entry_col);
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }
