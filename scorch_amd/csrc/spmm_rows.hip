@@ -225,18 +225,42 @@ __global__ __launch_bounds__(kBlockThreads) void csr_inspect_kernel(int M, int K
     longest = len > longest ? len : longest;
     empty += len == 0;
   }
-  for (int64_t p = first; p < nnz; p += stride) bad_cols |= (unsigned)col_idx[p] >= (unsigned)K;
-  // one atomic of each kind per wavefront that has something to say
+  {
+    // four column indices per thread in flight
+    int64_t p = first;
+    for (; p + 3 * stride < nnz; p += 4 * stride) {
+      const unsigned c0 = (unsigned)col_idx[p], c1 = (unsigned)col_idx[p + stride];
+      const unsigned c2 = (unsigned)col_idx[p + 2 * stride], c3 = (unsigned)col_idx[p + 3 * stride];
+      bad_cols |= (c0 >= (unsigned)K) | (c1 >= (unsigned)K) | (c2 >= (unsigned)K) | (c3 >= (unsigned)K);
+    }
+    for (; p < nnz; p += stride) bad_cols |= (unsigned)col_idx[p] >= (unsigned)K;
+  }
+  // one atomic of each kind per workgroup that has something to say
 #pragma unroll
   for (int off = kWaveSize / 2; off > 0; off >>= 1) {
     const int other = __shfl_xor(longest, off);
     longest = other > longest ? other : longest;
     empty += __shfl_xor(empty, off);
   }
+  __shared__ int s_bad_rows, s_bad_cols, s_longest[kWavesPerBlock], s_empty[kWavesPerBlock];
+  if (threadIdx.x == 0) s_bad_rows = s_bad_cols = 0;
+  __syncthreads();
   const bool any_bad_rows = __any(bad_rows), any_bad_cols = __any(bad_cols);
   if (wave_lane() == 0) {
-    if (any_bad_rows) atomicOr(&report[0], 1);
-    if (any_bad_cols) atomicOr(&report[1], 1);
+    if (any_bad_rows) s_bad_rows = 1;
+    if (any_bad_cols) s_bad_cols = 1;
+    s_longest[threadIdx.x / kWaveSize] = longest;
+    s_empty[threadIdx.x / kWaveSize] = empty;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    longest = empty = 0;
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      longest = s_longest[w] > longest ? s_longest[w] : longest;
+      empty += s_empty[w];
+    }
+    if (s_bad_rows) atomicOr(&report[0], 1);
+    if (s_bad_cols) atomicOr(&report[1], 1);
     if (longest > 0) atomicMax(&report[2], longest);
     if (empty > 0) atomicAdd(&report[3], empty);  // at most M < 2^31 in all
   }
@@ -284,7 +308,7 @@ int scorch_hip_csr_inspect(int64_t M, int64_t K, int64_t nnz, const int32_t *row
   SCORCH_HIP_CHECK(hipGetLastError());
   const int64_t work = (M > nnz ? M : nnz) + 1;
   int64_t blocks = (work + scorch::kBlockThreads - 1) / scorch::kBlockThreads;
-  if (blocks > 4096) blocks = 4096;
+  if (blocks > 2048) blocks = 2048;
   scorch::csr_inspect_kernel<<<dim3((unsigned)blocks), scorch::kBlockThreads, 0, s>>>((int)M, (int)K, nnz, row_ptr,
                                                                                     col_idx, report);
   SCORCH_HIP_CHECK(hipGetLastError());
