@@ -416,6 +416,38 @@ def test_steps_replay_from_a_hip_graph():
             assert torch.equal(got, want)
 
 
+def test_a_two_layer_gcn_forward_captured_once_and_replayed():
+    """scorch_amd.graphs.capture: the layers of a small GCN (dense product, fused SpMM + bias +
+    ReLU, dense product, fused SpMM + bias) as one graph; replays on new features equal the
+    eager pass bit for bit, with eager work and synchronisations between the replays."""
+    import scorch_amd as scorch
+    from scorch_amd import STensor, graphs
+    rng = np.random.default_rng(23)
+    n, f_in, hidden, classes = 2708, 1433, 16, 7          # the shape of the Cora citation graph
+    rp, ci, v = random_csr(rng, n, n, 0.002)
+    A = STensor.from_csr_arrays(dev(rp), dev(ci), dev(v), (n, n))
+    X = torch.randn(n, f_in, device="cuda")
+    W1, b1 = torch.randn(f_in, hidden, device="cuda") * 0.05, torch.randn(hidden, device="cuda")
+    W2, b2 = torch.randn(hidden, classes, device="cuda") * 0.2, torch.randn(classes, device="cuda")
+
+    def forward(x):
+        h = scorch.spmm_bias_act(A, x @ W1, b1, relu=True)
+        return scorch.spmm_bias_act(A, h @ W2, b2)
+
+    step = graphs.capture(forward, X)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for _ in range(4):
+        X.copy_(torch.randn(X.shape, device="cuda", generator=gen))
+        want = forward(X).clone()
+        torch.cuda.synchronize()
+        got = step()
+        torch.cuda.synchronize()
+        assert got is step.result and torch.equal(got, want)
+    dense = torch.sparse_csr_tensor(dev(rp).long(), dev(ci).long(), dev(v), size=(n, n)).to_dense().double()
+    ref = dense @ (torch.relu(dense @ (X.double() @ W1.double()) + b1.double()) @ W2.double()) + b2.double()
+    np.testing.assert_allclose(host(step()), host(ref), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("a_fmt,b_fmt", [("oo", "dd"), ("ds", "oo"), ("oo", "ds"), ("oo", "oo"), ("dd", "ds"),
                                          ("dd", "oo"), ("ds", "ds")])
