@@ -45,13 +45,16 @@ def _canonical(expression: str) -> str:
     return "".join(out)
 
 
+def _not_on_device(device) -> RuntimeError:
+    return RuntimeError("scorch_amd runs sparse kernels on HIP devices only; this operand is on "
+                        f"{device}. Move it with STensor.to('cuda') (host tensors belong to the "
+                        "reference's CPU kernels).")
+
+
 def _require_device(*tensors: STensor) -> None:
     for t in tensors:
         if not t.values.is_cuda:
-            raise RuntimeError(
-                "scorch_amd runs sparse kernels on HIP devices only; this operand is on "
-                f"{t.values.device}. Move it with STensor.to('cuda') (host tensors belong to the "
-                "reference's CPU kernels).")
+            raise _not_on_device(t.values.device)
 
 
 def _wrap(result_cpp, shape, fmt) -> STensor:
@@ -133,6 +136,7 @@ def _run_converted_matmul(a: STensor, b: STensor, requested, time_dict) -> Optio
 # dense operand and the result in STensors (two nn.Module constructions, most of the general
 # path's 30 us per call, against a kernel of a few microseconds).
 _direct_matmul: dict = {}
+_direct_fused: dict = {}
 
 
 def _matmul_csr_dense_direct(a: STensor, b: torch.Tensor, kwargs) -> Optional[torch.Tensor]:
@@ -370,15 +374,28 @@ def spmm_bias_act(a: STensor, b: Union[torch.Tensor, STensor], bias: torch.Tenso
     """``act(a @ b + bias)`` in one kernel: the call the reference's
     ``@scorch.compile`` makes when it recognises matmul -> add(bias) [-> relu]
     (src/scorch/trace.py:232-301).  Returns an (M, N) tensor."""
-    if isinstance(b, torch.Tensor):
-        b = STensor.from_torch(b)
     kinds = ("add", "relu") if relu else ("add",)
-    resolved = resolve_prebuilt_fused(str(a.format), str(b.format), kinds, a.values.dtype)
-    if resolved is None or b.values.dtype != a.values.dtype:
-        raise _not_prebuilt(f"fused matmul+{'+'.join(kinds)} for {a.format} x {b.format}, "
-                            f"{a.values.dtype}")
-    _require_device(a, b)
-    M, N = a.shape[0], b.shape[1]
-    out = resolved.fn([M, N], list(a.shape), a.index.mode_indices, a.values, list(b.shape),
-                      b.index.mode_indices, b.values, bias)
+    if isinstance(b, torch.Tensor) and b.layout == torch.strided and b.dim() == 2:
+        # a dense torch operand is handed to the kernel as it is (no STensor around it)
+        b_format, b_shape, b_index, b_values = "d,d", tuple(b.shape), [[], []], b.reshape(-1)
+        if b_values is not b and b_values.data_ptr() == b.data_ptr():
+            b_values._scorch_origin = b
+    else:
+        if isinstance(b, torch.Tensor):
+            b = STensor.from_torch(b)
+        b_format, b_shape, b_index, b_values = str(b.format), tuple(b.shape), b.index.mode_indices, b.values
+    key = (str(a.format), b_format, kinds, a.values.dtype)
+    fn = _direct_fused.get(key)
+    if fn is None:
+        resolved = resolve_prebuilt_fused(key[0], b_format, kinds, a.values.dtype)
+        if resolved is None:
+            raise _not_prebuilt(f"fused matmul+{'+'.join(kinds)} for {a.format} x {b_format}, {a.values.dtype}")
+        fn = _direct_fused[key] = resolved.fn
+    if b_values.dtype != a.values.dtype:
+        raise _not_prebuilt(f"fused matmul+{'+'.join(kinds)} for {a.values.dtype} x {b_values.dtype}")
+    for values in (a.values, b_values):
+        if not values.is_cuda:
+            raise _not_on_device(values.device)
+    M, N = a.shape[0], b_shape[1]
+    out = fn((M, N), a.shape, a.index.mode_indices, a.values, b_shape, b_index, b_values, bias)
     return out.storage.value.view(M, N)
