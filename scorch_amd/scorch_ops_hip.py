@@ -29,6 +29,11 @@ import torch
 
 from . import native
 
+# Every buffer this module allocates comes from these two names, so that a test can put a
+# poisoning allocator in their place: no kernel may depend on what a fresh buffer holds.
+_empty = torch.empty
+_empty_like = torch.empty_like
+
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
 
@@ -71,11 +76,11 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     same stream use, or that was replaced by a larger one and returned to the
     allocator since the capture."""
     if torch.cuda.is_current_stream_capturing():
-        return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        return _empty(max(nbytes, 256), dtype=torch.uint8, device=device)
     key = (device.index, stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        buf = _empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
 
@@ -197,7 +202,7 @@ def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, wha
     if torch.cuda.is_current_stream_capturing():
         return None
     dev = pos.device
-    report = torch.empty(4, dtype=torch.int32, device=dev)
+    report = _empty(4, dtype=torch.int32, device=dev)
     with _on_device(dev):
         native.check(native.lib().scorch_hip_csr_inspect(n_rows, n_cols, crd.numel(), pos.data_ptr(),
                                                          crd.data_ptr(), report.data_ptr(), _stream(dev)))
@@ -221,7 +226,7 @@ def _chunk_bounds(plan: CsrPlan, pos: torch.Tensor, M: int, nnz: int, N: int, el
     """Chunk boundaries of the merge-path split for dense width N, computed once."""
     bounds = plan.bounds.get((N, elem))
     if bounds is None:
-        bounds = torch.empty(L.scorch_hip_spmm_csr_bounds_bytes(M, nnz, N, elem), dtype=torch.uint8,
+        bounds = _empty(L.scorch_hip_spmm_csr_bounds_bytes(M, nnz, N, elem), dtype=torch.uint8,
                              device=pos.device)
         native.check(L.scorch_hip_spmm_csr_bounds(M, nnz, N, elem, pos.data_ptr(), bounds.data_ptr(),
                                                   bounds.numel(), stream))
@@ -253,7 +258,7 @@ def prepare_dense_operand(values: torch.Tensor, K: int, N: int) -> Optional[torc
     dev = values.device
     L = native.lib()
     flat = values if values.is_contiguous() else values.contiguous()
-    bt = torch.empty(L.scorch_hip_dense_tiled_bytes(K, N, 4) // 4, dtype=torch.float32, device=dev)
+    bt = _empty(L.scorch_hip_dense_tiled_bytes(K, N, 4) // 4, dtype=torch.float32, device=dev)
     with _on_device(dev):
         native.check(L.scorch_hip_dense_to_tiled_f32(K, N, flat.data_ptr(), bt.data_ptr(), bt.numel() * 4,
                                                      _stream(dev)))
@@ -309,7 +314,7 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
     if SPMM_PATH not in SPMM_PATHS:
         raise ValueError(f"scorch_ops_hip: SPMM_PATH is {SPMM_PATH!r}, expected one of {SPMM_PATHS}")
     plan = csr_plan(pos, crd, M, K, "A")
-    out = torch.empty(M * N, dtype=dtype, device=dev)
+    out = _empty(M * N, dtype=dtype, device=dev)
     L = native.lib()
     suffix = _SUFFIX[dtype]
     elem = a_val.element_size()
@@ -420,7 +425,7 @@ def _make_spgemm(dtype):
             stream = _stream(dev)
             need = L.scorch_hip_spgemm_csr_workspace_bytes(M, N, a_val.element_size())
             ws = _workspace(dev, stream, need)
-            c_pos = torch.empty(M + 1, dtype=torch.int32, device=dev)
+            c_pos = _empty(M + 1, dtype=torch.int32, device=dev)
             native.check(L.scorch_hip_spgemm_csr_symbolic(M, K, N, a_pos.data_ptr(), a_crd.data_ptr(),
                                                           b_pos.data_ptr(), b_crd.data_ptr(),
                                                           c_pos.data_ptr(), ws.data_ptr(), ws.numel(),
@@ -429,8 +434,8 @@ def _make_spgemm(dtype):
             if nnz < 0:
                 raise native.ScorchHipError(native.EUNSUPPORTED,
                                             "SpGEMM: the result has 2^31 entries or more, beyond its int32 row pointer")
-            c_crd = torch.empty(nnz, dtype=torch.int32, device=dev)
-            c_val = torch.empty(nnz, dtype=dtype, device=dev)
+            c_crd = _empty(nnz, dtype=torch.int32, device=dev)
+            c_val = _empty(nnz, dtype=dtype, device=dev)
             fn = getattr(L, "scorch_hip_spgemm_csr_numeric_" + _SUFFIX[dtype])
             native.check(fn(M, K, N, a_pos.data_ptr(), a_crd.data_ptr(), a_val.data_ptr(),
                             b_pos.data_ptr(), b_crd.data_ptr(), b_val.data_ptr(), c_pos.data_ptr(),
@@ -522,7 +527,7 @@ def _make_spmv(dtype):
             raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
         dev = _device_of(pos, crd, a_val, x)
         csr_plan(pos, crd, M, K, "A")
-        y = torch.empty(M, dtype=dtype, device=dev)
+        y = _empty(M, dtype=dtype, device=dev)
         L = native.lib()
         with _on_device(dev):
             stream = _stream(dev)
@@ -564,7 +569,7 @@ def _sddmm_lists(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, K: int,
         if plan.sddmm_lists is None and (plan.sddmm_uses < 2 or torch.cuda.is_current_stream_capturing()):
             return None
     if plan.sddmm_lists is None:
-        lists = torch.empty(L.scorch_hip_sddmm_csr_lists_bytes(crd.numel()), dtype=torch.uint8, device=pos.device)
+        lists = _empty(L.scorch_hip_sddmm_csr_lists_bytes(crd.numel()), dtype=torch.uint8, device=pos.device)
         native.check(L.scorch_hip_sddmm_csr_lists(M, n_cols, crd.numel(), pos.data_ptr(), crd.data_ptr(),
                                                   lists.data_ptr(), lists.numel(), stream))
         plan.sddmm_lists = lists
@@ -598,7 +603,7 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
     if row.numel() != s_val.numel() or col.numel() != s_val.numel():
         raise ValueError("scorch_ops_hip: S index and value lengths differ")
     dev = _device_of(row, col, s_val, a, b)
-    out = torch.empty_like(s_val)
+    out = _empty_like(s_val)
     with _on_device(dev):
         rc = native.lib().scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(),
                                                    col.data_ptr(), s_val.data_ptr(), a.data_ptr(),
@@ -619,8 +624,8 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
     dev = _device_of(pos, crd, s_val, a, b)
     plan = csr_plan(pos, crd, M, n_cols, "S")
-    out = torch.empty_like(s_val)
-    rows = torch.empty_like(crd)
+    out = _empty_like(s_val)
+    rows = _empty_like(crd)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
@@ -656,7 +661,7 @@ def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float 
     pos = _index(row_ptr, "row_ptr")
     v = _flat(values, torch.float32, "values")
     dev = _device_of(pos, v)
-    out = torch.empty_like(v)
+    out = _empty_like(v)
     L = native.lib()
     longest = _known_longest_row(pos, pos.numel() - 1, v.numel())
     with _on_device(dev):
@@ -678,7 +683,7 @@ def csr_row_indices(row_ptr: torch.Tensor, nnz: int) -> torch.Tensor:
     """Row of every stored entry of a CSR pattern (int32[nnz])."""
     pos = _index(row_ptr, "row_ptr")
     dev = _device_of(pos)
-    rows = torch.empty(nnz, dtype=torch.int32, device=dev)
+    rows = _empty(nnz, dtype=torch.int32, device=dev)
     with _on_device(dev):
         rc = native.lib().scorch_hip_csr_row_indices(pos.numel() - 1, nnz, pos.data_ptr(),
                                                      rows.data_ptr(), _stream(dev))
@@ -691,7 +696,7 @@ def coo_row_ptr(row_idx: torch.Tensor, n_rows: int) -> Optional[torch.Tensor]:
     if they are not sorted or lie outside [0, n_rows).  One host read of a flag."""
     rows = _index(row_idx, "row coordinates")
     dev = _device_of(rows)
-    pos = torch.empty(n_rows + 1, dtype=torch.int32, device=dev)
+    pos = _empty(n_rows + 1, dtype=torch.int32, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     with _on_device(dev):
         rc = native.lib().scorch_hip_coo_row_ptr(n_rows, rows.numel(), rows.data_ptr(), pos.data_ptr(),
@@ -770,8 +775,8 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     dev = _device_of(pos, crd, s_val, a, b)
     plan = csr_plan(pos, crd, M, n_cols, "S")
     nnz = s_val.numel()
-    out = torch.empty((H, nnz), dtype=torch.float32, device=dev)
-    rows = torch.empty_like(crd)
+    out = _empty((H, nnz), dtype=torch.float32, device=dev)
+    rows = _empty_like(crd)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
@@ -797,7 +802,7 @@ def softmax_csr_float_batched(row_ptr: torch.Tensor, values: torch.Tensor, scale
     v = values if values.is_contiguous() else values.contiguous()
     dev = _device_of(pos, v)
     H, nnz = int(v.shape[0]), int(v.shape[1])
-    out = torch.empty_like(v)
+    out = _empty_like(v)
     L = native.lib()
     longest = _known_longest_row(pos, pos.numel() - 1, nnz)
     with _on_device(dev):
@@ -831,7 +836,7 @@ def spmm_csr_float_batched(A_shape, A_mode_indices, A_values: torch.Tensor, B: t
         raise ValueError("scorch_ops_hip: array lengths do not match the shapes")
     dev = _device_of(pos, crd, a_val, b)
     plan = csr_plan(pos, crd, M, K, "A")
-    out = torch.empty((H, M, N), dtype=torch.float32, device=dev)
+    out = _empty((H, M, N), dtype=torch.float32, device=dev)
     if H == 0 or M == 0 or N == 0:
         return out
     L = native.lib()
@@ -1023,7 +1028,7 @@ def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     H, S, D = q.shape
     if S != bm.S:
         raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
-    out = torch.empty_like(q)
+    out = _empty_like(q)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
@@ -1059,7 +1064,7 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     H, S, D = q.shape
     if brp.numel() != S // block + 1:
         raise ValueError("scorch_ops_hip: block_row_ptr length does not match S / block")
-    out = torch.empty_like(q)
+    out = _empty_like(q)
     if block_mask_index is None:
         with _on_device(dev):
             rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),

@@ -26,6 +26,29 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(autouse=True)
+def poisoned_device_buffers(request, monkeypatch):
+    """Every GPU test runs with the package's fresh device buffers (results, workspaces, plans)
+    filled with NaN (floating point) or 0x7f bytes (everything else) before a kernel sees them:
+    a kernel that read memory it had not been given, or left part of a result unwritten, would
+    show here and not only when recycled memory happens to hold something harmful."""
+    if "gpu" not in request.keywords:
+        return
+    import torch
+    from scorch_amd import scorch_ops_hip as H
+
+    def poison(t):
+        if t.is_cuda and t.numel():
+            if t.dtype.is_floating_point:
+                t.fill_(float("nan"))
+            else:
+                t.view(torch.uint8).fill_(0x7F)
+        return t
+
+    monkeypatch.setattr(H, "_empty", lambda *a, **k: poison(torch.empty(*a, **k)))
+    monkeypatch.setattr(H, "_empty_like", lambda *a, **k: poison(torch.empty_like(*a, **k)))
+
+
 class Golden:
     """Cases of tests/golden/golden_ref.npz: golden.case("spmm_rect") -> dict of arrays."""
 
