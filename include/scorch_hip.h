@@ -398,7 +398,7 @@ SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int3
                                size_t workspace_bytes, void *stream);
 /* The same for `batch` value arrays over one pattern, for a caller that knows that no row has more
  * than 4096 entries (scorch_hip_csr_inspect reports the longest row): one launch, no workspace.
- * A longer row would be left unnormalised. */
+ * The entries of `out` that belong to a longer row would be left unwritten. */
 SCORCH_HIP_API int scorch_hip_softmax_csr_short_rows_f32(int64_t batch, int64_t M, int64_t nnz,
                                const int32_t *row_ptr, const float *vals, float scale, float *out,
                                void *stream);
