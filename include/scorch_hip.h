@@ -62,6 +62,12 @@ enum scorch_hip_status {
 
 /* Epilogue selector of scorch_hip_spmm_csr_bias_act_f32. */
 enum scorch_hip_act { SCORCH_HIP_ACT_NONE = 0, SCORCH_HIP_ACT_RELU = 1 };
+/* May be or-ed into the `act` argument of scorch_hip_spmm_csr_planned_<T>: the caller knows
+ * (scorch_hip_csr_inspect reports it) that most rows of A are empty.  C is then zeroed with one
+ * streaming fill and only the rows that have entries are written, as the reference does
+ * (csrc/spmm.h:2024-2025, 2052: memset, then empty rows skipped), instead of a row-sized store of
+ * zeros per empty row between the gathers.  Same result; ignored with a bias. */
+#define SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS 0x100
 
 /* ABI version of the loaded library (SCORCH_HIP_ABI_VERSION at build time). */
 SCORCH_HIP_API int scorch_hip_abi_version(void);

@@ -33,13 +33,21 @@
 
 namespace scorch {
 
+// C = 0 in 16-byte pieces with streaming stores (grid-stride).
+__global__ __launch_bounds__(kBlockThreads) void zero_fill_kernel(uint4 *__restrict__ out, int64_t pieces) {
+  const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+  typedef unsigned Native __attribute__((ext_vector_type(4)));
+  for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < pieces; i += stride)
+    __builtin_nontemporal_store(Native{0u, 0u, 0u, 0u}, reinterpret_cast<Native *>(out + i));
+}
+
 template <typename T, int VEC, int EPI>
 __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     int M, int N, const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
     const T *__restrict__ vals, const T *__restrict__ B, T *__restrict__ C,
     const T *__restrict__ bias, int64_t total_items, int items_per_chunk, int snap, int n_tiles,
     int64_t blocks_per_tile, int *__restrict__ carry_row, T *__restrict__ carry_val,
-    const Boundary *__restrict__ bounds, SpmmBatch batch) {
+    const Boundary *__restrict__ bounds, SpmmBatch batch, int zero_filled) {
   using A = typename Acc<T>::type;
   using VecT = Vec<T, VEC>;
   constexpr int kSlots = kItemsPerWave + kSnapItems;
@@ -94,9 +102,13 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 
   int x = x0;  // next row to finish
   int next_end = uniform(s_rp[w][1]);
+  // zero_filled: C holds zeros already (a matrix most of whose rows are empty: one streaming
+  // fill and then only the other rows, instead of row-sized zero stores mixed into the gathers);
+  // a row none of whose entries this chunk has seen then needs no store
+  bool touched = !zero_filled;
 
   auto flush_row = [&]() {
-    if (active) {
+    if (active && touched) {
       const bool partial = carry_in && x == x0;
       VecT o;
 #pragma unroll
@@ -106,6 +118,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = (A)0;
+    touched = !zero_filled;
     ++x;
     next_end = uniform(s_rp[w][x - x0 + 1]);
   };
@@ -124,6 +137,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_merge_kernel(
 
   auto consume = [&](int k, const VecT &b) {
     while (y0 + k == next_end) flush_row();  // markers that precede nonzero y0 + k
+    touched = true;
     const A a = (A)s_val[w][k];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
@@ -361,7 +375,7 @@ struct KernelTimer {
 template <typename T, int VEC, int EPI>
 int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_idx, const T *vals,
                 const T *B, const T *bias, T *C, void *workspace, hipStream_t stream,
-                KernelTimer *timer, const Boundary *bounds, int batch, int64_t K) {
+                KernelTimer *timer, const Boundary *bounds, int batch, int64_t K, bool zero_fill = false) {
   const SpmmSplit split = spmm_split(M, nnz, N, sizeof(T));
   const int64_t chunks = split.spans;
   const SpmmBatch strides = {nnz, K * N, (int64_t)M * N, chunks * N};
@@ -379,9 +393,18 @@ int launch_spmm(int M, int N, int64_t nnz, const int *row_ptr, const int *col_id
   const dim3 grid((unsigned)(blocks_per_tile * n_tiles), (unsigned)batch);
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[0], stream));
   mark_launch(stream);
+  zero_fill = zero_fill && EPI == kEpiNone && aligned_to(C, 16) && ((int64_t)batch * M * N * (int64_t)sizeof(T)) % 16 == 0;
+  if (zero_fill) {
+    const int64_t pieces = (int64_t)batch * M * N * (int64_t)sizeof(T) / 16;
+    const int64_t fill_blocks = (pieces + kBlockThreads * 8 - 1) / (kBlockThreads * 8);
+    zero_fill_kernel<<<dim3((unsigned)(fill_blocks < 65536 ? fill_blocks : 65536)), kBlockThreads, 0, stream>>>(
+        reinterpret_cast<uint4 *>(C), pieces);
+    SCORCH_HIP_CHECK(hipGetLastError());
+    mark_launch(stream);
+  }
   spmm_merge_kernel<T, VEC, EPI><<<grid, kBlockThreads, 0, stream>>>(
       M, N, row_ptr, col_idx, vals, B, C, bias, (int64_t)M + nnz, split.items_per_chunk,
-      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val, bounds, strides);
+      split.snap, n_tiles, blocks_per_tile, carry_row, carry_val, bounds, strides, zero_fill ? 1 : 0);
   SCORCH_HIP_CHECK(hipGetLastError());
   if (timer) SCORCH_HIP_CHECK(hipEventRecord(timer->ev[1], stream));
   mark_launch(stream);
@@ -457,7 +480,7 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
                const int32_t *col_idx, const T *vals, const T *B, const T *bias, T *C,
                void *workspace, size_t workspace_bytes, void *stream,
                KernelTimer *timer = nullptr, const void *bounds_buffer = nullptr, size_t bounds_bytes = 0,
-               int64_t batch = 1) {
+               int64_t batch = 1, bool mostly_empty_rows = false) {
   if (batch < 0 || batch > 65535)
     return fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
   if (batch == 0) return SCORCH_HIP_OK;
@@ -518,13 +541,13 @@ int spmm_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, con
   if constexpr (sizeof(T) == 4) {
     if (vec == 4)
       return launch_spmm<T, 4, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
-                                  (int)batch, K);
+                                  (int)batch, K, mostly_empty_rows);
   }
   if (vec == 2)
     return launch_spmm<T, 2, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
-                                  (int)batch, K);
+                                  (int)batch, K, mostly_empty_rows);
   return launch_spmm<T, 1, EPI>(m, n, nnz, row_ptr, col_idx, vals, B, bias, C, workspace, s, timer, bounds,
-                                  (int)batch, K);
+                                  (int)batch, K, mostly_empty_rows);
 }
 
 
@@ -911,10 +934,12 @@ int scorch_hip_spmm_csr_bounds(int64_t M, int64_t nnz, int64_t N, size_t elem_si
                                            size_t bounds_bytes, void *workspace, size_t workspace_bytes,    \
                                            void *stream) {                                                  \
     const char *fn = "scorch_hip_spmm_csr_planned_" #SUFFIX;                                                \
+    const bool mostly_empty = (act & SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS) != 0;                               \
+    act &= ~SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS;                                                              \
     if (!bias && act == SCORCH_HIP_ACT_NONE)                                                                \
       return scorch::spmm_entry<T, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, nullptr,  \
                                                      C, workspace, workspace_bytes, stream, nullptr,        \
-                                                     bounds, bounds_bytes);                                 \
+                                                     bounds, bounds_bytes, 1, mostly_empty);                \
     if (bias && act == SCORCH_HIP_ACT_NONE)                                                                 \
       return scorch::spmm_entry<T, scorch::kEpiBias>(fn, M, K, N, nnz, row_ptr, col_idx, vals, B, bias, C,  \
                                                      workspace, workspace_bytes, stream, nullptr, bounds,   \

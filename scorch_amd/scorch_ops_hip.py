@@ -34,6 +34,7 @@ from . import native
 _empty = torch.empty
 _empty_like = torch.empty_like
 
+HINT_MOSTLY_EMPTY_ROWS = 0x100      # SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS of include/scorch_hip.h
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
 
@@ -327,7 +328,10 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
             tiled = _tiled_operand(B_values, K, N, nnz, L)
         elif path == "tiled" and dtype == torch.float32:
             tiled = prepare_dense_operand(B_values, K, N)
-        if tiled is None and (path == "rows" or (path == "auto" and plan is not None
+        # most rows empty and a result large enough for two more launches not to show: one streaming
+        # fill of the result, then only the rows that have entries (merge-path kernel)
+        fill_first = plan is not None and bias is None and 2 * plan.empty_rows >= M and M * N * elem >= (32 << 20)
+        if tiled is None and (path == "rows" or (path == "auto" and plan is not None and not fill_first
                                                  and plan.max_row <= ROWS_KERNEL_MAX_ROW)):
             # every row is short: one launch of the row-split kernel, no workspace
             rc = getattr(L, "scorch_hip_spmm_csr_rows_" + suffix)(
@@ -344,9 +348,10 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
                                                  tiled.data_ptr(), tiled.numel() * 4, bias_ptr, act, out.data_ptr(),
                                                  bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
         else:
+            hint = HINT_MOSTLY_EMPTY_ROWS if fill_first else 0
             rc = getattr(L, "scorch_hip_spmm_csr_planned_" + suffix)(
-                M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(), bias_ptr, act,
-                out.data_ptr(), bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
+                M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(), b_val.data_ptr(), bias_ptr,
+                act | hint, out.data_ptr(), bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
     native.check(rc)
     result = Tensor(out, [[], []])
     result.workspace = ws      # a buffer handed out during a graph capture lives as long as the result

@@ -132,6 +132,44 @@ def test_precomputed_boundaries_change_nothing(N):
     assert np.array_equal(planned, searched)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+@pytest.mark.parametrize("N", [128, 520])
+def test_mostly_empty_rows_one_fill_then_only_the_rows_with_entries(oracle, dtype, N):
+    """SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS through the C ABI: the same result bit for bit as
+    without the hint, rows cut by chunk boundaries and a row of thousands of entries included;
+    and the Python layer takes that route by itself for a large result with mostly empty rows."""
+    rng = np.random.default_rng(31)
+    M, K = 70_000, 9_000
+    lens = np.where(rng.random(M) < 0.08, rng.integers(1, 40, M), 0).astype(np.int64)
+    lens[123] = 7000
+    lens[M - 1] = 300
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens if n]).astype(np.int32)
+    v = (rng.integers(-9, 9, ci.size) if np.issubdtype(dtype, np.integer) else rng.uniform(-1, 1, ci.size)).astype(dtype)
+    B = (rng.integers(-9, 9, (K, N)) if np.issubdtype(dtype, np.integer) else rng.standard_normal((K, N))).astype(dtype)
+    t_rp, t_ci, t_v, t_B = dev(rp), dev(ci), dev(v), dev(B).reshape(-1)
+    L = native.lib()
+    suffix = {np.float32: "f32", np.float64: "f64", np.int32: "i32"}[dtype]
+    elem = np.dtype(dtype).itemsize
+    ws = torch.empty(L.scorch_hip_spmm_csr_workspace_bytes(M, ci.size, N, elem), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for act in (0, H.HINT_MOSTLY_EMPTY_ROWS):
+        out = torch.full((M * N,), 77, dtype=t_v.dtype, device="cuda")
+        native.check(getattr(L, "scorch_hip_spmm_csr_planned_" + suffix)(
+            M, K, N, ci.size, t_rp.data_ptr(), t_ci.data_ptr(), t_v.data_ptr(), t_B.data_ptr(), None, act,
+            out.data_ptr(), None, 0, ws.data_ptr(), ws.numel(), stream))
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    want = oracle.spmm_fp64(rp, ci, v, B)
+    if np.issubdtype(dtype, np.integer):
+        assert np.array_equal(host(outs[1]).reshape(M, N), want.astype(dtype))
+    else:
+        assert oracle.rel_fro(host(outs[1]).reshape(M, N), want) <= TOL
+    auto = hip_spmm(rp, ci, v, B, path="auto")          # 36 MB and more of result, 92 % of the rows empty
+    assert np.array_equal(auto, host(outs[0]).reshape(M, N))
+
+
 def test_row_split_kernel_is_bit_reproducible_and_matches_the_reference(oracle):
     w = workloads.spmm_uniform()
     with spmm_path("rows"):
