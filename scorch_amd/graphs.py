@@ -11,7 +11,12 @@ What has to happen before the capture, and what ``capture`` therefore does:
 plans (index inspection, chunk boundaries, tiled copies, entry lists, block
 masks) are built on an operand's first or second use and need a
 synchronisation, which a capturing stream does not allow; the step is run
-eagerly on a side stream first, ``warmup`` times, so that they exist.
+eagerly on a side stream first, ``warmup`` times, so that they exist.  The plans
+of a sparse operand's index arrays (and of an attention mask) become part of the
+recording: values may be rewritten in place between replays, index arrays may
+not.  Plans that copy an operand's values (the column-tile copy of a wide dense
+operand) are never recorded; inside a graph such a product runs from the
+operand itself.
 
 The reference has no counterpart: its kernels run on the host.
 """

@@ -275,12 +275,16 @@ def _tiled_operand(values: torch.Tensor, K: int, N: int, nnz: int, L) -> Optiona
         return None
     if not tiled_operands_enabled() or not L.scorch_hip_dense_tiled_recommended(K, N, nnz, 4):
         return None
+    if torch.cuda.is_current_stream_capturing():
+        # a copy of the operand's values must not be recorded into a graph: a replay after the
+        # operand has been rewritten in place would read the old values, with nothing to notice it
+        return None
     owner = _dense_owner(values)
     stamp = (owner._version, values.data_ptr(), K, N)
     cached = getattr(owner, "_scorch_tiled", None)
     if cached is not None and cached[:4] == stamp:
         return cached[4]
-    if getattr(owner, "_scorch_seen", None) == stamp and not torch.cuda.is_current_stream_capturing():
+    if getattr(owner, "_scorch_seen", None) == stamp:
         return prepare_dense_operand(values, K, N)
     try:
         owner._scorch_seen = stamp

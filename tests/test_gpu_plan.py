@@ -229,6 +229,25 @@ def test_a_dense_operand_seen_twice_is_tiled_and_tracks_changes(oracle):
     assert oracle.rel_fro(host(fifth).reshape(512, 1024), 2 * ref64) <= TOL
 
 
+def test_a_recorded_step_never_reads_a_tiled_copy(oracle):
+    """A wide dense operand that has a column-tile copy (built during the warm-up) and is then
+    rewritten in place between replays of a captured step: every replay sees the new values."""
+    from scorch_amd import graphs
+    rng = np.random.default_rng(41)
+    M, K, N = 512, 2048, 2048
+    rp, ci, v = random_csr(rng, M, K, 0.01)
+    t_rp, t_ci, t_v = dev(rp), dev(ci), dev(v)
+    B = torch.randn(K * N, device="cuda")
+    product = lambda b: H.spmm_csr_float_v2([M, N], [M, K], [[], [t_rp, t_ci]], t_v, [K, N], [[], []], b).storage.value
+    step = graphs.capture(product, B, warmup=3)
+    assert getattr(B, "_scorch_tiled", None) is not None        # the eager warm-up did build the copy
+    for _ in range(3):
+        B.copy_(torch.randn(K * N, device="cuda"))
+        got = step().clone()
+        assert oracle.rel_fro(host(got).reshape(M, N), oracle.spmm_fp64(rp, ci, v, host(B).reshape(K, N))) <= TOL
+        assert torch.equal(got, product(B))                     # the eager call re-tiles and agrees bit for bit
+
+
 def test_matmul_keeps_the_tiled_copy_on_the_callers_tensor(oracle):
     import scorch_amd as scorch
     w = workloads.sae_decoder(M=256, K=2048, N=1024, k=16)
