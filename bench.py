@@ -490,6 +490,12 @@ def run_attention(args):
                                                 vf[h].reshape(-1)).storage.value)
             return outs
 
+        bm32 = H.BlockMask(S, w["block"], brp, bci, None, None, int(bci.numel()) * w["block"] * w["block"])
+        rec["fused_fp32"] = _vendor_time(
+            "the same attention in one fp32 kernel (fp32 operands, probabilities and sums; this package)",
+            lambda: H.attn_blocksparse_f32(qf, kf, vf, bm32, float(w["scale"])), max(args.steps // 2, 2), 2)
+        rec["fused_fp32"]["tflops"] = round(flops / rec["fused_fp32"]["ms_per_step"] / 1e9, 1)
+        rec["fused_fp32"]["frac_of_fp32_matrix_peak_157.3"] = round(rec["fused_fp32"]["tflops"] / 157.3, 3)
         rec["unfused_fp32_pipeline"] = _vendor_time("SDDMM -> softmax -> SpMM, one launch each for all heads "
                                                     "(this package, fp32)", unfused, max(args.steps // 4, 2), 1)
         rec["unfused_fp32_pipeline_per_head"] = _vendor_time(
@@ -611,6 +617,10 @@ def run_extra(args):
                              "distinct_block_masks": bm.n_masks,
                              "live_share_of_active_blocks": round(bm.density_in_blocks, 4),
                              "rel_fro_vs_fp32_pipeline": float(diff)}
+        # ... and through the fused fp32 kernel (fp32 operands, probabilities and sums)
+        ms_fused32 = _time_steps(lambda: H.sparse_attention_f32(q, k, v, rp, ci, scale), args.steps, args.warmup)
+        diff32 = (H.sparse_attention_f32(q, k, v, rp, ci, scale) - fn()).norm() / fn().norm()
+        out["fused_fp32"] = {"ms_per_step": round(ms_fused32, 5), "rel_fro_vs_fp32_pipeline": float(diff32)}
         if args.vendor:
             import torch.nn.functional as F
             rows = torch.repeat_interleave(torch.arange(S, device="cuda"), (rp[1:] - rp[:-1]).long())

@@ -463,6 +463,31 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_split_bf16(
     void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Fused block-sparse attention in fp32: the same computation as
+ * scorch_hip_attn_blocksparse_masked_bf16 / _split_bf16 with fp32 Q, K, V, O
+ * (H, S, D), fp32 probabilities and fp32 accumulation on the fp32 matrix
+ * instruction: the per-head SDDMM -> row softmax -> SpMM composition of
+ * bench/bench_sparse_transformer.py:354-372 in one kernel and at that
+ * composition's precision.  D = 32, 64 or 128, 64 x 64 blocks.
+ * block_mask_index may be NULL (every listed block fully live).  With
+ * n_items = 0 every block row is one workgroup's (block_row_ptr is read); with
+ * n_items > 0 the work items are `items` (4 x int32 each: block row, first and
+ * one-past-last position in block_col_idx, partial slot or -1), the block rows
+ * that were shared out are `split_rows` (block row, first slot, stretches, 0)
+ * and `workspace` (256-byte aligned,
+ * scorch_hip_attn_blocksparse_f32_workspace_bytes(H, n_slots, D)) takes their
+ * partial results; block_row_ptr is then not read.  The reference has no fused
+ * kernel.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API size_t scorch_hip_attn_blocksparse_f32_workspace_bytes(int64_t H, int64_t n_slots, int64_t D);
+SCORCH_HIP_API int scorch_hip_attn_blocksparse_f32(
+    int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, const int32_t *block_row_ptr,
+    const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks, const uint64_t *block_masks,
+    int64_t n_items, const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
+    const float *Q, const float *K, const float *V, float scale, float *O, void *workspace, size_t workspace_bytes,
+    void *stream);
+
+/* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's
  * sparse attention -- SDDMM, row softmax, SpMM, which its benchmark runs head by
  * head from a Python loop (bench/bench_sparse_transformer.py:325,354-372) -- each

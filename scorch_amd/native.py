@@ -100,6 +100,10 @@ SIGNATURES = {
     "scorch_hip_attn_blocksparse_split_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, _i64, _ptr, _i64,
                                                               _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, ctypes.c_float,
                                                               _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_attn_blocksparse_f32_workspace_bytes": (_size, [_i64, _i64, _i64]),
+    "scorch_hip_attn_blocksparse_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _i64,
+                                                       _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, ctypes.c_float, _ptr,
+                                                       _ptr, _size, _ptr]),
     "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "scorch_hip_coo_row_ptr": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
 }

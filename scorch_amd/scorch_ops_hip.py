@@ -1020,6 +1020,53 @@ def sparse_attention_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row
     return attn_blocksparse_split_bf16(q, k, v, bm, scale)
 
 
+def sparse_attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_ptr: torch.Tensor,
+                         col_idx: torch.Tensor, scale: float) -> torch.Tensor:
+    """softmax(scale * q k^T restricted to a CSR mask) v for fp32 q, k, v of shape (H, S, D), D in
+    {32, 64, 128}, S a multiple of 64, in one fused kernel with fp32 probabilities and sums: what
+    sparse_attention_csr computes in three launches (the reference's per-head composition,
+    bench/bench_sparse_transformer.py:354-372), to fp32 rounding.  The kernel computes every
+    64 x 64 block that holds an entry, so it pays for masks that fill their blocks reasonably."""
+    return attn_blocksparse_f32(q, k, v, attention_block_mask(row_ptr, col_idx, int(q.shape[1])), scale)
+
+
+def attn_blocksparse_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: BlockMask, scale: float) -> torch.Tensor:
+    """The fp32 fused attention kernel over a BlockMask (block_mask_index / block_masks may be None:
+    every listed block fully live; rows that split_long_block_rows shared out go through a
+    workspace and a second kernel)."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dtype != torch.float32 or t.dim() != 3:
+            raise TypeError(f"scorch_ops_hip: {name} must be a float32 tensor of shape (H, S, D)")
+    if q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
+    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+    index_tensors = [t for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index, bm.block_masks, bm.items,
+                                 bm.split_rows) if t is not None]
+    dev = _device_of(q, k, v, *index_tensors)
+    H, S, D = q.shape
+    if S != bm.S:
+        raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
+    ptr = lambda t: t.data_ptr() if t is not None and t.numel() else None
+    n_items = bm.items.numel() // 4 if bm.items is not None else 0
+    n_split = bm.split_rows.numel() // 4 if bm.split_rows is not None else 0
+    out = _empty_like(q)
+    L = native.lib()
+    with _on_device(dev):
+        stream = _stream(dev)
+        need = L.scorch_hip_attn_blocksparse_f32_workspace_bytes(H, bm.n_slots, D) if n_items else 0
+        ws = _workspace(dev, stream, need) if need else None
+        rc = L.scorch_hip_attn_blocksparse_f32(
+            H, S, D, bm.block, bm.n_active_blocks, ptr(bm.block_row_ptr), ptr(bm.block_col_idx),
+            ptr(bm.block_mask_index), bm.n_masks if bm.block_masks is not None else 0, ptr(bm.block_masks),
+            n_items, ptr(bm.items), n_split, ptr(bm.split_rows), bm.n_slots if n_items else 0,
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream)
+    native.check(rc)
+    if ws is not None:
+        out._scorch_workspace = ws     # a buffer handed out during a graph capture lives as long as the result
+    return out
+
+
 def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: BlockMask,
                                 scale: float) -> torch.Tensor:
     """attn_blocksparse_bf16 over a BlockMask whose long block rows split_long_block_rows has
