@@ -887,7 +887,7 @@ class BlockMask:
     of its 64-word bit mask (bit j of word r: query r of the block row attends to key j of the
     block).  Blocks with equal masks share one."""
     __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz",
-                 "items", "split_rows", "n_slots")
+                 "items", "split_rows", "n_slots", "schedule32")
 
     def __init__(self, S, block, block_row_ptr, block_col_idx, block_mask_index, block_masks, nnz):
         self.S, self.block, self.nnz = S, block, nnz
@@ -896,6 +896,7 @@ class BlockMask:
         # set by split_long_block_rows when some block row is shared out among workgroups
         self.items = self.split_rows = None
         self.n_slots = 0
+        self.schedule32 = None      # the fp32 kernel's own sharing-out (see _fp32_schedule)
 
     @property
     def n_active_blocks(self) -> int:
@@ -953,13 +954,14 @@ def block_mask_from_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) ->
                      masks.contiguous().view(-1), nnz)
 
 
-def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None) -> BlockMask:
+def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_unequal_rows: bool = False) -> BlockMask:
     """Share block rows with more than `longest` key blocks out among several workgroups (in
     stretches of equal length up to `longest`); by default `longest` is twice the mean number of
     key blocks per block row, at least 8, so that masks whose rows are of similar length are left
     alone and a row that attends to everything (a global token) is not the one workgroup the whole
     launch waits for.  Fills bm.items / bm.split_rows / bm.n_slots (None / None / 0 when no row is
-    long enough)."""
+    long enough -- unless `list_unequal_rows` asks for the rows, longest first, whenever they differ
+    in length)."""
     brp = bm.block_row_ptr.cpu().tolist()
     nb = len(brp) - 1
     lens = [brp[i + 1] - brp[i] for i in range(nb)]
@@ -968,7 +970,8 @@ def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None) -> Block
     bm.items = bm.split_rows = None
     bm.n_slots = 0
     if longest < 1 or max(lens, default=0) <= longest:
-        return bm
+        if not (list_unequal_rows and lens and min(lens) != max(lens)):
+            return bm
     items, split_rows, slot = [], [], 0
     for row, n in enumerate(lens):
         if n <= longest:
@@ -1030,6 +1033,31 @@ def sparse_attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, row_
     return attn_blocksparse_f32(q, k, v, attention_block_mask(row_ptr, col_idx, int(q.shape[1])), scale)
 
 
+FP32_ATTENTION_STRETCH = 16
+
+
+def _fp32_schedule(bm: BlockMask):
+    """(items, split_rows, n_slots) for the fp32 attention kernel, kept with the BlockMask.  Its
+    key blocks take six times as long as the bf16 kernel's, so what a stretch's partial results
+    cost matters little and an even load matters much: where block rows differ in length by more
+    than a quarter of the mean they go out in stretches of at most 16 key blocks (and at most
+    twice the mean, at least 8), longest first (a causal mask at S = 4096: a quarter less time);
+    rows of similar length stay whole.  Under stream capture a BlockMask that has no schedule yet
+    is served by whole rows."""
+    if bm.schedule32 is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None, None, 0
+        plain = BlockMask(bm.S, bm.block, bm.block_row_ptr, bm.block_col_idx, None, None, bm.nnz)
+        lens = (bm.block_row_ptr[1:] - bm.block_row_ptr[:-1]).cpu().tolist()
+        mean = sum(lens) / max(len(lens), 1)
+        longest = max(lens, default=0)
+        if longest > 1.25 * mean:      # (rows of similar length are best left whole)
+            longest = min(FP32_ATTENTION_STRETCH, max(8, 2 * math.ceil(mean)))
+        split_long_block_rows(plain, longest, list_unequal_rows=True)
+        bm.schedule32 = (plain.items, plain.split_rows, plain.n_slots)
+    return bm.schedule32
+
+
 def attn_blocksparse_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: BlockMask, scale: float) -> torch.Tensor:
     """The fp32 fused attention kernel over a BlockMask (block_mask_index / block_masks may be None:
     every listed block fully live; rows that split_long_block_rows shared out go through a
@@ -1040,25 +1068,26 @@ def attn_blocksparse_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: 
     if q.shape != k.shape or q.shape != v.shape:
         raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
     q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
-    index_tensors = [t for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index, bm.block_masks, bm.items,
-                                 bm.split_rows) if t is not None]
+    index_tensors = [t for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index, bm.block_masks)
+                     if t is not None]
     dev = _device_of(q, k, v, *index_tensors)
     H, S, D = q.shape
     if S != bm.S:
         raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
     ptr = lambda t: t.data_ptr() if t is not None and t.numel() else None
-    n_items = bm.items.numel() // 4 if bm.items is not None else 0
-    n_split = bm.split_rows.numel() // 4 if bm.split_rows is not None else 0
+    items, split_rows, n_slots = _fp32_schedule(bm)
+    n_items = items.numel() // 4 if items is not None else 0
+    n_split = split_rows.numel() // 4 if split_rows is not None else 0
     out = _empty_like(q)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
-        need = L.scorch_hip_attn_blocksparse_f32_workspace_bytes(H, bm.n_slots, D) if n_items else 0
+        need = L.scorch_hip_attn_blocksparse_f32_workspace_bytes(H, n_slots, D) if n_items else 0
         ws = _workspace(dev, stream, need) if need else None
         rc = L.scorch_hip_attn_blocksparse_f32(
             H, S, D, bm.block, bm.n_active_blocks, ptr(bm.block_row_ptr), ptr(bm.block_col_idx),
             ptr(bm.block_mask_index), bm.n_masks if bm.block_masks is not None else 0, ptr(bm.block_masks),
-            n_items, ptr(bm.items), n_split, ptr(bm.split_rows), bm.n_slots if n_items else 0,
+            n_items, ptr(items), n_split, ptr(split_rows), n_slots if n_items else 0,
             q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), out.data_ptr(),
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream)
     native.check(rc)
