@@ -1045,7 +1045,7 @@ def _fp32_schedule(bm: BlockMask):
     rows of similar length stay whole.  Under stream capture a BlockMask that has no schedule yet
     is served by whole rows."""
     if bm.schedule32 is None:
-        if torch.cuda.is_current_stream_capturing():
+        if bm.block_row_ptr.is_cuda and torch.cuda.is_current_stream_capturing():
             return None, None, 0
         plain = BlockMask(bm.S, bm.block, bm.block_row_ptr, bm.block_col_idx, None, None, bm.nnz)
         lens = (bm.block_row_ptr[1:] - bm.block_row_ptr[:-1]).cpu().tolist()

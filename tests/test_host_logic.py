@@ -422,3 +422,28 @@ def test_validate_accepts_well_formed_tensors_and_names_what_is_wrong():
     coo = STensor.from_coo(indices=torch.tensor([[0, 1, 2], [1, 0, 2]]), values=vals, shape=(2, 3))
     with pytest.raises(ValueError, match=r"outside \[0, 2\)"):
         coo.validate()
+
+
+def test_fp32_attention_schedule_covers_every_block_once_in_short_stretches():
+    from scorch_amd import scorch_ops_hip as H
+    nb = 64
+    brp = torch.tensor(np.concatenate([[0], np.cumsum(np.arange(1, nb + 1))]), dtype=torch.int32)      # causal
+    bci = torch.tensor(np.concatenate([np.arange(i + 1) for i in range(nb)]), dtype=torch.int32)
+    bm = H.BlockMask(nb * 64, 64, brp, bci, None, None, int(bci.numel()) * 4096)
+    items, split_rows, n_slots = H._fp32_schedule(bm)
+    items = items.view(-1, 4).tolist()
+    lengths = [e - b for _, b, e, _ in items]
+    assert max(lengths) <= H.FP32_ATTENTION_STRETCH and lengths == sorted(lengths, reverse=True)
+    covered = sorted(p for _, b, e, _ in items for p in range(b, e))
+    assert covered == list(range(bci.numel()))
+    for row, b, e, slot in items:
+        assert brp[row] <= b < e <= brp[row + 1] and (slot >= 0) == (brp[row + 1] - brp[row] > H.FP32_ATTENTION_STRETCH)
+    slots = sorted(slot for *_, slot in items if slot >= 0)
+    assert slots == list(range(n_slots))
+    for row, first, parts, _ in split_rows.view(-1, 4).tolist():
+        assert [it[3] for it in items if it[0] == row and it[3] >= 0].__len__() == parts and first >= 0
+    assert H._fp32_schedule(bm) is bm.schedule32                       # kept with the mask
+    # rows of equal length: nothing to list
+    even = H.BlockMask(256, 64, torch.arange(0, 17, 4, dtype=torch.int32), torch.arange(4, dtype=torch.int32).repeat(4),
+                       None, None, 16 * 4096)
+    assert H._fp32_schedule(even) == (None, None, 0)
