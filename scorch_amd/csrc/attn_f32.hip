@@ -172,9 +172,11 @@ __global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
     // a block that is only partly live: bit j of word i of its mask says whether query i of the
     // block row attends to key j of the block
     unsigned long long live = ~0ull;
+    bool partly_live = false;  // the same for the whole workgroup
     if (block_mask_index) {
       const int mask_at = uniform(block_mask_index[it]);
       if (mask_at >= 0) {
+        partly_live = true;
         live = block_masks[(size_t)mask_at * kBlock + my_query_in_block] >> (4 * g);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -191,23 +193,33 @@ __global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) mx = fmaxf(mx, st[t][r]);
     mx = combine_query_lanes(mx, [](float a, float b) { return fmaxf(a, b); });
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // (no maximum yet: exp2(0) on sums that are 0)
-    m_run = m_new;
-    l_run *= alpha;
+    if (__any(mx > m_run)) {  // some query's maximum rises: after a row's first key blocks, seldom
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // (no maximum yet: the sums are 0)
+      m_run = m_new;
+      l_run *= alpha;
 #pragma unroll
-    for (int dt = 0; dt < kFeat; ++dt)
+      for (int dt = 0; dt < kFeat; ++dt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
+        for (int r = 0; r < 4; ++r) o_acc[dt][r] *= alpha;
+    }
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float p = __builtin_amdgcn_exp2f(st[t][r] - m_run);
-        if (!((live >> (16 * t + r)) & 1ull)) p = 0.0f;  // (a query with no live key so far has m_run = kDead)
-        st[t][r] = p;
-        l_run += p;
-      }
+      for (int r = 0; r < 4; ++r) st[t][r] = __builtin_amdgcn_exp2f(st[t][r] - m_run);
+    if (partly_live) {
+      // an entry the mask leaves out: exp2(kDead - m_run) is 0 already unless the query has had no
+      // live key so far (m_run = kDead), so it is set
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (!((live >> (16 * t + r)) & 1ull)) st[t][r] = 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) l_run += st[t][r];
 
     // O^T += V^T P^T: step (t, r) contracts keys 16 t + 4 g + r, whose probabilities lane (g, n)
     // holds for query n; the V^T operand is V[that key][16 dt + n]
