@@ -11,8 +11,8 @@
 // v_mfma_f32_16x16x4_f32, which contracts four values per lane group at a sixteenth of the bf16
 // rate, so the kernel is bound by the matrix cores and everything around them is kept simple:
 // tiles go through registers into LDS rows padded by 16 bytes (no bank conflicts for either
-// operand), one tile in LDS and the next in registers, the running maximum is updated at every
-// key block.
+// operand), one tile in LDS and the next in registers, the accumulators are rescaled whenever a
+// query's running maximum rises.
 //
 // Lane (g, n) = (lane / 16, lane % 16).  An MFMA takes A[i = n][k = g] and B[k = g][j = n] and
 // adds to C[4g .. 4g+3][n].  Which four values of the contraction index a group of four MFMAs
