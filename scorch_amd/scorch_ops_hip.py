@@ -174,7 +174,7 @@ class CsrPlan:
     chunk boundaries of the merge-path kernels.  Lives as an attribute of the
     row-pointer tensor, so it is dropped with the operand, and is rebuilt when
     either index tensor has been written to since."""
-    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses")
+    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows")
 
     def __init__(self, key, max_row: int, empty_rows: int):
         self.key = key
@@ -183,6 +183,7 @@ class CsrPlan:
         self.bounds: Dict[Tuple[int, int], torch.Tensor] = {}
         self.sddmm_lists: Optional[torch.Tensor] = None   # the mask's entries listed per XCD (SDDMM)
         self.sddmm_uses = 0                                # SDDMM calls that could have used them
+        self.rows: Optional[torch.Tensor] = None           # the row coordinate of every entry (SDDMM results)
 
 
 def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, what: str = "operand") -> Optional[CsrPlan]:
@@ -621,6 +622,20 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
     return Tensor(out, S_mode_indices)
 
 
+def _result_rows(plan: Optional[CsrPlan], crd: torch.Tensor):
+    """The tensor of row coordinates for an SDDMM result over a CSR mask, and the pointer the
+    kernel is to write them through (None: nothing to write).  The coordinates depend on the
+    mask's pattern only: the first product with a planned mask writes them, later ones hand out
+    the same tensor -- as the reference hands out a coordinate mask's own index tensors
+    (src/scorch/ops.py:416-423) -- so a result's index tensors are not for writing to."""
+    if plan is not None and plan.rows is not None:
+        return plan.rows, None
+    rows = _empty_like(crd)
+    if plan is not None and not torch.cuda.is_current_stream_capturing():
+        plan.rows = rows
+    return rows, rows.data_ptr()
+
+
 def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_mode_indices, A_values,
                     B_shape, B_mode_indices, B_values):
     """SDDMM with a CSR mask.  The result is in coordinate format, one entry per
@@ -634,7 +649,7 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     dev = _device_of(pos, crd, s_val, a, b)
     plan = csr_plan(pos, crd, M, n_cols, "S")
     out = _empty_like(s_val)
-    rows = _empty_like(crd)
+    rows, rows_ptr = _result_rows(plan, crd)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
@@ -642,11 +657,11 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
         if lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                   rows.data_ptr(), stream)
+                                                   rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(), crd.data_ptr(),
                                             s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                            rows.data_ptr(), stream)
+                                            rows_ptr, stream)
     native.check(rc)
     return Tensor(out, [[rows], [crd]])
 
@@ -785,7 +800,7 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     plan = csr_plan(pos, crd, M, n_cols, "S")
     nnz = s_val.numel()
     out = _empty((H, nnz), dtype=torch.float32, device=dev)
-    rows = _empty_like(crd)
+    rows, rows_ptr = _result_rows(plan, crd)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
@@ -793,11 +808,11 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
         if lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                   rows.data_ptr(), stream)
+                                                   rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),
                                                     s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                    rows.data_ptr(), stream)
+                                                    rows_ptr, stream)
     native.check(rc)
     return out, rows
 

@@ -228,3 +228,28 @@ def test_einsum_with_dense_torch_operands_takes_the_direct_route(mask_format):
     times = {}
     again = scorch.einsum("ab,ac,bc->ab", S, Q, K, time_dict=times)      # other index names, same expression
     assert torch.equal(again.values, direct.values) and times["eval_time"] > 0
+
+
+def test_row_coordinates_of_a_planned_mask_are_written_once(oracle):
+    """The row coordinates of a CSR mask's SDDMM result depend on the pattern only: the first
+    product writes them, later ones hand out the same tensor (as the reference hands out a
+    coordinate mask's own index tensors), a changed pattern gets new ones."""
+    rng = np.random.default_rng(61)
+    M, C, K = 300, 200, 32
+    rp, ci, s = random_csr(rng, M, C, 0.1)
+    t_rp, t_ci, t_s = dev(rp), dev(ci), dev(s)
+    call = lambda A, B: H.sddmm_csr_float([M, C], [M, C], [[], [t_rp, t_ci]], t_s, [M, K], [[], []], A.reshape(-1),
+                                          [C, K], [[], []], B.reshape(-1))
+    A1, B1 = (torch.randn(n, K, device="cuda") for n in (M, C))
+    A2, B2 = (torch.randn(n, K, device="cuda") for n in (M, C))
+    first, second = call(A1, B1), call(A2, B2)
+    rows1, rows2 = first.storage.index.mode_indices[0][0], second.storage.index.mode_indices[0][0]
+    assert rows2 is rows1 and np.array_equal(host(rows1), oracle.rows_of(rp))
+    ref = oracle.sddmm_fp64(oracle.rows_of(rp), ci, s, host(A2), host(B2))
+    assert oracle.rel_fro(host(second.storage.value), ref) <= 1e-5
+    t_ci.copy_(torch.roll(t_ci, 1))                       # (any write: the plan no longer holds)
+    t_ci.copy_(dev(ci))
+    third = call(A1, B1)
+    rows3 = third.storage.index.mode_indices[0][0]
+    assert rows3 is not rows1 and torch.equal(rows3, rows1)
+    assert torch.equal(third.storage.value, first.storage.value)
