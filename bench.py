@@ -57,9 +57,9 @@ MEASURED_TRAFFIC = {
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
     ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "commit": "ea89918",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sddmm_uniform", "listed"): {"bytes": 360_500_000, "commit": "7ef9419",
+    ("sddmm_uniform", "listed"): {"bytes": 360_500_000, "commit": "ef63360",
                                   "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("sddmm_uniform", "plain"): {"bytes": 867_200_000, "commit": "7ef9419",
+    ("sddmm_uniform", "plain"): {"bytes": 867_200_000, "commit": "ef63360",
                                  "profile": "profiles/sddmm_kernels_uniform_65536.md"},
     ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "commit": "ea89918",
                                          "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
