@@ -53,7 +53,8 @@ struct Tile {
 constexpr float kDead = -3.0e38f;  // score of an entry the mask leaves out; also "no maximum yet"
 
 template <int D>
-__global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
+__global__ __launch_bounds__(kBlockThreads)
+__attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 4))) void attn_f32_kernel(
     int S, int n_blocks, int n_heads, const int *__restrict__ block_row_ptr,
     const int *__restrict__ block_col_idx, const int *__restrict__ block_mask_index,
     const unsigned long long *__restrict__ block_masks, const float *__restrict__ Q,
@@ -122,14 +123,17 @@ __global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
 
   // Tile traffic: thread `tid` moves chunks tid, tid + 256, ... (16 bytes each) of a 64 x D tile.
   floatx4 k_next[kCpt], v_next[kCpt];
-  auto fetch_tile = [&](int it) {
+  auto fetch_k = [&](int it) {
     const size_t tile = (size_t)uniform(block_col_idx[it]) * kBlock * D;
 #pragma unroll
-    for (int u = 0; u < kCpt; ++u) {
-      const int chunk = tid + u * kBlockThreads;
-      k_next[u] = *reinterpret_cast<const floatx4 *>(Kh + tile + (size_t)chunk * 4);
-      v_next[u] = *reinterpret_cast<const floatx4 *>(Vh + tile + (size_t)chunk * 4);
-    }
+    for (int u = 0; u < kCpt; ++u)
+      k_next[u] = *reinterpret_cast<const floatx4 *>(Kh + tile + (size_t)(tid + u * kBlockThreads) * 4);
+  };
+  auto fetch_v = [&](int it) {
+    const size_t tile = (size_t)uniform(block_col_idx[it]) * kBlock * D;
+#pragma unroll
+    for (int u = 0; u < kCpt; ++u)
+      v_next[u] = *reinterpret_cast<const floatx4 *>(Vh + tile + (size_t)(tid + u * kBlockThreads) * 4);
   };
   auto store_tile = [&]() {
 #pragma unroll
@@ -143,14 +147,17 @@ __global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
   const int my_query_in_block = w * 16 + n;
 
   if (kb_begin < kb_end) {
-    fetch_tile(kb_begin);
+    fetch_k(kb_begin);
+    fetch_v(kb_begin);
     store_tile();
   }
   __syncthreads();
 
   for (int it = kb_begin; it < kb_end; ++it) {
     const bool more = it + 1 < kb_end;
-    if (more) fetch_tile(it + 1);  // in flight while this block is computed
+    if (more) fetch_k(it + 1);  // in flight while this block is computed (V follows after the scores:
+                                // the two sets of staging registers are then not live at once with
+                                // the K operands)
 
     // S^T = K Q^T: tile t holds keys 16 t + 4 g + r (r = 0 .. 3) against query n
     floatx4 st[4];
@@ -168,6 +175,8 @@ __global__ __launch_bounds__(kBlockThreads) void attn_f32_kernel(
         for (int t = 0; t < 4; ++t)
           st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(k_op[t][c], q_op[j][c], st[t], 0, 0, 0);
     }
+
+    if (more) fetch_v(it + 1);
 
     // a block that is only partly live: bit j of word i of its mask says whether query i of the
     // block row attends to key j of the block
