@@ -488,6 +488,41 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_f32(
     void *stream);
 
 /* ------------------------------------------------------------------------
+ * SDDMM and SpMM in fp32 for a CSR operand whose entries cluster in 64 x 64
+ * blocks (attention masks), on the fp32 matrix instruction: the same results
+ * as scorch_hip_sddmm_csr_batched_f32 and scorch_hip_spmm_csr_batched_f32 (the
+ * reference's csrc/kernels.h:508-570 and csrc/spmm.h:2007-2089 for every head,
+ * as bench/bench_sparse_transformer.py:354-372 composes them), up to the order
+ * of the fp32 sums, for a pattern the caller has described by blocks:
+ *   block_col_idx[n_active_blocks]    block column of every active block, block
+ *                                     row major;
+ *   block_words[n_active_blocks * 64] bit c of word r of a block: column c of
+ *                                     the block is stored in row r of it;
+ *   block_off[n_active_blocks * 64]   position in the CSR arrays of the first
+ *                                     stored entry of row r inside the block.
+ * Every row's column indices must increase strictly (the entry of bit c is
+ * then block_off + the number of set bits below c); the arrays are trusted.
+ * M and the sparse operand's column count must be multiples of 64, the dense
+ * operands 32, 64 or 128 wide.  `items` (4 x int32 each: block row, first and
+ * one-past-last position in block_col_idx, 0) are the work items: for the
+ * SDDMM any cover of the active blocks by stretches of block rows, for the
+ * SpMM every block row exactly once and whole (a block row without blocks
+ * gives zero rows).  A is (H, M, K), B is (H, n_cols, K) [SDDMM] or (H, K, N)
+ * [SpMM], mask_vals is [nnz] (shared by the heads), vals and out_vals are
+ * (H, nnz), C is (H, M, N).  out_row_idx (may be NULL) receives the row of
+ * every entry.  No workspace.
+ * ---------------------------------------------------------------------- */
+SCORCH_HIP_API int scorch_hip_sddmm_csr_blocked_f32(
+    int64_t H, int64_t M, int64_t n_cols, int64_t K, int64_t nnz, int64_t n_active_blocks,
+    const int32_t *block_col_idx, const uint64_t *block_words, const int32_t *block_off, int64_t n_items,
+    const int32_t *items, const float *mask_vals, const float *A, const float *B, float *out_vals,
+    int32_t *out_row_idx, void *stream);
+SCORCH_HIP_API int scorch_hip_spmm_csr_blocked_f32(
+    int64_t H, int64_t M, int64_t K, int64_t N, int64_t nnz, int64_t n_active_blocks, const int32_t *block_col_idx,
+    const uint64_t *block_words, const int32_t *block_off, int64_t n_items, const int32_t *items, const float *vals,
+    const float *B, float *C, void *stream);
+
+/* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's
  * sparse attention -- SDDMM, row softmax, SpMM, which its benchmark runs head by
  * head from a Python loop (bench/bench_sparse_transformer.py:325,354-372) -- each

@@ -174,7 +174,7 @@ class CsrPlan:
     chunk boundaries of the merge-path kernels.  Lives as an attribute of the
     row-pointer tensor, so it is dropped with the operand, and is rebuilt when
     either index tensor has been written to since."""
-    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows")
+    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows", "blocked")
 
     def __init__(self, key, max_row: int, empty_rows: int):
         self.key = key
@@ -184,6 +184,7 @@ class CsrPlan:
         self.sddmm_lists: Optional[torch.Tensor] = None   # the mask's entries listed per XCD (SDDMM)
         self.sddmm_uses = 0                                # SDDMM calls that could have used them
         self.rows: Optional[torch.Tensor] = None           # the row coordinate of every entry (SDDMM results)
+        self.blocked = None                                # BlockedCsr, False (looked at: not blocky), None (not yet)
 
 
 def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, what: str = "operand") -> Optional[CsrPlan]:
@@ -234,6 +235,123 @@ def _chunk_bounds(plan: CsrPlan, pos: torch.Tensor, M: int, nnz: int, N: int, el
                                                   bounds.numel(), stream))
         plan.bounds[(N, elem)] = bounds
     return bounds
+
+
+# A CSR operand whose entries cluster in 64 x 64 blocks (an attention mask) is multiplied on the
+# fp32 matrix instruction, block by block, when its dense partner is 32, 64 or 128 wide.  "auto"
+# (SCORCH_HIP_BLOCKED overrides it at import) decides on the operand's first use, from the
+# share of the active blocks' positions that are stored; "off" keeps the general kernels,
+# "always" takes the block kernels for every operand they can serve, however thinly filled.
+BLOCKED_PATHS = ("auto", "off", "always")
+BLOCKED_PATH = os.environ.get("SCORCH_HIP_BLOCKED", "auto")
+# dense width -> share of the active blocks' positions that must be stored for the block kernels to
+# be the faster ones (measured on uniformly filled 4,096 x 4,096 masks, 8 heads: the general
+# kernels' time grows with the entries, the block kernels' with the blocks)
+BLOCKED_MIN_FILL = {32: 0.17, 64: 0.15, 128: 0.12}
+BLOCKED_WIDTHS = tuple(BLOCKED_MIN_FILL)
+BLOCKED_STRETCH = 16         # blocks per SDDMM work item at most
+BLOCKED_MAX_BLOCKS = 1 << 24  # blocks of the whole matrix: beyond, the operand is a graph, not a mask
+BLOCKED_MAX_NNZ = 1 << 27
+
+
+class BlockedCsr:
+    """A CSR pattern described by 64 x 64 blocks, for scorch_hip_{sddmm,spmm}_csr_blocked_f32:
+    the active blocks in block row major order, per block and row a word of stored columns and
+    the CSR position of the row's first entry in the block, and the two lists of work items."""
+    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "sddmm_items", "n_sddmm_items",
+                 "spmm_items", "n_block_rows", "longest_block_row", "fill")
+
+
+def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_fill: float) -> Optional[BlockedCsr]:
+    """The block description of (pos, crd), or None when the pattern is not one the block kernels
+    serve (dimensions not multiples of 64, rows not strictly increasing, blocks too thinly filled).
+    Torch operations on the operand's device and a few reads on the host; once per pattern."""
+    block = 64
+    nnz = int(crd.numel())
+    if M % block or n_cols % block or nnz == 0 or nnz > BLOCKED_MAX_NNZ:
+        return None
+    nbr, nbc = M // block, n_cols // block
+    if nbr * nbc > BLOCKED_MAX_BLOCKS or nnz < min_fill * block * M:   # (every block row has a block, usually)
+        return None
+    dev = pos.device
+    pos64, crd64 = pos.to(torch.int64), crd.to(torch.int64)
+    if min_fill > 0 and nbr > 3:
+        # three block rows tell a graph from a mask before anything of the operand's size is computed
+        picks = sorted({0, nbr // 2, nbr - 1})
+        ends = pos64[torch.tensor([x for b in picks for x in (b * block, (b + 1) * block)], device=dev)].tolist()
+        stored, blocks = 0, 0
+        for i, b in enumerate(picks):
+            lo, hi = ends[2 * i], ends[2 * i + 1]
+            if hi > lo:
+                stored += hi - lo
+                blocks += int(torch.unique(crd64[lo:hi] // block).numel())
+        if blocks == 0 or stored < 0.5 * min_fill * blocks * block * block:
+            return None
+    rows = torch.repeat_interleave(torch.arange(M, device=dev, dtype=torch.int64), pos64[1:] - pos64[:-1],
+                                   output_size=nnz)
+    if nnz > 1 and not bool(((crd64[1:] > crd64[:-1]) | (rows[1:] != rows[:-1])).all()):
+        return None                                   # a row with repeated or unordered columns
+    blocks, block_of = torch.unique(rows // block * nbc + crd64 // block, return_inverse=True)
+    n_active = int(blocks.numel())
+    fill = nnz / (n_active * block * block)
+    if fill < min_fill:
+        return None
+    key = block_of * block + rows % block
+    words = torch.zeros(n_active * block, dtype=torch.int64, device=dev)
+    # distinct bits: the sum is the union (1 << 63 wraps to the sign bit, as it should)
+    words.index_add_(0, key, torch.ones_like(crd64) << (crd64 % block))
+    first = torch.full((n_active * block,), nnz, dtype=torch.int64, device=dev)
+    first.scatter_reduce_(0, key, torch.arange(nnz, device=dev, dtype=torch.int64), "amin")
+    first[first == nnz] = 0
+    lens = torch.bincount(blocks // nbc, minlength=nbr).cpu().tolist()
+    sddmm_items, spmm_items, at = [], [], 0
+    for row, n in enumerate(lens):
+        spmm_items.append((n, row, at, at + n, 0))
+        parts = -(-n // BLOCKED_STRETCH)
+        for part in range(parts):
+            lo, hi = at + n * part // parts, at + n * (part + 1) // parts
+            sddmm_items.append((hi - lo, row, lo, hi, 0))
+        at += n
+    sddmm_items.sort(key=lambda it: -it[0])           # longest first
+    spmm_items.sort(key=lambda it: -it[0])
+    bl = BlockedCsr()
+    bl.n_active = n_active
+    bl.block_col_idx = (blocks % nbc).to(torch.int32)
+    bl.block_words = words
+    bl.block_off = first.to(torch.int32)
+    bl.sddmm_items = torch.tensor([it[1:] for it in sddmm_items], dtype=torch.int32, device=dev).reshape(-1)
+    bl.n_sddmm_items = len(sddmm_items)
+    bl.spmm_items = torch.tensor([it[1:] for it in spmm_items], dtype=torch.int32, device=dev).reshape(-1)
+    bl.n_block_rows = nbr
+    bl.longest_block_row = max(lens)
+    bl.fill = fill
+    return bl
+
+
+def _blocked(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, width: int) -> Optional[BlockedCsr]:
+    """The operand's block description if products with it go to the block kernels (decided on
+    its first use; never under a stream capture unless it was decided before)."""
+    if BLOCKED_PATH not in BLOCKED_PATHS:
+        raise ValueError(f"scorch_ops_hip: BLOCKED_PATH is {BLOCKED_PATH!r}, expected one of {BLOCKED_PATHS}")
+    if BLOCKED_PATH == "off" or plan is None or width not in BLOCKED_WIDTHS:
+        return None
+    if plan.blocked is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        least = 0.0 if BLOCKED_PATH == "always" else min(BLOCKED_MIN_FILL.values())
+        plan.blocked = _blocked_csr(pos, crd, M, n_cols, least) or False
+    bl = plan.blocked or None
+    if bl is not None and BLOCKED_PATH == "auto" and bl.fill < BLOCKED_MIN_FILL[width]:
+        return None
+    return bl
+
+
+def _blocked_spmm_balanced(bl: BlockedCsr) -> bool:
+    """A block row is one workgroup's work in the block SpMM: the longest must not be what the
+    launch waits for (a row that attends to everything among rows that attend to a window).
+    Judged from the pattern alone, so that a product takes the same kernel whatever the number
+    of heads it is batched with."""
+    return bl.longest_block_row <= max(8, 2 * -(-bl.n_active // bl.n_block_rows))
 
 
 def tiled_operands_enabled() -> bool:
@@ -336,6 +454,14 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
         # most rows empty and a result large enough for two more launches not to show: one streaming
         # fill of the result, then only the rows that have entries (merge-path kernel)
         fill_first = plan is not None and bias is None and 2 * plan.empty_rows >= M and M * N * elem >= (32 << 20)
+        if path == "auto" and tiled is None and dtype == torch.float32 and bias is None and act == 0:
+            bl = _blocked(plan, pos, crd, M, K, N)
+            if bl is not None and _blocked_spmm_balanced(bl):
+                native.check(L.scorch_hip_spmm_csr_blocked_f32(
+                    1, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
+                    bl.block_off.data_ptr(), bl.n_block_rows, bl.spmm_items.data_ptr(), a_val.data_ptr(),
+                    b_val.data_ptr(), out.data_ptr(), stream))
+                return Tensor(out, [[], []])
         if tiled is None and (path == "rows" or (path == "auto" and plan is not None and not fill_first
                                                  and plan.max_row <= ROWS_KERNEL_MAX_ROW)):
             # every row is short: one launch of the row-split kernel, no workspace
@@ -653,8 +779,15 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
-        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream)
-        if lists is not None:
+        bl = _blocked(plan, pos, crd, M, n_cols, K)
+        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
+        if bl is not None:
+            rc = L.scorch_hip_sddmm_csr_blocked_f32(1, M, n_cols, K, s_val.numel(), bl.n_active,
+                                                    bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
+                                                    bl.block_off.data_ptr(), bl.n_sddmm_items,
+                                                    bl.sddmm_items.data_ptr(), s_val.data_ptr(), a.data_ptr(),
+                                                    b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+        elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
                                                    rows_ptr, stream)
@@ -804,8 +937,14 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
-        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream)
-        if lists is not None:
+        bl = _blocked(plan, pos, crd, M, n_cols, K) if H > 0 else None
+        lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
+        if bl is not None:
+            rc = L.scorch_hip_sddmm_csr_blocked_f32(H, M, n_cols, K, nnz, bl.n_active, bl.block_col_idx.data_ptr(),
+                                                    bl.block_words.data_ptr(), bl.block_off.data_ptr(),
+                                                    bl.n_sddmm_items, bl.sddmm_items.data_ptr(), s_val.data_ptr(),
+                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+        elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
                                                    rows_ptr, stream)
@@ -866,7 +1005,13 @@ def spmm_csr_float_batched(A_shape, A_mode_indices, A_values: torch.Tensor, B: t
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
-        if SPMM_PATH == "rows" or (SPMM_PATH == "auto" and plan is not None and plan.max_row <= ROWS_KERNEL_MAX_ROW):
+        bl = _blocked(plan, pos, crd, M, K, N) if SPMM_PATH == "auto" else None
+        if bl is not None and _blocked_spmm_balanced(bl):
+            rc = L.scorch_hip_spmm_csr_blocked_f32(H, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(),
+                                                   bl.block_words.data_ptr(), bl.block_off.data_ptr(),
+                                                   bl.n_block_rows, bl.spmm_items.data_ptr(), a_val.data_ptr(),
+                                                   b.data_ptr(), out.data_ptr(), stream)
+        elif SPMM_PATH == "rows" or (SPMM_PATH == "auto" and plan is not None and plan.max_row <= ROWS_KERNEL_MAX_ROW):
             rc = L.scorch_hip_spmm_csr_rows_batched_f32(H, M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
                                                         a_val.data_ptr(), b.data_ptr(), out.data_ptr(), stream)
         else:

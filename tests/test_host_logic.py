@@ -447,3 +447,49 @@ def test_fp32_attention_schedule_covers_every_block_once_in_short_stretches():
     even = H.BlockMask(256, 64, torch.arange(0, 17, 4, dtype=torch.int32), torch.arange(4, dtype=torch.int32).repeat(4),
                        None, None, 16 * 4096)
     assert H._fp32_schedule(even) == (None, None, 0)
+
+
+def test_block_description_of_a_csr_pattern():
+    """_blocked_csr against a direct reading of the pattern: every stored entry is found at
+    block_off + (stored columns below it), every work-item list covers what it must."""
+    import numpy as np
+    import torch
+    from scorch_amd import scorch_ops_hip as H
+    rng = np.random.default_rng(0)
+    M, n_cols = 192, 320
+    mask = rng.random((M, n_cols)) < 0.3
+    mask[64:128] = False                                          # a block row without blocks
+    mask[:, 128:192] = False                                      # a block column without blocks
+    mask[130, :] = False                                          # an empty row inside an active block row
+    rp = np.zeros(M + 1, dtype=np.int32)
+    rp[1:] = np.cumsum(mask.sum(axis=1))
+    ci = np.nonzero(mask)[1].astype(np.int32)
+    bl = H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(ci), M, n_cols, 0.1)
+    assert bl is not None and bl.n_block_rows == 3 and abs(bl.fill - ci.size / (bl.n_active * 4096)) < 1e-12
+    cols = bl.block_col_idx.tolist()
+    words = bl.block_words.view(-1, 64).numpy().view(np.uint64)
+    offs = bl.block_off.view(-1, 64).numpy()
+    spmm_items = sorted(bl.spmm_items.view(-1, 4).tolist())
+    assert [it[0] for it in spmm_items] == [0, 1, 2] and spmm_items[1][1] == spmm_items[1][2]
+    seen = np.zeros(ci.size, dtype=bool)
+    for row_block, lo, hi, _ in spmm_items:
+        assert cols[lo:hi] == sorted(cols[lo:hi]) and 2 not in cols[lo:hi]
+        for b in range(lo, hi):
+            for r in range(64):
+                row = 64 * row_block + r
+                stored = [c for c in range(64) if mask[row, 64 * cols[b] + c]]
+                assert int(words[b, r]) == sum(1 << c for c in stored)
+                for rank, c in enumerate(stored):
+                    at = offs[b, r] + rank
+                    assert rp[row] <= at < rp[row + 1] and ci[at] == 64 * cols[b] + c and not seen[at]
+                    seen[at] = True
+    assert seen.all()
+    covered = sorted((lo, hi) for _, lo, hi, _ in bl.sddmm_items.view(-1, 4).tolist())
+    assert covered[0][0] == 0 and covered[-1][1] == bl.n_active
+    assert all(a[1] == b[0] for a, b in zip(covered, covered[1:])) and all(hi - lo <= H.BLOCKED_STRETCH for lo, hi in covered)
+    # what the description is not built for
+    assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(ci), M, n_cols, 0.5) is None     # too thinly filled
+    assert H._blocked_csr(torch.from_numpy(rp[:-1]), torch.from_numpy(ci[:rp[-2]]), M - 1, n_cols, 0.0) is None
+    backwards = ci.copy()
+    backwards[rp[3]:rp[4]] = backwards[rp[3]:rp[4]][::-1]
+    assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(backwards), M, n_cols, 0.0) is None
