@@ -508,8 +508,9 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_f32(
  * SDDMM any cover of the active blocks by stretches of block rows, for the
  * SpMM every block row exactly once and whole (a block row without blocks
  * gives zero rows).  A is (H, M, K), B is (H, n_cols, K) [SDDMM] or (H, K, N)
- * [SpMM], mask_vals is [nnz] (shared by the heads), vals and out_vals are
- * (H, nnz), C is (H, M, N).  out_row_idx (may be NULL) receives the row of
+ * [SpMM], mask_vals is [nnz] (shared by the heads; NULL: every value is 1, an
+ * attention mask, and nothing is read for it), vals and out_vals are (H, nnz),
+ * C is (H, M, N).  out_row_idx (may be NULL) receives the row of
  * every entry.  No workspace.
  * ---------------------------------------------------------------------- */
 SCORCH_HIP_API int scorch_hip_sddmm_csr_blocked_f32(

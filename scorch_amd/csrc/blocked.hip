@@ -83,8 +83,9 @@ __device__ __forceinline__ int bits_below_lane(unsigned long long word) {
 }
 
 // out[h][p] = mask_vals[p] * <A[h][row of p], B[h][column of p]> for the entries p of a stretch of
-// a block row.  items: x = block row, y and z = the stretch within block_col_idx.
-template <int D>
+// a block row (SCALED = false: mask_vals is not read, every value is taken to be 1 -- an
+// attention mask).  items: x = block row, y and z = the stretch within block_col_idx.
+template <int D, bool SCALED>
 __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 4))) void sddmm_blocked_kernel(
     int M, int n_cols, long long nnz, int n_heads, const int *__restrict__ block_col_idx,
     const unsigned long long *__restrict__ block_words, const int *__restrict__ block_off,
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
     // row's first plus c): its mask values are asked for before the products
     const bool whole = __all(word == ~0ull);
     float scale_of[16];
-    if (whole) {
+    if (SCALED && whole) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) scale_of[r] = mask_vals[__builtin_amdgcn_readlane(off, r) + lane];
     }
@@ -189,7 +190,8 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int at = __builtin_amdgcn_readlane(off, r) + lane;
-        store_streaming(out_h + at, scale_of[r] * mine[r * kRowStride + lane]);
+        const float x = mine[r * kRowStride + lane];
+        store_streaming(out_h + at, SCALED ? scale_of[r] * x : x);
         if (rows_out) rows_out[at] = first_row + r;
       }
     } else {
@@ -198,7 +200,8 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
         const unsigned long long stored = row_word(word, r);
         if ((stored >> lane) & 1ull) {
           const int at = __builtin_amdgcn_readlane(off, r) + bits_below_lane(stored);
-          store_streaming(out_h + at, mask_vals[at] * mine[r * kRowStride + lane]);
+          const float x = mine[r * kRowStride + lane];
+          store_streaming(out_h + at, SCALED ? mask_vals[at] * x : x);
           if (rows_out) rows_out[at] = first_row + r;
         }
       }
@@ -360,7 +363,7 @@ extern "C" int scorch_hip_sddmm_csr_blocked_f32(int64_t H, int64_t M, int64_t n_
                                         block_off, n_items, items);
   if (rc != SCORCH_HIP_OK) return rc;
   if (H == 0 || nnz == 0 || n_items == 0) return SCORCH_HIP_OK;
-  SCORCH_REQUIRE(mask_vals && A && B && out_vals, "%s: NULL operand", fn);
+  SCORCH_REQUIRE(A && B && out_vals, "%s: NULL operand", fn);
   SCORCH_REQUIRE(aligned_to(A, 16) && aligned_to(B, 16) && aligned_to(out_vals, 4) && aligned_to(mask_vals, 4),
                  "%s: A and B must be 16-byte aligned", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -368,13 +371,19 @@ extern "C" int scorch_hip_sddmm_csr_blocked_f32(int64_t H, int64_t M, int64_t n_
   const unsigned long long *words = reinterpret_cast<const unsigned long long *>(block_words);
   const int4 *item_list = reinterpret_cast<const int4 *>(items);
   mark_launch(s);
-#define SCORCH_BLOCKED_SDDMM(DIM)                                                                                  \
-  blocked::sddmm_blocked_kernel<DIM><<<grid, kBlockThreads, 0, s>>>((int)M, (int)n_cols, (long long)nnz, (int)H,   \
-                                                                    block_col_idx, words, block_off, mask_vals, A, \
-                                                                    B, out_vals, out_row_idx, (int)n_items, item_list)
-  if (K == 32) SCORCH_BLOCKED_SDDMM(32);
-  else if (K == 64) SCORCH_BLOCKED_SDDMM(64);
-  else SCORCH_BLOCKED_SDDMM(128);
+#define SCORCH_BLOCKED_SDDMM(DIM, SCALED)                                                                           \
+  blocked::sddmm_blocked_kernel<DIM, SCALED><<<grid, kBlockThreads, 0, s>>>(                                        \
+      (int)M, (int)n_cols, (long long)nnz, (int)H, block_col_idx, words, block_off, mask_vals, A, B, out_vals,      \
+      out_row_idx, (int)n_items, item_list)
+  if (mask_vals) {
+    if (K == 32) SCORCH_BLOCKED_SDDMM(32, true);
+    else if (K == 64) SCORCH_BLOCKED_SDDMM(64, true);
+    else SCORCH_BLOCKED_SDDMM(128, true);
+  } else {
+    if (K == 32) SCORCH_BLOCKED_SDDMM(32, false);
+    else if (K == 64) SCORCH_BLOCKED_SDDMM(64, false);
+    else SCORCH_BLOCKED_SDDMM(128, false);
+  }
 #undef SCORCH_BLOCKED_SDDMM
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);

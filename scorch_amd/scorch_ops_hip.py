@@ -346,6 +346,24 @@ def _blocked(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, width: int)
     return bl
 
 
+def _known_all_ones(values: torch.Tensor) -> bool:
+    """Whether a mask's values are known to be all 1 (an attention mask; the block SDDMM then
+    reads nothing for them).  Looked at when the same tensor comes back unchanged -- one
+    reduction and one read of its result -- and remembered with the tensor."""
+    key = (values.data_ptr(), values._version, values.numel())
+    seen = getattr(values, "_scorch_ones", None)
+    if seen is not None and seen[0] == key:
+        if seen[1] is None and not torch.cuda.is_current_stream_capturing():
+            seen = (key, bool((values == 1).all()))
+            values._scorch_ones = seen
+        return bool(seen[1])
+    try:
+        values._scorch_ones = (key, None)
+    except (AttributeError, RuntimeError):
+        pass
+    return False
+
+
 def _blocked_spmm_balanced(bl: BlockedCsr) -> bool:
     """A block row is one workgroup's work in the block SpMM: the longest must not be what the
     launch waits for (a row that attends to everything among rows that attend to a window).
@@ -785,8 +803,9 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
             rc = L.scorch_hip_sddmm_csr_blocked_f32(1, M, n_cols, K, s_val.numel(), bl.n_active,
                                                     bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
                                                     bl.block_off.data_ptr(), bl.n_sddmm_items,
-                                                    bl.sddmm_items.data_ptr(), s_val.data_ptr(), a.data_ptr(),
-                                                    b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+                                                    bl.sddmm_items.data_ptr(),
+                                                    None if _known_all_ones(s_val) else s_val.data_ptr(),
+                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
@@ -921,29 +940,35 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     """out[h, p] = S.val[p] * <A[h, i_p, :], B[h, j_p, :]> for every head h and stored entry p of
     the CSR mask S: the SDDMM step of the reference's sparse attention for all heads in one launch
     (bench/bench_sparse_transformer.py:354-361 runs it per head).  A is (H, M, K), B is (H, n_cols, K).
+    S_values may be None: every stored entry of the mask is 1 (a tensor of ones is made only if
+    the kernel that serves the mask reads one).
     Returns (values of shape (H, nnz), row coordinates int32[nnz])."""
     M, n_cols = int(S_shape[0]), int(S_shape[1])
     pos, crd = _csr_parts(S_mode_indices, "S")
-    s_val = _flat(S_values, torch.float32, "S values")
+    s_val = _flat(S_values, torch.float32, "S values") if S_values is not None else None
     H, K = int(A.shape[0]), int(A.shape[2])
     a, b = _batched_dense(A, H, M, K, "A"), _batched_dense(B, H, n_cols, K, "B")
-    if pos.numel() != M + 1 or crd.numel() != s_val.numel():
+    nnz = crd.numel()
+    if pos.numel() != M + 1 or (s_val is not None and nnz != s_val.numel()):
         raise ValueError("scorch_ops_hip: S array lengths do not match its shape")
-    dev = _device_of(pos, crd, s_val, a, b)
+    dev = _device_of(pos, crd, a, b) if s_val is None else _device_of(pos, crd, s_val, a, b)
     plan = csr_plan(pos, crd, M, n_cols, "S")
-    nnz = s_val.numel()
     out = _empty((H, nnz), dtype=torch.float32, device=dev)
     rows, rows_ptr = _result_rows(plan, crd)
     L = native.lib()
     with _on_device(dev):
         stream = _stream(dev)
         bl = _blocked(plan, pos, crd, M, n_cols, K) if H > 0 else None
+        if bl is None and s_val is None:
+            s_val = torch.ones(nnz, dtype=torch.float32, device=dev)
         lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
         if bl is not None:
+            ones = s_val is None or _known_all_ones(s_val)
             rc = L.scorch_hip_sddmm_csr_blocked_f32(H, M, n_cols, K, nnz, bl.n_active, bl.block_col_idx.data_ptr(),
                                                     bl.block_words.data_ptr(), bl.block_off.data_ptr(),
-                                                    bl.n_sddmm_items, bl.sddmm_items.data_ptr(), s_val.data_ptr(),
-                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+                                                    bl.n_sddmm_items, bl.sddmm_items.data_ptr(),
+                                                    None if ones else s_val.data_ptr(), a.data_ptr(), b.data_ptr(),
+                                                    out.data_ptr(), rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
@@ -1034,9 +1059,8 @@ def sparse_attention_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, q: torch.
     SpMM per head) as three launches for all heads.  Any mask, any head dimension; rows of the mask
     without entries give zero rows."""
     H, S, D = (int(x) for x in q.shape)
-    ones = torch.ones(col_idx.numel(), dtype=torch.float32, device=q.device)
     mask = [[], [row_ptr, col_idx]]
-    scores, _ = sddmm_csr_float_batched([S, S], mask, ones, q, k)
+    scores, _ = sddmm_csr_float_batched([S, S], mask, None, q, k)
     probs = softmax_csr_float_batched(row_ptr, scores, scale)
     return spmm_csr_float_batched([S, S], mask, probs, v)
 

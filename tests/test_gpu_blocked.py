@@ -250,3 +250,28 @@ def test_entry_points_refuse_what_they_do_not_serve():
         1, 128, 64, 64, 4096, 1, col.data_ptr(), words.data_ptr(), off.data_ptr(), n_items, items.data_ptr(),
         z.data_ptr(), z.data_ptr(), torch.zeros(128 * 64, device="cuda").data_ptr(), None)
     assert spmm(1) == native.EINVAL and "every block row" in native.last_error()
+
+
+def test_a_mask_of_ones_is_not_read(oracle):
+    rng = np.random.default_rng(13)
+    M = n_cols = 256
+    rp, ci = csr_of(pattern("causal", M, n_cols, rng))
+    _, A, B, _, _ = operands(rng, 2, M, n_cols, 64, ci.size)
+    pos, crd, a, b = dev(rp), dev(ci), dev(A), dev(B)
+    idx = [[], [pos, crd]]
+    ones = torch.ones(ci.size, device="cuda")
+    first, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)      # first sight of the values: read
+    assert ones._scorch_ones[1] is None
+    second, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)     # back unchanged: looked at, all 1
+    assert ones._scorch_ones[1] is True
+    third, _ = H.sddmm_csr_float_batched([M, n_cols], idx, None, a, b)
+    assert torch.equal(first, second) and torch.equal(first, third)
+    ref_rows = oracle.rows_of(rp)
+    assert oracle.rel_fro(host(first[1]), oracle.sddmm_fp64(ref_rows, ci, np.ones(ci.size, np.float32), A[1], B[1])) <= TOL
+    ones[7] = -2.0                                                           # written to: looked at again
+    changed, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)
+    again, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)
+    assert ones._scorch_ones[1] is False and torch.equal(changed, again)
+    expect = first.clone()
+    expect[:, 7] *= -2.0
+    assert torch.equal(changed, expect)
