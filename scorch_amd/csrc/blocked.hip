@@ -272,11 +272,16 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
   };
   float row_next[16];
   auto fetch_values = [&]() {
+    if (__all(word_next == ~0ull)) {  // every row of the 16 fully stored: lane c's entry is the row's first plus c
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const unsigned long long stored = row_word(word_next, r);
-      const int at = __builtin_amdgcn_readlane(off_next, r) + bits_below_lane(stored);
-      row_next[r] = (stored >> lane) & 1ull ? vals_h[at] : 0.0f;
+      for (int r = 0; r < 16; ++r) row_next[r] = vals_h[__builtin_amdgcn_readlane(off_next, r) + lane];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const unsigned long long stored = row_word(word_next, r);
+        const int at = __builtin_amdgcn_readlane(off_next, r) + bits_below_lane(stored);
+        row_next[r] = (stored >> lane) & 1ull ? vals_h[at] : 0.0f;
+      }
     }
   };
 
