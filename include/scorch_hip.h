@@ -505,23 +505,30 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_f32(
  * M and the sparse operand's column count must be multiples of 64, the dense
  * operands 32, 64 or 128 wide.  `items` (4 x int32 each: block row, first and
  * one-past-last position in block_col_idx, 0) are the work items: for the
- * SDDMM any cover of the active blocks by stretches of block rows, for the
- * SpMM every block row exactly once and whole (a block row without blocks
- * gives zero rows).  A is (H, M, K), B is (H, n_cols, K) [SDDMM] or (H, K, N)
+ * SDDMM any cover of the active blocks by stretches of block rows (the fourth
+ * integer is not read); for the SpMM every block row either once and whole
+ * (fourth integer -1; a block row without blocks gives zero rows) or as
+ * consecutive stretches whose fourth integers are consecutive slots of
+ * `workspace` (256-byte aligned,
+ * scorch_hip_spmm_csr_blocked_workspace_bytes(H, n_slots, N)), named in
+ * `split_rows` (block row, first slot, stretches, 0): a second kernel adds a
+ * row's stretches up in their order, so the result does not depend on timing.  A is (H, M, K), B is (H, n_cols, K) [SDDMM] or (H, K, N)
  * [SpMM], mask_vals is [nnz] (shared by the heads; NULL: every value is 1, an
  * attention mask, and nothing is read for it), vals and out_vals are (H, nnz),
  * C is (H, M, N).  out_row_idx (may be NULL) receives the row of
- * every entry.  No workspace.
+ * every entry.
  * ---------------------------------------------------------------------- */
 SCORCH_HIP_API int scorch_hip_sddmm_csr_blocked_f32(
     int64_t H, int64_t M, int64_t n_cols, int64_t K, int64_t nnz, int64_t n_active_blocks,
     const int32_t *block_col_idx, const uint64_t *block_words, const int32_t *block_off, int64_t n_items,
     const int32_t *items, const float *mask_vals, const float *A, const float *B, float *out_vals,
     int32_t *out_row_idx, void *stream);
+SCORCH_HIP_API size_t scorch_hip_spmm_csr_blocked_workspace_bytes(int64_t H, int64_t n_slots, int64_t N);
 SCORCH_HIP_API int scorch_hip_spmm_csr_blocked_f32(
     int64_t H, int64_t M, int64_t K, int64_t N, int64_t nnz, int64_t n_active_blocks, const int32_t *block_col_idx,
-    const uint64_t *block_words, const int32_t *block_off, int64_t n_items, const int32_t *items, const float *vals,
-    const float *B, float *C, void *stream);
+    const uint64_t *block_words, const int32_t *block_off, int64_t n_items, const int32_t *items,
+    int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots, const float *vals, const float *B, float *C,
+    void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's

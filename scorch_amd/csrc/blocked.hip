@@ -213,14 +213,16 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
   }
 }
 
-// C[h][row] = sum over the row's entries p of vals[h][p] * B[h][column of p] for a block row.
-// items: x = block row, y and z = its range within block_col_idx (possibly empty: zero rows).
+// C[h][row] = sum over the row's entries p of vals[h][p] * B[h][column of p] for a block row or a
+// stretch of one.  items: x = block row, y and z = the range within block_col_idx (possibly empty:
+// zero rows), w = -1 if the item is the whole block row and writes C, else the slot of `partials`
+// (H x n_slots tiles of 64 x D) its sums go to, for spmm_blocked_merge_kernel to add up.
 template <int D>
 __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 4))) void spmm_blocked_kernel(
     int M, int K, long long nnz, int n_heads, const int *__restrict__ block_col_idx,
     const unsigned long long *__restrict__ block_words, const int *__restrict__ block_off,
     const float *__restrict__ vals, const float *__restrict__ B, float *__restrict__ C, int n_items,
-    const int4 *__restrict__ items) {
+    const int4 *__restrict__ items, int n_slots, float *__restrict__ partials) {
   using T = Tile<D>;
   constexpr int kStride = T::kStride;
   constexpr int kFeat = D / 16;
@@ -325,9 +327,34 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
     lds_barrier();
   }
 
-  float *c_row = C + ((size_t)head * M + row) * D;
+  const int slot = uniform(item.w);
+  float *c_row = slot < 0 ? C + ((size_t)head * M + row) * D
+                          : partials + (((size_t)head * n_slots + slot) * kBlock + in_block) * D;
 #pragma unroll
   for (int dt = 0; dt < kFeat; ++dt) *reinterpret_cast<floatx4 *>(c_row + 16 * dt + 4 * g) = acc[dt];
+}
+
+// The block rows that went out in stretches: C = the stretches' sums added in their order.
+// One workgroup per (split row, head); split_rows: x = block row, y = first slot, z = stretches.
+template <int D>
+__global__ __launch_bounds__(kBlockThreads) void spmm_blocked_merge_kernel(int M, int n_slots,
+                                                                           const int4 *__restrict__ split_rows,
+                                                                           const float *__restrict__ partials,
+                                                                           float *__restrict__ C) {
+  const int4 row = split_rows[blockIdx.x];
+  const int head = blockIdx.y;
+  constexpr int kTile = kBlock * D;  // floats; 256 threads x 4 floats per pass
+  const float *base = partials + ((size_t)head * n_slots + row.y) * kTile;
+  float *out = C + ((size_t)head * M + (size_t)row.x * kBlock) * D;
+  for (int at = threadIdx.x * 4; at < kTile; at += kBlockThreads * 4) {
+    floatx4 sum = *reinterpret_cast<const floatx4 *>(base + at);
+    for (int p = 1; p < row.z; ++p) {
+      const floatx4 x = *reinterpret_cast<const floatx4 *>(base + (size_t)p * kTile + at);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[r] += x[r];
+    }
+    *reinterpret_cast<floatx4 *>(out + at) = sum;
+  }
 }
 
 static int check_blocked(const char *fn, int64_t H, int64_t M, int64_t K, int64_t D, int64_t nnz, int64_t n_active,
@@ -395,37 +422,67 @@ extern "C" int scorch_hip_sddmm_csr_blocked_f32(int64_t H, int64_t M, int64_t n_
   return SCORCH_HIP_OK;
 }
 
+extern "C" size_t scorch_hip_spmm_csr_blocked_workspace_bytes(int64_t H, int64_t n_slots, int64_t N) {
+  if (H <= 0 || n_slots <= 0 || N <= 0) return 0;
+  return (size_t)H * (size_t)n_slots * scorch::blocked::kBlock * (size_t)N * sizeof(float);
+}
+
 extern "C" int scorch_hip_spmm_csr_blocked_f32(int64_t H, int64_t M, int64_t K, int64_t N, int64_t nnz,
                                                int64_t n_active_blocks, const int32_t *block_col_idx,
                                                const uint64_t *block_words, const int32_t *block_off,
-                                               int64_t n_items, const int32_t *items, const float *vals,
-                                               const float *B, float *C, void *stream) {
+                                               int64_t n_items, const int32_t *items, int64_t n_split_rows,
+                                               const int32_t *split_rows, int64_t n_slots, const float *vals,
+                                               const float *B, float *C, void *workspace, size_t workspace_bytes,
+                                               void *stream) {
   using namespace scorch;
   const char *fn = "scorch_hip_spmm_csr_blocked_f32";
   const int rc = blocked::check_blocked(fn, H, M, K, N, nnz, n_active_blocks, block_col_idx, block_words, block_off,
                                         n_items, items);
   if (rc != SCORCH_HIP_OK) return rc;
   if (H == 0 || M == 0) return SCORCH_HIP_OK;
-  if (n_items != M / blocked::kBlock)
-    return fail(SCORCH_HIP_EINVAL, "%s: %lld items for %lld block rows (every block row must be listed once)", fn,
+  if (n_split_rows < 0 || n_slots < 0 || n_slots > INT32_MAX || (n_split_rows == 0) != (n_slots == 0))
+    return fail(SCORCH_HIP_EINVAL, "%s: %lld split rows with %lld slots", fn, (long long)n_split_rows,
+                (long long)n_slots);
+  if (n_items < M / blocked::kBlock)
+    return fail(SCORCH_HIP_EINVAL, "%s: %lld items for %lld block rows (every block row must be covered)", fn,
                 (long long)n_items, (long long)(M / blocked::kBlock));
   SCORCH_REQUIRE((nnz == 0 || vals) && B && C, "%s: NULL operand", fn);
   SCORCH_REQUIRE(aligned_to(B, 16) && aligned_to(C, 16) && aligned_to(vals, 4), "%s: B and C must be 16-byte aligned",
                  fn);
+  float *partials = nullptr;
+  if (n_split_rows > 0) {
+    SCORCH_REQUIRE(split_rows != nullptr && aligned_to(split_rows, 16), "%s: split_rows must be 16-byte aligned", fn);
+    const size_t need = scorch_hip_spmm_csr_blocked_workspace_bytes(H, n_slots, N);
+    if (!workspace || workspace_bytes < need || !aligned_to(workspace, 256))
+      return fail(SCORCH_HIP_EWORKSPACE, "%s: a 256-byte aligned workspace of %zu bytes is needed, %zu given", fn,
+                  need, workspace ? workspace_bytes : (size_t)0);
+    partials = static_cast<float *>(workspace);
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(n_items * H));
+  const dim3 merge_grid((unsigned)n_split_rows, (unsigned)H);
   const unsigned long long *words = reinterpret_cast<const unsigned long long *>(block_words);
   const int4 *item_list = reinterpret_cast<const int4 *>(items);
+  const int4 *rows = reinterpret_cast<const int4 *>(split_rows);
   mark_launch(s);
-#define SCORCH_BLOCKED_SPMM(DIM)                                                                                \
-  blocked::spmm_blocked_kernel<DIM><<<grid, kBlockThreads, 0, s>>>((int)M, (int)K, (long long)nnz, (int)H,      \
-                                                                   block_col_idx, words, block_off, vals, B, C, \
-                                                                   (int)n_items, item_list)
+#define SCORCH_BLOCKED_SPMM(DIM)                                                                                  \
+  do {                                                                                                            \
+    blocked::spmm_blocked_kernel<DIM><<<grid, kBlockThreads, 0, s>>>((int)M, (int)K, (long long)nnz, (int)H,      \
+                                                                     block_col_idx, words, block_off, vals, B, C, \
+                                                                     (int)n_items, item_list, (int)n_slots,       \
+                                                                     partials);                                   \
+    SCORCH_HIP_CHECK(hipGetLastError());                                                                          \
+    mark_launch(s);                                                                                               \
+    if (n_split_rows > 0) {                                                                                       \
+      blocked::spmm_blocked_merge_kernel<DIM><<<merge_grid, kBlockThreads, 0, s>>>((int)M, (int)n_slots, rows,    \
+                                                                                   partials, C);                  \
+      SCORCH_HIP_CHECK(hipGetLastError());                                                                        \
+      mark_launch(s);                                                                                             \
+    }                                                                                                             \
+  } while (0)
   if (N == 32) SCORCH_BLOCKED_SPMM(32);
   else if (N == 64) SCORCH_BLOCKED_SPMM(64);
   else SCORCH_BLOCKED_SPMM(128);
 #undef SCORCH_BLOCKED_SPMM
-  SCORCH_HIP_CHECK(hipGetLastError());
-  mark_launch(s);
   return SCORCH_HIP_OK;
 }

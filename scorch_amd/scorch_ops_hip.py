@@ -259,7 +259,8 @@ class BlockedCsr:
     the active blocks in block row major order, per block and row a word of stored columns and
     the CSR position of the row's first entry in the block, and the two lists of work items."""
     __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "sddmm_items", "n_sddmm_items",
-                 "spmm_items", "n_block_rows", "longest_block_row", "fill")
+                 "spmm_items", "n_spmm_items", "spmm_split_rows", "n_spmm_split_rows", "n_spmm_slots",
+                 "n_block_rows", "longest_block_row", "fill")
 
 
 def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_fill: float) -> Optional[BlockedCsr]:
@@ -304,13 +305,27 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     first.scatter_reduce_(0, key, torch.arange(nnz, device=dev, dtype=torch.int64), "amin")
     first[first == nnz] = 0
     lens = torch.bincount(blocks // nbc, minlength=nbr).cpu().tolist()
-    sddmm_items, spmm_items, at = [], [], 0
+    # Work items.  SDDMM: stretches of at most BLOCKED_STRETCH blocks.  SpMM: a block row sums into one
+    # tile of the result, so it stays whole unless the rows differ by more than a quarter of their mean;
+    # then rows longer than twice the mean (8 to BLOCKED_STRETCH blocks) go out in stretches whose sums a
+    # second kernel adds up in order.
+    mean = n_active / nbr
+    spmm_longest = min(BLOCKED_STRETCH, max(8, 2 * -(-n_active // nbr))) if max(lens) > 1.25 * mean else max(lens)
+    sddmm_items, spmm_items, split_rows, at, slot = [], [], [], 0, 0
     for row, n in enumerate(lens):
-        spmm_items.append((n, row, at, at + n, 0))
         parts = -(-n // BLOCKED_STRETCH)
         for part in range(parts):
             lo, hi = at + n * part // parts, at + n * (part + 1) // parts
             sddmm_items.append((hi - lo, row, lo, hi, 0))
+        if n <= spmm_longest:
+            spmm_items.append((n, row, at, at + n, -1))
+        else:
+            parts = -(-n // spmm_longest)
+            split_rows.append((row, slot, parts, 0))
+            for part in range(parts):
+                lo, hi = at + n * part // parts, at + n * (part + 1) // parts
+                spmm_items.append((hi - lo, row, lo, hi, slot))
+                slot += 1
         at += n
     sddmm_items.sort(key=lambda it: -it[0])           # longest first
     spmm_items.sort(key=lambda it: -it[0])
@@ -322,6 +337,10 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     bl.sddmm_items = torch.tensor([it[1:] for it in sddmm_items], dtype=torch.int32, device=dev).reshape(-1)
     bl.n_sddmm_items = len(sddmm_items)
     bl.spmm_items = torch.tensor([it[1:] for it in spmm_items], dtype=torch.int32, device=dev).reshape(-1)
+    bl.n_spmm_items = len(spmm_items)
+    bl.spmm_split_rows = torch.tensor(split_rows, dtype=torch.int32, device=dev).reshape(-1)
+    bl.n_spmm_split_rows = len(split_rows)
+    bl.n_spmm_slots = slot
     bl.n_block_rows = nbr
     bl.longest_block_row = max(lens)
     bl.fill = fill
@@ -364,12 +383,20 @@ def _known_all_ones(values: torch.Tensor) -> bool:
     return False
 
 
-def _blocked_spmm_balanced(bl: BlockedCsr) -> bool:
-    """A block row is one workgroup's work in the block SpMM: the longest must not be what the
-    launch waits for (a row that attends to everything among rows that attend to a window).
-    Judged from the pattern alone, so that a product takes the same kernel whatever the number
-    of heads it is batched with."""
-    return bl.longest_block_row <= max(8, 2 * -(-bl.n_active // bl.n_block_rows))
+def _blocked_spmm(L, bl: BlockedCsr, heads: int, M: int, K: int, N: int, nnz: int, vals: torch.Tensor,
+                  b: torch.Tensor, out: torch.Tensor, stream: int) -> int:
+    """Launch the block SpMM for `heads` value arrays over one pattern."""
+    ws = None
+    if bl.n_spmm_slots:
+        ws = _workspace(out.device, stream, L.scorch_hip_spmm_csr_blocked_workspace_bytes(heads, bl.n_spmm_slots, N))
+        if torch.cuda.is_current_stream_capturing():
+            out._scorch_workspace = ws      # a buffer handed out during a capture lives as long as the result
+    return L.scorch_hip_spmm_csr_blocked_f32(
+        heads, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
+        bl.block_off.data_ptr(), bl.n_spmm_items, bl.spmm_items.data_ptr(), bl.n_spmm_split_rows,
+        bl.spmm_split_rows.data_ptr() if bl.n_spmm_split_rows else None, bl.n_spmm_slots, vals.data_ptr(),
+        b.data_ptr(), out.data_ptr(), ws.data_ptr() if ws is not None else None,
+        ws.numel() if ws is not None else 0, stream)
 
 
 def tiled_operands_enabled() -> bool:
@@ -474,11 +501,8 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
         fill_first = plan is not None and bias is None and 2 * plan.empty_rows >= M and M * N * elem >= (32 << 20)
         if path == "auto" and tiled is None and dtype == torch.float32 and bias is None and act == 0:
             bl = _blocked(plan, pos, crd, M, K, N)
-            if bl is not None and _blocked_spmm_balanced(bl):
-                native.check(L.scorch_hip_spmm_csr_blocked_f32(
-                    1, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
-                    bl.block_off.data_ptr(), bl.n_block_rows, bl.spmm_items.data_ptr(), a_val.data_ptr(),
-                    b_val.data_ptr(), out.data_ptr(), stream))
+            if bl is not None:
+                native.check(_blocked_spmm(L, bl, 1, M, K, N, nnz, a_val, b_val, out, stream))
                 return Tensor(out, [[], []])
         if tiled is None and (path == "rows" or (path == "auto" and plan is not None and not fill_first
                                                  and plan.max_row <= ROWS_KERNEL_MAX_ROW)):
@@ -1031,11 +1055,8 @@ def spmm_csr_float_batched(A_shape, A_mode_indices, A_values: torch.Tensor, B: t
     with _on_device(dev):
         stream = _stream(dev)
         bl = _blocked(plan, pos, crd, M, K, N) if SPMM_PATH == "auto" else None
-        if bl is not None and _blocked_spmm_balanced(bl):
-            rc = L.scorch_hip_spmm_csr_blocked_f32(H, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(),
-                                                   bl.block_words.data_ptr(), bl.block_off.data_ptr(),
-                                                   bl.n_block_rows, bl.spmm_items.data_ptr(), a_val.data_ptr(),
-                                                   b.data_ptr(), out.data_ptr(), stream)
+        if bl is not None:
+            rc = _blocked_spmm(L, bl, H, M, K, N, nnz, a_val, b, out, stream)
         elif SPMM_PATH == "rows" or (SPMM_PATH == "auto" and plan is not None and plan.max_row <= ROWS_KERNEL_MAX_ROW):
             rc = L.scorch_hip_spmm_csr_rows_batched_f32(H, M, K, N, nnz, pos.data_ptr(), crd.data_ptr(),
                                                         a_val.data_ptr(), b.data_ptr(), out.data_ptr(), stream)

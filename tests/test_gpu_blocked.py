@@ -147,10 +147,15 @@ def test_what_goes_to_the_block_kernels():
     assert H._blocked(plan, pos, crd, 256, 256, 32) is None
     with blocked_path("off"):
         assert f("causal", 256, 256) is None
-    # a row that holds everything among rows that hold a window: SDDMM by blocks, SpMM not
+    # a row that holds everything among rows that hold a window: its block row goes out in stretches
     pos, crd = (dev(x) for x in csr_of(pattern("window_global", 1024, 1024, rng)))
     bl = H._blocked(H.csr_plan(pos, crd, 1024, 1024), pos, crd, 1024, 1024, 64)
-    assert bl is not None and bl.longest_block_row == 16 and not H._blocked_spmm_balanced(bl)
+    assert bl is not None and bl.longest_block_row == 16
+    assert bl.spmm_split_rows.tolist() == [0, 0, 2, 0] and bl.n_spmm_slots == 2 and bl.n_spmm_items == 17
+    # rows of similar length stay whole
+    pos, crd = (dev(x) for x in csr_of(pattern("window", 1024, 1024, rng)))
+    bl = H._blocked(H.csr_plan(pos, crd, 1024, 1024), pos, crd, 1024, 1024, 64)
+    assert bl.n_spmm_slots == 0 and bl.n_spmm_items == 16
 
 
 def test_unbalanced_mask_values(oracle):
@@ -246,10 +251,15 @@ def test_entry_points_refuse_what_they_do_not_serve():
     assert L.scorch_hip_sddmm_csr_blocked_f32(*args(60, 64, 64)) == native.EUNSUPPORTED
     assert L.scorch_hip_sddmm_csr_blocked_f32(*args(64, 64, 64)) == 0
     torch.cuda.synchronize()
-    spmm = lambda n_items: L.scorch_hip_spmm_csr_blocked_f32(
+    c = torch.zeros(128 * 64, device="cuda")
+    spmm = lambda n_items, n_split=0, n_slots=0, ws=None, ws_bytes=0: L.scorch_hip_spmm_csr_blocked_f32(
         1, 128, 64, 64, 4096, 1, col.data_ptr(), words.data_ptr(), off.data_ptr(), n_items, items.data_ptr(),
-        z.data_ptr(), z.data_ptr(), torch.zeros(128 * 64, device="cuda").data_ptr(), None)
+        n_split, items.data_ptr() if n_split else None, n_slots, z.data_ptr(), z.data_ptr(), c.data_ptr(), ws,
+        ws_bytes, None)
     assert spmm(1) == native.EINVAL and "every block row" in native.last_error()
+    assert spmm(2, 1, 0) == native.EINVAL                        # split rows without slots
+    assert spmm(2, 1, 2) == native.EWORKSPACE and "workspace" in native.last_error()
+    assert L.scorch_hip_spmm_csr_blocked_workspace_bytes(3, 2, 64) == 3 * 2 * 64 * 64 * 4
 
 
 def test_a_mask_of_ones_is_not_read(oracle):
