@@ -174,7 +174,8 @@ class CsrPlan:
     chunk boundaries of the merge-path kernels.  Lives as an attribute of the
     row-pointer tensor, so it is dropped with the operand, and is rebuilt when
     either index tensor has been written to since."""
-    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows", "blocked")
+    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows", "blocked",
+                 "blocked_uses")
 
     def __init__(self, key, max_row: int, empty_rows: int):
         self.key = key
@@ -185,6 +186,7 @@ class CsrPlan:
         self.sddmm_uses = 0                                # SDDMM calls that could have used them
         self.rows: Optional[torch.Tensor] = None           # the row coordinate of every entry (SDDMM results)
         self.blocked = None                                # BlockedCsr, False (looked at: not blocky), None (not yet)
+        self.blocked_uses = 0                              # products that could have gone to the block kernels
 
 
 def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, what: str = "operand") -> Optional[CsrPlan]:
@@ -239,9 +241,10 @@ def _chunk_bounds(plan: CsrPlan, pos: torch.Tensor, M: int, nnz: int, N: int, el
 
 # A CSR operand whose entries cluster in 64 x 64 blocks (an attention mask) is multiplied on the
 # fp32 matrix instruction, block by block, when its dense partner is 32, 64 or 128 wide.  "auto"
-# (SCORCH_HIP_BLOCKED overrides it at import) decides on the operand's first use, from the
-# share of the active blocks' positions that are stored; "off" keeps the general kernels,
-# "always" takes the block kernels for every operand they can serve, however thinly filled.
+# (SCORCH_HIP_BLOCKED overrides it at import) decides when an operand comes back for its second
+# product, from the share of the active blocks' positions that are stored; "off" keeps the
+# general kernels, "always" takes the block kernels for every operand they can serve, however
+# thinly filled, from its first product on.
 BLOCKED_PATHS = ("auto", "off", "always")
 BLOCKED_PATH = os.environ.get("SCORCH_HIP_BLOCKED", "auto")
 # dense width -> share of the active blocks' positions that must be stored for the block kernels to
@@ -348,14 +351,18 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
 
 
 def _blocked(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, width: int) -> Optional[BlockedCsr]:
-    """The operand's block description if products with it go to the block kernels (decided on
-    its first use; never under a stream capture unless it was decided before)."""
+    """The operand's block description if products with it go to the block kernels.  Decided when
+    the operand (the same index tensors, unchanged) comes back for a second product: describing
+    a pattern costs a pass of torch operations over its entries, which an operand that is built
+    anew for every call -- the probabilities of an attention head wrapped in a fresh STensor --
+    would pay each time.  Never under a stream capture unless it was decided before."""
     if BLOCKED_PATH not in BLOCKED_PATHS:
         raise ValueError(f"scorch_ops_hip: BLOCKED_PATH is {BLOCKED_PATH!r}, expected one of {BLOCKED_PATHS}")
     if BLOCKED_PATH == "off" or plan is None or width not in BLOCKED_WIDTHS:
         return None
     if plan.blocked is None:
-        if torch.cuda.is_current_stream_capturing():
+        plan.blocked_uses += 1
+        if torch.cuda.is_current_stream_capturing() or (plan.blocked_uses < 2 and BLOCKED_PATH != "always"):
             return None
         least = 0.0 if BLOCKED_PATH == "always" else min(BLOCKED_MIN_FILL.values())
         plan.blocked = _blocked_csr(pos, crd, M, n_cols, least) or False

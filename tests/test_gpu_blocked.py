@@ -67,8 +67,11 @@ def products(rp, ci, mask_vals, A, B, P, V):
     M, n_cols = len(rp) - 1, B.shape[1]
     pos, crd = dev(rp), dev(ci)
     idx = [[], [pos, crd]]
+    first, _ = H.sddmm_csr_float_batched([M, n_cols], idx, dev(mask_vals), dev(A), dev(B))
+    # (the pattern's first product: general kernel; what serves it from now on is decided when it comes back)
     out, rows = H.sddmm_csr_float_batched([M, n_cols], idx, dev(mask_vals), dev(A), dev(B))
     c = H.spmm_csr_float_batched([M, n_cols], idx, dev(P), dev(V))
+    np.testing.assert_allclose(host(first), host(out), rtol=1e-4, atol=1e-4)
     return host(out), host(rows), host(c), pos._scorch_plan
 
 
@@ -133,8 +136,12 @@ def test_thinly_filled_blocks_when_forced(oracle, D):
 
 def test_what_goes_to_the_block_kernels():
     rng = np.random.default_rng(3)
-    f = lambda kind, M, n, D=64, width=None: H._blocked(
-        H.csr_plan(*(p := [dev(x) for x in csr_of(pattern(kind, M, n, rng))]), M, n), p[0], p[1], M, n, D)
+    def second_use(pos, crd, M, n, D):
+        plan = H.csr_plan(pos, crd, M, n)
+        assert H._blocked(plan, pos, crd, M, n, D) is None or H.BLOCKED_PATH == "always"   # first product: not yet
+        return H._blocked(plan, pos, crd, M, n, D)
+
+    f = lambda kind, M, n, D=64: second_use(*[dev(x) for x in csr_of(pattern(kind, M, n, rng))], M, n, D)
     assert f("causal", 256, 256) is not None
     assert f("causal", 256, 256, D=48) is None                  # dense width without a kernel
     assert f("causal", 250, 256) is None                        # rows not a multiple of 64
@@ -143,18 +150,18 @@ def test_what_goes_to_the_block_kernels():
     m = rng.random((256, 256)) < 0.135
     pos, crd = (dev(x) for x in csr_of(m))
     plan = H.csr_plan(pos, crd, 256, 256)
-    assert H._blocked(plan, pos, crd, 256, 256, 128) is not None
+    assert second_use(pos, crd, 256, 256, 128) is not None
     assert H._blocked(plan, pos, crd, 256, 256, 32) is None
     with blocked_path("off"):
         assert f("causal", 256, 256) is None
     # a row that holds everything among rows that hold a window: its block row goes out in stretches
     pos, crd = (dev(x) for x in csr_of(pattern("window_global", 1024, 1024, rng)))
-    bl = H._blocked(H.csr_plan(pos, crd, 1024, 1024), pos, crd, 1024, 1024, 64)
+    bl = second_use(pos, crd, 1024, 1024, 64)
     assert bl is not None and bl.longest_block_row == 16
     assert bl.spmm_split_rows.tolist() == [0, 0, 2, 0] and bl.n_spmm_slots == 2 and bl.n_spmm_items == 17
     # rows of similar length stay whole
     pos, crd = (dev(x) for x in csr_of(pattern("window", 1024, 1024, rng)))
-    bl = H._blocked(H.csr_plan(pos, crd, 1024, 1024), pos, crd, 1024, 1024, 64)
+    bl = second_use(pos, crd, 1024, 1024, 64)
     assert bl.n_spmm_slots == 0 and bl.n_spmm_items == 16
 
 
@@ -191,6 +198,7 @@ def test_batched_equals_per_head_and_repeats_bit_for_bit():
     mv, A, B, P, V = operands(rng, 4, M, n_cols, 64, ci.size)
     pos, crd = dev(rp), dev(ci)
     idx = [[], [pos, crd]]
+    H.sddmm_csr_float_batched([M, n_cols], idx, dev(mv), dev(A), dev(B))       # (first product: general kernel)
     out, rows = H.sddmm_csr_float_batched([M, n_cols], idx, dev(mv), dev(A), dev(B))
     c = H.spmm_csr_float_batched([M, n_cols], idx, dev(P), dev(V))
     assert isinstance(pos._scorch_plan.blocked, H.BlockedCsr)
@@ -213,6 +221,7 @@ def test_sparse_attention_through_the_block_kernels(oracle):
     rp, ci = csr_of(mask)
     q, k, v = (rng.standard_normal((heads, S, D)).astype(np.float32) for _ in range(3))
     pos, crd = dev(rp), dev(ci)
+    H.sparse_attention_csr(pos, crd, dev(q), dev(k), dev(v), D ** -0.5)
     got = host(H.sparse_attention_csr(pos, crd, dev(q), dev(k), dev(v), D ** -0.5))
     assert isinstance(pos._scorch_plan.blocked, H.BlockedCsr)
     for h in range(heads):
@@ -270,7 +279,10 @@ def test_a_mask_of_ones_is_not_read(oracle):
     pos, crd, a, b = dev(rp), dev(ci), dev(A), dev(B)
     idx = [[], [pos, crd]]
     ones = torch.ones(ci.size, device="cuda")
+    general, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)    # the pattern's first product
     first, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)      # first sight of the values: read
+    assert isinstance(pos._scorch_plan.blocked, H.BlockedCsr)
+    np.testing.assert_allclose(host(general), host(first), rtol=1e-4, atol=1e-4)
     assert ones._scorch_ones[1] is None
     second, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)     # back unchanged: looked at, all 1
     assert ones._scorch_ones[1] is True
