@@ -17,10 +17,10 @@
 // the row's first stored entry inside the block (block_off).  Rows must hold strictly increasing
 // column indices: the entry of bit c is then block_off + (number of set bits below c).
 //
-// Lane (g, n) = (lane / 16, lane % 16); a wavefront serves 16 rows of the block row, lane (g, n)
-// holds row n's values for columns 16 t + 4 g + r (t, r = 0 .. 3) of a block -- 16 bytes of the
-// CSR value array when the row is fully stored in the block -- which is both the layout in which
-// v_mfma_f32_16x16x4_f32 returns K Q^T and the one in which it takes P^T for V^T P^T.
+// Lane (g, n) = (lane / 16, lane % 16); a wavefront serves 16 rows of the block row, and around
+// the MFMAs lane (g, n) holds row n's values for columns 16 t + 4 g + r (t, r = 0 .. 3) of a
+// block: the layout in which v_mfma_f32_16x16x4_f32 returns (B A^T) and the one in which it takes
+// P^T for B^T P^T.  To and from memory the values travel a row at a time (below).
 #include "common.hpp"
 
 namespace scorch {
