@@ -499,7 +499,11 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_f32(
  *   block_words[n_active_blocks * 64] bit c of word r of a block: column c of
  *                                     the block is stored in row r of it;
  *   block_off[n_active_blocks * 64]   position in the CSR arrays of the first
- *                                     stored entry of row r inside the block.
+ *                                     stored entry of row r inside the block;
+ *   block_cols[n_active_blocks]       (SpMM; may be NULL) bit c: some row of the
+ *                                     block stores column c.  A row of B that
+ *                                     no entry of a block refers to is then not
+ *                                     used for that block, whatever it holds.
  * Every row's column indices must increase strictly (the entry of bit c is
  * then block_off + the number of set bits below c); the arrays are trusted.
  * M and the sparse operand's column count must be multiples of 64, the dense
@@ -526,9 +530,9 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_blocked_f32(
 SCORCH_HIP_API size_t scorch_hip_spmm_csr_blocked_workspace_bytes(int64_t H, int64_t n_slots, int64_t N);
 SCORCH_HIP_API int scorch_hip_spmm_csr_blocked_f32(
     int64_t H, int64_t M, int64_t K, int64_t N, int64_t nnz, int64_t n_active_blocks, const int32_t *block_col_idx,
-    const uint64_t *block_words, const int32_t *block_off, int64_t n_items, const int32_t *items,
-    int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots, const float *vals, const float *B, float *C,
-    void *workspace, size_t workspace_bytes, void *stream);
+    const uint64_t *block_words, const int32_t *block_off, const uint64_t *block_cols, int64_t n_items,
+    const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots, const float *vals,
+    const float *B, float *C, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's

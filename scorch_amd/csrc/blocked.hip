@@ -221,7 +221,7 @@ template <int D>
 __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 4))) void spmm_blocked_kernel(
     int M, int K, long long nnz, int n_heads, const int *__restrict__ block_col_idx,
     const unsigned long long *__restrict__ block_words, const int *__restrict__ block_off,
-    const float *__restrict__ vals, const float *__restrict__ B, float *__restrict__ C, int n_items,
+    const unsigned long long *__restrict__ block_cols, const float *__restrict__ vals, const float *__restrict__ B, float *__restrict__ C, int n_items,
     const int4 *__restrict__ items, int n_slots, float *__restrict__ partials) {
   using T = Tile<D>;
   constexpr int kStride = T::kStride;
@@ -249,9 +249,15 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
 #pragma unroll
   for (int dt = 0; dt < kFeat; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // A row of B that no entry of the block refers to is not used: it goes into LDS as zeros, so
+  // that whatever it holds (the padding of a batch, never written) meets the zeros standing for
+  // "not stored" as 0 x 0.  (A row that some of the block's rows refer to meets the other rows'
+  // zeros as it is: a NaN or infinity in it reaches all 64 rows of the block.)
   floatx4 b_next[kCpt];
+  unsigned long long cols_next = ~0ull;  // bit c: some row of the tile's block stores column c
   auto fetch = [&](int it) {
     const size_t tile = (size_t)uniform(block_col_idx[it]) * kBlock * D;
+    if (block_cols) cols_next = block_cols[it];
 #pragma unroll
     for (int u = 0; u < kCpt; ++u)
       b_next[u] = *reinterpret_cast<const floatx4 *>(Bh + tile + (size_t)(tid + u * kBlockThreads) * 4);
@@ -260,8 +266,10 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(D
 #pragma unroll
     for (int u = 0; u < kCpt; ++u) {
       const int chunk = tid + u * kBlockThreads;
-      *reinterpret_cast<floatx4 *>(&s_b[(chunk / T::kChunksPerRow) * kStride + (chunk % T::kChunksPerRow) * 4]) =
-          b_next[u];
+      const int tile_row = chunk / T::kChunksPerRow;
+      const bool used = (cols_next >> tile_row) & 1ull;
+      *reinterpret_cast<floatx4 *>(&s_b[tile_row * kStride + (chunk % T::kChunksPerRow) * 4]) =
+          used ? b_next[u] : floatx4{0.f, 0.f, 0.f, 0.f};
     }
   };
   // The values of a block, a row at a time (lane c: column c; zero where nothing is stored), and
@@ -430,7 +438,8 @@ extern "C" size_t scorch_hip_spmm_csr_blocked_workspace_bytes(int64_t H, int64_t
 extern "C" int scorch_hip_spmm_csr_blocked_f32(int64_t H, int64_t M, int64_t K, int64_t N, int64_t nnz,
                                                int64_t n_active_blocks, const int32_t *block_col_idx,
                                                const uint64_t *block_words, const int32_t *block_off,
-                                               int64_t n_items, const int32_t *items, int64_t n_split_rows,
+                                               const uint64_t *block_cols, int64_t n_items, const int32_t *items,
+                                               int64_t n_split_rows,
                                                const int32_t *split_rows, int64_t n_slots, const float *vals,
                                                const float *B, float *C, void *workspace, size_t workspace_bytes,
                                                void *stream) {
@@ -461,14 +470,17 @@ extern "C" int scorch_hip_spmm_csr_blocked_f32(int64_t H, int64_t M, int64_t K, 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(n_items * H));
   const dim3 merge_grid((unsigned)n_split_rows, (unsigned)H);
+  SCORCH_REQUIRE(aligned_to(block_cols, 8), "%s: block_cols must be 8-byte aligned", fn);
   const unsigned long long *words = reinterpret_cast<const unsigned long long *>(block_words);
+  const unsigned long long *cols = reinterpret_cast<const unsigned long long *>(block_cols);
   const int4 *item_list = reinterpret_cast<const int4 *>(items);
   const int4 *rows = reinterpret_cast<const int4 *>(split_rows);
   mark_launch(s);
 #define SCORCH_BLOCKED_SPMM(DIM)                                                                                  \
   do {                                                                                                            \
     blocked::spmm_blocked_kernel<DIM><<<grid, kBlockThreads, 0, s>>>((int)M, (int)K, (long long)nnz, (int)H,      \
-                                                                     block_col_idx, words, block_off, vals, B, C, \
+                                                                     block_col_idx, words, block_off, cols, vals, \
+                                                                     B, C,                                        \
                                                                      (int)n_items, item_list, (int)n_slots,       \
                                                                      partials);                                   \
     SCORCH_HIP_CHECK(hipGetLastError());                                                                          \

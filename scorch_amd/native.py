@@ -107,8 +107,8 @@ SIGNATURES = {
     "scorch_hip_sddmm_csr_blocked_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr,
                                                         _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "scorch_hip_spmm_csr_blocked_workspace_bytes": (_size, [_i64, _i64, _i64]),
-    "scorch_hip_spmm_csr_blocked_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr,
-                                                       _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
+    "scorch_hip_spmm_csr_blocked_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _i64,
+                                                       _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
     "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "scorch_hip_coo_row_ptr": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
 }

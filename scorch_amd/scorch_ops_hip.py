@@ -261,7 +261,7 @@ class BlockedCsr:
     """A CSR pattern described by 64 x 64 blocks, for scorch_hip_{sddmm,spmm}_csr_blocked_f32:
     the active blocks in block row major order, per block and row a word of stored columns and
     the CSR position of the row's first entry in the block, and the two lists of work items."""
-    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "sddmm_items", "n_sddmm_items",
+    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "block_cols", "sddmm_items", "n_sddmm_items",
                  "spmm_items", "n_spmm_items", "spmm_split_rows", "n_spmm_split_rows", "n_spmm_slots",
                  "n_block_rows", "longest_block_row", "fill")
 
@@ -337,6 +337,10 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     bl.block_col_idx = (blocks % nbc).to(torch.int32)
     bl.block_words = words
     bl.block_off = first.to(torch.int32)
+    used = words.view(n_active, block)                # columns some row of the block stores: the rows' words or-ed
+    while used.shape[1] > 1:
+        used = used[:, 0::2] | used[:, 1::2]
+    bl.block_cols = used.reshape(-1).contiguous()
     bl.sddmm_items = torch.tensor([it[1:] for it in sddmm_items], dtype=torch.int32, device=dev).reshape(-1)
     bl.n_sddmm_items = len(sddmm_items)
     bl.spmm_items = torch.tensor([it[1:] for it in spmm_items], dtype=torch.int32, device=dev).reshape(-1)
@@ -400,7 +404,8 @@ def _blocked_spmm(L, bl: BlockedCsr, heads: int, M: int, K: int, N: int, nnz: in
             out._scorch_workspace = ws      # a buffer handed out during a capture lives as long as the result
     return L.scorch_hip_spmm_csr_blocked_f32(
         heads, M, K, N, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
-        bl.block_off.data_ptr(), bl.n_spmm_items, bl.spmm_items.data_ptr(), bl.n_spmm_split_rows,
+        bl.block_off.data_ptr(), bl.block_cols.data_ptr(), bl.n_spmm_items, bl.spmm_items.data_ptr(),
+        bl.n_spmm_split_rows,
         bl.spmm_split_rows.data_ptr() if bl.n_spmm_split_rows else None, bl.n_spmm_slots, vals.data_ptr(),
         b.data_ptr(), out.data_ptr(), ws.data_ptr() if ws is not None else None,
         ws.numel() if ws is not None else 0, stream)

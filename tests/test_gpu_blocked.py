@@ -262,7 +262,7 @@ def test_entry_points_refuse_what_they_do_not_serve():
     torch.cuda.synchronize()
     c = torch.zeros(128 * 64, device="cuda")
     spmm = lambda n_items, n_split=0, n_slots=0, ws=None, ws_bytes=0: L.scorch_hip_spmm_csr_blocked_f32(
-        1, 128, 64, 64, 4096, 1, col.data_ptr(), words.data_ptr(), off.data_ptr(), n_items, items.data_ptr(),
+        1, 128, 64, 64, 4096, 1, col.data_ptr(), words.data_ptr(), off.data_ptr(), None, n_items, items.data_ptr(),
         n_split, items.data_ptr() if n_split else None, n_slots, z.data_ptr(), z.data_ptr(), c.data_ptr(), ws,
         ws_bytes, None)
     assert spmm(1) == native.EINVAL and "every block row" in native.last_error()
@@ -297,3 +297,22 @@ def test_a_mask_of_ones_is_not_read(oracle):
     expect = first.clone()
     expect[:, 7] *= -2.0
     assert torch.equal(changed, expect)
+
+
+def test_rows_of_the_dense_operand_that_no_entry_refers_to_are_not_used(oracle):
+    """Columns the mask leaves out altogether (the padding of a batch): whatever the dense operands
+    hold there -- NaN here -- stays out of both products, as with the general kernels."""
+    rng = np.random.default_rng(14)
+    M = n_cols = 256
+    mask = pattern("causal", M, n_cols, rng)
+    padded = np.r_[40:64, 130:131, 200:256]
+    mask[:, padded] = False
+    rp, ci = csr_of(mask)
+    mv, A, B, P, V = operands(rng, 2, M, n_cols, 64, ci.size)
+    B_bad, V_bad = B.copy(), V.copy()
+    B_bad[:, padded] = np.nan
+    V_bad[:, padded] = np.nan
+    out, rows, c, plan = products(rp, ci, mv, A, B_bad, P, V_bad)
+    assert isinstance(plan.blocked, H.BlockedCsr)
+    assert np.isfinite(out).all() and np.isfinite(c).all()
+    check_values(oracle, rp, ci, mv, A, B, P, V, out, rows, c)

@@ -471,10 +471,13 @@ def test_block_description_of_a_csr_pattern():
     offs = bl.block_off.view(-1, 64).numpy()
     spmm_items = sorted(bl.spmm_items.view(-1, 4).tolist())
     assert [it[0] for it in spmm_items] == [0, 1, 2] and spmm_items[1][1] == spmm_items[1][2]
+    used = bl.block_cols.numpy().view(np.uint64)
     seen = np.zeros(ci.size, dtype=bool)
     for row_block, lo, hi, _ in spmm_items:
         assert cols[lo:hi] == sorted(cols[lo:hi]) and 2 not in cols[lo:hi]
         for b in range(lo, hi):
+            block = mask[64 * row_block:64 * row_block + 64, 64 * cols[b]:64 * cols[b] + 64]
+            assert int(used[b]) == sum(1 << c for c in range(64) if block[:, c].any())
             for r in range(64):
                 row = 64 * row_block + r
                 stored = [c for c in range(64) if mask[row, 64 * cols[b] + c]]
