@@ -111,3 +111,26 @@ def test_arguments_are_checked():
     q48 = torch.zeros(1, 128, 48, device="cuda")
     with pytest.raises(RuntimeError, match="head dimensions 32, 64 and 128"):
         H.attn_blocksparse_f32(q48, q48, q48, bm, 1.0)
+
+
+def test_keys_the_mask_leaves_out_may_hold_anything_in_k(oracle):
+    """Padding keys that no query attends to: their rows of K may be NaN (their scores are replaced
+    before they are looked at); their rows of V are multiplied by zero probabilities, so V has to be
+    finite there.  Both fused kernels, against the fp64 result on clean operands."""
+    S, heads, D = 256, 2, 64
+    rng = np.random.default_rng(21)
+    i, j = np.arange(S)[:, None], np.arange(S)[None, :]
+    mask = j <= i
+    padded = np.r_[50:64, 130:131, 192:256]         # part of a block, one key, a whole block column
+    mask[:, padded] = False
+    mask[padded, 0] = True                           # (the padded queries attend to the first key)
+    q, k, v = (rng.standard_normal((heads, S, D)).astype(np.float32) for _ in range(3))
+    k_bad = k.copy()
+    k_bad[:, padded] = np.nan
+    rp, ci = csr_of(mask)
+    ref = np.stack([oracle.attention_dense_fp64(q[h], k[h], v[h], mask, D ** -0.5) for h in range(heads)])
+    out32 = H.sparse_attention_f32(dev(q), dev(k_bad), dev(v), dev(rp), dev(ci), D ** -0.5).cpu().numpy()
+    assert np.isfinite(out32).all() and oracle.rel_fro(out32, ref) <= TOL
+    to16 = lambda a: dev(a).to(torch.bfloat16)
+    out16 = H.sparse_attention_bf16(to16(q), to16(k_bad), to16(v), dev(rp), dev(ci), D ** -0.5).float().cpu().numpy()
+    assert np.isfinite(out16).all() and oracle.rel_fro(out16, ref) <= 1e-2
