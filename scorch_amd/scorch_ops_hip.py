@@ -780,6 +780,33 @@ def _sddmm_dense_args(S_shape, A_shape, A_values, B_shape, B_values):
     return M, n_cols, K, a, b
 
 
+def _coo_mask_row_ptr(row: torch.Tensor, col: torch.Tensor, M: int, n_cols: int, K: int) -> Optional[torch.Tensor]:
+    """The row pointer of a coordinate mask that may be one for the block kernels (dimensions
+    multiples of 64, a dense width they serve, eight entries per row or more), once the same
+    coordinate tensors have come back unchanged; None otherwise, and for coordinates that are
+    not in row order.  Kept with the row tensor (one kernel and one host read, once)."""
+    if BLOCKED_PATH == "off" or not plans_enabled() or K not in BLOCKED_WIDTHS or M % 64 or n_cols % 64 \
+            or row.numel() < 8 * M or M == 0:
+        return None
+    key = (row._version, col.data_ptr(), col._version, col.numel(), M)
+    seen = getattr(row, "_scorch_coo_pos", None)
+    if seen is not None and seen[0] == key:
+        if seen[1] is None and not torch.cuda.is_current_stream_capturing():
+            pos = coo_row_ptr(row, M)
+            seen = (key, pos if pos is not None else False)
+            row._scorch_coo_pos = seen
+            if pos is not None:
+                plan = csr_plan(pos, col, M, n_cols, "S")
+                if plan is not None:
+                    plan.blocked_uses = 1           # this is the mask's second product already
+        return seen[1] if isinstance(seen[1], torch.Tensor) else None
+    try:
+        row._scorch_coo_pos = (key, None)
+    except (AttributeError, RuntimeError):
+        pass
+    return None
+
+
 def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_mode_indices,
                              A_values, B_shape, B_mode_indices, B_values):
     """D = S * (A @ B^T) at S's entries, S in coordinate format
@@ -794,10 +821,23 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
         raise ValueError("scorch_ops_hip: S index and value lengths differ")
     dev = _device_of(row, col, s_val, a, b)
     out = _empty_like(s_val)
+    L = native.lib()
     with _on_device(dev):
-        rc = native.lib().scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(),
-                                                   col.data_ptr(), s_val.data_ptr(), a.data_ptr(),
-                                                   b.data_ptr(), out.data_ptr(), _stream(dev))
+        stream = _stream(dev)
+        pos = _coo_mask_row_ptr(row, col, M, n_cols, K)
+        bl = _blocked(csr_plan(pos, col, M, n_cols, "S"), pos, col, M, n_cols, K) if pos is not None else None
+        if bl is not None:
+            # a mask made of 64 x 64 blocks, its coordinates in row-major order: the block kernel
+            # writes the values in that same order
+            rc = L.scorch_hip_sddmm_csr_blocked_f32(1, M, n_cols, K, s_val.numel(), bl.n_active,
+                                                    bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
+                                                    bl.block_off.data_ptr(), bl.n_sddmm_items,
+                                                    bl.sddmm_items.data_ptr(),
+                                                    None if _known_all_ones(s_val) else s_val.data_ptr(),
+                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), None, stream)
+        else:
+            rc = L.scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(), col.data_ptr(),
+                                            s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(), stream)
     native.check(rc)
     return Tensor(out, S_mode_indices)
 

@@ -316,3 +316,40 @@ def test_rows_of_the_dense_operand_that_no_entry_refers_to_are_not_used(oracle):
     assert isinstance(plan.blocked, H.BlockedCsr)
     assert np.isfinite(out).all() and np.isfinite(c).all()
     check_values(oracle, rp, ci, mv, A, B, P, V, out, rows, c)
+
+
+def test_coordinate_mask_made_of_blocks(oracle):
+    """The reference's prebuilt SDDMM takes a coordinate mask (csrc/kernels.h:508-570): one made
+    of blocks, in row-major order, goes to the block kernel once it has come back; the result
+    carries the mask's own index tensors either way."""
+    rng = np.random.default_rng(15)
+    M, n_cols, K = 256, 320, 64
+    mask = pattern("random30", M, n_cols, rng)
+    rp, ci = csr_of(mask)
+    rows_np = oracle.rows_of(rp)
+    mv = rng.standard_normal(ci.size).astype(np.float32)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((n_cols, K)).astype(np.float32)
+    r, c, v, a, b = dev(rows_np), dev(ci), dev(mv), dev(A).reshape(-1), dev(B).reshape(-1)
+    call = lambda: H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[r], [c]], v, [M, K], [[], []], a,
+                                              [n_cols, K], [[], []], b)
+    ref64 = oracle.sddmm_fp64(rows_np, ci, mv, A, B)
+    first = call()                                       # general kernel
+    assert r._scorch_coo_pos[1] is None
+    second = call()                                      # the mask has come back: by blocks from here on
+    assert isinstance(r._scorch_coo_pos[1], torch.Tensor) and np.array_equal(host(r._scorch_coo_pos[1]), rp)
+    assert isinstance(r._scorch_coo_pos[1]._scorch_plan.blocked, H.BlockedCsr)
+    third = call()
+    for out in (first, second, third):
+        assert out.storage.index.mode_indices[0][0] is r and out.storage.index.mode_indices[1][0] is c
+        assert oracle.rel_fro(host(out.storage.value), ref64) <= TOL
+    assert torch.equal(second.storage.value, third.storage.value)
+    assert not torch.equal(first.storage.value, second.storage.value)      # (another order of the fp32 sums)
+    # coordinates that are not in row order keep the general kernel
+    perm = rng.permutation(ci.size)
+    r2, c2, v2 = dev(rows_np[perm]), dev(ci[perm]), dev(mv[perm])
+    for _ in range(3):
+        out = H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[r2], [c2]], v2, [M, K], [[], []], a,
+                                         [n_cols, K], [[], []], b)
+    assert r2._scorch_coo_pos[1] is False
+    assert oracle.rel_fro(host(out.storage.value), ref64[perm]) <= TOL
