@@ -353,3 +353,25 @@ def test_coordinate_mask_made_of_blocks(oracle):
                                          [n_cols, K], [[], []], b)
     assert r2._scorch_coo_pos[1] is False
     assert oracle.rel_fro(host(out.storage.value), ref64[perm]) <= TOL
+
+
+def test_through_matmul_and_einsum():
+    """The reference's own calls (src/scorch/ops.py:248-372, 396-423) with a mask that is kept
+    across calls, as its attention benchmark keeps it (bench/bench_sparse_transformer.py:236,357)."""
+    import scorch_amd as scorch
+    torch.manual_seed(16)
+    S, D = 256, 32
+    dense_mask = torch.tril(torch.ones(S, S))
+    mask = scorch.STensor.from_csr(dense_mask.to_sparse_csr()).to("cuda")
+    q, k, v = (torch.randn(S, D, device="cuda") for _ in range(3))
+    live = dense_mask.bool().cuda()
+    want_scores = (q.double() @ k.double().T)[live]
+    probs = scorch.STensor.from_csr(torch.rand(S, S).tril().to_sparse_csr()).to("cuda")
+    want_out = probs.to_torch(in_place=False).to_dense().double() @ v.double()
+    for call in range(3):
+        scores = scorch.einsum("ij,ik,jk->ij", mask, q, k)
+        assert ((scores.values.double() - want_scores).norm() / want_scores.norm()).item() <= TOL
+        out = scorch.matmul(probs, v)
+        assert ((out.double() - want_out).norm() / want_out.norm()).item() <= TOL
+    for operand in (mask, probs):
+        assert isinstance(operand.index.mode_indices[1][0]._scorch_plan.blocked, H.BlockedCsr)
