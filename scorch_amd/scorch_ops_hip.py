@@ -252,7 +252,8 @@ BLOCKED_PATH = os.environ.get("SCORCH_HIP_BLOCKED", "auto")
 # kernels' time grows with the entries, the block kernels' with the blocks)
 BLOCKED_MIN_FILL = {32: 0.17, 64: 0.15, 128: 0.12}
 BLOCKED_WIDTHS = tuple(BLOCKED_MIN_FILL)
-BLOCKED_STRETCH = 16         # blocks per SDDMM work item at most
+BLOCKED_STRETCH = 16         # blocks per work item at most
+BLOCKED_STRETCHES = (16, 4, 1)   # the SDDMM's work items exist in these sizes: a small launch takes smaller ones
 BLOCKED_MAX_BLOCKS = 1 << 24  # blocks of the whole matrix: beyond, the operand is a graph, not a mask
 BLOCKED_MAX_NNZ = 1 << 27
 
@@ -261,7 +262,7 @@ class BlockedCsr:
     """A CSR pattern described by 64 x 64 blocks, for scorch_hip_{sddmm,spmm}_csr_blocked_f32:
     the active blocks in block row major order, per block and row a word of stored columns and
     the CSR position of the row's first entry in the block, and the two lists of work items."""
-    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "block_cols", "sddmm_items", "n_sddmm_items",
+    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "block_cols", "sddmm_items",
                  "spmm_items", "n_spmm_items", "spmm_split_rows", "n_spmm_split_rows", "n_spmm_slots",
                  "n_block_rows", "longest_block_row", "fill")
 
@@ -308,18 +309,22 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     first.scatter_reduce_(0, key, torch.arange(nnz, device=dev, dtype=torch.int64), "amin")
     first[first == nnz] = 0
     lens = torch.bincount(blocks // nbc, minlength=nbr).cpu().tolist()
-    # Work items.  SDDMM: stretches of at most BLOCKED_STRETCH blocks.  SpMM: a block row sums into one
-    # tile of the result, so it stays whole unless the rows differ by more than a quarter of their mean;
-    # then rows longer than twice the mean (8 to BLOCKED_STRETCH blocks) go out in stretches whose sums a
-    # second kernel adds up in order.
+    # Work items.  SDDMM: stretches of block rows, in several sizes (the entries do not depend on how
+    # they are shared out, so a launch picks the size that fills the chip).  SpMM: a block row sums into
+    # one tile of the result, so it stays whole unless the rows differ by more than a quarter of their
+    # mean; then rows longer than the mean by more than a block (4 to BLOCKED_STRETCH blocks) go out in
+    # stretches whose sums a second kernel adds up in order -- the same stretches whatever the number of
+    # heads, so that a head's result does not depend on what it is batched with.
     mean = n_active / nbr
-    spmm_longest = min(BLOCKED_STRETCH, max(8, 2 * -(-n_active // nbr))) if max(lens) > 1.25 * mean else max(lens)
-    sddmm_items, spmm_items, split_rows, at, slot = [], [], [], 0, 0
+    spmm_longest = min(BLOCKED_STRETCH, max(4, -(-n_active // nbr) + 1)) if max(lens) > 1.25 * mean else max(lens)
+    sddmm_items = {stretch: [] for stretch in BLOCKED_STRETCHES}
+    spmm_items, split_rows, at, slot = [], [], 0, 0
     for row, n in enumerate(lens):
-        parts = -(-n // BLOCKED_STRETCH)
-        for part in range(parts):
-            lo, hi = at + n * part // parts, at + n * (part + 1) // parts
-            sddmm_items.append((hi - lo, row, lo, hi, 0))
+        for stretch, items in sddmm_items.items():
+            parts = -(-n // stretch)
+            for part in range(parts):
+                lo, hi = at + n * part // parts, at + n * (part + 1) // parts
+                items.append((hi - lo, row, lo, hi, 0))
         if n <= spmm_longest:
             spmm_items.append((n, row, at, at + n, -1))
         else:
@@ -330,7 +335,8 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
                 spmm_items.append((hi - lo, row, lo, hi, slot))
                 slot += 1
         at += n
-    sddmm_items.sort(key=lambda it: -it[0])           # longest first
+    for items in sddmm_items.values():
+        items.sort(key=lambda it: -it[0])             # longest first
     spmm_items.sort(key=lambda it: -it[0])
     bl = BlockedCsr()
     bl.n_active = n_active
@@ -341,8 +347,8 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     while used.shape[1] > 1:
         used = used[:, 0::2] | used[:, 1::2]
     bl.block_cols = used.reshape(-1).contiguous()
-    bl.sddmm_items = torch.tensor([it[1:] for it in sddmm_items], dtype=torch.int32, device=dev).reshape(-1)
-    bl.n_sddmm_items = len(sddmm_items)
+    bl.sddmm_items = {stretch: (torch.tensor([it[1:] for it in items], dtype=torch.int32, device=dev).reshape(-1),
+                                len(items)) for stretch, items in sddmm_items.items()}
     bl.spmm_items = torch.tensor([it[1:] for it in spmm_items], dtype=torch.int32, device=dev).reshape(-1)
     bl.n_spmm_items = len(spmm_items)
     bl.spmm_split_rows = torch.tensor(split_rows, dtype=torch.int32, device=dev).reshape(-1)
@@ -374,6 +380,22 @@ def _blocked(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, width: int)
     if bl is not None and BLOCKED_PATH == "auto" and bl.fill < BLOCKED_MIN_FILL[width]:
         return None
     return bl
+
+
+def _blocked_sddmm(L, bl: BlockedCsr, heads: int, M: int, n_cols: int, K: int, nnz: int, mask_vals,
+                   a: torch.Tensor, b: torch.Tensor, out: torch.Tensor, rows_ptr, stream: int) -> int:
+    """Launch the block SDDMM for `heads` pairs of dense operands over one pattern: with the
+    largest work items that still give every workgroup slot of the chip one (1,024: 256 CUs x 4),
+    else the smallest."""
+    for stretch in BLOCKED_STRETCHES:
+        items, n_items = bl.sddmm_items[stretch]
+        if n_items * heads >= 1024:
+            break
+    return L.scorch_hip_sddmm_csr_blocked_f32(
+        heads, M, n_cols, K, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
+        bl.block_off.data_ptr(), n_items, items.data_ptr(),
+        None if mask_vals is None or _known_all_ones(mask_vals) else mask_vals.data_ptr(), a.data_ptr(),
+        b.data_ptr(), out.data_ptr(), rows_ptr, stream)
 
 
 def _known_all_ones(values: torch.Tensor) -> bool:
@@ -829,12 +851,7 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
         if bl is not None:
             # a mask made of 64 x 64 blocks, its coordinates in row-major order: the block kernel
             # writes the values in that same order
-            rc = L.scorch_hip_sddmm_csr_blocked_f32(1, M, n_cols, K, s_val.numel(), bl.n_active,
-                                                    bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
-                                                    bl.block_off.data_ptr(), bl.n_sddmm_items,
-                                                    bl.sddmm_items.data_ptr(),
-                                                    None if _known_all_ones(s_val) else s_val.data_ptr(),
-                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), None, stream)
+            rc = _blocked_sddmm(L, bl, 1, M, n_cols, K, s_val.numel(), s_val, a, b, out, None, stream)
         else:
             rc = L.scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(), col.data_ptr(),
                                             s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(), stream)
@@ -876,12 +893,7 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
         bl = _blocked(plan, pos, crd, M, n_cols, K)
         lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
         if bl is not None:
-            rc = L.scorch_hip_sddmm_csr_blocked_f32(1, M, n_cols, K, s_val.numel(), bl.n_active,
-                                                    bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
-                                                    bl.block_off.data_ptr(), bl.n_sddmm_items,
-                                                    bl.sddmm_items.data_ptr(),
-                                                    None if _known_all_ones(s_val) else s_val.data_ptr(),
-                                                    a.data_ptr(), b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+            rc = _blocked_sddmm(L, bl, 1, M, n_cols, K, s_val.numel(), s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
@@ -1039,12 +1051,7 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
             s_val = torch.ones(nnz, dtype=torch.float32, device=dev)
         lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
         if bl is not None:
-            ones = s_val is None or _known_all_ones(s_val)
-            rc = L.scorch_hip_sddmm_csr_blocked_f32(H, M, n_cols, K, nnz, bl.n_active, bl.block_col_idx.data_ptr(),
-                                                    bl.block_words.data_ptr(), bl.block_off.data_ptr(),
-                                                    bl.n_sddmm_items, bl.sddmm_items.data_ptr(),
-                                                    None if ones else s_val.data_ptr(), a.data_ptr(), b.data_ptr(),
-                                                    out.data_ptr(), rows_ptr, stream)
+            rc = _blocked_sddmm(L, bl, H, M, n_cols, K, nnz, s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),

@@ -158,7 +158,7 @@ def test_what_goes_to_the_block_kernels():
     pos, crd = (dev(x) for x in csr_of(pattern("window_global", 1024, 1024, rng)))
     bl = second_use(pos, crd, 1024, 1024, 64)
     assert bl is not None and bl.longest_block_row == 16
-    assert bl.spmm_split_rows.tolist() == [0, 0, 2, 0] and bl.n_spmm_slots == 2 and bl.n_spmm_items == 17
+    assert bl.spmm_split_rows.tolist() == [0, 0, 3, 0] and bl.n_spmm_slots == 3 and bl.n_spmm_items == 18
     # rows of similar length stay whole
     pos, crd = (dev(x) for x in csr_of(pattern("window", 1024, 1024, rng)))
     bl = second_use(pos, crd, 1024, 1024, 64)

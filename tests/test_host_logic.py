@@ -487,9 +487,11 @@ def test_block_description_of_a_csr_pattern():
                     assert rp[row] <= at < rp[row + 1] and ci[at] == 64 * cols[b] + c and not seen[at]
                     seen[at] = True
     assert seen.all()
-    covered = sorted((lo, hi) for _, lo, hi, _ in bl.sddmm_items.view(-1, 4).tolist())
-    assert covered[0][0] == 0 and covered[-1][1] == bl.n_active
-    assert all(a[1] == b[0] for a, b in zip(covered, covered[1:])) and all(hi - lo <= H.BLOCKED_STRETCH for lo, hi in covered)
+    for stretch, (items, n_items) in bl.sddmm_items.items():
+        covered = sorted((lo, hi) for _, lo, hi, _ in items.view(-1, 4).tolist())
+        assert len(covered) == n_items and covered[0][0] == 0 and covered[-1][1] == bl.n_active
+        assert all(a[1] == b[0] for a, b in zip(covered, covered[1:])) and all(hi - lo <= stretch for lo, hi in covered)
+    assert set(bl.sddmm_items) == set(H.BLOCKED_STRETCHES) and bl.sddmm_items[1][1] == bl.n_active
     # what the description is not built for
     assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(ci), M, n_cols, 0.5) is None     # too thinly filled
     assert H._blocked_csr(torch.from_numpy(rp[:-1]), torch.from_numpy(ci[:rp[-2]]), M - 1, n_cols, 0.0) is None
