@@ -36,6 +36,10 @@ constexpr int kTileBytes = 128;                // bytes of one row of a column t
 constexpr int64_t kTiledSliceMax = 3 << 20;    // K * kTileBytes must fit an L2 beside A
 constexpr int kTiledGroupRowMax = 64;          // longer in-chunk rows are shared by all groups
 constexpr int kTiledItemsMax = 320;            // most merge items per chunk (the split may exceed the usual 256)
+// A chunk stages what lies between its two boundaries, and its end may move forward by up to
+// kSnapItems items to a row's end (chunk_boundary), so a wavefront's staging arrays hold this many.
+constexpr int kTiledSlots = kTiledItemsMax + kSnapItems;
+static_assert(kTiledItemsMax >= kItemsPerWave, "the usual split must fit the staging arrays too");
 constexpr int kTiledBatch = 8;                 // tile-row loads in flight per lane group (16 measured slower)
 constexpr int kTiledMaxWorkgroupsPerXcd = 256; // 32 CUs x 8 workgroups
 constexpr int kPacePolls = 400;                // polls after which a wavefront stops waiting for the others
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
   constexpr int LPR = kTileBytes / 16;
   constexpr int TC = LPR * VEC;
   constexpr int G = kWaveSize / LPR;
-  constexpr int kSlots = kItemsPerWave + kSnapItems;
+  constexpr int kSlots = kTiledSlots;
   using VecT = Vec<T, VEC>;
 
   __shared__ int s_col[kWavesPerBlock][kSlots];
@@ -303,6 +307,9 @@ int spmm_tiled_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nn
       bounds = nullptr;
     }
   }
+  if (split.items_per_chunk + split.snap > kTiledSlots)
+    return fail(SCORCH_HIP_ERUNTIME, "%s: chunks of %d + %d items exceed the %d staging slots", fn,
+                split.items_per_chunk, split.snap, kTiledSlots);
   if (bounds) {
     const size_t have = (size_t)(split.spans + 1) * sizeof(Boundary);
     if (bounds_bytes < have)

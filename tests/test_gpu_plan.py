@@ -277,3 +277,23 @@ def test_tiled_kernel_with_rows_cut_by_chunks_and_an_epilogue(oracle, relu):
         assert oracle.rel_fro(got, want) <= TOL
         again = hip_spmm(rp, ci, v, B, bias=bias, relu=relu, path="tiled")
         assert np.array_equal(got, again)
+
+
+def test_tiled_kernel_when_the_even_resplit_makes_chunks_longer_than_the_usual_ones(oracle):
+    """4096 rows of 32 entries with a hundred rows of 330 to 600: the tiled kernel re-splits the work
+    into a multiple of 128 chunks of more than 256 items, and a chunk that ends inside one of the
+    long rows stages up to 64 items more.  Checked against fp64 and against the merge path."""
+    rng = np.random.default_rng(3)
+    M, K, N = 4096, 4096, 4096
+    lens = np.full(M, 32, np.int64)
+    lens[rng.choice(M, 100, replace=False)] = rng.integers(330, 601, 100)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ci = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens]).astype(np.int32)
+    v = rng.uniform(-1, 1, ci.size).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    want = oracle.spmm_fp64(rp, ci, v, B)
+    got = hip_spmm(rp, ci, v, B, path="tiled")
+    assert oracle.rel_fro(got, want) <= TOL
+    merge = hip_spmm(rp, ci, v, B, path="merge")
+    np.testing.assert_allclose(got, merge, rtol=1e-4, atol=1e-5)
+    assert np.array_equal(got, hip_spmm(rp, ci, v, B, path="tiled"))

@@ -2,6 +2,8 @@
 tensor model, the prebuilt-kernel registry and the routing decisions of
 matmul / einsum.  Mirrors tests/test_scorch/test_prebuilt_kernel_registry.py
 and the format checks of the reference; runs without a GPU."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -498,3 +500,74 @@ def test_block_description_of_a_csr_pattern():
     backwards = ci.copy()
     backwards[rp[3]:rp[4]] = backwards[rp[3]:rp[4]][::-1]
     assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(backwards), M, n_cols, 0.0) is None
+
+
+# ---- the work split of the SpMM kernels, replayed on the host ---------------------------------------
+def _kernel_constant(name, *files):
+    import re
+    for f in files:
+        text = open(os.path.join(os.path.dirname(scorch_ops_hip.__file__), "csrc", f)).read()
+        m = re.search(r"constexpr\s+int\s+" + name + r"\s*=\s*([^;]+);", text)
+        if m:
+            expr = m.group(1)
+            for other in re.findall(r"k[A-Z]\w+", expr):
+                expr = expr.replace(other, str(_kernel_constant(other, *files)))
+            return int(eval(expr, {"__builtins__": {}}))
+    raise KeyError(name)
+
+
+def _spmm_split(M, nnz, N, elem, items_max=256, items_min=32, snap_items=64):
+    """spmm_split of scorch_amd/csrc/spmm.hpp."""
+    total = M + nnz
+    tiles = max((N * elem + 1023) // 1024, 1)
+    per_wave = total * tiles // 8192
+    ipc = items_min
+    while ipc < items_max and ipc * 2 <= per_wave:
+        ipc *= 2
+    return ipc, min(ipc, snap_items), -(-total // ipc)
+
+
+def _chunk_boundary(d, M, total, row_ptr, snap):
+    """chunk_boundary of scorch_amd/csrc/spmm.hpp: (rows finished, entries before) at merged position d."""
+    if d >= total:
+        return M, total - M
+    keys = row_ptr[1:] + np.arange(M)                   # the position of row i's end marker
+    x = int(np.searchsorted(keys, d, side="left"))      # rows whose marker lies before d
+    y = d - x
+    if x < M:
+        begin, end = int(row_ptr[x]), int(row_ptr[x + 1])
+        if begin < y and end + x + 1 - d <= snap:
+            x, y = x + 1, end
+    return x, y
+
+
+def test_every_chunk_of_the_tiled_split_fits_the_staging_arrays():
+    """The kernel for a dense operand stored by column tiles re-splits the work into a multiple of
+    128 chunks of up to kTiledItemsMax items; a chunk's end may move forward to a row's end by up to
+    kSnapItems more.  What a wavefront stages must fit kTiledSlots: replayed here for a matrix of 32
+    entries per row with a hundred rows of 330 to 600."""
+    files = ("spmm_tiled.hip", "spmm.hpp")
+    items_max, snap_items = _kernel_constant("kTiledItemsMax", *files), _kernel_constant("kSnapItems", *files)
+    slots = _kernel_constant("kTiledSlots", *files)
+    assert slots >= items_max + snap_items
+    rng = np.random.default_rng(3)
+    M, N = 4096, 4096
+    lens = np.full(M, 32, np.int64)
+    lens[rng.choice(M, 100, replace=False)] = rng.integers(330, 601, 100)
+    row_ptr = np.concatenate([[0], np.cumsum(lens)])
+    nnz = int(row_ptr[-1])
+    ipc, snap, spans = _spmm_split(M, nnz, N, 4, _kernel_constant("kItemsPerWave", *files))
+    max_wgs = _kernel_constant("kTiledMaxWorkgroupsPerXcd", *files)
+    assert 128 < spans <= max_wgs * 4
+    even = spans // 128 * 128
+    resplit = -(-(M + nnz) // even)
+    assert even != spans and ipc < resplit <= items_max           # the case takes the re-split
+    ipc, spans = resplit, -(-(M + nnz) // resplit)
+    largest = 0
+    for c in range(spans):
+        x0, y0 = _chunk_boundary(c * ipc, M, M + nnz, row_ptr, snap)
+        x1, y1 = _chunk_boundary((c + 1) * ipc, M, M + nnz, row_ptr, snap)
+        assert 0 <= y1 - y0 and 0 <= x1 - x0
+        largest = max(largest, y1 - y0, x1 - x0 + 2)
+    assert largest > _kernel_constant("kItemsPerWave", *files) + snap_items   # more than the usual split stages
+    assert largest <= slots
