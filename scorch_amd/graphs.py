@@ -14,9 +14,17 @@ synchronisation, which a capturing stream does not allow; the step is run
 eagerly on a side stream first, ``warmup`` times, so that they exist.  The plans
 of a sparse operand's index arrays (and of an attention mask) become part of the
 recording: values may be rewritten in place between replays, index arrays may
-not.  Plans that copy an operand's values (the column-tile copy of a wide dense
-operand) are never recorded; inside a graph such a product runs from the
-operand itself.
+not.  Nothing derived from an operand's *values* is recorded (the column-tile
+copy of a wide dense operand, the verdict that a mask's values are all 1): a
+recorded product runs from the operand itself and reads every value array it
+was given.
+
+A replay writes the results, and whatever the caller copied into the static
+inputs arrived there, without PyTorch's version counters necessarily noticing.
+``capture`` therefore marks the static inputs and the results volatile
+(scorch_ops_hip.mark_volatile: eager calls that take them as operands keep
+nothing derived from their values), and every replay bumps the results' version
+counters, so that data other code derived from them is seen to be stale.
 
 The reference has no counterpart: its kernels run on the host.
 """
@@ -25,6 +33,8 @@ from __future__ import annotations
 from typing import Any, Callable
 
 import torch
+
+from . import scorch_ops_hip
 
 
 class CapturedStep:
@@ -38,6 +48,7 @@ class CapturedStep:
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError("scorch_amd.graphs: capture() called while the stream is already capturing")
         self.args = args
+        scorch_ops_hip.mark_volatile(args)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -48,9 +59,14 @@ class CapturedStep:
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.result = fn(*args)
+        self._result_tensors = list(scorch_ops_hip._tensors_of(self.result))
+        scorch_ops_hip.mark_volatile(self._result_tensors)
 
     def replay(self) -> Any:
         self.graph.replay()
+        if self._result_tensors:
+            # the replay has rewritten them in place behind the version counters' back
+            torch.autograd.graph.increment_version(self._result_tensors)
         return self.result
 
     __call__ = replay

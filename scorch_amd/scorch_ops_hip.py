@@ -148,6 +148,98 @@ class _on_device:
         return False
 
 
+# ---- what is kept beside tensors between calls, and how a caller drops it ---------------------
+# The reference's call is stateless (src/scorch/prebuilt_kernels.py:198-224); its only cache is keyed
+# on the expression and the formats, never on values (src/scorch/ops.py:425-488).  This module keeps
+# derived data as attributes of the tensors it was derived from:
+#   from index tensors   the CsrPlan (validity, longest row, chunk boundaries, entry lists, block
+#                        description), the row pointer of a coordinate mask, an attention mask's blocks
+#   from value tensors   the column-tile copy of a wide dense operand, "this mask's values are all 1"
+# Each is stamped with the tensor's address, its version counter and its epoch (below), and rebuilt
+# when the stamp no longer matches.  PyTorch bumps the version counter for every in-place operation
+# of its own on the tensor or on a view of it.  It does not for writes through ``t.data``, a raw
+# pointer, a numpy or DLPack alias, a kernel of another library, or the replay of a recorded graph:
+# after such a write call forget(t), or mark the tensor volatile once.
+_CACHE_ATTRIBUTES = ("_scorch_plan", "_scorch_tiled", "_scorch_seen", "_scorch_ones", "_scorch_coo_pos",
+                     "_scorch_block_mask", "_scorch_mask_checked")
+
+
+def _tensors_of(obj, seen=None):
+    """The torch tensors reachable from `obj`: a tensor, an STensor (values and index arrays), a result
+    carrier of this module, or lists / tuples / dicts of those."""
+    if seen is None:
+        seen = set()
+    if obj is None or id(obj) in seen:
+        return
+    seen.add(id(obj))
+    if isinstance(obj, torch.Tensor):
+        yield obj
+        origin = getattr(obj, "_scorch_origin", None)
+        if origin is not None:
+            yield from _tensors_of(origin, seen)
+    elif isinstance(obj, (list, tuple)):
+        for x in obj:
+            yield from _tensors_of(x, seen)
+    elif isinstance(obj, dict):
+        for x in obj.values():
+            yield from _tensors_of(x, seen)
+    elif isinstance(obj, (Tensor, TensorStorage, TensorIndex)) or hasattr(obj, "storage"):
+        storage = obj if isinstance(obj, TensorStorage) else getattr(obj, "storage", None)
+        if isinstance(obj, TensorIndex):
+            yield from _tensors_of(obj.mode_indices, seen)
+        elif storage is not None:
+            yield from _tensors_of(getattr(storage, "value", None), seen)
+            yield from _tensors_of(getattr(getattr(storage, "index", None), "mode_indices", None), seen)
+
+
+def _epoch(t: torch.Tensor) -> int:
+    return getattr(t, "_scorch_epoch", 0)
+
+
+def _stamp(t: torch.Tensor):
+    """What must be unchanged for data derived from `t` to be served again."""
+    return (t.data_ptr(), t._version, _epoch(t), t.numel())
+
+
+def forget(*objs) -> None:
+    """Drop everything this module has derived from the given tensors (or from the tensors of the
+    given STensors, results, lists): the next call inspects, plans and copies anew.  For writes that
+    PyTorch's version counter does not see -- ``t.data``, raw pointers, numpy / DLPack aliases,
+    kernels of other libraries, replays of recorded graphs."""
+    for t in _tensors_of(objs):
+        for name in _CACHE_ATTRIBUTES:
+            if hasattr(t, name):
+                try:
+                    delattr(t, name)
+                except AttributeError:
+                    pass
+        try:
+            t._scorch_epoch = _epoch(t) + 1      # plans that live on a partner tensor name this one's epoch
+        except (AttributeError, RuntimeError):
+            pass
+
+
+def mark_volatile(*objs, volatile: bool = True) -> None:
+    """Tensors whose *values* change behind PyTorch's back (the static inputs and the results of a
+    recorded graph, buffers another library writes): nothing derived from their values -- the
+    column-tile copy, the all-ones verdict -- is kept or used from now on.  What is derived from an
+    index tensor (a sparsity pattern) is not affected: use forget() when a pattern is rewritten."""
+    for t in _tensors_of(objs):
+        if volatile:
+            for name in ("_scorch_tiled", "_scorch_seen", "_scorch_ones"):
+                if hasattr(t, name):
+                    delattr(t, name)
+        try:
+            t._scorch_volatile = bool(volatile)
+        except (AttributeError, RuntimeError):
+            pass
+
+
+def is_volatile(t: torch.Tensor) -> bool:
+    return bool(getattr(t, "_scorch_volatile", False)) or \
+        bool(getattr(getattr(t, "_scorch_origin", None), "_scorch_volatile", False))
+
+
 # ---- what is computed once per operand ---------------------------------------------
 def plans_enabled() -> bool:
     """Sparse operands are inspected and planned unless SCORCH_HIP_PLAN=0."""
@@ -196,7 +288,7 @@ def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, wha
     len(crd) or decrease, column indices outside [0, n_cols) -- before any
     kernel dereferences it.  None when planning is switched off or the stream
     is being captured (no synchronisation is possible there)."""
-    key = (pos._version, crd.data_ptr(), crd._version, crd.numel(), n_rows, n_cols)
+    key = (_stamp(pos), _stamp(crd), n_rows, n_cols)
     plan = getattr(pos, "_scorch_plan", None)
     if plan is not None and plan.key == key:
         return plan
@@ -402,10 +494,13 @@ def _known_all_ones(values: torch.Tensor) -> bool:
     """Whether a mask's values are known to be all 1 (an attention mask; the block SDDMM then
     reads nothing for them).  Looked at when the same tensor comes back unchanged -- one
     reduction and one read of its result -- and remembered with the tensor."""
-    key = (values.data_ptr(), values._version, values.numel())
+    if torch.cuda.is_current_stream_capturing() or is_volatile(values):
+        # a recording holds pointers, not verdicts: the values may be rewritten before a replay
+        return False
+    key = _stamp(values)
     seen = getattr(values, "_scorch_ones", None)
     if seen is not None and seen[0] == key:
-        if seen[1] is None and not torch.cuda.is_current_stream_capturing():
+        if seen[1] is None:
             seen = (key, bool((values == 1).all()))
             values._scorch_ones = seen
         return bool(seen[1])
@@ -461,7 +556,7 @@ def prepare_dense_operand(values: torch.Tensor, K: int, N: int) -> Optional[torc
     with _on_device(dev):
         native.check(L.scorch_hip_dense_to_tiled_f32(K, N, flat.data_ptr(), bt.data_ptr(), bt.numel() * 4,
                                                      _stream(dev)))
-    owner._scorch_tiled = (owner._version, values.data_ptr(), K, N, bt)
+    owner._scorch_tiled = (owner._version, values.data_ptr(), K, N, bt, _epoch(owner))
     return bt
 
 
@@ -478,10 +573,13 @@ def _tiled_operand(values: torch.Tensor, K: int, N: int, nnz: int, L) -> Optiona
         # operand has been rewritten in place would read the old values, with nothing to notice it
         return None
     owner = _dense_owner(values)
+    if is_volatile(owner) or is_volatile(values):
+        return None
     stamp = (owner._version, values.data_ptr(), K, N)
     cached = getattr(owner, "_scorch_tiled", None)
-    if cached is not None and cached[:4] == stamp:
+    if cached is not None and cached[:4] == stamp and cached[5] == _epoch(owner):
         return cached[4]
+    stamp = stamp + (_epoch(owner),)
     if getattr(owner, "_scorch_seen", None) == stamp:
         return prepare_dense_operand(values, K, N)
     try:
@@ -810,7 +908,7 @@ def _coo_mask_row_ptr(row: torch.Tensor, col: torch.Tensor, M: int, n_cols: int,
     if BLOCKED_PATH == "off" or not plans_enabled() or K not in BLOCKED_WIDTHS or M % 64 or n_cols % 64 \
             or row.numel() < 8 * M or M == 0:
         return None
-    key = (row._version, col.data_ptr(), col._version, col.numel(), M)
+    key = (_stamp(row), _stamp(col), M)
     seen = getattr(row, "_scorch_coo_pos", None)
     if seen is not None and seen[0] == key:
         if seen[1] is None and not torch.cuda.is_current_stream_capturing():
@@ -914,7 +1012,7 @@ def _known_longest_row(pos: torch.Tensor, n_rows: int, nnz: int) -> Optional[int
     """The longest row of the pattern if a plan made for this row pointer says so (a product with
     the same pattern has inspected it), else None."""
     plan = getattr(pos, "_scorch_plan", None)
-    if plan is not None and plan.key[0] == pos._version and plan.key[3] == nnz and plan.key[4] == n_rows:
+    if plan is not None and plan.key[0] == _stamp(pos) and plan.key[1][3] == nnz and plan.key[2] == n_rows:
         return plan.max_row
     return None
 
@@ -1258,7 +1356,7 @@ def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_une
 def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -> BlockMask:
     """block_mask_from_csr, kept with the mask's row_ptr tensor and rebuilt when either index
     array is replaced or written to."""
-    key = (row_ptr.data_ptr(), row_ptr._version, col_idx.data_ptr(), col_idx._version, int(col_idx.numel()), S)
+    key = (_stamp(row_ptr), _stamp(col_idx), S)
     cached = getattr(row_ptr, "_scorch_block_mask", None)
     if cached is not None and cached[0] == key:
         return cached[1]
@@ -1432,11 +1530,11 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     n_masks = block_masks.numel() // block
     # the kernel trusts the mask indices as it trusts block_col_idx; a caller that built them by
     # hand gets them checked here, once per index tensor
-    if getattr(bmi, "_scorch_mask_checked", None) != (bmi._version, n_masks):
+    if getattr(bmi, "_scorch_mask_checked", None) != (_stamp(bmi), n_masks):
         if bmi.numel() and int(bmi.max()) >= n_masks:
             raise ValueError("scorch_ops_hip: block_mask_index names a mask beyond block_masks")
         try:
-            bmi._scorch_mask_checked = (bmi._version, n_masks)
+            bmi._scorch_mask_checked = (_stamp(bmi), n_masks)
         except AttributeError:
             pass
     with _on_device(dev):

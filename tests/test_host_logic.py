@@ -571,3 +571,49 @@ def test_every_chunk_of_the_tiled_split_fits_the_staging_arrays():
         largest = max(largest, y1 - y0, x1 - x0 + 2)
     assert largest > _kernel_constant("kItemsPerWave", *files) + snap_items   # more than the usual split stages
     assert largest <= slots
+
+
+# ---- what the device module keeps beside tensors ----------------------------------------------------
+def test_forget_and_mark_volatile_reach_every_tensor_of_an_operand():
+    H = scorch_ops_hip
+    dense = torch.arange(12.0).reshape(3, 4)
+    A = STensor.from_torch(dense.to_sparse_csr(), "A")
+    pos, crd = A.index.mode_indices[1]
+    found = list(H._tensors_of([A, {"x": dense}, (None, 3)]))
+    assert any(t is pos for t in found) and any(t is crd for t in found) and any(t is A.values for t in found)
+    assert any(t is dense for t in found)
+    before = (H._stamp(pos), H._stamp(crd))
+    pos._scorch_plan = object()
+    A.values._scorch_ones = (H._stamp(A.values), True)
+    H.forget(A)
+    assert not hasattr(pos, "_scorch_plan") and not hasattr(A.values, "_scorch_ones")
+    assert H._stamp(pos) != before[0] and H._stamp(crd) != before[1]     # plans kept on a partner tensor go stale too
+    assert not H.is_volatile(dense)
+    dense._scorch_tiled = ("stale",)
+    H.mark_volatile(dense)
+    assert H.is_volatile(dense) and not hasattr(dense, "_scorch_tiled")
+    flat = dense.flatten()
+    flat._scorch_origin = dense            # what STensor.from_torch and matmul note on the flat view of a device tensor
+    assert H.is_volatile(flat)
+    H.mark_volatile(dense, volatile=False)
+    assert not H.is_volatile(flat)
+    result = H.Tensor(torch.zeros(3), [[], [pos, crd]])
+    assert sum(1 for _ in H._tensors_of(result)) == 3
+
+
+def test_writes_the_version_counter_misses_are_the_ones_forget_is_for():
+    """The stamps follow PyTorch's version counter: in-place operations and writes through views
+    change them, writes through .data do not -- which is what forget() exists for."""
+    H = scorch_ops_hip
+    t = torch.zeros(8)
+    s0 = H._stamp(t)
+    t.add_(1)
+    s1 = H._stamp(t)
+    assert s1 != s0
+    t.view(2, 4)[0].mul_(2)
+    s2 = H._stamp(t)
+    assert s2 != s1
+    t.data.add_(1)
+    assert H._stamp(t) == s2
+    H.forget(t)
+    assert H._stamp(t) != s2
