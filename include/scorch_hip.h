@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define SCORCH_HIP_ABI_VERSION 1
+#define SCORCH_HIP_ABI_VERSION 2
 
 /* Every function below is exported from libscorch_hip.so. */
 #if defined(__GNUC__)
@@ -166,19 +166,29 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_f32_timed(int64_t M, int64_t K, int64_t N
  * loop, bench/README_sparse_autoencoder.md:86).  All of it lives in memory the
  * caller owns; the library keeps no state.
  *
- * scorch_hip_csr_inspect writes four int32 to `report` (device):
+ * scorch_hip_csr_inspect writes SCORCH_HIP_INSPECT_REPORT_INTS int32 to `report` (device):
  *   [0] 1 if row_ptr is malformed (row_ptr[0] != 0, row_ptr[M] != nnz, or a
  *       pointer below its predecessor), else 0
  *   [1] 1 if a column index lies outside [0, K), else 0
  *   [2] the longest row
  *   [3] the number of empty rows
+ *   [4] the number of entries that do not exceed the entry before them in their
+ *       row (0: every row's column indices increase strictly)
+ *   [5] the number of runs: maximal stretches of a row's entries that increase
+ *       and lie in one aligned group of 64 columns.  nnz / (64 * runs) bounds
+ *       from above the share of stored positions in the 64 x 64 blocks the
+ *       pattern touches: a graph is told from a mask made of blocks without
+ *       looking at blocks
+ *   [6], [7] 0 (reserved)
+ * ([4] and [5] mean what they say only when [0] is 0.)
  * It reads row_ptr[0..M] and col_idx[0..nnz) only, so it is safe on malformed
  * input; a caller that reads the report back (one synchronisation) can refuse
  * the operand before any kernel dereferences it, and knows whether all rows
  * are short.
  * ---------------------------------------------------------------------- */
+#define SCORCH_HIP_INSPECT_REPORT_INTS 8
 SCORCH_HIP_API int scorch_hip_csr_inspect(int64_t M, int64_t K, int64_t nnz, const int32_t *row_ptr,
-                           const int32_t *col_idx, int32_t *report /* device, [4] */, void *stream);
+                           const int32_t *col_idx, int32_t *report /* device, [8] */, void *stream);
 
 /* Row-split SpMM for matrices whose rows are all short: C = act(A * B + bias)
  * in one launch, without workspace (a team of lanes per row; no rows are cut,
@@ -533,6 +543,28 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_blocked_f32(
     const uint64_t *block_words, const int32_t *block_off, const uint64_t *block_cols, int64_t n_items,
     const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots, const float *vals,
     const float *B, float *C, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The block description of a CSR pattern, built on the device in two calls with one host read
+ * between them.  The reference's attention loop wraps fresh operands for every head and call
+ * (bench/bench_sparse_transformer.py:354-372), so describing a pattern must cost about what one
+ * product costs.  M and n_cols multiples of 64, at most 131,072 block columns.
+ *   _block_count  block_row_ptr[M / 64 + 1]: running count of the active blocks (those that hold
+ *                 a stored entry) per block row.  The caller reads block_row_ptr[M / 64] back,
+ *                 the number of active blocks, and allocates the arrays of the second call.
+ *   _block_fill   block_col_idx, block_words, block_off, block_cols as described above, and
+ *                 block_nnz[n_active_blocks], the number of stored positions of every block
+ *                 (4096: fully stored).  Entries may repeat and rows need not be sorted for
+ *                 block_words / block_cols / block_nnz to be right; block_off is what the block
+ *                 kernels need only when every row's columns increase strictly
+ *                 (scorch_hip_csr_inspect, report[4] == 0).  Column indices outside [0, n_cols)
+ *                 are skipped by both calls. */
+SCORCH_HIP_API int scorch_hip_csr_block_count(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
+                                              const int32_t *col_idx, int32_t *block_row_ptr, void *stream);
+SCORCH_HIP_API int scorch_hip_csr_block_fill(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
+                                             const int32_t *col_idx, const int32_t *block_row_ptr,
+                                             int64_t n_active_blocks, int32_t *block_col_idx,
+                                             uint64_t *block_words, int32_t *block_off, uint64_t *block_cols,
+                                             int32_t *block_nnz, void *stream);
 
 /* ------------------------------------------------------------------------
  * One sparsity pattern, `batch` value arrays: the three steps of the reference's

@@ -206,9 +206,20 @@ int spmm_rows_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz
 // report[1]  1 if a column index lies outside [0, K)
 // report[2]  the longest row
 // report[3]  the number of empty rows
-// Only row_ptr[0 .. M] and col_idx[0 .. nnz) are read, whatever they contain.
+// report[4]  the number of entries that do not exceed the entry before them in the same row
+//            (0: every row's columns increase strictly)
+// report[5]  the number of runs: maximal stretches of a row's entries that lie in one aligned
+//            group of 64 columns and increase.  nnz / (64 runs) bounds from above the share of
+//            stored positions in the 64 x 64 blocks the pattern touches (a block's row holds one
+//            run at least when it holds anything), so a graph is told from a mask made of blocks
+//            without looking at blocks
+// report[6], report[7]  0 (reserved)
+// Only row_ptr[0 .. M] and col_idx[0 .. nnz) are read, whatever they contain; [4] and [5] mean
+// what they say only when [0] is 0.
+constexpr int kInspectReportInts = 8;
+
 __global__ void csr_inspect_clear_kernel(int *__restrict__ report) {
-  if (threadIdx.x < 4) report[threadIdx.x] = 0;
+  if (threadIdx.x < kInspectReportInts) report[threadIdx.x] = 0;
 }
 
 __global__ __launch_bounds__(kBlockThreads) void csr_inspect_kernel(int M, int K, int64_t nnz,
@@ -218,22 +229,49 @@ __global__ __launch_bounds__(kBlockThreads) void csr_inspect_kernel(int M, int K
   const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
   const int64_t first = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
   int bad_rows = 0, bad_cols = 0, longest = 0, empty = 0;
-  if (first == 0 && (row_ptr[0] != 0 || (int64_t)row_ptr[M] != nnz)) bad_rows = 1;
+  // The entry loop below does not know where rows begin: it counts an entry as a descent when it
+  // does not exceed its predecessor, and as the head of a run when it is a descent or lies in
+  // another group of 64 columns than its predecessor.  Every row's first entry is the head of a
+  // run and never a descent, whatever its predecessor: the row loop corrects both counts.
+  int descents = 0, runs = 0;
+  if (first == 0) {
+    if (row_ptr[0] != 0 || (int64_t)row_ptr[M] != nnz) bad_rows = 1;
+    if (nnz > 0) runs = 1;  // entry 0
+  }
   for (int64_t i = first; i < M; i += stride) {
-    const int len = row_ptr[i + 1] - row_ptr[i];
+    const int begin = row_ptr[i], len = row_ptr[i + 1] - begin;
     bad_rows |= len < 0;
     longest = len > longest ? len : longest;
     empty += len == 0;
+    if (len > 0 && begin > 0 && (int64_t)begin < nnz) {
+      const int before = col_idx[begin - 1], here = col_idx[begin];
+      const bool descent = here <= before;
+      const bool head = descent || ((unsigned)here >> 6) != ((unsigned)before >> 6);
+      descents -= descent;
+      runs += !head;
+    }
   }
   {
-    // four column indices per thread in flight
+    // four column indices per thread in flight, each with its predecessor (the same cache line
+    // another lane reads, except for the wavefront's first lane)
+    auto look = [&](int64_t p) {
+      const int here = col_idx[p];
+      bad_cols |= (unsigned)here >= (unsigned)K;
+      if (p > 0) {
+        const int before = col_idx[p - 1];
+        const bool descent = here <= before;
+        descents += descent;
+        runs += descent || ((unsigned)here >> 6) != ((unsigned)before >> 6);
+      }
+    };
     int64_t p = first;
     for (; p + 3 * stride < nnz; p += 4 * stride) {
-      const unsigned c0 = (unsigned)col_idx[p], c1 = (unsigned)col_idx[p + stride];
-      const unsigned c2 = (unsigned)col_idx[p + 2 * stride], c3 = (unsigned)col_idx[p + 3 * stride];
-      bad_cols |= (c0 >= (unsigned)K) | (c1 >= (unsigned)K) | (c2 >= (unsigned)K) | (c3 >= (unsigned)K);
+      look(p);
+      look(p + stride);
+      look(p + 2 * stride);
+      look(p + 3 * stride);
     }
-    for (; p < nnz; p += stride) bad_cols |= (unsigned)col_idx[p] >= (unsigned)K;
+    for (; p < nnz; p += stride) look(p);
   }
   // one atomic of each kind per workgroup that has something to say
 #pragma unroll
@@ -241,8 +279,11 @@ __global__ __launch_bounds__(kBlockThreads) void csr_inspect_kernel(int M, int K
     const int other = __shfl_xor(longest, off);
     longest = other > longest ? other : longest;
     empty += __shfl_xor(empty, off);
+    descents += __shfl_xor(descents, off);
+    runs += __shfl_xor(runs, off);
   }
   __shared__ int s_bad_rows, s_bad_cols, s_longest[kWavesPerBlock], s_empty[kWavesPerBlock];
+  __shared__ int s_descents[kWavesPerBlock], s_runs[kWavesPerBlock];
   if (threadIdx.x == 0) s_bad_rows = s_bad_cols = 0;
   __syncthreads();
   const bool any_bad_rows = __any(bad_rows), any_bad_cols = __any(bad_cols);
@@ -251,18 +292,25 @@ __global__ __launch_bounds__(kBlockThreads) void csr_inspect_kernel(int M, int K
     if (any_bad_cols) s_bad_cols = 1;
     s_longest[threadIdx.x / kWaveSize] = longest;
     s_empty[threadIdx.x / kWaveSize] = empty;
+    s_descents[threadIdx.x / kWaveSize] = descents;
+    s_runs[threadIdx.x / kWaveSize] = runs;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    longest = empty = 0;
+    longest = empty = descents = runs = 0;
     for (int w = 0; w < kWavesPerBlock; ++w) {
       longest = s_longest[w] > longest ? s_longest[w] : longest;
       empty += s_empty[w];
+      descents += s_descents[w];
+      runs += s_runs[w];
     }
     if (s_bad_rows) atomicOr(&report[0], 1);
     if (s_bad_cols) atomicOr(&report[1], 1);
     if (longest > 0) atomicMax(&report[2], longest);
     if (empty > 0) atomicAdd(&report[3], empty);  // at most M < 2^31 in all
+    // partial sums may be negative (the row loop's corrections); the totals lie in [0, nnz]
+    if (descents != 0) atomicAdd(&report[4], descents);
+    if (runs != 0) atomicAdd(&report[5], runs);
   }
 }
 

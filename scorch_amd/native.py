@@ -111,6 +111,9 @@ SIGNATURES = {
                                                        _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
     "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "scorch_hip_coo_row_ptr": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_csr_block_count": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_csr_block_fill": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr,
+                                                 _ptr, _ptr]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import math
 import os
+import weakref
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -35,6 +36,7 @@ _empty = torch.empty
 _empty_like = torch.empty_like
 
 HINT_MOSTLY_EMPTY_ROWS = 0x100      # SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS of include/scorch_hip.h
+INSPECT_REPORT_INTS = 8             # SCORCH_HIP_INSPECT_REPORT_INTS
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
 
@@ -201,6 +203,14 @@ def _stamp(t: torch.Tensor):
     return (t.data_ptr(), t._version, _epoch(t), t.numel())
 
 
+def _same(ref, t: torch.Tensor) -> bool:
+    """Whether the weak reference `ref` still names the tensor object `t`.  Derived data lives on
+    one tensor of an operand (the row pointer) and names its partner (the column indices) by stamp;
+    a stamp alone would also match another tensor that the allocator has since put at the freed
+    partner's address."""
+    return ref is not None and ref() is t
+
+
 def forget(*objs) -> None:
     """Drop everything this module has derived from the given tensors (or from the tensors of the
     given STensors, results, lists): the next call inspects, plans and copies anew.  For writes that
@@ -266,13 +276,16 @@ class CsrPlan:
     chunk boundaries of the merge-path kernels.  Lives as an attribute of the
     row-pointer tensor, so it is dropped with the operand, and is rebuilt when
     either index tensor has been written to since."""
-    __slots__ = ("key", "max_row", "empty_rows", "bounds", "sddmm_lists", "sddmm_uses", "rows", "blocked",
-                 "blocked_uses")
+    __slots__ = ("key", "partner", "max_row", "empty_rows", "sorted_rows", "runs", "bounds", "sddmm_lists",
+                 "sddmm_uses", "rows", "blocked", "blocked_uses")
 
-    def __init__(self, key, max_row: int, empty_rows: int):
+    def __init__(self, key, max_row: int, empty_rows: int, sorted_rows: bool = False, runs: int = 0):
         self.key = key
+        self.partner = None                                # weak reference to the column-index tensor (see _same)
         self.max_row = max_row
         self.empty_rows = empty_rows
+        self.sorted_rows = sorted_rows                     # every row's column indices increase strictly
+        self.runs = runs                                   # stretches of a row inside one aligned group of 64 columns
         self.bounds: Dict[Tuple[int, int], torch.Tensor] = {}
         self.sddmm_lists: Optional[torch.Tensor] = None   # the mask's entries listed per XCD (SDDMM)
         self.sddmm_uses = 0                                # SDDMM calls that could have used them
@@ -290,7 +303,7 @@ def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, wha
     is being captured (no synchronisation is possible there)."""
     key = (_stamp(pos), _stamp(crd), n_rows, n_cols)
     plan = getattr(pos, "_scorch_plan", None)
-    if plan is not None and plan.key == key:
+    if plan is not None and plan.key == key and _same(plan.partner, crd):
         return plan
     if not plans_enabled():
         return None
@@ -299,11 +312,11 @@ def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, wha
     if torch.cuda.is_current_stream_capturing():
         return None
     dev = pos.device
-    report = _empty(4, dtype=torch.int32, device=dev)
+    report = _empty(INSPECT_REPORT_INTS, dtype=torch.int32, device=dev)
     with _on_device(dev):
         native.check(native.lib().scorch_hip_csr_inspect(n_rows, n_cols, crd.numel(), pos.data_ptr(),
                                                          crd.data_ptr(), report.data_ptr(), _stream(dev)))
-    bad_rows, bad_cols, max_row, empty_rows = report.tolist()
+    bad_rows, bad_cols, max_row, empty_rows, descents, runs = report.tolist()[:6]
     if bad_rows or bad_cols:
         problems = []
         if bad_rows:
@@ -311,7 +324,8 @@ def csr_plan(pos: torch.Tensor, crd: torch.Tensor, n_rows: int, n_cols: int, wha
         if bad_cols:
             problems.append(f"a column index lies outside [0, {n_cols})")
         raise ValueError(f"scorch_ops_hip: {what}: malformed CSR index: " + "; ".join(problems))
-    plan = CsrPlan(key, max_row, empty_rows)
+    plan = CsrPlan(key, max_row, empty_rows, descents == 0, runs)
+    plan.partner = weakref.ref(crd)
     try:
         pos._scorch_plan = plan
     except (AttributeError, RuntimeError):      # an object that takes no attributes: plan per call
@@ -348,59 +362,103 @@ BLOCKED_STRETCH = 16         # blocks per work item at most
 BLOCKED_STRETCHES = (16, 4, 1)   # the SDDMM's work items exist in these sizes: a small launch takes smaller ones
 BLOCKED_MAX_BLOCKS = 1 << 24  # blocks of the whole matrix: beyond, the operand is a graph, not a mask
 BLOCKED_MAX_NNZ = 1 << 27
+BLOCKED_MAX_BLOCK_COLS = 1 << 17  # what scorch_hip_csr_block_count takes
 
 
 class BlockedCsr:
     """A CSR pattern described by 64 x 64 blocks, for scorch_hip_{sddmm,spmm}_csr_blocked_f32:
     the active blocks in block row major order, per block and row a word of stored columns and
     the CSR position of the row's first entry in the block, and the two lists of work items."""
-    __slots__ = ("n_active", "block_col_idx", "block_words", "block_off", "block_cols", "sddmm_items",
-                 "spmm_items", "n_spmm_items", "spmm_split_rows", "n_spmm_split_rows", "n_spmm_slots",
+    __slots__ = ("n_active", "block_row_ptr", "block_col_idx", "block_words", "block_off", "block_cols", "block_nnz",
+                 "sddmm_items", "spmm_items", "n_spmm_items", "spmm_split_rows", "n_spmm_split_rows", "n_spmm_slots",
                  "n_block_rows", "longest_block_row", "fill")
 
 
-def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_fill: float) -> Optional[BlockedCsr]:
+def _describe_blocks(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_fill: float = 0.0):
+    """(block_row_ptr on the host as a numpy array, the device arrays of scorch_hip_csr_block_fill) for
+    the pattern (pos, crd): two kernel passes over the entries and, between them, one host read of
+    the block rows' counts, which sizes the second pass's arrays.  None instead of the arrays when
+    the active blocks hold less than `min_fill` of their positions (the second pass is then not run)."""
+    L = native.lib()
+    dev = pos.device
+    nnz = int(crd.numel())
+    nbr = M // 64
+    block_row_ptr = _empty(nbr + 1, dtype=torch.int32, device=dev)
+    with _on_device(dev):
+        stream = _stream(dev)
+        native.check(L.scorch_hip_csr_block_count(M, n_cols, nnz, pos.data_ptr(), crd.data_ptr(),
+                                                  block_row_ptr.data_ptr(), stream))
+        brp = block_row_ptr.cpu().numpy()                  # the one synchronisation
+        n_active = int(brp[-1])
+        if n_active == 0 or nnz < min_fill * n_active * 4096:
+            return brp, None
+        arrays = {
+            "block_row_ptr": block_row_ptr,
+            "block_col_idx": _empty(n_active, dtype=torch.int32, device=dev),
+            "block_words": _empty(n_active * 64, dtype=torch.int64, device=dev),
+            "block_off": _empty(n_active * 64, dtype=torch.int32, device=dev),
+            "block_cols": _empty(n_active, dtype=torch.int64, device=dev),
+            "block_nnz": _empty(n_active, dtype=torch.int32, device=dev),
+        }
+        native.check(L.scorch_hip_csr_block_fill(
+            M, n_cols, nnz, pos.data_ptr(), crd.data_ptr(), block_row_ptr.data_ptr(), n_active,
+            arrays["block_col_idx"].data_ptr(), arrays["block_words"].data_ptr(), arrays["block_off"].data_ptr(),
+            arrays["block_cols"].data_ptr(), arrays["block_nnz"].data_ptr(), stream))
+    return brp, arrays
+
+
+def _stretches(lens, longest, split_slots: bool):
+    """Work items (block row, begin, end, slot) over block rows of `lens` active blocks each, as an
+    int32 array of shape (n, 4) sorted longest first (ties in row order): a block row with more
+    than `longest` blocks goes out in ceil(n / longest) stretches of nearly equal length.  With
+    `split_slots` a whole row's slot is -1 and the stretches of a shared-out row get consecutive
+    slots, returned with the list of those rows (block row, first slot, stretches, 0) and the number
+    of slots; otherwise the slot is 0."""
+    import numpy as np
+    lens = np.asarray(lens, dtype=np.int64)
+    at = np.concatenate([[0], np.cumsum(lens)])[:-1]
+    parts = np.maximum(-(-lens // max(int(longest), 1)), 1)
+    row = np.repeat(np.arange(lens.size, dtype=np.int64), parts)
+    part = np.arange(row.size, dtype=np.int64) - np.repeat(np.cumsum(parts) - parts, parts)
+    lo = at[row] + lens[row] * part // parts[row]
+    hi = at[row] + lens[row] * (part + 1) // parts[row]
+    slot = np.zeros(row.size, dtype=np.int64)
+    split_rows, n_slots = np.zeros((0, 4), dtype=np.int32), 0
+    if split_slots:
+        shared = parts > 1
+        first_slot = np.cumsum(np.where(shared, parts, 0)) - np.where(shared, parts, 0)
+        slot = np.where(shared[row], first_slot[row] + part, -1)
+        n_slots = int(parts[shared].sum())
+        rows = np.nonzero(shared)[0]
+        split_rows = np.stack([rows, first_slot[rows], parts[rows], np.zeros_like(rows)], axis=1).astype(np.int32)
+    order = np.argsort(-(hi - lo), kind="stable")          # longest first
+    items = np.stack([row, lo, hi, slot], axis=1)[order].astype(np.int32)
+    return items, split_rows, n_slots
+
+
+def _blocked_csr(plan: "CsrPlan", pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int,
+                 min_fill: float) -> Optional[BlockedCsr]:
     """The block description of (pos, crd), or None when the pattern is not one the block kernels
     serve (dimensions not multiples of 64, rows not strictly increasing, blocks too thinly filled).
-    Torch operations on the operand's device and a few reads on the host; once per pattern."""
+    The inspection has already counted the pattern's runs, which bound the blocks' fill from above:
+    a graph is turned away here without a kernel.  Otherwise two kernel passes (_describe_blocks)
+    and the work-item lists, computed on the host from the block rows' lengths."""
     block = 64
     nnz = int(crd.numel())
     if M % block or n_cols % block or nnz == 0 or nnz > BLOCKED_MAX_NNZ:
         return None
     nbr, nbc = M // block, n_cols // block
-    if nbr * nbc > BLOCKED_MAX_BLOCKS or nnz < min_fill * block * M:   # (every block row has a block, usually)
+    if nbr * nbc > BLOCKED_MAX_BLOCKS or nbc > BLOCKED_MAX_BLOCK_COLS or nnz < min_fill * block * M:
+        return None                                        # (every block row has a block, usually)
+    if not plan.sorted_rows or nnz < min_fill * block * plan.runs:
         return None
     dev = pos.device
-    pos64, crd64 = pos.to(torch.int64), crd.to(torch.int64)
-    if min_fill > 0 and nbr > 3:
-        # three block rows tell a graph from a mask before anything of the operand's size is computed
-        picks = sorted({0, nbr // 2, nbr - 1})
-        ends = pos64[torch.tensor([x for b in picks for x in (b * block, (b + 1) * block)], device=dev)].tolist()
-        stored, blocks = 0, 0
-        for i, b in enumerate(picks):
-            lo, hi = ends[2 * i], ends[2 * i + 1]
-            if hi > lo:
-                stored += hi - lo
-                blocks += int(torch.unique(crd64[lo:hi] // block).numel())
-        if blocks == 0 or stored < 0.5 * min_fill * blocks * block * block:
-            return None
-    rows = torch.repeat_interleave(torch.arange(M, device=dev, dtype=torch.int64), pos64[1:] - pos64[:-1],
-                                   output_size=nnz)
-    if nnz > 1 and not bool(((crd64[1:] > crd64[:-1]) | (rows[1:] != rows[:-1])).all()):
-        return None                                   # a row with repeated or unordered columns
-    blocks, block_of = torch.unique(rows // block * nbc + crd64 // block, return_inverse=True)
-    n_active = int(blocks.numel())
-    fill = nnz / (n_active * block * block)
-    if fill < min_fill:
+    brp, arrays = _describe_blocks(pos, crd, M, n_cols, min_fill)
+    if arrays is None:
         return None
-    key = block_of * block + rows % block
-    words = torch.zeros(n_active * block, dtype=torch.int64, device=dev)
-    # distinct bits: the sum is the union (1 << 63 wraps to the sign bit, as it should)
-    words.index_add_(0, key, torch.ones_like(crd64) << (crd64 % block))
-    first = torch.full((n_active * block,), nnz, dtype=torch.int64, device=dev)
-    first.scatter_reduce_(0, key, torch.arange(nnz, device=dev, dtype=torch.int64), "amin")
-    first[first == nnz] = 0
-    lens = torch.bincount(blocks // nbc, minlength=nbr).cpu().tolist()
+    import numpy as np
+    lens = np.diff(brp).astype(np.int64)
+    n_active = int(brp[-1])
     # Work items.  SDDMM: stretches of block rows, in several sizes (the entries do not depend on how
     # they are shared out, so a launch picks the size that fills the chip).  SpMM: a block row sums into
     # one tile of the result, so it stays whole unless the rows differ by more than a quarter of their
@@ -408,47 +466,31 @@ def _blocked_csr(pos: torch.Tensor, crd: torch.Tensor, M: int, n_cols: int, min_
     # stretches whose sums a second kernel adds up in order -- the same stretches whatever the number of
     # heads, so that a head's result does not depend on what it is batched with.
     mean = n_active / nbr
-    spmm_longest = min(BLOCKED_STRETCH, max(4, -(-n_active // nbr) + 1)) if max(lens) > 1.25 * mean else max(lens)
-    sddmm_items = {stretch: [] for stretch in BLOCKED_STRETCHES}
-    spmm_items, split_rows, at, slot = [], [], 0, 0
-    for row, n in enumerate(lens):
-        for stretch, items in sddmm_items.items():
-            parts = -(-n // stretch)
-            for part in range(parts):
-                lo, hi = at + n * part // parts, at + n * (part + 1) // parts
-                items.append((hi - lo, row, lo, hi, 0))
-        if n <= spmm_longest:
-            spmm_items.append((n, row, at, at + n, -1))
-        else:
-            parts = -(-n // spmm_longest)
-            split_rows.append((row, slot, parts, 0))
-            for part in range(parts):
-                lo, hi = at + n * part // parts, at + n * (part + 1) // parts
-                spmm_items.append((hi - lo, row, lo, hi, slot))
-                slot += 1
-        at += n
-    for items in sddmm_items.values():
-        items.sort(key=lambda it: -it[0])             # longest first
-    spmm_items.sort(key=lambda it: -it[0])
+    longest = int(lens.max())
+    spmm_longest = min(BLOCKED_STRETCH, max(4, -(-n_active // nbr) + 1)) if longest > 1.25 * mean else longest
+    to_device = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev).reshape(-1)
     bl = BlockedCsr()
     bl.n_active = n_active
-    bl.block_col_idx = (blocks % nbc).to(torch.int32)
-    bl.block_words = words
-    bl.block_off = first.to(torch.int32)
-    used = words.view(n_active, block)                # columns some row of the block stores: the rows' words or-ed
-    while used.shape[1] > 1:
-        used = used[:, 0::2] | used[:, 1::2]
-    bl.block_cols = used.reshape(-1).contiguous()
-    bl.sddmm_items = {stretch: (torch.tensor([it[1:] for it in items], dtype=torch.int32, device=dev).reshape(-1),
-                                len(items)) for stretch, items in sddmm_items.items()}
-    bl.spmm_items = torch.tensor([it[1:] for it in spmm_items], dtype=torch.int32, device=dev).reshape(-1)
-    bl.n_spmm_items = len(spmm_items)
-    bl.spmm_split_rows = torch.tensor(split_rows, dtype=torch.int32, device=dev).reshape(-1)
-    bl.n_spmm_split_rows = len(split_rows)
-    bl.n_spmm_slots = slot
+    bl.block_row_ptr = arrays["block_row_ptr"]
+    bl.block_col_idx = arrays["block_col_idx"]
+    bl.block_words = arrays["block_words"]
+    bl.block_off = arrays["block_off"]
+    bl.block_cols = arrays["block_cols"]
+    bl.block_nnz = arrays["block_nnz"]
+    bl.sddmm_items = {}
+    for stretch in BLOCKED_STRETCHES:
+        items, _, _ = _stretches(lens, stretch, False)
+        items = items[items[:, 2] > items[:, 1]]           # a block row without blocks has no entries to compute
+        bl.sddmm_items[stretch] = (to_device(items), int(items.shape[0]))
+    items, split_rows, n_slots = _stretches(lens, spmm_longest, True)
+    bl.spmm_items = to_device(items)
+    bl.n_spmm_items = int(items.shape[0])
+    bl.spmm_split_rows = to_device(split_rows)
+    bl.n_spmm_split_rows = int(split_rows.shape[0])
+    bl.n_spmm_slots = n_slots
     bl.n_block_rows = nbr
-    bl.longest_block_row = max(lens)
-    bl.fill = fill
+    bl.longest_block_row = longest
+    bl.fill = nnz / (n_active * block * block)
     return bl
 
 
@@ -467,7 +509,7 @@ def _blocked(plan: Optional[CsrPlan], pos, crd, M: int, n_cols: int, width: int)
         if torch.cuda.is_current_stream_capturing() or (plan.blocked_uses < 2 and BLOCKED_PATH != "always"):
             return None
         least = 0.0 if BLOCKED_PATH == "always" else min(BLOCKED_MIN_FILL.values())
-        plan.blocked = _blocked_csr(pos, crd, M, n_cols, least) or False
+        plan.blocked = _blocked_csr(plan, pos, crd, M, n_cols, least) or False
     bl = plan.blocked or None
     if bl is not None and BLOCKED_PATH == "auto" and bl.fill < BLOCKED_MIN_FILL[width]:
         return None
@@ -910,10 +952,10 @@ def _coo_mask_row_ptr(row: torch.Tensor, col: torch.Tensor, M: int, n_cols: int,
         return None
     key = (_stamp(row), _stamp(col), M)
     seen = getattr(row, "_scorch_coo_pos", None)
-    if seen is not None and seen[0] == key:
+    if seen is not None and seen[0] == key and _same(seen[2], col):
         if seen[1] is None and not torch.cuda.is_current_stream_capturing():
             pos = coo_row_ptr(row, M)
-            seen = (key, pos if pos is not None else False)
+            seen = (key, pos if pos is not None else False, seen[2])
             row._scorch_coo_pos = seen
             if pos is not None:
                 plan = csr_plan(pos, col, M, n_cols, "S")
@@ -921,7 +963,7 @@ def _coo_mask_row_ptr(row: torch.Tensor, col: torch.Tensor, M: int, n_cols: int,
                     plan.blocked_uses = 1           # this is the mask's second product already
         return seen[1] if isinstance(seen[1], torch.Tensor) else None
     try:
-        row._scorch_coo_pos = (key, None)
+        row._scorch_coo_pos = (key, None, weakref.ref(col))
     except (AttributeError, RuntimeError):
         pass
     return None
@@ -1249,7 +1291,7 @@ class BlockMask:
     of its 64-word bit mask (bit j of word r: query r of the block row attends to key j of the
     block).  Blocks with equal masks share one."""
     __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz",
-                 "items", "split_rows", "n_slots", "schedule32")
+                 "items", "split_rows", "n_slots", "schedule32", "block_row_lens")
 
     def __init__(self, S, block, block_row_ptr, block_col_idx, block_mask_index, block_masks, nnz):
         self.S, self.block, self.nnz = S, block, nnz
@@ -1259,6 +1301,15 @@ class BlockMask:
         self.items = self.split_rows = None
         self.n_slots = 0
         self.schedule32 = None      # the fp32 kernel's own sharing-out (see _fp32_schedule)
+        self.block_row_lens = None  # active blocks per block row, on the host (numpy), once it has been read
+
+    def row_lens(self):
+        """Active blocks per block row as a numpy array on the host (read from the device once)."""
+        if self.block_row_lens is None:
+            import numpy as np
+            brp = self.block_row_ptr.cpu().numpy().astype(np.int64)
+            self.block_row_lens = brp[1:] - brp[:-1]
+        return self.block_row_lens
 
     @property
     def n_active_blocks(self) -> int:
@@ -1276,44 +1327,39 @@ class BlockMask:
 
 
 def block_mask_from_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -> BlockMask:
-    """Regroup an S x S CSR mask (S a multiple of 64) into a BlockMask, with torch operations on
-    the device the mask lives on.  Done once per mask (see attention_block_mask for the cached
-    form); duplicate entries are tolerated."""
+    """Regroup an S x S CSR mask (S a multiple of 64) on a HIP device into a BlockMask: the two
+    kernel passes of _describe_blocks over the entries, then the blocks that are not fully stored
+    are compared with one another so that equal masks are kept once.  Done once per mask (see
+    attention_block_mask for the cached form); repeated entries and unsorted rows are tolerated."""
     block = 64
     if S % block:
         raise ValueError("scorch_ops_hip: S must be a multiple of 64")
-    dev = row_ptr.device
-    nb = S // block
-    rp = row_ptr.to(torch.int64)
-    if rp.numel() != S + 1:
+    pos, crd = _index(row_ptr, "row_ptr"), _index(col_idx, "col_idx")
+    dev = _device_of(pos, crd)
+    if pos.numel() != S + 1:
         raise ValueError("scorch_ops_hip: row_ptr length does not match S")
-    cols = col_idx.to(torch.int64)
-    rows = torch.repeat_interleave(torch.arange(S, device=dev, dtype=torch.int64), rp[1:] - rp[:-1])
-    if rows.numel() != cols.numel():
-        raise ValueError("scorch_ops_hip: row_ptr does not describe col_idx")
-    if cols.numel() and (int(cols.min()) < 0 or int(cols.max()) >= S):
-        raise ValueError("scorch_ops_hip: column index out of range")
-    entry = torch.unique((rows // block * nb + cols // block) * (block * block) + rows % block * block + cols % block)
-    nnz = int(entry.numel())
-    blocks, block_of = torch.unique(entry // (block * block), return_inverse=True)  # sorted: block row major
-    n_active = int(blocks.numel())
-    words = torch.zeros(n_active * block, dtype=torch.int64, device=dev)
-    within = entry % (block * block)
-    # distinct bits: the sum is the union (1 << 63 wraps to the sign bit, as it should)
-    words.index_add_(0, block_of * block + within // block, torch.ones_like(within) << (within % block))
-    words = words.view(n_active, block)
-    full = (words == -1).all(dim=1)
+    csr_plan(pos, crd, S, S, "mask")                      # validates the index (ValueError), once per tensor pair
+    nb = S // block
+    brp, arrays = _describe_blocks(pos, crd, S, S)
+    if arrays is None:                                    # no entries at all
+        empty = lambda dtype: torch.zeros(0, dtype=dtype, device=dev)
+        bm = BlockMask(S, block, torch.zeros(nb + 1, dtype=torch.int32, device=dev), empty(torch.int32),
+                       empty(torch.int32), empty(torch.int64), 0)
+        bm.block_row_lens = brp[1:] - brp[:-1]
+        return bm
+    stored = arrays["block_nnz"]
+    n_active = int(stored.numel())
     mask_index = torch.full((n_active,), -1, dtype=torch.int32, device=dev)
-    partial = torch.nonzero(~full).flatten()
+    partial = torch.nonzero(stored != block * block).flatten()
     if partial.numel():
-        masks, which = torch.unique(words[partial], dim=0, return_inverse=True)
+        masks, which = torch.unique(arrays["block_words"].view(n_active, block)[partial], dim=0, return_inverse=True)
         mask_index[partial] = which.to(torch.int32)
     else:
         masks = torch.zeros((0, block), dtype=torch.int64, device=dev)
-    block_row_ptr = torch.zeros(nb + 1, dtype=torch.int64, device=dev)
-    block_row_ptr[1:] = torch.cumsum(torch.bincount(blocks // nb, minlength=nb), 0)
-    return BlockMask(S, block, block_row_ptr.to(torch.int32), (blocks % nb).to(torch.int32), mask_index,
-                     masks.contiguous().view(-1), nnz)
+    bm = BlockMask(S, block, arrays["block_row_ptr"], arrays["block_col_idx"], mask_index,
+                   masks.contiguous().view(-1), int(stored.sum()))
+    bm.block_row_lens = brp[1:] - brp[:-1]
+    return bm
 
 
 def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_unequal_rows: bool = False) -> BlockMask:
@@ -1324,32 +1370,21 @@ def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_une
     launch waits for.  Fills bm.items / bm.split_rows / bm.n_slots (None / None / 0 when no row is
     long enough -- unless `list_unequal_rows` asks for the rows, longest first, whenever they differ
     in length)."""
-    brp = bm.block_row_ptr.cpu().tolist()
-    nb = len(brp) - 1
-    lens = [brp[i + 1] - brp[i] for i in range(nb)]
+    lens = bm.row_lens()
+    nb = int(lens.size)
     if longest is None:
-        longest = max(8, 2 * -(-sum(lens) // max(nb, 1)))
+        longest = max(8, 2 * -(-int(lens.sum()) // max(nb, 1)))
     bm.items = bm.split_rows = None
     bm.n_slots = 0
-    if longest < 1 or max(lens, default=0) <= longest:
-        if not (list_unequal_rows and lens and min(lens) != max(lens)):
+    most = int(lens.max()) if nb else 0
+    if longest < 1 or most <= longest:
+        if not (list_unequal_rows and nb and int(lens.min()) != most):
             return bm
-    items, split_rows, slot = [], [], 0
-    for row, n in enumerate(lens):
-        if n <= longest:
-            items.append((n, row, brp[row], brp[row + 1], -1))
-            continue
-        parts = -(-n // longest)
-        split_rows.append((row, slot, parts, 0))
-        for part in range(parts):
-            lo, hi = brp[row] + n * part // parts, brp[row] + n * (part + 1) // parts
-            items.append((hi - lo, row, lo, hi, slot))
-            slot += 1
-    items.sort(key=lambda it: -it[0])                     # longest first
+    items, split_rows, n_slots = _stretches(lens, longest if longest >= 1 else max(most, 1), True)
     dev = bm.block_row_ptr.device
-    bm.items = torch.tensor([it[1:] for it in items], dtype=torch.int32, device=dev).reshape(-1)
-    bm.split_rows = torch.tensor(split_rows, dtype=torch.int32, device=dev).reshape(-1)
-    bm.n_slots = slot
+    bm.items = torch.from_numpy(items).to(dev).reshape(-1)
+    bm.split_rows = torch.from_numpy(split_rows).to(dev).reshape(-1)
+    bm.n_slots = n_slots
     return bm
 
 
@@ -1358,14 +1393,14 @@ def attention_block_mask(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) -
     array is replaced or written to."""
     key = (_stamp(row_ptr), _stamp(col_idx), S)
     cached = getattr(row_ptr, "_scorch_block_mask", None)
-    if cached is not None and cached[0] == key:
+    if cached is not None and cached[0] == key and _same(cached[2], col_idx):
         return cached[1]
     if torch.cuda.is_current_stream_capturing():
         raise RuntimeError("scorch_ops_hip: the block form of an attention mask is built with host reads; call "
                            "attention_block_mask(row_ptr, col_idx, S) once before capturing")
     bm = split_long_block_rows(block_mask_from_csr(row_ptr, col_idx, S))
     try:
-        row_ptr._scorch_block_mask = (key, bm)
+        row_ptr._scorch_block_mask = (key, bm, weakref.ref(col_idx))
     except AttributeError:
         pass
     return bm
@@ -1410,9 +1445,10 @@ def _fp32_schedule(bm: BlockMask):
         if bm.block_row_ptr.is_cuda and torch.cuda.is_current_stream_capturing():
             return None, None, 0
         plain = BlockMask(bm.S, bm.block, bm.block_row_ptr, bm.block_col_idx, None, None, bm.nnz)
-        lens = (bm.block_row_ptr[1:] - bm.block_row_ptr[:-1]).cpu().tolist()
-        mean = sum(lens) / max(len(lens), 1)
-        longest = max(lens, default=0)
+        lens = bm.row_lens()
+        plain.block_row_lens = lens
+        mean = float(lens.sum()) / max(int(lens.size), 1)
+        longest = int(lens.max()) if lens.size else 0
         if longest > 1.25 * mean:      # (rows of similar length are best left whole)
             longest = min(FP32_ATTENTION_STRETCH, max(8, 2 * math.ceil(mean)))
         split_long_block_rows(plain, longest, list_unequal_rows=True)

@@ -15,10 +15,12 @@ TOL = 1e-5
 
 
 def _inspect(rp, ci, n_cols):
-    report = torch.full((4,), -7, dtype=torch.int32, device="cuda")
+    report = torch.full((H.INSPECT_REPORT_INTS + 1,), -7, dtype=torch.int32, device="cuda")
     native.check(native.lib().scorch_hip_csr_inspect(rp.numel() - 1, n_cols, ci.numel(), rp.data_ptr(), ci.data_ptr(),
                                                      report.data_ptr(), torch.cuda.current_stream().cuda_stream))
-    return report.tolist()
+    report = report.tolist()
+    assert report[6:] == [0, 0, -7]              # reserved fields cleared, nothing written past the report
+    return report[:4]
 
 
 def test_inspection_report():
@@ -230,8 +232,9 @@ def test_a_dense_operand_seen_twice_is_tiled_and_tracks_changes(oracle):
 
 
 def test_a_recorded_step_never_reads_a_tiled_copy(oracle):
-    """A wide dense operand that has a column-tile copy (built during the warm-up) and is then
-    rewritten in place between replays of a captured step: every replay sees the new values."""
+    """A wide dense operand that has a column-tile copy (built by eager products) and is then
+    handed to a captured step and rewritten in place between replays: every replay sees the new
+    values, and the capture has made the operand volatile, so no copy of it is kept any more."""
     from scorch_amd import graphs
     rng = np.random.default_rng(41)
     M, K, N = 512, 2048, 2048
@@ -239,13 +242,16 @@ def test_a_recorded_step_never_reads_a_tiled_copy(oracle):
     t_rp, t_ci, t_v = dev(rp), dev(ci), dev(v)
     B = torch.randn(K * N, device="cuda")
     product = lambda b: H.spmm_csr_float_v2([M, N], [M, K], [[], [t_rp, t_ci]], t_v, [K, N], [[], []], b).storage.value
+    for _ in range(3):
+        product(B)
+    assert getattr(B, "_scorch_tiled", None) is not None        # eager products built the copy
     step = graphs.capture(product, B, warmup=3)
-    assert getattr(B, "_scorch_tiled", None) is not None        # the eager warm-up did build the copy
+    assert H.is_volatile(B) and getattr(B, "_scorch_tiled", None) is None
     for _ in range(3):
         B.copy_(torch.randn(K * N, device="cuda"))
         got = step().clone()
         assert oracle.rel_fro(host(got).reshape(M, N), oracle.spmm_fp64(rp, ci, v, host(B).reshape(K, N))) <= TOL
-        assert torch.equal(got, product(B))                     # the eager call re-tiles and agrees bit for bit
+        assert torch.equal(got, product(B))                     # the eager call runs from the operand itself too
 
 
 def test_matmul_keeps_the_tiled_copy_on_the_callers_tensor(oracle):
@@ -295,5 +301,6 @@ def test_tiled_kernel_when_the_even_resplit_makes_chunks_longer_than_the_usual_o
     got = hip_spmm(rp, ci, v, B, path="tiled")
     assert oracle.rel_fro(got, want) <= TOL
     merge = hip_spmm(rp, ci, v, B, path="merge")
-    np.testing.assert_allclose(got, merge, rtol=1e-4, atol=1e-5)
+    assert oracle.rel_fro(got, merge) <= 1e-6                # (long rows are summed in another grouping)
+    np.testing.assert_allclose(got, merge, rtol=1e-2, atol=1e-4)
     assert np.array_equal(got, hip_spmm(rp, ci, v, B, path="tiled"))

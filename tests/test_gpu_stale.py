@@ -174,3 +174,24 @@ def test_an_index_rewritten_through_data_is_inspected_again_after_forget():
     H.forget(A)
     with pytest.raises(ValueError, match="row_ptr"):
         scorch.matmul(A, B.reshape(K, N), format="dd")
+
+
+def test_a_new_index_tensor_at_a_freed_tensors_address_is_not_taken_for_it():
+    """The plan lives on the row pointer and names the column indices by address, version and
+    length -- and by identity: the allocator hands a freed tensor's address to the next tensor of
+    its size, which must be inspected as the new operand it is."""
+    pos = dev(np.array([0, 2, 4], np.int32))
+    B = torch.ones(8 * 16, device="cuda")
+    vals = torch.ones(4, device="cuda")
+    product = lambda crd: H.spmm_csr_float_v2([2, 16], [2, 8], [[], [pos, crd]], vals, [8, 16], [[], []], B)
+    crd = dev(np.array([0, 3, 1, 7], np.int32))
+    address = crd.data_ptr()
+    product(crd)
+    assert pos._scorch_plan.partner() is crd
+    del crd
+    for _ in range(4):                                       # the caching allocator reuses the block
+        crd = dev(np.array([0, 3, 1, 8], np.int32))          # column 8 of 8
+        if crd.data_ptr() == address:
+            break
+    with pytest.raises(ValueError, match="column index"):
+        product(crd)

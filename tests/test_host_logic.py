@@ -308,6 +308,16 @@ def _csr_of(mask):
     return torch.from_numpy(rp), torch.from_numpy(np.nonzero(mask)[1].astype(np.int32))
 
 
+def _block_mask_of(active):
+    """BlockMask of a mask made of whole 64 x 64 blocks, active[i, j] saying which."""
+    nb = active.shape[0]
+    brp = np.concatenate([[0], np.cumsum(active.sum(1))]).astype(np.int32)
+    bci = np.nonzero(active)[1].astype(np.int32)
+    return scorch_ops_hip.BlockMask(64 * nb, 64, torch.from_numpy(brp), torch.from_numpy(bci),
+                                    torch.full((bci.size,), -1, dtype=torch.int32), torch.zeros(0, dtype=torch.int64),
+                                    int(bci.size) * 4096)
+
+
 def _mask_of(bm):
     """The dense mask a BlockMask stands for."""
     brp, bci, bmi = (t.numpy() for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index))
@@ -321,51 +331,6 @@ def _mask_of(bm):
     return out
 
 
-def test_block_mask_from_csr_round_trips_and_shares_equal_masks():
-    rng = np.random.default_rng(40)
-    S = 320
-    mask = rng.random((S, S)) < 0.03
-    mask[0:64, 64:128] = True                      # a full block
-    mask[128:192, :] = False                       # an empty block row
-    mask[64:128, 0:64] = np.tri(64, dtype=bool)    # two equal partial blocks
-    mask[256:320, 192:256] = np.tri(64, dtype=bool)
-    mask[100, 319] = True                          # bit 63 of a word
-    rp, ci = _csr_of(mask)
-    bm = scorch_ops_hip.block_mask_from_csr(rp, ci, S)
-    assert np.array_equal(_mask_of(bm), mask) and bm.nnz == int(mask.sum())
-    brp, bci, bmi = (t.numpy() for t in (bm.block_row_ptr, bm.block_col_idx, bm.block_mask_index))
-    at = {(br, int(bci[i])): int(bmi[i]) for br in range(5) for i in range(brp[br], brp[br + 1])}
-    assert at[(0, 1)] == -1 and at[(1, 0)] == at[(4, 3)] >= 0 and brp[3] == brp[2]
-    assert bm.n_masks < bm.n_active_blocks
-    # duplicate entries are tolerated
-    rp2 = torch.tensor([0, 3] + [3] * 63, dtype=torch.int32)
-    bm2 = scorch_ops_hip.block_mask_from_csr(rp2, torch.tensor([5, 5, 7], dtype=torch.int32), 64)
-    assert bm2.nnz == 2 and int(bm2.block_masks[0]) == (1 << 5) | (1 << 7)
-    with pytest.raises(ValueError):
-        scorch_ops_hip.block_mask_from_csr(rp2, torch.tensor([5, 64, 7], dtype=torch.int32), 64)
-    with pytest.raises(ValueError):
-        scorch_ops_hip.block_mask_from_csr(rp, ci, 100)
-
-
-def test_longformer_mask_in_block_form():
-    """The reference's Longformer pattern (window 64, one global token) at S = 4096: 314 active
-    blocks, 6 distinct masks, and only the global token's block row is shared out."""
-    from scorch_amd import workloads
-    rp, ci = workloads.longformer_mask(4096)
-    bm = scorch_ops_hip.split_long_block_rows(
-        scorch_ops_hip.block_mask_from_csr(torch.from_numpy(rp), torch.from_numpy(ci), 4096))
-    assert (bm.n_active_blocks, bm.n_masks, bm.nnz) == (314, 6, 532286)
-    assert bm.split_rows.tolist() == [0, 0, 7, 0] and bm.n_slots == 7
-    items = bm.items.view(-1, 4).numpy()
-    lengths = items[:, 2] - items[:, 1]
-    assert (np.diff(lengths) <= 0).all() and lengths.max() <= 10          # longest first, none long
-    covered = np.zeros(314, int)
-    for _, lo, hi, _ in items:
-        covered[lo:hi] += 1
-    assert (covered == 1).all()
-    assert sorted(items[items[:, 3] >= 0, 3].tolist()) == list(range(7))
-
-
 @pytest.mark.parametrize("longest", [1, 2, 5])
 def test_split_long_block_rows_covers_every_block_once(longest):
     rng = np.random.default_rng(41 + longest)
@@ -373,9 +338,7 @@ def test_split_long_block_rows_covers_every_block_once(longest):
     active = rng.random((nb, nb)) < 0.5
     active[3, :] = True
     active[7, :] = False
-    mask = np.kron(active, np.ones((64, 64), bool))
-    rp, ci = _csr_of(mask)
-    bm = scorch_ops_hip.split_long_block_rows(scorch_ops_hip.block_mask_from_csr(rp, ci, 64 * nb), longest)
+    bm = scorch_ops_hip.split_long_block_rows(_block_mask_of(active), longest)
     items = bm.items.view(-1, 4).numpy()
     brp = bm.block_row_ptr.numpy()
     covered = np.zeros(bm.n_active_blocks, int)
@@ -389,8 +352,20 @@ def test_split_long_block_rows_covers_every_block_once(longest):
         mine = items[items[:, 0] == row]
         assert sorted(mine[:, 3].tolist()) == list(range(first, first + parts))
     # a mask whose rows are all short enough is left alone
-    bm = scorch_ops_hip.split_long_block_rows(scorch_ops_hip.block_mask_from_csr(rp, ci, 64 * nb), nb)
+    bm = scorch_ops_hip.split_long_block_rows(_block_mask_of(active), nb)
     assert bm.items is None and bm.n_slots == 0
+
+
+@pytest.mark.parametrize("longest,split", [(1, True), (3, True), (4, False), (16, True), (100, False)])
+def test_work_items_by_array_operations_equal_the_plain_loops(longest, split):
+    from blockdesc_reference import stretches
+    rng = np.random.default_rng(longest)
+    lens = rng.integers(0, 40, 57)
+    lens[[3, 20]] = [0, 97]
+    items, split_rows, n_slots = scorch_ops_hip._stretches(lens, longest, split)
+    want_items, want_rows, want_slots = stretches(lens, longest, split)
+    assert items.dtype == np.int32 and items.tolist() == [list(it) for it in want_items]
+    assert split_rows.tolist() == [list(r) for r in want_rows] and n_slots == want_slots
 
 
 def test_names_the_package_lacks_resolve_to_torch():
@@ -449,57 +424,6 @@ def test_fp32_attention_schedule_covers_every_block_once_in_short_stretches():
     even = H.BlockMask(256, 64, torch.arange(0, 17, 4, dtype=torch.int32), torch.arange(4, dtype=torch.int32).repeat(4),
                        None, None, 16 * 4096)
     assert H._fp32_schedule(even) == (None, None, 0)
-
-
-def test_block_description_of_a_csr_pattern():
-    """_blocked_csr against a direct reading of the pattern: every stored entry is found at
-    block_off + (stored columns below it), every work-item list covers what it must."""
-    import numpy as np
-    import torch
-    from scorch_amd import scorch_ops_hip as H
-    rng = np.random.default_rng(0)
-    M, n_cols = 192, 320
-    mask = rng.random((M, n_cols)) < 0.3
-    mask[64:128] = False                                          # a block row without blocks
-    mask[:, 128:192] = False                                      # a block column without blocks
-    mask[130, :] = False                                          # an empty row inside an active block row
-    rp = np.zeros(M + 1, dtype=np.int32)
-    rp[1:] = np.cumsum(mask.sum(axis=1))
-    ci = np.nonzero(mask)[1].astype(np.int32)
-    bl = H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(ci), M, n_cols, 0.1)
-    assert bl is not None and bl.n_block_rows == 3 and abs(bl.fill - ci.size / (bl.n_active * 4096)) < 1e-12
-    cols = bl.block_col_idx.tolist()
-    words = bl.block_words.view(-1, 64).numpy().view(np.uint64)
-    offs = bl.block_off.view(-1, 64).numpy()
-    spmm_items = sorted(bl.spmm_items.view(-1, 4).tolist())
-    assert [it[0] for it in spmm_items] == [0, 1, 2] and spmm_items[1][1] == spmm_items[1][2]
-    used = bl.block_cols.numpy().view(np.uint64)
-    seen = np.zeros(ci.size, dtype=bool)
-    for row_block, lo, hi, _ in spmm_items:
-        assert cols[lo:hi] == sorted(cols[lo:hi]) and 2 not in cols[lo:hi]
-        for b in range(lo, hi):
-            block = mask[64 * row_block:64 * row_block + 64, 64 * cols[b]:64 * cols[b] + 64]
-            assert int(used[b]) == sum(1 << c for c in range(64) if block[:, c].any())
-            for r in range(64):
-                row = 64 * row_block + r
-                stored = [c for c in range(64) if mask[row, 64 * cols[b] + c]]
-                assert int(words[b, r]) == sum(1 << c for c in stored)
-                for rank, c in enumerate(stored):
-                    at = offs[b, r] + rank
-                    assert rp[row] <= at < rp[row + 1] and ci[at] == 64 * cols[b] + c and not seen[at]
-                    seen[at] = True
-    assert seen.all()
-    for stretch, (items, n_items) in bl.sddmm_items.items():
-        covered = sorted((lo, hi) for _, lo, hi, _ in items.view(-1, 4).tolist())
-        assert len(covered) == n_items and covered[0][0] == 0 and covered[-1][1] == bl.n_active
-        assert all(a[1] == b[0] for a, b in zip(covered, covered[1:])) and all(hi - lo <= stretch for lo, hi in covered)
-    assert set(bl.sddmm_items) == set(H.BLOCKED_STRETCHES) and bl.sddmm_items[1][1] == bl.n_active
-    # what the description is not built for
-    assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(ci), M, n_cols, 0.5) is None     # too thinly filled
-    assert H._blocked_csr(torch.from_numpy(rp[:-1]), torch.from_numpy(ci[:rp[-2]]), M - 1, n_cols, 0.0) is None
-    backwards = ci.copy()
-    backwards[rp[3]:rp[4]] = backwards[rp[3]:rp[4]][::-1]
-    assert H._blocked_csr(torch.from_numpy(rp), torch.from_numpy(backwards), M, n_cols, 0.0) is None
 
 
 # ---- the work split of the SpMM kernels, replayed on the host ---------------------------------------
