@@ -42,35 +42,53 @@ CONFIG_WORKLOADS = ("spmm_uniform", "sddmm_uniform", "attention_blocksparse", "s
 # Bytes through the L2-to-fabric boundary per launch of each configuration's
 # dominant kernel at its default size: FETCH_SIZE (KiB, x 2.0: the factor a
 # 1 GiB device copy gives for this counter on gfx950) + WRITE_SIZE (KiB, x 1.0)
-# from two rocprofv3 --pmc runs of `python3 bench.py --workload NAME --no-cpu`.
-# Measured constants: valid for the default sizes and for the kernels as they
-# stood at the named commit only (null for anything else); the summaries with
-# the commands are the named files.
-# bytes = FETCH_SIZE [KiB] x 1024 x 2.0 + WRITE_SIZE [KiB] x 1024 of the dominant kernel, the factors
-# being what the same counters read for a copy of known size (profiles/copy_calibration.md).
+# from two rocprofv3 --pmc runs of `python3 bench.py --workload NAME --no-cpu`
+# (the factors are what the same counters read for a copy of known size,
+# profiles/copy_calibration.md).  A measured constant holds for the default size
+# and for the kernel as its source files stood when it was measured: "sha16" is
+# the hash of those files then (source_hash below; `python bench.py
+# --source-hashes` prints the current ones), and a record whose files have
+# changed since reports "traffic": null until it is measured again.
+_CSRC = "scorch_amd/csrc/"
+_SPMM_SOURCES = (_CSRC + "spmm.hip", _CSRC + "spmm.hpp", _CSRC + "common.hpp")
 MEASURED_TRAFFIC = {
-    ("gcn_powerlaw", "merge"): {"bytes": 9_790_400_000, "commit": "41c9d10",
+    ("gcn_powerlaw", "merge"): {"bytes": 9_790_400_000, "sources": _SPMM_SOURCES, "sha16": "f83608455ca9b538",
                                 "profile": "profiles/spmm_merge_kernel_gcn_powerlaw.md"},
-    ("spmm_uniform", "rows"): {"bytes": 10_820_000, "commit": "ea89918",
+    ("spmm_uniform", "rows"): {"bytes": 10_820_000, "sources": (_CSRC + "spmm_rows.hip", _CSRC + "spmm.hpp",
+                                                                _CSRC + "common.hpp"), "sha16": "",
                                "profile": "profiles/spmm_rows_kernel_uniform_4096.md"},
-    ("sae_decoder", "tiled"): {"bytes": 666_300_000, "commit": "ea89918",
+    ("sae_decoder", "tiled"): {"bytes": 666_300_000, "sources": (_CSRC + "spmm_tiled.hip", _CSRC + "spmm.hpp",
+                                                                 _CSRC + "common.hpp"), "sha16": "",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "commit": "ea89918",
+    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "sources": _SPMM_SOURCES, "sha16": "f83608455ca9b538",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sddmm_uniform", "listed"): {"bytes": 360_500_000, "commit": "ef63360",
-                                  "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("sddmm_uniform", "plain"): {"bytes": 867_200_000, "commit": "ef63360",
-                                 "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "commit": "ea89918",
-                                         "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
+    ("sddmm_uniform", "listed"): {"bytes": 360_500_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
+                                  "sha16": "54b07aaa7167ed6f", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("sddmm_uniform", "plain"): {"bytes": 867_200_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
+                                 "sha16": "54b07aaa7167ed6f", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "sources": (_CSRC + "attn.hip", _CSRC + "common.hpp"),
+                                         "sha16": "680980df0b40e9db", "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
 }
+
+
+def source_hash(files):
+    """First 16 hex digits of the SHA-256 over the named files' bytes, in order."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic(name, path, default_size):
     rec = MEASURED_TRAFFIC.get((name, path))
     if rec is None or not default_size:
         return None, None
-    return rec["bytes"], {"commit": rec["commit"], "profile": rec["profile"]}
+    if source_hash(rec["sources"]) != rec["sha16"]:
+        return None, {"profile": rec["profile"], "stale": "the kernel's source files have changed since the "
+                                                          "counters were read"}
+    return rec["bytes"], {"sha16": rec["sha16"], "profile": rec["profile"]}
 
 
 def spmm_algorithmic_bytes(M, K, N, nnz):
@@ -84,27 +102,39 @@ def spmm_gather_bytes(M, N, nnz):
 
 
 # ---- CPU baselines: the reference's own kernels (oracle/_ref) on the host cores ------------------
-def _timed_calls(fn, repeats):
+# Protocol of the reference's benchmarks (bench/_utils.py:295-310): 3 warm-up calls, 10 timed,
+# median.  Two figures where they differ: the kernel's loop alone, and the call as the reference's
+# dispatch times it (src/scorch/prebuilt_kernels.py:217-222: the whole native call, which for SpMM
+# allocates and zero-fills the result, csrc/spmm.h:2024-2025).
+CPU_WARMUP, CPU_REPEATS = 3, 10
+
+
+def _timed_calls(fn, repeats=CPU_REPEATS, warmup=CPU_WARMUP):
     times = []
-    for i in range(repeats + 1):
+    for i in range(warmup + repeats):
         t0 = time.perf_counter()
         out = fn()
         dt = time.perf_counter() - t0
         del out
-        if i:
+        if i >= warmup:
             times.append(dt)
     return statistics.median(times)
 
 
-def cpu_baseline_spmm(w, repeats=5):
-    """The reference's spmm_csr_float_v2 (oracle/_ref, compiled from the
-    reference's sources) or, where that module is absent, this repository's C
-    restatement of it, on the host cores and the same inputs.  The timed region
-    is the whole native call, as the reference's own eval_time is: it includes
-    allocating and zero-filling C."""
+_PROTOCOL = f"median of {CPU_REPEATS} calls after {CPU_WARMUP} warm-up calls"
+
+
+def cpu_baseline_spmm(w):
+    """Two timings on the host cores and the same inputs.  as_reference_times_it_ms: the
+    reference's spmm_csr_float_v2 itself (oracle/_ref, compiled from the reference's sources;
+    this repository's C restatement of it where that module is absent or this host cannot run
+    it), the whole native call -- it allocates and zero-fills C.  kernel_only_ms: the
+    restatement's loop into a result that is already allocated and zeroed (the compiled reference
+    cannot be entered past its allocation).  `value` is computed from the first."""
+    import numpy as np
     from oracle import oracle as O
     M, N, nnz = w["M"], w["N"], int(w["col_idx"].size)
-    kind, med = "port", None
+    kind, whole = "port", None
     if O.have_ref():
         try:
             import torch
@@ -112,23 +142,31 @@ def cpu_baseline_spmm(w, repeats=5):
             pos, crd = torch.from_numpy(w["row_ptr"]), torch.from_numpy(w["col_idx"])
             val, Bf = torch.from_numpy(w["vals"]), torch.from_numpy(w["B"]).reshape(-1)
             args = ([M, N], [M, w["K"]], [[], [pos, crd]], val, [w["K"], N], [[], []], Bf)
-            med = _timed_calls(lambda: mod.spmm_csr_float_v2(*args), repeats)
+            whole = _timed_calls(lambda: mod.spmm_csr_float_v2(*args))
             kind = "reference"
-        except Exception as exc:  # module built for another host
+        except Exception as exc:  # module built against another torch
             print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
-    if med is None:
-        import numpy as np
-        out = np.empty((M, N), dtype=np.float32)
-        med = _timed_calls(lambda: O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"], out=out), repeats)
-    return {"value": round(2.0 * nnz * N / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
-            "kind": kind, "ms_per_step": round(med * 1e3, 3),
-            "sample": f"full workload (M={M}, nnz={nnz}, N={N}), median of {repeats} calls after 1 "
-                      "warm-up, whole native call incl. allocating and zeroing C"}
+    if whole is None:
+        whole = _timed_calls(lambda: O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"]))
+    out = np.zeros((M, N), dtype=np.float32)
+
+    def loop_only():
+        O.spmm_csr_f32_v2(w["row_ptr"], w["col_idx"], w["vals"], w["B"], out=out, zero_fill=False)
+
+    loop = _timed_calls(loop_only)
+    return {"value": round(2.0 * nnz * N / whole / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
+            "kind": kind, "ms_per_step": round(whole * 1e3, 3),
+            "as_reference_times_it_ms": round(whole * 1e3, 3), "kernel_only_ms": round(loop * 1e3, 3),
+            "kernel_only_kind": "port",
+            "sample": f"full workload (M={M}, nnz={nnz}, N={N}), {_PROTOCOL}; as_reference_times_it_ms: the "
+                      "whole native call incl. allocating and zeroing C; kernel_only_ms: the restatement's "
+                      "loop into a result allocated and zeroed beforehand"}
 
 
-def cpu_baseline_sddmm(w, repeats=5):
-    """The reference's sddmm_coo_float_prebuilt (oracle/_ref) or the C
-    restatement of it, on the host cores, coordinate mask, same inputs."""
+def cpu_baseline_sddmm(w):
+    """The reference's sddmm_coo_float_prebuilt (oracle/_ref) or the C restatement of it, on the
+    host cores, coordinate mask, same inputs: the whole call as the reference's dispatch times it
+    (it allocates the result's values), and the restatement's loop alone."""
     from oracle import oracle as O
     nnz, K = int(w["col_idx"].size), w["K"]
     kind = "reference" if O.have_ref() else "port"
@@ -140,19 +178,23 @@ def cpu_baseline_sddmm(w, repeats=5):
         return O.sddmm_coo_f32(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])
 
     try:
-        med = _timed_calls(ref if kind == "reference" else port, repeats)
-    except Exception as exc:  # module built for another host
+        whole = _timed_calls(ref if kind == "reference" else port)
+    except Exception as exc:  # module built against another torch
         if kind == "port":
             raise
         print(f"[bench] reference module unusable here ({exc}); timing the C restatement", file=sys.stderr)
-        kind, med = "port", _timed_calls(port, repeats)
-    return {"value": round((2.0 * nnz * K + nnz) / med / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
-            "kind": kind, "ms_per_step": round(med * 1e3, 3),
-            "sample": f"full workload (nnz={nnz}, K={K}), median of {repeats} calls after 1 warm-up, "
-                      "incl. wrapping the operands"}
+        kind, whole = "port", _timed_calls(port)
+    loop = whole if kind == "port" else _timed_calls(port)
+    return {"value": round((2.0 * nnz * K + nnz) / whole / 1e9, 3), "unit": "GFLOP/s", "cores": O.num_threads(),
+            "kind": kind, "ms_per_step": round(whole * 1e3, 3),
+            "as_reference_times_it_ms": round(whole * 1e3, 3), "kernel_only_ms": round(loop * 1e3, 3),
+            "kernel_only_kind": "port",
+            "sample": f"full workload (nnz={nnz}, K={K}), {_PROTOCOL}; as_reference_times_it_ms incl. wrapping "
+                      "the operands and copying the result's index arrays; kernel_only_ms: the restatement's "
+                      "loop with its result array"}
 
 
-def cpu_baseline_attention(w, heads=2, pattern=None):
+def cpu_baseline_attention(w, heads=4, pattern=None):
     """The per-head composition of the reference's attention benchmark
     (bench/bench_sparse_transformer.py:354-372) on the host cores, fp32, for a
     sample of the heads: its SDDMM and SpMM kernels (oracle/_ref, or the C
@@ -186,16 +228,20 @@ def cpu_baseline_attention(w, heads=2, pattern=None):
         print(f"[bench] reference module unusable here ({exc}); timing the C restatements", file=sys.stderr)
         kind = "port"
         head(0, False)
-    t0 = time.perf_counter()
+    times = []
     for h in range(heads):
+        t0 = time.perf_counter()
         head(h, kind == "reference")
-    per_head = (time.perf_counter() - t0) / heads
+        times.append(time.perf_counter() - t0)
+    per_head = statistics.median(times)
     nnz = int(crd.size)
     return {"value": round(4.0 * nnz * D / per_head / 1e12, 4), "unit": "TFLOP/s", "cores": O.num_threads(),
             "kind": kind, "ms_per_step": round(per_head * H * 1e3, 1),
-            "sample": f"{heads} of {H} heads after 1 warm-up head (nnz per head {nnz}); ms_per_step is the per-head "
-                      f"time x {H}; SDDMM -> row softmax -> SpMM per head in fp32, the softmax leg is the "
-                      "oracle's C restatement of the benchmark's torch ops"}
+            "as_reference_times_it_ms": round(per_head * H * 1e3, 1),
+            "sample": f"{heads} of {H} heads after 1 warm-up head (nnz per head {nnz}), median; ms_per_step is the "
+                      f"per-head time x {H}; SDDMM -> row softmax -> SpMM per head in fp32, each product the whole "
+                      "native call as the reference times it; the softmax leg is the oracle's C restatement of "
+                      "the benchmark's torch ops"}
 
 
 # ---- device timing ----------------------------------------------------------------------------
@@ -238,7 +284,17 @@ def _time_steps(fn, steps, warmup, rounds=3, min_round_ms=4.0):
         results = []
     while len(results) < rounds:
         results.append(one_round(n))
+    global _last_timing
+    _last_timing = {"steps": n, "rounds": len(results)}
     return statistics.median(results)
+
+
+_last_timing = {"steps": 0, "rounds": 0}
+
+
+def _timed_as():
+    """How the last _time_steps call was timed: steps per round and rounds (median taken)."""
+    return dict(_last_timing)
 
 
 def _kernel_times(fn, samples):
@@ -278,6 +334,7 @@ def _hbm_roofline(kernel, kernel_ms, algo, traffic, provenance, extra=None):
            "kernel_ms_avg": round(kernel_ms, 5)}
     if provenance:
         out["traffic_measured_at"] = provenance
+    if traffic is not None:
         # what the memory system moved per second for this kernel: the distance to the HBM peak that
         # remains once the re-reads the access pattern forces are counted
         out["traffic_gbps"] = round(traffic / (kernel_ms * 1e-3) / 1e9, 1)
@@ -325,8 +382,10 @@ def run_spmm(name, args, headline=False):
         torch.cuda.synchronize()
         ms_per_step = (time.perf_counter() - t_begin) * 1e3 / args.steps
         event_ms = start.elapsed_time(stop) / args.steps
+        timed = {"steps": args.steps, "rounds": 1}
     else:
         ms_per_step = event_ms = _time_steps(fn, args.steps, 0)
+        timed = _timed_as()
 
     tiled = getattr(B, "_scorch_tiled", None) is not None
     plan = getattr(pos, "_scorch_plan", None)
@@ -342,9 +401,10 @@ def run_spmm(name, args, headline=False):
         names = [f"spmm_merge_kernel<float,{vec},0>" if N * 4 > 256 else "spmm_grouped_kernel<float,...>",
                  "spmm_fixup_kernel<float,...>"]
     dominant = max(range(len(kernels)), key=lambda i: kernels[i])
-    # a single-launch step: the queued per-step time is the kernel's duration without the events'
-    # own overhead, which matters for kernels of a few microseconds
-    kernel_ms = event_ms if len(kernels) == 1 and not headline else kernels[dominant]
+    # the named kernel's own duration, HIP events around its launch (for a kernel of a few
+    # microseconds that includes the dispatch of an isolated launch, which back-to-back launches
+    # hide: ms_per_step, the queued time per step, can be the smaller figure)
+    kernel_ms = kernels[dominant]
 
     flops = 2.0 * nnz * N
     algo, gather = spmm_algorithmic_bytes(M, K, N, nnz), spmm_gather_bytes(M, N, nnz)
@@ -353,7 +413,8 @@ def run_spmm(name, args, headline=False):
         "metric": "CSR SpMM GFLOP/s + HBM GB/s (% peak), power-law 1M rows, N=128 fp32" if headline
                   else "CSR SpMM GFLOP/s",
         "value": round(flops / (ms_per_step * 1e-3) / 1e9, 2), "unit": "GFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "n_gpus": 1, "steps": timed["steps"], "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "timed_rounds": timed["rounds"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": name + "_spmm_fp32" if name == "gcn_powerlaw" else name + "_fp32",
                    "rows": M, "cols": K, "nnz": nnz, "features": N,
@@ -409,6 +470,8 @@ def run_sddmm(args):
                                              [n_cols, K], [[], []], Bf)
     warm = _warmup_calls(csr, args.warmup)
     ms = _time_steps(csr, args.steps, 0)
+    timed = _timed_as()
+    kernel_ms = max(_kernel_times(csr, min(args.steps, 10)))
     ms_coo = _time_steps(coo, args.steps, 2)
     flops = 2.0 * nnz * K + nnz
     # every array once: row_ptr, col_idx, mask values, A, B, result values; the CSR-mask kernel
@@ -419,15 +482,17 @@ def run_sddmm(args):
     listed = plan is not None and plan.sddmm_lists is not None
     traffic, provenance = measured_traffic("sddmm_uniform", "listed" if listed else "plain", True)
     rec = {"metric": "CSR SDDMM GFLOP/s", "value": round(flops / ms / 1e6, 2), "unit": "GFLOP/s",
-           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+           "n_gpus": 1, "steps": timed["steps"], "timed_rounds": timed["rounds"], "warmup": args.warmup,
+           "ms_per_step": round(ms, 5),
            "ms_per_step_coo_mask": round(ms_coo, 5), "higher_is_better": True, "dtype": "f32", "data": "synthetic",
            "config": {"workload": "sddmm_uniform_fp32", "rows": M, "cols": n_cols, "nnz": nnz, "K": K,
                       "seed": workloads.SEEDS["sddmm_uniform"]},
            "warmup_ms": warm,
            "path": "listed" if listed else "plain",
-           "roofline": _hbm_roofline("sddmm_listed_kernel<16,4>" if listed else "sddmm_kernel<16,4,false,false>", ms, algo, traffic, provenance,
+           "roofline": _hbm_roofline("sddmm_listed_kernel<16,4>" if listed else "sddmm_kernel<16,4,false,false>",
+                                     kernel_ms, algo, traffic, provenance,
                                      {"row_coordinate_output_bytes": 4 * nnz, "gather_model_bytes": gather,
-                                      "gather_model_gbps": round(gather / ms / 1e6, 1)})}
+                                      "gather_model_gbps": round(gather / kernel_ms / 1e6, 1)})}
     if args.vendor:
         mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
         Bt = B.t().contiguous()
@@ -452,22 +517,27 @@ def run_attention(args):
     fn = lambda: H.attn_blocksparse_bf16(q, k, v, brp, bci, float(w["scale"]))
     warm = _warmup_calls(fn, args.warmup)
     ms = _time_steps(fn, args.steps, 0)
+    timed = _timed_as()
+    kernel_ms = max(_kernel_times(fn, min(args.steps, 10)))
     flops = 4.0 * nnz * D * Hh
     algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
     achieved = flops / ms / 1e9
+    kernel_achieved = flops / kernel_ms / 1e9
     traffic, provenance = measured_traffic("attention_blocksparse", "fused", True)
     rec = {"metric": "fused block-sparse attention TFLOP/s", "value": round(achieved, 2), "unit": "TFLOP/s",
-           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+           "n_gpus": 1, "steps": timed["steps"], "timed_rounds": timed["rounds"], "warmup": args.warmup,
+           "ms_per_step": round(ms, 5),
            "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
            "config": {"workload": "attention_blocksparse_bf16", "S": S, "H": Hh, "D": D, "block": w["block"],
                       "active_blocks": int(bci.numel()), "nnz_per_head": nnz,
                       "seed": workloads.SEEDS["attention_blocksparse"]},
            "warmup_ms": warm,
-           "roofline": {"bound": "mfma", "kernel": "attn_blocksparse_kernel<64, false, false>", "achieved": round(achieved, 1),
+           "roofline": {"bound": "mfma", "kernel": "attn_blocksparse_kernel<64, false, false>",
+                        "achieved": round(kernel_achieved, 1),
                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
-                        "flops": flops, "algorithmic_bytes": algo, "kernel_ms_avg": round(ms, 5),
-                        "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
+                        "frac": round(kernel_achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
+                        "flops": flops, "algorithmic_bytes": algo, "kernel_ms_avg": round(kernel_ms, 5),
+                        "hbm_gbps_algorithmic": round(algo / kernel_ms / 1e6, 1),
                         **({"traffic_measured_at": provenance} if provenance else {})}}
     # the same attention at the reference's precision: fp32 operands, probabilities and sums, one kernel
     q32, k32, v32 = q.float(), k.float(), v.float()
@@ -731,7 +801,14 @@ def main() -> int:
                     help="also time torch's own sparse routine on the same operands")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replay (SpMM side workloads)")
+    ap.add_argument("--source-hashes", action="store_true",
+                    help="print the current hash of every kernel's source files named in MEASURED_TRAFFIC and exit")
     args = ap.parse_args()
+    if args.source_hashes:
+        for key, rec in MEASURED_TRAFFIC.items():
+            now = source_hash(rec["sources"])
+            print(f"{key}: {now}" + ("" if now == rec["sha16"] else f"  (recorded: {rec['sha16'] or 'none'})"))
+        return 0
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (the kernel shards by rows "
               "of A, every GPU writing its own rows of C, with no reduction). Run with --gpus 1.", file=sys.stderr)

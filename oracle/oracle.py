@@ -59,14 +59,37 @@ def build(force: bool = False) -> None:
 
 
 _lib = None
+_NATIVE_LIB_PATH = os.path.join(_HERE, "liboracle_native.so")
+
+
+def host_has_avx512() -> bool:
+    """The prebuilt binaries here are compiled for x86-64-v4 (oracle/Makefile): on a host without
+    AVX-512 their first vector instruction would kill the process with SIGILL, which no
+    ``try`` can catch -- so the flags are read before anything is loaded."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("flags"):
+                    flags = set(line.split(":", 1)[1].split())
+                    return {"avx512f", "avx512bw", "avx512cd", "avx512dq", "avx512vl"} <= flags
+    except OSError:
+        pass
+    return False
 
 
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
+        path = _LIB_PATH
+        if not host_has_avx512():
+            # this host cannot run the prebuilt library: compile the restatement for it
+            path = _NATIVE_LIB_PATH
+            if not os.path.exists(path):
+                subprocess.run(["make", "-C", _HERE, "-B", "MARCH=native", "LIB=liboracle_native.so",
+                                "liboracle_native.so"], check=True, stdout=subprocess.DEVNULL)
+        elif not os.path.exists(path):
             build()
-        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib = ctypes.CDLL(path)
         _lib.oracle_num_threads.restype = ctypes.c_int
     return _lib
 
@@ -337,7 +360,9 @@ _ref_mod = None
 
 
 def have_ref() -> bool:
-    return os.path.exists(_REF_PATH)
+    """The compiled reference module is there and this host can run it (it is built for
+    x86-64-v4; see host_has_avx512)."""
+    return os.path.exists(_REF_PATH) and host_has_avx512()
 
 
 def ref_module():
