@@ -302,6 +302,10 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_bias_act_f32(int64_t M, int64_t K, int64_
  * (src/scorch/ops.py:638-666, src/scorch/compiler/cin_lowerer.py:2286-2326).
  * out_row_idx, when not NULL, receives the row of every entry (the result's
  * mode_indices[0][0]); its mode_indices[1][0] is col_idx itself.
+ *
+ * mask_vals may be NULL in every SDDMM entry point: every stored entry of the
+ * mask is then taken to be 1 (an attention mask, the mask of this benchmark's
+ * SDDMM configuration) and nothing is read for it.
  * ---------------------------------------------------------------------- */
 SCORCH_HIP_API int scorch_hip_sddmm_coo_f32(int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
                              const int32_t *row_idx, const int32_t *col_idx,

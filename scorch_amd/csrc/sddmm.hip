@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_kernel(
     float scale = 0.0f;
     if (valid) {
       col = col_idx[p];
-      scale = mask_vals[p];
+      scale = mask_vals ? mask_vals[p] : 1.0f;  // (no value array: every stored entry is 1)
       if (COO) {
         row = rows[p];
       } else {
@@ -154,8 +154,9 @@ constexpr int kBuckets = 8;  // one per XCD
 // Workgroups per XCD of the kernel that walks the lists: a grid that is resident as a whole,
 // workgroup id & 7 being the XCD it runs on (checked against the hardware's XCC_ID register: no
 // workgroup of 102,400 was elsewhere, also with 256 per XCD).  65,536^2 mask, 64 per row, K = 64:
-// 128 per XCD 0.165 ms (fewer wavefronts hide less latency), 192 and 256 the same 0.109 ms.
-constexpr int kListedWorkgroupsPerXcd = 192;
+// 64 per XCD 0.222 ms, 128 0.136, 192 0.105, 256 0.098 (fewer wavefronts hide less latency); more
+// than the 256 a XCD holds change nothing.
+constexpr int kListedWorkgroupsPerXcd = 256;
 
 __device__ __forceinline__ int sddmm_entry_row(const int *__restrict__ row_ptr, int row_lo, int row_hi, int64_t p) {
   int lo = row_lo, hi = row_hi;  // answer in [lo, hi]
@@ -340,7 +341,8 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
       cols_of[b] = valid ? entry_col[e] : 0;
     }
 #pragma unroll
-    for (int b = 0; b < kBatches; ++b) scale_of[b] = pos_of[b] >= 0 ? mask_vals[pos_of[b]] : 0.0f;
+    for (int b = 0; b < kBatches; ++b)  // (no value array: every stored entry is 1)
+      scale_of[b] = pos_of[b] >= 0 ? (mask_vals ? mask_vals[pos_of[b]] : 1.0f) : 0.0f;
 #pragma unroll
     for (int b = 0; b < kBatches; ++b) {
       if (first + b * kWaveSize >= last) break;
@@ -455,7 +457,7 @@ int sddmm_entry(const char *fn, int64_t M, int64_t n_cols, int64_t K, int64_t nn
   SCORCH_REQUIRE(COO || rows != nullptr, "%s: row_ptr is NULL", fn);
   if (nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(M > 0 && n_cols > 0, "%s: nnz=%lld in an empty mask", fn, (long long)nnz);
-  SCORCH_REQUIRE(rows && col_idx && mask_vals && out_vals, "%s: NULL index/value array", fn);
+  SCORCH_REQUIRE(rows && col_idx && out_vals, "%s: NULL index/value array", fn);
   SCORCH_REQUIRE(K == 0 || (A && B), "%s: NULL dense operand", fn);
   SCORCH_REQUIRE(aligned_to(rows, 4) && aligned_to(col_idx, 4) && aligned_to(mask_vals, 4) &&
                      aligned_to(out_vals, 4) && aligned_to(A, 4) && aligned_to(B, 4) &&
@@ -578,7 +580,7 @@ int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, in
   if (M >= INT32_MAX || n_cols > INT32_MAX || K > INT32_MAX || nnz > INT32_MAX)
     return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
   if (batch == 0 || nnz == 0) return SCORCH_HIP_OK;
-  SCORCH_REQUIRE(lists && mask_vals && out_vals, "%s: NULL lists or value array", fn);
+  SCORCH_REQUIRE(lists && out_vals, "%s: NULL lists or value array", fn);
   SCORCH_REQUIRE(K == 0 || (A && B), "%s: NULL dense operand", fn);
   SCORCH_REQUIRE(scorch::aligned_to(lists, 256) && scorch::aligned_to(mask_vals, 4) && scorch::aligned_to(out_vals, 4) &&
                      scorch::aligned_to(A, 4) && scorch::aligned_to(B, 4) && scorch::aligned_to(out_row_idx, 4),

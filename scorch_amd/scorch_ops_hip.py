@@ -530,8 +530,13 @@ def _blocked_sddmm(L, bl: BlockedCsr, heads: int, M: int, n_cols: int, K: int, n
     return L.scorch_hip_sddmm_csr_blocked_f32(
         heads, M, n_cols, K, nnz, bl.n_active, bl.block_col_idx.data_ptr(), bl.block_words.data_ptr(),
         bl.block_off.data_ptr(), n_items, items.data_ptr(),
-        None if mask_vals is None or _known_all_ones(mask_vals) else mask_vals.data_ptr(), a.data_ptr(),
-        b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+        _mask_values_pointer(mask_vals), a.data_ptr(), b.data_ptr(), out.data_ptr(), rows_ptr, stream)
+
+
+def _mask_values_pointer(values: Optional[torch.Tensor]):
+    """What an SDDMM kernel is handed for its mask's values: nothing when they are known to be all 1
+    (the kernel then reads nothing for them), else the array."""
+    return None if values is None or _known_all_ones(values) else values.data_ptr()
 
 
 def _known_all_ones(values: torch.Tensor) -> bool:
@@ -998,7 +1003,8 @@ def sddmm_coo_float_prebuilt(result_shape, S_shape, S_mode_indices, S_values, A_
             rc = _blocked_sddmm(L, bl, 1, M, n_cols, K, s_val.numel(), s_val, a, b, out, None, stream)
         else:
             rc = L.scorch_hip_sddmm_coo_f32(M, n_cols, K, s_val.numel(), row.data_ptr(), col.data_ptr(),
-                                            s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(), stream)
+                                            _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                            stream)
     native.check(rc)
     return Tensor(out, S_mode_indices)
 
@@ -1040,11 +1046,11 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
             rc = _blocked_sddmm(L, bl, 1, M, n_cols, K, s_val.numel(), s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
-                                                   s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                   rows_ptr, stream)
+                                                   _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(),
+                                                   out.data_ptr(), rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(), crd.data_ptr(),
-                                            s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                            _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(), out.data_ptr(),
                                             rows_ptr, stream)
     native.check(rc)
     return Tensor(out, [[rows], [crd]])
@@ -1172,8 +1178,7 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     """out[h, p] = S.val[p] * <A[h, i_p, :], B[h, j_p, :]> for every head h and stored entry p of
     the CSR mask S: the SDDMM step of the reference's sparse attention for all heads in one launch
     (bench/bench_sparse_transformer.py:354-361 runs it per head).  A is (H, M, K), B is (H, n_cols, K).
-    S_values may be None: every stored entry of the mask is 1 (a tensor of ones is made only if
-    the kernel that serves the mask reads one).
+    S_values may be None: every stored entry of the mask is 1 (no kernel reads anything for them).
     Returns (values of shape (H, nnz), row coordinates int32[nnz])."""
     M, n_cols = int(S_shape[0]), int(S_shape[1])
     pos, crd = _csr_parts(S_mode_indices, "S")
@@ -1191,19 +1196,17 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
     with _on_device(dev):
         stream = _stream(dev)
         bl = _blocked(plan, pos, crd, M, n_cols, K) if H > 0 else None
-        if bl is None and s_val is None:
-            s_val = torch.ones(nnz, dtype=torch.float32, device=dev)
         lists = _sddmm_lists(plan, pos, crd, M, n_cols, K, L, stream) if bl is None else None
         if bl is not None:
             rc = _blocked_sddmm(L, bl, H, M, n_cols, K, nnz, s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
-                                                   s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                   rows_ptr, stream)
+                                                   _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(),
+                                                   out.data_ptr(), rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),
-                                                    s_val.data_ptr(), a.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                                    rows_ptr, stream)
+                                                    _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(),
+                                                    out.data_ptr(), rows_ptr, stream)
     native.check(rc)
     return out, rows
 

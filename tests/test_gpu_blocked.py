@@ -279,13 +279,13 @@ def test_a_mask_of_ones_is_not_read(oracle):
     pos, crd, a, b = dev(rp), dev(ci), dev(A), dev(B)
     idx = [[], [pos, crd]]
     ones = torch.ones(ci.size, device="cuda")
-    general, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)    # the pattern's first product
-    first, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)      # first sight of the values: read
+    general, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)    # the pattern's first product,
+    assert ones._scorch_ones[1] is None                                     # first sight of the values: read
+    first, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)      # back unchanged: looked at, all 1
     assert isinstance(pos._scorch_plan.blocked, H.BlockedCsr)
     np.testing.assert_allclose(host(general), host(first), rtol=1e-4, atol=1e-4)
-    assert ones._scorch_ones[1] is None
-    second, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)     # back unchanged: looked at, all 1
     assert ones._scorch_ones[1] is True
+    second, _ = H.sddmm_csr_float_batched([M, n_cols], idx, ones, a, b)
     third, _ = H.sddmm_csr_float_batched([M, n_cols], idx, None, a, b)
     assert torch.equal(first, second) and torch.equal(first, third)
     ref_rows = oracle.rows_of(rp)

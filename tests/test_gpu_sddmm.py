@@ -253,3 +253,56 @@ def test_row_coordinates_of_a_planned_mask_are_written_once(oracle):
     rows3 = third.storage.index.mode_indices[0][0]
     assert rows3 is not rows1 and torch.equal(rows3, rows1)
     assert torch.equal(third.storage.value, first.storage.value)
+
+
+@pytest.mark.parametrize("path", ["plain", "listed", "coo"])
+def test_a_mask_without_a_value_array_is_a_mask_of_ones(oracle, monkeypatch, path):
+    """mask_vals = NULL through the C ABI (what the wrappers pass once a mask's values are known to
+    be all 1): bit for bit the result with an array of ones, and the fp64 recomputation."""
+    from scorch_amd import native
+    from scorch_amd import scorch_ops_hip as H
+    w = workloads.sddmm_uniform(M=1500, n_cols=2200, per_row=30, K=48, seed=9, unit_mask=True)
+    M, n_cols, K, nnz = 1500, 2200, 48, int(w["col_idx"].size)
+    rp, ci, rows = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["row_idx"])
+    ones = torch.ones(nnz, device="cuda")
+    A, B = dev(w["A"]).reshape(-1), dev(w["B"]).reshape(-1)
+    L, stream = native.lib(), torch.cuda.current_stream().cuda_stream
+    lists = None
+    if path == "listed":
+        lists = torch.empty(L.scorch_hip_sddmm_csr_lists_bytes(nnz), dtype=torch.uint8, device="cuda")
+        native.check(L.scorch_hip_sddmm_csr_lists(M, n_cols, nnz, rp.data_ptr(), ci.data_ptr(), lists.data_ptr(),
+                                                  lists.numel(), stream))
+
+    def run(values):
+        out = torch.full((nnz,), float("nan"), device="cuda")
+        v = values.data_ptr() if values is not None else None
+        if path == "plain":
+            rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, nnz, rp.data_ptr(), ci.data_ptr(), v, A.data_ptr(),
+                                            B.data_ptr(), out.data_ptr(), None, stream)
+        elif path == "listed":
+            rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(), v,
+                                                   A.data_ptr(), B.data_ptr(), out.data_ptr(), None, stream)
+        else:
+            rc = L.scorch_hip_sddmm_coo_f32(M, n_cols, K, nnz, rows.data_ptr(), ci.data_ptr(), v, A.data_ptr(),
+                                            B.data_ptr(), out.data_ptr(), stream)
+        native.check(rc)
+        return out
+
+    with_ones, without = run(ones), run(None)
+    assert torch.equal(with_ones, without)
+    assert oracle.rel_fro(host(without), oracle.sddmm_fp64(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])) <= 1e-5
+    # through the wrappers: the verdict is reached when the same value tensor comes back unchanged
+    monkeypatch.setattr(H, "SDDMM_PATH", "plain" if path == "coo" else path)
+    if path == "coo":
+        call = lambda: H.sddmm_coo_float_prebuilt([M, n_cols], [M, n_cols], [[rows], [ci]], ones, [M, K], [[], []], A,
+                                                  [n_cols, K], [[], []], B).storage.value
+    else:
+        call = lambda: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [rp, ci]], ones, [M, K], [[], []], A,
+                                         [n_cols, K], [[], []], B).storage.value
+    results = [call() for _ in range(3)]
+    assert ones._scorch_ones[1] is True and all(torch.equal(r, with_ones) for r in results)
+    ones[11] = 3.0                                            # no longer a mask of ones
+    changed = call()
+    expect = with_ones.clone()
+    expect[11] *= 3.0
+    assert torch.equal(changed, expect)
