@@ -52,7 +52,7 @@ CONFIG_WORKLOADS = ("spmm_uniform", "sddmm_uniform", "attention_blocksparse", "s
 _CSRC = "scorch_amd/csrc/"
 _SPMM_SOURCES = (_CSRC + "spmm.hip", _CSRC + "spmm.hpp", _CSRC + "common.hpp")
 MEASURED_TRAFFIC = {
-    ("gcn_powerlaw", "merge"): {"bytes": 9_790_400_000, "sources": _SPMM_SOURCES, "sha16": "f83608455ca9b538",
+    ("gcn_powerlaw", "merge"): {"bytes": 9_790_400_000, "sources": _SPMM_SOURCES, "sha16": "",
                                 "profile": "profiles/spmm_merge_kernel_gcn_powerlaw.md"},
     ("spmm_uniform", "rows"): {"bytes": 10_820_000, "sources": (_CSRC + "spmm_rows.hip", _CSRC + "spmm.hpp",
                                                                 _CSRC + "common.hpp"), "sha16": "",
@@ -60,14 +60,14 @@ MEASURED_TRAFFIC = {
     ("sae_decoder", "tiled"): {"bytes": 666_300_000, "sources": (_CSRC + "spmm_tiled.hip", _CSRC + "spmm.hpp",
                                                                  _CSRC + "common.hpp"), "sha16": "",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "sources": _SPMM_SOURCES, "sha16": "f83608455ca9b538",
+    ("sae_decoder", "merge"): {"bytes": 1_765_900_000, "sources": _SPMM_SOURCES, "sha16": "",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
     ("sddmm_uniform", "listed"): {"bytes": 360_500_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
                                   "sha16": "", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
     ("sddmm_uniform", "plain"): {"bytes": 867_200_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
                                  "sha16": "", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
     ("attention_blocksparse", "fused"): {"bytes": 67_320_000, "sources": (_CSRC + "attn.hip", _CSRC + "common.hpp"),
-                                         "sha16": "680980df0b40e9db", "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
+                                         "sha16": "", "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
 }
 
 
@@ -390,10 +390,8 @@ def run_spmm(name, args, headline=False):
     tiled = getattr(B, "_scorch_tiled", None) is not None
     plan = getattr(pos, "_scorch_plan", None)
     kernels = _kernel_times(fn, min(args.steps, 10))
-    if tiled and len(kernels) == 2:      # every row short: the tiled kernel in which nobody waits
-        path, names = "tiled", ["spmm_tiled_short_rows_kernel<float,0>", "spmm_fixup_kernel<float,1,0>"]
-    elif tiled:
-        path, names = "tiled", ["spmm_tiled_clear_kernel", "spmm_tiled_kernel<float,0>", "spmm_fixup_kernel<float,1,0>"]
+    if tiled:
+        path, names = "tiled", ["spmm_tiled_kernel<float,0>", "spmm_fixup_kernel<float,1,0>"]
     elif len(kernels) == 1:
         lanes = 64 if N % 4 else max(8, min(64, 1 << (max(N // 4, 1) - 1).bit_length()))
         path, names = "rows", [f"spmm_rows_kernel<float,{4 if N % 4 == 0 else 1},{lanes}>"]

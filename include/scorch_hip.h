@@ -68,12 +68,6 @@ enum scorch_hip_act { SCORCH_HIP_ACT_NONE = 0, SCORCH_HIP_ACT_RELU = 1 };
  * (csrc/spmm.h:2024-2025, 2052: memset, then empty rows skipped), instead of a row-sized store of
  * zeros per empty row between the gathers.  Same result; ignored with a bias. */
 #define SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS 0x100
-/* May be or-ed into the `act` argument of scorch_hip_spmm_csr_tiled_f32: the caller knows
- * (scorch_hip_csr_inspect reports the longest row) that no row of A has more than 64 entries.
- * The product then takes a kernel in which every row is one lane group's and no workgroup waits
- * for another; same result bit for bit.  With a longer row the result is still right, the call
- * slower. */
-#define SCORCH_HIP_HINT_SHORT_ROWS 0x200
 
 /* ABI version of the loaded library (SCORCH_HIP_ABI_VERSION at build time). */
 SCORCH_HIP_API int scorch_hip_abi_version(void);

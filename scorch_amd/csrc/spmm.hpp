@@ -139,19 +139,16 @@ inline int64_t spmm_num_chunks(int64_t M, int64_t nnz, int64_t N, size_t elem) {
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Workspace layout: carry_row int32[num_chunks] padded to 256 bytes, then
-// carry_val T[num_chunks * N] padded likewise, then kPaceBytes of counters
-// that only the kernel for column-tiled operands uses (spmm_tiled.hip).
-constexpr int kPaceStride = 32;  // ints between two XCDs' pace counters (a cache line each)
-constexpr size_t kPaceBytes = 8 * kPaceStride * sizeof(int);
+// carry_val T[num_chunks * N] padded likewise.
 inline size_t spmm_workspace_bytes(int64_t M, int64_t nnz, int64_t N, size_t elem) {
   const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
-  return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256) + kPaceBytes;
+  return align_up(chunks * sizeof(int), 256) + align_up(chunks * (size_t)N * elem, 256);
 }
 
 // A batch of products over one pattern: one carry_row array, then carry_val for every problem.
 inline size_t spmm_batched_workspace_bytes(int64_t batch, int64_t M, int64_t nnz, int64_t N, size_t elem) {
   const size_t chunks = (size_t)spmm_num_chunks(M, nnz, N, elem);
-  return align_up(chunks * sizeof(int), 256) + align_up((size_t)batch * chunks * (size_t)N * elem, 256) + kPaceBytes;
+  return align_up(chunks * sizeof(int), 256) + align_up((size_t)batch * chunks * (size_t)N * elem, 256);
 }
 
 // Elements per lane.  Preferred: the widest vector (at most 16 bytes) that

@@ -36,8 +36,6 @@ _empty = torch.empty
 _empty_like = torch.empty_like
 
 HINT_MOSTLY_EMPTY_ROWS = 0x100      # SCORCH_HIP_HINT_MOSTLY_EMPTY_ROWS of include/scorch_hip.h
-HINT_SHORT_ROWS = 0x200             # SCORCH_HIP_HINT_SHORT_ROWS
-TILED_SHORT_ROW = 64                # longest row for which the tiled kernel for short rows is asked for
 INSPECT_REPORT_INTS = 8             # SCORCH_HIP_INSPECT_REPORT_INTS
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32", torch.int64: "i64"}
 
@@ -698,10 +696,8 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
             if plan is not None and path != "merge_unplanned" else None
         bounds_ptr, bounds_bytes = (bounds.data_ptr(), bounds.numel()) if bounds is not None else (None, 0)
         if tiled is not None:
-            hint = HINT_SHORT_ROWS if plan is not None and plan.max_row <= TILED_SHORT_ROW else 0
             rc = L.scorch_hip_spmm_csr_tiled_f32(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(),
-                                                 tiled.data_ptr(), tiled.numel() * 4, bias_ptr, act | hint,
-                                                 out.data_ptr(),
+                                                 tiled.data_ptr(), tiled.numel() * 4, bias_ptr, act, out.data_ptr(),
                                                  bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
         else:
             hint = HINT_MOSTLY_EMPTY_ROWS if fill_first else 0

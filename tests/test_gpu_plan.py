@@ -306,12 +306,12 @@ def test_tiled_kernel_when_the_even_resplit_makes_chunks_longer_than_the_usual_o
     assert np.array_equal(got, hip_spmm(rp, ci, v, B, path="tiled"))
 
 
-@pytest.mark.parametrize("longest", [1, 7, 33, 64])
+@pytest.mark.parametrize("longest", [1, 7, 33, 64, 200])
 @pytest.mark.parametrize("relu", [None, False, True])
-def test_tiled_kernel_for_short_rows_equals_the_general_one(oracle, monkeypatch, longest, relu):
-    """Operands whose longest row has at most 64 entries take a tiled kernel of their own (every row
-    one lane group's, no workgroup waits for another): bit for bit the general tiled kernel's result,
-    with empty rows, rows cut by chunk boundaries, an epilogue, and N not a multiple of the tile width."""
+def test_tiled_kernel_over_row_lengths_and_epilogues(oracle, longest, relu):
+    """The tiled kernel against fp64 and, bit for bit where no row is shared by all lane groups
+    (at most 64 entries), against the merge path: empty rows, rows cut by chunk boundaries, an
+    epilogue, N not a multiple of the tile width."""
     rng = np.random.default_rng(100 * longest + (0 if relu is None else 1 + relu))
     M, K = 3000, 1500
     lens = rng.integers(0, longest + 1, M)
@@ -325,31 +325,6 @@ def test_tiled_kernel_for_short_rows_equals_the_general_one(oracle, monkeypatch,
         want = oracle.spmm_fp64(rp, ci, v, B)
         if bias is not None:
             want = np.maximum(want + bias, 0) if relu else want + bias
-        monkeypatch.setattr(H, "TILED_SHORT_ROW", 64)
         got = hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled")
         assert oracle.rel_fro(got, want) <= TOL
-        monkeypatch.setattr(H, "TILED_SHORT_ROW", -1)                     # the hint withheld: the general kernel
-        general = hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled")
-        assert np.array_equal(got, general)
-
-
-def test_tiled_kernel_for_short_rows_when_a_row_is_longer_than_promised(oracle):
-    """The hint is a promise about speed, not about correctness: with it, rows of a few hundred
-    entries still come out right."""
-    rng = np.random.default_rng(77)
-    M, K, N = 600, 900, 1000
-    lens = rng.integers(0, 40, M); lens[[0, 300, 599]] = [700, 333, 420]
-    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-    ci = rng.integers(0, K, int(rp[-1])).astype(np.int32)
-    v = rng.uniform(-1, 1, ci.size).astype(np.float32)
-    B = rng.standard_normal((K, N)).astype(np.float32)
-    L = native.lib()
-    pos, crd, val, Bd = dev(rp), dev(ci), dev(v), dev(B).reshape(-1)
-    bt = H.prepare_dense_operand(Bd, K, N)
-    out = torch.full((M * N,), float("nan"), device="cuda")
-    ws = torch.empty(L.scorch_hip_spmm_csr_workspace_bytes(M, ci.size, N, 4), dtype=torch.uint8, device="cuda")
-    native.check(L.scorch_hip_spmm_csr_tiled_f32(M, K, N, ci.size, pos.data_ptr(), crd.data_ptr(), val.data_ptr(),
-                                                 bt.data_ptr(), bt.numel() * 4, None, H.HINT_SHORT_ROWS, out.data_ptr(),
-                                                 None, 0, ws.data_ptr(), ws.numel(),
-                                                 torch.cuda.current_stream().cuda_stream))
-    assert oracle.rel_fro(host(out).reshape(M, N), oracle.spmm_fp64(rp, ci, v, B)) <= TOL
+        assert np.array_equal(got, hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled"))
