@@ -35,6 +35,13 @@ LaunchMarks *launch_marks() {
 // read twice: a running maximum and sum first, the write second; the next
 // row's entries are requested before the current row's phases start): however such rows are placed in the matrix, few among
 // many short ones or all of them long, they are spread over the whole chip.
+// A row of more than kSoftmaxSplitRow entries is not one workgroup's either (the reference's
+// softmax is torch scatter operations over entries, bench/bench_sparse_transformer.py:277-297:
+// a single row of millions costs it what any other four million entries cost): the giant-row
+// kernel only enters it in a second list, cut into up to 1024 stretches, and two more kernels
+// serve the stretches -- softmax_split_partial_kernel a stretch's maximum and its sum of
+// exponentials relative to that, softmax_split_finish_kernel the row's maximum and sum from its
+// stretches' (in stretch order: the same bits on every run) and the stretch's results.
 // Values are loaded raw and scaled at their first use, so that a row's loads
 // are all issued before any of them is waited for.
 constexpr int kSoftmaxRegs = 4;
@@ -49,6 +56,10 @@ constexpr int kSoftmaxWaveRowMax = kSoftmaxRegs * kWaveSize;
 constexpr int kSoftmaxLongWaveRowMax = kSoftmaxBlockRegs * kWaveSize;
 constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
 constexpr int kSoftmaxGiantThreads = 1024;
+constexpr int kSoftmaxSplitRow = 65536;     // rows longer than this are shared out in stretches
+constexpr int kSoftmaxStretch = 16384;      // entries of a stretch, at least
+constexpr int kSoftmaxMaxStretches = 1024;  // stretches of a row, at most (one per thread of the combining workgroup)
+constexpr int kSoftmaxSplitBlocks = 2048;   // most workgroups the two stretch kernels start
 constexpr int kSoftmaxGiantBlocks = 1024;  // most workgroups the giant-row kernel starts
 constexpr float kSoftmaxLowest = -3.402823466e38f;
 
@@ -273,15 +284,121 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   }
 }
 
-__global__ void softmax_reset_kernel(int *giant_count) {
-  if (threadIdx.x == 0) *giant_count = 0;
+// counters[0]: giant rows listed; [1]: rows served in stretches; [2]: their stretches in all
+__global__ void softmax_reset_kernel(int *counters) {
+  if (threadIdx.x < 3) counters[threadIdx.x] = 0;
+}
+
+// The rows that are served in stretches, in the caller's workspace: rows[j] = (row, its first
+// stretch's number, its stretches, entries per stretch), units[u] = (j, number of the stretch within
+// its row), partials[u] = (the stretch's maximum, its sum of exponentials relative to that).
+struct SoftmaxSplit {
+  int *counters;
+  int4 *rows;
+  int2 *units;
+  float2 *partials;
+};
+
+// (maximum, sum of exponentials relative to it) of the entries of a stretch, for every stretch.
+__global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_split_partial_kernel(
+    const int *__restrict__ row_ptr, const float *__restrict__ vals, float scale, SoftmaxSplit split) {
+  constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
+  __shared__ float s_red[kWaves];
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  auto reduce = [&](float v, bool take_max) {
+    v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
+    __syncthreads();
+    if (lane == 0) s_red[w] = v;
+    __syncthreads();
+    float r = s_red[0];
+#pragma unroll
+    for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
+    return r;
+  };
+  const int n_units = split.counters[2];
+  for (int u = blockIdx.x; u < n_units; u += gridDim.x) {  // uniform over the workgroup
+    const int2 unit = split.units[u];
+    const int4 row = split.rows[unit.x];
+    const int begin = row_ptr[row.x] + unit.y * row.w;
+    const int row_end = row_ptr[row.x + 1];
+    const int end = row_end - begin > row.w ? begin + row.w : row_end;  // (no overflow near 2^31 entries)
+    constexpr int kBatch = 8;
+    float mx = kSoftmaxLowest, sum = 0.0f;
+    for (int p0 = begin + (int)threadIdx.x; p0 < end; p0 += kBatch * kSoftmaxGiantThreads) {
+      float raw[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const int p = p0 + k * kSoftmaxGiantThreads;
+        raw[k] = p < end ? vals[p] : 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        if (p0 + k * kSoftmaxGiantThreads >= end) break;
+        const float x = raw[k] * scale;
+        const float e = expf(-fabsf(x - mx));
+        const bool higher = x > mx;
+        sum = higher ? sum * e + 1.0f : sum + e;
+        mx = higher ? x : mx;
+      }
+    }
+    const float unit_max = reduce(mx, true);
+    const float unit_sum = reduce(sum * expf(mx - unit_max), false);  // (a thread without entries: 0 * exp(lowest - max) = 0)
+    if (threadIdx.x == 0) split.partials[u] = make_float2(unit_max, unit_sum);
+  }
+}
+
+// The row's maximum and sum from its stretches', then the stretch's results.
+__global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_split_finish_kernel(
+    const int *__restrict__ row_ptr, const float *vals, float scale, float *out, SoftmaxSplit split) {
+  constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
+  __shared__ float s_red[kWaves];
+  const int lane = wave_lane();
+  const int w = threadIdx.x / kWaveSize;
+  auto reduce = [&](float v, bool take_max) {
+    v = softmax_shuffle_reduce<kWaveSize>(v, take_max);
+    __syncthreads();
+    if (lane == 0) s_red[w] = v;
+    __syncthreads();
+    float r = s_red[0];
+#pragma unroll
+    for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
+    return r;
+  };
+  const int n_units = split.counters[2];
+  for (int u = blockIdx.x; u < n_units; u += gridDim.x) {  // uniform over the workgroup
+    const int2 unit = split.units[u];
+    const int4 row = split.rows[unit.x];
+    float2 part = make_float2(kSoftmaxLowest, 0.0f);  // thread t: stretch t of the row
+    if ((int)threadIdx.x < row.z) part = split.partials[row.y + threadIdx.x];
+    const float row_max = reduce(part.x, true);
+    const float row_sum = reduce(part.y * expf(part.x - row_max), false);
+    const int begin = row_ptr[row.x] + unit.y * row.w;
+    const int row_end = row_ptr[row.x + 1];
+    const int end = row_end - begin > row.w ? begin + row.w : row_end;  // (no overflow near 2^31 entries)
+    constexpr int kBatch = 8;  // (loads issued together: out may alias vals, see softmax_finish)
+    for (int p0 = begin + (int)threadIdx.x; p0 < end; p0 += kBatch * kSoftmaxGiantThreads) {
+      float raw[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const int p = p0 + k * kSoftmaxGiantThreads;
+        raw[k] = p < end ? vals[p] : 0.0f;
+      }
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const int p = p0 + k * kSoftmaxGiantThreads;
+        if (p < end) out[p] = expf(raw[k] * scale - row_max) / row_sum;
+      }
+    }
+  }
 }
 
 __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel(
     const int *__restrict__ row_ptr, const float *vals, float scale, float *out,
-    const int *__restrict__ giant_count, const int *__restrict__ giant_rows, int64_t nnz) {
+    const int *__restrict__ giant_count, const int *__restrict__ giant_rows, int64_t nnz, SoftmaxSplit split) {
   constexpr int kWaves = kSoftmaxGiantThreads / kWaveSize;
   __shared__ float s_red[kWaves];
+  __shared__ int s_claim[2];
   vals += blockIdx.y * nnz;  // problem blockIdx.y of a batch over one pattern
   out += blockIdx.y * nnz;
   const int n = *giant_count;
@@ -298,6 +415,27 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
     for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
     return r;
   };
+  // A row of more than kSoftmaxSplitRow entries is entered in the list of rows that are served in
+  // stretches (by problem 0 of a batch: the pattern is the same for all) and skipped here.
+  // Uniform over the workgroup.
+  auto leave_to_the_stretch_kernels = [&](int row, int lo, int &hi) {
+    const int len = hi - lo;
+    if (len <= kSoftmaxSplitRow || split.rows == nullptr) return;
+    hi = lo;
+    if (blockIdx.y != 0) return;
+    int stretch = (len + kSoftmaxMaxStretches - 1) / kSoftmaxMaxStretches;
+    stretch = stretch < kSoftmaxStretch ? kSoftmaxStretch : (stretch + 1023) / 1024 * 1024;
+    const int n_units = (len + stretch - 1) / stretch;
+    __syncthreads();  // (s_claim may still be read from the row before)
+    if (threadIdx.x == 0) {
+      s_claim[0] = atomicAdd(split.counters + 1, 1);
+      s_claim[1] = atomicAdd(split.counters + 2, n_units);
+    }
+    __syncthreads();
+    const int j = s_claim[0], first = s_claim[1];
+    if (threadIdx.x == 0) split.rows[j] = make_int4(row, first, n_units, stretch);
+    if ((int)threadIdx.x < n_units) split.units[first + threadIdx.x] = make_int2(j, (int)threadIdx.x);
+  };
   // The next row's first entries are requested before this row's phases begin,
   // so that its memory latency passes behind their barriers.  (out may alias
   // vals: rows do not overlap, so the early read sees the row unchanged.)
@@ -305,6 +443,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
   if (i >= n) return;
   int row = giant_rows[i];
   int lo = row_ptr[row], hi = row_ptr[row + 1];
+  leave_to_the_stretch_kernels(row, lo, hi);
   float v[kSoftmaxGiantRegs];
   softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo, hi, t, vals, v);
   for (;;) {  // uniform over the workgroup
@@ -315,6 +454,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
       const int row_next = giant_rows[i_next];
       lo_next = row_ptr[row_next];
       hi_next = row_ptr[row_next + 1];
+      leave_to_the_stretch_kernels(row_next, lo_next, hi_next);
     }
     softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo_next, hi_next, t, vals, v_next);
     softmax_finish<kSoftmaxGiantThreads, kSoftmaxGiantRegs, true>(lo, hi, t, vals, scale, out, v, reduce);
@@ -334,9 +474,40 @@ inline int64_t softmax_giant_capacity(int64_t M, int64_t nnz) {
   return by_entries < M ? by_entries : M;
 }
 
+// Rows that may have to be served in stretches, and stretches in all.
+inline int64_t softmax_split_rows(int64_t M, int64_t nnz) {
+  const int64_t by_entries = nnz / (kSoftmaxSplitRow + 1);
+  return by_entries < M ? by_entries : M;
+}
+inline int64_t softmax_split_units(int64_t M, int64_t nnz) {
+  const int64_t rows = softmax_split_rows(M, nnz);
+  return rows > 0 ? nnz / kSoftmaxStretch + rows : 0;
+}
+inline size_t softmax_round_256(size_t v) { return (v + 255) / 256 * 256; }
+
+// Workspace: three counters (256 bytes), the giant rows' numbers, then -- only when a row can be
+// long enough -- the rows served in stretches, the stretches and their partial results.
 inline size_t softmax_workspace_bytes(int64_t M, int64_t nnz) {
   const int64_t rows = softmax_giant_capacity(M, nnz);
-  return rows > 0 ? 256 + ((size_t)rows * sizeof(int) + 255) / 256 * 256 : 0;
+  if (rows <= 0) return 0;
+  const size_t split_rows = (size_t)softmax_split_rows(M, nnz), units = (size_t)softmax_split_units(M, nnz);
+  return 256 + softmax_round_256((size_t)rows * sizeof(int)) + softmax_round_256(split_rows * sizeof(int4)) +
+         softmax_round_256(units * sizeof(int2)) + softmax_round_256(units * sizeof(float2));
+}
+
+inline SoftmaxSplit softmax_split_layout(void *workspace, int64_t M, int64_t nnz) {
+  SoftmaxSplit split{nullptr, nullptr, nullptr, nullptr};
+  const size_t split_rows = (size_t)softmax_split_rows(M, nnz), units = (size_t)softmax_split_units(M, nnz);
+  if (split_rows == 0) return split;
+  char *base = static_cast<char *>(workspace);
+  size_t at = 256 + softmax_round_256((size_t)softmax_giant_capacity(M, nnz) * sizeof(int));
+  split.counters = reinterpret_cast<int *>(base);
+  split.rows = reinterpret_cast<int4 *>(base + at);
+  at += softmax_round_256(split_rows * sizeof(int4));
+  split.units = reinterpret_cast<int2 *>(base + at);
+  at += softmax_round_256(units * sizeof(int2));
+  split.partials = reinterpret_cast<float2 *>(base + at);
+  return split;
 }
 
 // ---- CSR -> coordinate rows ---------------------------------------------------
@@ -472,9 +643,23 @@ static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t n
     if (most > scorch::kSoftmaxGiantBlocks) most = scorch::kSoftmaxGiantBlocks;
     if (batch > 1 && most > 128) most = 128;  // every problem brings its own workgroups
     const dim3 giant_grid((unsigned)most, (unsigned)batch);
+    const scorch::SoftmaxSplit split = scorch::softmax_split_layout(workspace, M, nnz);
     scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(
-        row_ptr, vals, scale, out, giant_count, giant_rows, nnz);
+        row_ptr, vals, scale, out, giant_count, giant_rows, nnz, split);
     SCORCH_HIP_CHECK(hipGetLastError());
+    if (split.rows != nullptr) {  // a row can be long enough to be served in stretches
+      int64_t blocks = scorch::softmax_split_units(M, nnz);
+      if (blocks > scorch::kSoftmaxSplitBlocks) blocks = scorch::kSoftmaxSplitBlocks;
+      // the stretches' partial results are one problem's: the problems of a batch take their turns
+      for (int64_t h = 0; h < batch; ++h) {
+        scorch::softmax_split_partial_kernel<<<dim3((unsigned)blocks), scorch::kSoftmaxGiantThreads, 0, s>>>(
+            row_ptr, vals + h * nnz, scale, split);
+        SCORCH_HIP_CHECK(hipGetLastError());
+        scorch::softmax_split_finish_kernel<<<dim3((unsigned)blocks), scorch::kSoftmaxGiantThreads, 0, s>>>(
+            row_ptr, vals + h * nnz, scale, out + h * nnz, split);
+        SCORCH_HIP_CHECK(hipGetLastError());
+      }
+    }
   }
   return SCORCH_HIP_OK;
 }

@@ -129,7 +129,10 @@ def test_spmv_softmax_rows_reject_bad_arguments(L):
     # rows longer than 4096 entries are possible from nnz = 4097 on: a workspace is needed then
     assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4096) == 0
     assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4097) == 512
-    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 17_000_000) == 256 + 16640
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 60_000) == 256 + 256
+    # from 65,537 entries on a row can be long enough to be served in stretches: three more arrays
+    # (259 such rows at most here, 1,037 + 259 stretches)
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 17_000_000) == 256 + 16640 + 4352 + 2 * 10496
     assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, NULL, 0, NULL) == native.EWORKSPACE
     assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, FAKE, 256, NULL) == native.EWORKSPACE
     assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL

@@ -134,6 +134,39 @@ def test_softmax_in_place(oracle):
     assert oracle.rel_fro(host(v), oracle.softmax_csr_fp64(rp, vals, 0.5)) <= TOL
 
 
+@pytest.mark.parametrize("lens", [[4_200_000], [3, 70_000, 0, 1_500_000, 12, 65_536, 65_537, 5000, 200_000]])
+def test_softmax_rows_shared_out_among_workgroups(oracle, lens):
+    """Rows of more than 65,536 entries are served in stretches by many workgroups (a single row of
+    millions would otherwise be one workgroup's): against the fp64 recomputation, the same bits on
+    every run, in place, and for a batch of value arrays over the pattern."""
+    lens = np.array(lens, np.int64)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(int(lens.sum()) % 1000)
+    vals = (rng.standard_normal(int(rp[-1])) * 4).astype(np.float32)
+    vals[int(rp[-1]) // 2] = 40.0                          # one entry that towers over its row
+    pos, v = dev(rp), dev(vals)
+    out = H.softmax_csr_float(pos, v, 0.5)
+    want = oracle.softmax_csr_fp64(rp, vals, 0.5)
+    assert oracle.rel_fro(host(out), want) <= TOL
+    np.testing.assert_allclose(host(out), want, rtol=5e-5, atol=1e-30)
+    assert torch.equal(out, H.softmax_csr_float(pos, v, 0.5))
+    sums = np.add.reduceat(host(out).astype(np.float64), rp[:-1][lens > 0])
+    np.testing.assert_allclose(sums, 1.0, rtol=1e-5)
+    # a batch: every problem's rows, also the ones served in stretches
+    batch = torch.stack([v, v * 0.5 + 1.0, -v])
+    got = H.softmax_csr_float_batched(pos, batch, 0.5)
+    for h in range(3):
+        assert torch.equal(got[h], H.softmax_csr_float(pos, batch[h].contiguous(), 0.5))
+    # in place through the C ABI
+    L = H.native.lib()
+    need = L.scorch_hip_softmax_csr_workspace_bytes(len(lens), v.numel())
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    inplace = v.clone()
+    rc = L.scorch_hip_softmax_csr_f32(len(lens), v.numel(), pos.data_ptr(), inplace.data_ptr(), 0.5, inplace.data_ptr(),
+                                      ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(inplace, out)
+
+
 def test_softmax_with_empty_rows_and_large_values(oracle):
     rp = np.array([0, 0, 4, 4, 5], np.int32)
     vals = np.array([1000.0, 1001.0, 999.0, 1000.5, -3.0], np.float32)
