@@ -466,12 +466,16 @@ SCORCH_HIP_API int scorch_hip_attn_blocksparse_masked_bf16(
  * stretches, 0.  Partial results (unnormalised sums, reference maximum, row sum per query) go
  * through `workspace` (256-byte aligned, scorch_hip_attn_blocksparse_split_workspace_bytes(H,
  * n_slots, D) bytes; not to be shared by calls that may overlap in time) and a second kernel
- * combines them.  block_mask_index may be NULL (every block fully live).  No counterpart in the
+ * combines them.  block_mask_index may be NULL (every block fully live).  With pair_items != 0 a
+ * workgroup takes two items, the k-th longest and then the k-th shortest of the list, so that all
+ * workgroups carry about the same work and half as many start: it pays where the items differ in
+ * length (or are very short) and the launch is about one to four times what the chip holds at
+ * once, and costs a few per cent elsewhere; same results bit for bit.  No counterpart in the
  * reference, like the two entry points above. */
 SCORCH_HIP_API size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, int64_t n_slots, int64_t D);
 SCORCH_HIP_API int scorch_hip_attn_blocksparse_split_bf16(
     int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
-    const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
+    const int32_t *items, int pair_items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
     const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
     const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
     void *workspace, size_t workspace_bytes, void *stream);

@@ -105,7 +105,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     const unsigned long long *__restrict__ block_masks, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O, int n_items, const int4 *__restrict__ items, int n_slots,
-    float *__restrict__ partials) {
+    float *__restrict__ partials, int pairs) {
   using Tile = AttnTile<D>;
   constexpr int kTileBytes = Tile::kBytes;
   constexpr int kRowBytes = Tile::kRowBytes;
@@ -133,27 +133,33 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     // (2 * S * 128 bytes) are fetched into one L2 only and an XCD works through its
     // heads one after the other.
     const int id = blockIdx.x;
+    const int n_ranks = pairs ? (n_items + 1) >> 1 : n_items;
     if (n_heads % 8 == 0) {
       const int xcd = id & 7, slot = id >> 3;
-      head = xcd + 8 * (slot / n_items);
-      rank = slot % n_items;
+      head = xcd + 8 * (slot / n_ranks);
+      rank = slot % n_ranks;
     } else {
-      head = id / n_items;
-      rank = id % n_items;
+      head = id / n_ranks;
+      rank = id % n_ranks;
     }
   }
+  // pairs: a workgroup takes two items, the rank-th longest and the rank-th shortest, one after
+  // the other, so that all workgroups carry about the same work and fit the chip in one round
+  for (int pass = 0; pass < (pairs ? 2 : 1); ++pass) {
+  const int item_rank = pass == 0 ? rank : n_items - 1 - rank;
+  if (pass == 1 && item_rank <= rank) break;
   // A workgroup's work item is a block row, or -- when `items` is given -- a stretch of a block
   // row's key blocks (x: block row, y and z: the stretch within block_col_idx, w: where its
   // partial result goes, or -1 for a whole row that writes O itself).  Items come longest first.
   int qb, kb_begin, kb_end, part_slot = -1;
   if (items) {
-    const int4 item = items[rank];
+    const int4 item = items[item_rank];
     qb = uniform(item.x);
     kb_begin = uniform(item.y);
     kb_end = uniform(item.z);
     part_slot = uniform(item.w);
   } else {
-    qb = n_blocks - 1 - rank;  // (masks with longer block rows further down: longest first)
+    qb = n_blocks - 1 - item_rank;  // (masks with longer block rows further down: longest first)
     kb_begin = block_row_ptr[qb];
     kb_end = block_row_ptr[qb + 1];
   }
@@ -354,7 +360,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
       part[D] = m_run;
       part[D + 1] = l;
     }
-    return;
+    continue;
   }
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // queries without a live key give zeros
   __bf16 *out = O + head_off + (size_t)query * D;
@@ -365,6 +371,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     for (int r = 0; r < 4; ++r) o[r] = (__bf16)(o_acc[dt][r] * inv);
     *reinterpret_cast<bf16x4 *>(out + 16 * dt + 4 * g) = o;
   }
+  }  // pass
 }
 
 // Combines the stretches of a block row that was shared out: with m* the largest of the
@@ -418,11 +425,11 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
                             const int32_t *block_row_ptr, const int32_t *block_col_idx,
                             const int32_t *block_mask_index, const unsigned long long *block_masks,
                             const __bf16 *q, const __bf16 *k, const __bf16 *v, float scale_log2e,
-                            __bf16 *o, int n_items, const int4 *items, int n_slots, float *partials) {
+                            __bf16 *o, int n_items, const int4 *items, int n_slots, float *partials, int pairs) {
 #define SCORCH_ATTN_LAUNCH(NEG, MASKED)                                                          \
   attn_blocksparse_kernel<D, NEG, MASKED><<<grid, kBlockThreads, 0, s>>>(                        \
       S, n_blocks, H, block_row_ptr, block_col_idx, block_mask_index, block_masks, q, k, v,      \
-      scale_log2e, o, n_items, items, n_slots, partials)
+      scale_log2e, o, n_items, items, n_slots, partials, pairs)
   const bool masked = block_mask_index != nullptr;
   if (negative) {
     if (masked) SCORCH_ATTN_LAUNCH(true, true); else SCORCH_ATTN_LAUNCH(true, false);
@@ -435,6 +442,7 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
 // Block rows shared out among several workgroups (scorch_hip_attn_blocksparse_split_bf16).
 struct AttnSplit {
   int64_t n_items = 0, n_split_rows = 0, n_slots = 0;
+  bool pair_items = false;              // a workgroup takes the k-th longest and then the k-th shortest item
   const int32_t *items = nullptr;       // 4 per item: block row, begin, end, slot (-1: writes O itself)
   const int32_t *split_rows = nullptr;  // 4 per split row: block row, first slot, stretches, 0
   void *workspace = nullptr;
@@ -491,7 +499,9 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
     items = reinterpret_cast<const int4 *>(split->items);
     partials = static_cast<float *>(split->workspace);
   }
-  const dim3 grid((unsigned)(n_items * H));
+  // pairs: every workgroup takes two items, see the kernel (asked for through the work-list entry)
+  const int pairs = split && split->pair_items && n_items >= 2;
+  const dim3 grid((unsigned)((pairs ? (n_items + 1) / 2 : n_items) * H));
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const __bf16 *q = static_cast<const __bf16 *>(Q), *k = static_cast<const __bf16 *>(K),
@@ -501,13 +511,13 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
   mark_launch(s);
   if (D == 32)
     attn_launch_dim<32>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
   else if (D == 64)
     attn_launch_dim<64>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
   else
     attn_launch_dim<128>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                         block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials);
+                         block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
   if (split && split->n_split_rows > 0) {
@@ -560,7 +570,7 @@ extern "C" size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, i
 
 extern "C" int scorch_hip_attn_blocksparse_split_bf16(
     int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
-    const int32_t *items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
+    const int32_t *items, int pair_items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
     const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
     const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
     void *workspace, size_t workspace_bytes, void *stream) {
@@ -573,6 +583,7 @@ extern "C" int scorch_hip_attn_blocksparse_split_bf16(
   }
   AttnSplit split;
   split.n_items = n_items;
+  split.pair_items = pair_items != 0;
   split.n_split_rows = n_split_rows;
   split.n_slots = n_slots;
   split.items = items;

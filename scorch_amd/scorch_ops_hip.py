@@ -163,7 +163,7 @@ class _on_device:
 # pointer, a numpy or DLPack alias, a kernel of another library, or the replay of a recorded graph:
 # after such a write call forget(t), or mark the tensor volatile once.
 _CACHE_ATTRIBUTES = ("_scorch_plan", "_scorch_tiled", "_scorch_seen", "_scorch_ones", "_scorch_coo_pos",
-                     "_scorch_block_mask", "_scorch_mask_checked")
+                     "_scorch_block_mask", "_scorch_mask_checked", "_scorch_rows")
 
 
 def _tensors_of(obj, seen=None):
@@ -1294,7 +1294,7 @@ class BlockMask:
     of its 64-word bit mask (bit j of word r: query r of the block row attends to key j of the
     block).  Blocks with equal masks share one."""
     __slots__ = ("S", "block", "block_row_ptr", "block_col_idx", "block_mask_index", "block_masks", "nnz",
-                 "items", "split_rows", "n_slots", "schedule32", "block_row_lens")
+                 "items", "split_rows", "n_slots", "schedule32", "block_row_lens", "pairing")
 
     def __init__(self, S, block, block_row_ptr, block_col_idx, block_mask_index, block_masks, nnz):
         self.S, self.block, self.nnz = S, block, nnz
@@ -1305,6 +1305,7 @@ class BlockMask:
         self.n_slots = 0
         self.schedule32 = None      # the fp32 kernel's own sharing-out (see _fp32_schedule)
         self.block_row_lens = None  # active blocks per block row, on the host (numpy), once it has been read
+        self.pairing = {}           # (item list, heads, head dimension) -> whether workgroups take two items
 
     def row_lens(self):
         """Active blocks per block row as a numpy array on the host (read from the device once)."""
@@ -1363,6 +1364,40 @@ def block_mask_from_csr(row_ptr: torch.Tensor, col_idx: torch.Tensor, S: int) ->
                    masks.contiguous().view(-1), int(stored.sum()))
     bm.block_row_lens = brp[1:] - brp[:-1]
     return bm
+
+
+# workgroups of the fused bf16 attention kernel a CU holds at once, by head dimension
+ATTENTION_WORKGROUPS_PER_CU = {32: 6, 64: 4, 128: 2}
+
+
+_cu_counts: Dict[int, int] = {}
+
+
+def _cu_count(device) -> int:
+    index = torch.device(device).index or 0
+    if index not in _cu_counts:
+        _cu_counts[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _cu_counts[index]
+
+
+def pair_attention_items(lens, heads: int, D: int, n_cus: int = 256) -> bool:
+    """Whether the fused bf16 attention kernel should give every workgroup two work items, the
+    k-th longest and then the k-th shortest (scorch_hip_attn_blocksparse_split_bf16, pair_items).
+    `lens`: key blocks per item.  Pairing evens the workgroups out and halves their number; it
+    pays where the items differ in length, or are so short that a workgroup's start and end
+    weigh, and the launch is between about 0.6 and 4 times what the chip holds at once, and costs
+    elsewhere (S = 8192, 16 heads, D = 64, measured: the benchmark's causal strided mask -7 %,
+    four blocks in every row -9 %, twelve +1 %; a causal mask at S = 4096 -15 % with 16 heads,
+    +7 % with 4, -3 % with 128; at S = 16384 with D = 128 +3 %)."""
+    import numpy as np
+    lens = np.asarray(lens)
+    if lens.size < 2 or D not in ATTENTION_WORKGROUPS_PER_CU:
+        return False
+    slots = n_cus * ATTENTION_WORKGROUPS_PER_CU[D]
+    rounds = lens.size * heads / slots
+    mean = float(lens.mean())
+    uneven = float(lens.max()) > 1.25 * mean
+    return 0.6 <= rounds <= 4.0 and mean <= 64 and (uneven or mean <= 6)
 
 
 def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_unequal_rows: bool = False) -> BlockMask:
@@ -1497,6 +1532,51 @@ def attn_blocksparse_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: 
     return out
 
 
+def _attn_bf16_args(q, k, v):
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if t.dtype != torch.bfloat16 or t.dim() != 3:
+            raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
+    if q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
+    return tuple(t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+
+
+def _attn_bf16_items(q, k, v, bm: BlockMask, items: torch.Tensor, split_rows: Optional[torch.Tensor], n_slots: int,
+                     scale: float, pair: bool) -> torch.Tensor:
+    """The fused bf16 kernel over a list of work items (scorch_hip_attn_blocksparse_split_bf16)."""
+    tensors = [t for t in (bm.block_col_idx, bm.block_mask_index, bm.block_masks, items) if t is not None]
+    dev = _device_of(q, k, v, *tensors)
+    H, S, D = q.shape
+    if S != bm.S:
+        raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
+    ptr = lambda t: t.data_ptr() if t is not None and t.numel() else None
+    out = _empty_like(q)
+    L = native.lib()
+    with _on_device(dev):
+        stream = _stream(dev)
+        need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(H, n_slots, D)
+        ws = _workspace(dev, stream, need) if need else None
+        rc = L.scorch_hip_attn_blocksparse_split_bf16(
+            H, S, D, bm.block, bm.n_active_blocks, items.numel() // 4, items.data_ptr(), int(pair),
+            split_rows.numel() // 4 if split_rows is not None else 0, ptr(split_rows), n_slots,
+            ptr(bm.block_col_idx), ptr(bm.block_mask_index) if bm.block_mask_index is not None else None,
+            bm.n_masks if bm.block_masks is not None else 0, ptr(bm.block_masks), q.data_ptr(), k.data_ptr(),
+            v.data_ptr(), float(scale), out.data_ptr(), ws.data_ptr() if ws is not None else None,
+            ws.numel() if ws is not None else 0, stream)
+    native.check(rc)
+    if ws is not None:
+        out._scorch_workspace = ws     # a buffer handed out during a graph capture lives as long as the result
+    return out
+
+
+def _pairing(bm: BlockMask, kind: str, lens, heads: int, D: int, device) -> bool:
+    """pair_attention_items for one of the BlockMask's item lists, remembered per (list, heads, D)."""
+    key = (kind, int(heads), int(D))
+    if key not in bm.pairing:
+        bm.pairing[key] = pair_attention_items(lens, heads, D, _cu_count(device))
+    return bm.pairing[key]
+
+
 def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bm: BlockMask,
                                 scale: float) -> torch.Tensor:
     """attn_blocksparse_bf16 over a BlockMask whose long block rows split_long_block_rows has
@@ -1504,29 +1584,38 @@ def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     combines them.  Same result up to the rounding of the partial sums' combination."""
     if bm.items is None:
         raise ValueError("scorch_ops_hip: this BlockMask has no shared-out rows (split_long_block_rows)")
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        if t.dtype != torch.bfloat16 or t.dim() != 3:
-            raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
-    if q.shape != k.shape or q.shape != v.shape:
-        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
-    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
-    dev = _device_of(q, k, v, bm.block_col_idx, bm.block_mask_index, bm.block_masks, bm.items)
-    H, S, D = q.shape
-    if S != bm.S:
-        raise ValueError("scorch_ops_hip: the BlockMask was built for another sequence length")
-    out = _empty_like(q)
-    L = native.lib()
-    with _on_device(dev):
-        stream = _stream(dev)
-        need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(H, bm.n_slots, D)
-        ws = _workspace(dev, stream, need)
-        rc = L.scorch_hip_attn_blocksparse_split_bf16(
-            H, S, D, bm.block, bm.n_active_blocks, bm.items.numel() // 4, bm.items.data_ptr(),
-            bm.split_rows.numel() // 4, bm.split_rows.data_ptr(), bm.n_slots, bm.block_col_idx.data_ptr(),
-            bm.block_mask_index.data_ptr(), bm.n_masks, bm.block_masks.data_ptr(), q.data_ptr(), k.data_ptr(),
-            v.data_ptr(), float(scale), out.data_ptr(), ws.data_ptr(), ws.numel(), stream)
-    native.check(rc)
-    return out
+    q, k, v = _attn_bf16_args(q, k, v)
+    key = ("items", int(q.shape[0]), int(q.shape[2]))
+    if key not in bm.pairing:
+        if q.is_cuda and torch.cuda.is_current_stream_capturing():
+            bm_pair = False                       # (deciding needs a host read of the items)
+        else:
+            rows = bm.items.view(-1, 4)
+            bm_pair = _pairing(bm, "items", (rows[:, 2] - rows[:, 1]).cpu().numpy(), q.shape[0], q.shape[2], q.device)
+    else:
+        bm_pair = bm.pairing[key]
+    return _attn_bf16_items(q, k, v, bm, bm.items, bm.split_rows, bm.n_slots, scale, bm_pair)
+
+
+def _block_row_schedule(brp: torch.Tensor):
+    """(key blocks per block row on the host, the block rows as work items longest first, pairing
+    decisions) of a block row pointer, read back once and kept with the tensor; None while the
+    stream is capturing and nothing is known yet."""
+    import numpy as np
+    cached = getattr(brp, "_scorch_rows", None)
+    if cached is not None and cached[0] == _stamp(brp):
+        return cached[1:]
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    ptrs = brp.cpu().numpy().astype(np.int64)
+    lens = ptrs[1:] - ptrs[:-1]
+    items, _, _ = _stretches(lens, max(int(lens.max()), 1) if lens.size else 1, True)
+    entry = (_stamp(brp), lens, torch.from_numpy(items).to(brp.device).reshape(-1), {})
+    try:
+        brp._scorch_rows = entry
+    except (AttributeError, RuntimeError):
+        pass
+    return entry[1:]
 
 
 def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, block_row_ptr: torch.Tensor,
@@ -1538,48 +1627,53 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     per-head SDDMM -> softmax -> SpMM pipeline of
     bench/bench_sparse_transformer.py:354-372.  With block_mask_index (int32 per active block, -1
     = fully live) and block_masks (int64, 64 words per mask) a block is restricted to the entries
-    its bit mask names."""
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        if t.dtype != torch.bfloat16 or t.dim() != 3:
-            raise TypeError(f"scorch_ops_hip: {name} must be a bfloat16 tensor of shape (H, S, D)")
-    if q.shape != k.shape or q.shape != v.shape:
-        raise ValueError("scorch_ops_hip: q, k and v must have the same shape")
-    q, k, v = (t if t.is_contiguous() else t.contiguous() for t in (q, k, v))
+    its bit mask names.  Where it pays (pair_attention_items) the block rows go to the kernel as a
+    list of work items of which every workgroup takes two; the result is the same bit for bit."""
+    q, k, v = _attn_bf16_args(q, k, v)
     brp, bci = _index(block_row_ptr, "block_row_ptr"), _index(block_col_idx, "block_col_idx")
     dev = _device_of(q, k, v, brp, bci)
     H, S, D = q.shape
     if brp.numel() != S // block + 1:
         raise ValueError("scorch_ops_hip: block_row_ptr length does not match S / block")
+    bmi, n_masks = None, 0
+    if block_mask_index is not None:
+        bmi = _index(block_mask_index, "block_mask_index")
+        if block_masks is None or block_masks.dtype != torch.int64 or not block_masks.is_contiguous():
+            raise TypeError("scorch_ops_hip: block_masks must be a contiguous int64 tensor")
+        if bmi.numel() != bci.numel():
+            raise ValueError("scorch_ops_hip: block_mask_index must have one entry per active block")
+        if block_masks.numel() % block or block_masks.device != q.device or bmi.device != q.device:
+            raise ValueError("scorch_ops_hip: block_masks must hold 64 words per mask on the operands' device")
+        n_masks = block_masks.numel() // block
+        # the kernel trusts the mask indices as it trusts block_col_idx; a caller that built them by
+        # hand gets them checked here, once per index tensor
+        if getattr(bmi, "_scorch_mask_checked", None) != (_stamp(bmi), n_masks):
+            if bmi.numel() and int(bmi.max()) >= n_masks:
+                raise ValueError("scorch_ops_hip: block_mask_index names a mask beyond block_masks")
+            try:
+                bmi._scorch_mask_checked = (_stamp(bmi), n_masks)
+            except AttributeError:
+                pass
+    schedule = _block_row_schedule(brp) if block == 64 and D in ATTENTION_WORKGROUPS_PER_CU else None
+    if schedule is not None:
+        lens, items, pairing = schedule
+        key = (int(H), int(D))
+        if key not in pairing:
+            pairing[key] = pair_attention_items(lens, int(H), int(D), _cu_count(dev))
+        if pairing[key]:
+            rows = BlockMask(int(S), block, brp, bci, bmi, block_masks if bmi is not None else None, 0)
+            return _attn_bf16_items(q, k, v, rows, items, None, 0, scale, True)
     out = _empty_like(q)
-    if block_mask_index is None:
-        with _on_device(dev):
+    with _on_device(dev):
+        if bmi is None:
             rc = native.lib().scorch_hip_attn_blocksparse_bf16(H, S, D, block, bci.numel(), brp.data_ptr(),
                                                                bci.data_ptr(), q.data_ptr(), k.data_ptr(),
                                                                v.data_ptr(), float(scale), out.data_ptr(),
                                                                _stream(dev))
-        native.check(rc)
-        return out
-    bmi = _index(block_mask_index, "block_mask_index")
-    if block_masks is None or block_masks.dtype != torch.int64 or not block_masks.is_contiguous():
-        raise TypeError("scorch_ops_hip: block_masks must be a contiguous int64 tensor")
-    if bmi.numel() != bci.numel():
-        raise ValueError("scorch_ops_hip: block_mask_index must have one entry per active block")
-    if block_masks.numel() % block or block_masks.device != q.device or bmi.device != q.device:
-        raise ValueError("scorch_ops_hip: block_masks must hold 64 words per mask on the operands' device")
-    n_masks = block_masks.numel() // block
-    # the kernel trusts the mask indices as it trusts block_col_idx; a caller that built them by
-    # hand gets them checked here, once per index tensor
-    if getattr(bmi, "_scorch_mask_checked", None) != (_stamp(bmi), n_masks):
-        if bmi.numel() and int(bmi.max()) >= n_masks:
-            raise ValueError("scorch_ops_hip: block_mask_index names a mask beyond block_masks")
-        try:
-            bmi._scorch_mask_checked = (_stamp(bmi), n_masks)
-        except AttributeError:
-            pass
-    with _on_device(dev):
-        rc = native.lib().scorch_hip_attn_blocksparse_masked_bf16(
-            H, S, D, block, bci.numel(), brp.data_ptr(), bci.data_ptr(), bmi.data_ptr(), n_masks,
-            block_masks.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), out.data_ptr(),
-            _stream(dev))
+        else:
+            rc = native.lib().scorch_hip_attn_blocksparse_masked_bf16(
+                H, S, D, block, bci.numel(), brp.data_ptr(), bci.data_ptr(), bmi.data_ptr(), n_masks,
+                block_masks.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), float(scale), out.data_ptr(),
+                _stream(dev))
     native.check(rc)
     return out

@@ -319,3 +319,63 @@ def test_masks_with_rows_of_similar_length_are_not_shared_out():
     rp, ci = workloads.longformer_mask(4096)
     bm = H.attention_block_mask(dev(rp), dev(ci), 4096)
     assert bm.items is not None and bm.split_rows.cpu().tolist()[:3] == [0, 0, 7]
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("kind", ["strided", "causal", "random_with_bit_masks", "odd_count"])
+def test_workgroups_that_take_two_items_change_nothing(oracle, D, kind):
+    """pair_items of the work-list entry: every workgroup takes the k-th longest and then the k-th
+    shortest item.  Bit for bit the result of one item per workgroup, whole block rows and
+    shared-out stretches alike, with and without per-block bit masks, and an odd number of items."""
+    from scorch_amd import native
+    rng = np.random.default_rng(D + len(kind))
+    heads = 3
+    if kind == "random_with_bit_masks":
+        S = 512
+        mask = rng.random((S, S)) < 0.3
+        mask[64:128] = False
+        rp = np.concatenate([[0], np.cumsum(mask.sum(1))]).astype(np.int32)
+        bm = H.block_mask_from_csr(dev(rp), dev(np.nonzero(mask)[1].astype(np.int32)), S)
+    else:
+        nb = {"strided": 24, "causal": 16, "odd_count": 7}[kind]
+        S = 64 * nb
+        brp, bci = workloads.blocksparse_pattern(nb, window=3 if kind == "strided" else nb, stride=4)
+        bm = H.BlockMask(S, 64, dev(brp), dev(bci), None, None, int(bci.size) * 4096)
+    q, k, v = (torch.randn(heads, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))
+    for longest in (None, 2):                                     # whole rows; rows shared out in stretches of two
+        if longest is None:
+            items, split_rows, n_slots = H._stretches(bm.row_lens(), max(int(bm.row_lens().max()), 1), True)
+        else:
+            items, split_rows, n_slots = H._stretches(bm.row_lens(), longest, True)
+        t_items = torch.from_numpy(items).cuda().reshape(-1)
+        t_rows = torch.from_numpy(split_rows).cuda().reshape(-1) if n_slots else None
+        single = H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, False)
+        paired = H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, True)
+        assert torch.equal(single, paired)
+        if longest is None:
+            whole = single
+    plain = H.attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, D ** -0.5,
+                                    block_mask_index=bm.block_mask_index, block_masks=bm.block_masks)
+    assert torch.equal(plain, whole)
+    if kind != "random_with_bit_masks":
+        ref = oracle.attention_blocksparse_fp64(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(),
+                                                bm.block_row_ptr.cpu().numpy(), bm.block_col_idx.cpu().numpy(), 64, D ** -0.5)
+        assert oracle.rel_fro(whole.float().cpu().numpy(), ref) <= TOL_BF16
+
+
+def test_the_dispatch_pairs_items_where_it_was_measured_to_pay():
+    """A causal mask at S = 4096 with 16 heads fills the chip once with uneven workgroups: the
+    wrapper hands the block rows over as a paired work list; with 4 heads it does not.  Same bits."""
+    nb = 64
+    brp, bci = workloads.blocksparse_pattern(nb, window=nb, stride=1)
+    t_brp, t_bci = dev(brp), dev(bci)
+    for heads, expect in ((16, True), (4, False)):
+        q, k, v = (torch.randn(heads, 64 * nb, 64, device="cuda").to(torch.bfloat16) for _ in range(3))
+        out = H.attn_blocksparse_bf16(q, k, v, t_brp, t_bci, 0.125)
+        assert t_brp._scorch_rows[3][(heads, 64)] is expect
+        rc_out = torch.empty_like(q)
+        from scorch_amd import native
+        native.check(native.lib().scorch_hip_attn_blocksparse_bf16(
+            heads, 64 * nb, 64, 64, t_bci.numel(), t_brp.data_ptr(), t_bci.data_ptr(), q.data_ptr(), k.data_ptr(),
+            v.data_ptr(), 0.125, rc_out.data_ptr(), torch.cuda.current_stream().cuda_stream))
+        assert torch.equal(out, rc_out)

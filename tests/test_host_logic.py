@@ -541,3 +541,22 @@ def test_writes_the_version_counter_misses_are_the_ones_forget_is_for():
     assert H._stamp(t) == s2
     H.forget(t)
     assert H._stamp(t) != s2
+
+
+def test_when_attention_workgroups_take_two_items():
+    """pair_attention_items on the shapes it was measured on (256 CUs): uneven or very short block
+    rows, launches of 0.6 to 4 times what the chip holds at once, rows of 64 blocks at most."""
+    pair = scorch_ops_hip.pair_attention_items
+    nb = 128
+    bi = np.arange(nb)
+    c4 = np.array([int(((bi[:i + 1] >= i - 3) | ((i - bi[:i + 1]) % 8 == 0)).sum()) for i in range(nb)])   # the benchmark's mask
+    assert c4.sum() == 1466
+    causal = lambda n: np.arange(1, n + 1)
+    assert pair(c4, 16, 64) and not pair(c4, 64, 64) and not pair(c4, 4, 64)
+    assert pair(np.full(nb, 4), 16, 64) and not pair(np.full(nb, 12), 16, 64) and not pair(np.full(nb, 4), 64, 64)
+    assert pair(causal(64), 16, 64) and pair(causal(64), 64, 64) and not pair(causal(64), 4, 64)
+    assert not pair(causal(64), 128, 64)
+    assert pair(causal(64), 32, 128) and pair(causal(64), 16, 32)
+    assert not pair(causal(256), 8, 128)                       # rows of 128 blocks on average
+    assert not pair(np.full(nb, nb), 16, 64)                   # dense
+    assert not pair(np.array([5]), 16, 64) and not pair(c4, 16, 48)
