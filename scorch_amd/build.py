@@ -39,8 +39,8 @@ def sources():
 
 
 def _headers():
-    return glob.glob(os.path.join(SRC_DIR, "*.hpp")) + [
-        os.path.join(os.path.dirname(PKG_DIR), "include", "scorch_hip.h")]
+    return glob.glob(os.path.join(SRC_DIR, "*.hpp")) + glob.glob(
+        os.path.join(os.path.dirname(PKG_DIR), "include", "*.h"))
 
 
 def _newer(target, deps) -> bool:

@@ -8,7 +8,7 @@
 #include <cstdio>
 #include <type_traits>
 
-#include "../../include/scorch_hip.h"
+#include "../../include/scorch_hip_unstable.h"  // and, through it, scorch_hip.h
 
 namespace scorch {
 

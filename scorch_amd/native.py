@@ -1,4 +1,5 @@
-"""ctypes binding of libscorch_hip.so (declarations: include/scorch_hip.h).
+"""ctypes binding of libscorch_hip.so (declarations: include/scorch_hip.h and, for the single
+steps this package drives itself, include/scorch_hip_unstable.h).
 
 The library is loaded from this directory.  If it is not there it is built
 once with hipcc (scorch_amd.build); if that is impossible the import of the
@@ -26,10 +27,17 @@ _SPMM_PLANNED = [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, ctypes.c_
 _SPGEMM = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 _SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 
-# name -> (restype, argtypes); one entry per declaration in include/scorch_hip.h
+# name -> (restype, argtypes); one entry per declaration in the two headers
 SIGNATURES = {
     "scorch_hip_abi_version": (ctypes.c_int, []),
     "scorch_hip_last_error": (ctypes.c_char_p, []),
+    "scorch_hip_csr_plan_create": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, ctypes.POINTER(_ptr)]),
+    "scorch_hip_csr_plan_destroy": (ctypes.c_int, [_ptr]),
+    "scorch_hip_csr_plan_info": (ctypes.c_int, [_ptr, ctypes.POINTER(_i64)]),
+    "scorch_hip_csr_plan_prepare": (ctypes.c_int, [_ptr, ctypes.c_int, _i64, _ptr]),
+    "scorch_hip_spmm_csr_plan_f32": (ctypes.c_int, [_ptr, _i64, _ptr, _ptr, _ptr, ctypes.c_int, _ptr, _ptr]),
+    "scorch_hip_sddmm_csr_plan_f32": (ctypes.c_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_softmax_csr_plan_f32": (ctypes.c_int, [_ptr, _ptr, ctypes.c_float, _ptr, _ptr]),
     "scorch_hip_timing_begin": (ctypes.c_int, []),
     "scorch_hip_timing_end": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), ctypes.c_int,
                                              ctypes.POINTER(ctypes.c_int)]),

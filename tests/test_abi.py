@@ -1,6 +1,6 @@
 """The C-ABI library without a GPU: it loads, exports every symbol that
-include/scorch_hip.h declares, and rejects bad arguments on the host before
-launching anything.  No compute call is made here."""
+include/scorch_hip.h and include/scorch_hip_unstable.h declare, and rejects bad
+arguments on the host before launching anything.  No compute call is made here."""
 import ctypes
 import os
 import re
@@ -10,13 +10,19 @@ import pytest
 from scorch_amd import native
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "scorch_hip.h")
+HEADER = os.path.join(ROOT, "include", "scorch_hip.h")                    # the stable surface
+UNSTABLE_HEADER = os.path.join(ROOT, "include", "scorch_hip_unstable.h")  # the steps underneath
+HEADERS = (HEADER, UNSTABLE_HEADER)
 
 
-def declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"SCORCH_HIP_API[^;(]*?\b(scorch_hip_\w+)\s*\(", text)))
+def declared_symbols(headers=HEADERS):
+    names = []
+    for header in headers:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"SCORCH_HIP_API[^;(]*?\b(scorch_hip_\w+)\s*\(", text)
+    assert len(names) == len(set(names)), "a function is declared twice"
+    return sorted(names)
 
 
 @pytest.fixture(scope="module")
@@ -33,9 +39,25 @@ def test_header_declares_the_expected_entry_points():
     assert len(names) >= 16
 
 
+def test_the_stable_header_holds_no_plan_step():
+    """One call per operation and the plan handle in scorch_hip.h; inspection, boundaries, entry
+    lists, block descriptions, work-item lists, pinned kernels and timing aids in the other."""
+    stable = declared_symbols((HEADER,))
+    unstable = declared_symbols((UNSTABLE_HEADER,))
+    step = re.compile(r"inspect|bounds|planned|_rows_|tiled|lists|listed|short_rows|split|blocked|block_|batched|"
+                      r"timing|timed|attn_blocksparse_f32")
+    assert [n for n in stable if step.search(n)] == []
+    assert [n for n in unstable if not step.search(n)] == []
+    assert len(stable) <= 40
+    for name in ("create", "destroy", "info", "prepare"):
+        assert "scorch_hip_csr_plan_" + name in stable
+    for name in ("spmm", "sddmm", "softmax"):
+        assert f"scorch_hip_{name}_csr_plan_f32" in stable
+
+
 def test_library_exports_every_declared_symbol(L):
     for name in declared_symbols():
-        assert hasattr(L, name), f"{name} is declared in scorch_hip.h but not exported"
+        assert hasattr(L, name), f"{name} is declared in a header but not exported"
 
 
 def test_binding_table_matches_header(L):
@@ -198,6 +220,27 @@ def test_attention_rejects_unsupported_shapes(L):
     assert split(n_items=0, items=NULL) == native.OK
 
 
+def test_plan_handle_rejects_bad_arguments_on_the_host(L):
+    handle = ctypes.c_void_p()
+    ref = ctypes.byref(handle)
+    index = (ctypes.c_int32 * 8)()
+    at = ctypes.addressof(index)
+    assert L.scorch_hip_csr_plan_create(4, 4, 0, at, NULL, None, None) == native.EINVAL
+    assert b"plan is NULL" in L.scorch_hip_last_error()
+    assert L.scorch_hip_csr_plan_create(-1, 4, 0, at, NULL, None, ref) == native.EINVAL
+    assert L.scorch_hip_csr_plan_create(4, 4, 0, NULL, NULL, None, ref) == native.EINVAL
+    assert L.scorch_hip_csr_plan_create(4, 4, 3, at, NULL, None, ref) == native.EINVAL
+    assert L.scorch_hip_csr_plan_create(1 << 31, 4, 0, at, NULL, None, ref) == native.EUNSUPPORTED
+    assert handle.value is None
+    info = (ctypes.c_int64 * 8)()
+    assert L.scorch_hip_csr_plan_info(None, info) == native.EINVAL
+    assert L.scorch_hip_csr_plan_prepare(None, 0, 8, None) == native.EINVAL
+    assert L.scorch_hip_spmm_csr_plan_f32(None, 8, at, at, None, 0, at, None) == native.EINVAL
+    assert L.scorch_hip_sddmm_csr_plan_f32(None, 8, None, at, at, at, None, None) == native.EINVAL
+    assert L.scorch_hip_softmax_csr_plan_f32(None, at, 1.0, at, None) == native.EINVAL
+    assert L.scorch_hip_csr_plan_destroy(None) == native.OK
+
+
 def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):
     """The boundary is a C ABI: the header compiles as C99 and as C++11, and a C program linked
     against the library reads the ABI version and a workspace size (no GPU involved)."""
@@ -205,12 +248,12 @@ def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):
     import shutil
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    header = os.path.join(root, "include", "scorch_hip.h")
     gcc, gxx = shutil.which("gcc"), shutil.which("g++")
     if not gcc or not gxx:
         pytest.skip("no host compiler")
-    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", header], check=True)
-    subprocess.run([gxx, "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", header], check=True)
+    for header in HEADERS:
+        subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", header], check=True)
+        subprocess.run([gxx, "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", header], check=True)
     src = tmp_path / "host.c"
     src.write_text(
         '#include <stdio.h>\n#include "scorch_hip.h"\n'
