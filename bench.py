@@ -298,9 +298,19 @@ def _timed_as():
 
 
 def _kernel_times(fn, samples):
-    """Average duration (ms) of each kernel `fn` launches, in launch order."""
+    """Average duration (ms) of each kernel `fn` launches, in launch order: HIP events that the
+    library records on the kernels' stream before, between and after them.  A kernel that only
+    spins (no memory traffic, so the caches stay as the timed steps left them) is queued in front
+    of every sample, so that the events and the kernels between them are all enqueued before the
+    GPU reaches the first: an interval is then the kernel's time, without the host's time to
+    issue it, which for a kernel of a few microseconds would be most of the figure."""
+    import torch
     from scorch_amd import native
-    rows = [native.kernel_times(fn) for _ in range(samples)]
+
+    def sample():
+        torch.cuda._sleep(80_000)       # about 40 us
+        fn()
+    rows = [native.kernel_times(sample) for _ in range(samples)]
     width = min(len(r) for r in rows)
     return [sum(r[i] for r in rows) / len(rows) for i in range(width)]
 
@@ -401,10 +411,12 @@ def run_spmm(name, args, headline=False):
         names = [f"spmm_merge_kernel<float,{vec},0>" if N * 4 > 256 else "spmm_grouped_kernel<float,...>",
                  "spmm_fixup_kernel<float,...>"]
     dominant = max(range(len(kernels)), key=lambda i: kernels[i])
-    # the named kernel's own duration, HIP events around its launch (for a kernel of a few
-    # microseconds that includes the dispatch of an isolated launch, which back-to-back launches
-    # hide: ms_per_step, the queued time per step, can be the smaller figure)
-    kernel_ms = kernels[dominant]
+    # the named kernel's duration: its share (from the events around every single launch) of the
+    # time per step between the two events that enclose the timed region, where the launches run
+    # back to back as they do in use.  The bracket around one launch by itself (kernel_ms_bracketed)
+    # also holds the dispatch of an isolated launch and of its two events, 2 to 3 us: most of the
+    # figure for a kernel of 5 us, nothing for one of a millisecond.
+    kernel_ms = event_ms * kernels[dominant] / sum(kernels)
 
     flops = 2.0 * nnz * N
     algo, gather = spmm_algorithmic_bytes(M, K, N, nnz), spmm_gather_bytes(M, N, nnz)
@@ -426,7 +438,8 @@ def run_spmm(name, args, headline=False):
         "event_ms_per_step": round(event_ms, 5),
         "hbm_gbps_algorithmic": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
         "roofline": _hbm_roofline(names[dominant], kernel_ms, algo, traffic, provenance,
-                                  {"gather_model_bytes": gather,
+                                  {"kernel_ms_bracketed": round(kernels[dominant], 5),
+                                   "gather_model_bytes": gather,
                                    "gather_model_gbps": round(gather / (kernel_ms * 1e-3) / 1e9, 1)}),
     }
     if name == "gcn_powerlaw":
@@ -471,7 +484,8 @@ def run_sddmm(args):
     warm = _warmup_calls(csr, args.warmup)
     ms = _time_steps(csr, args.steps, 0)
     timed = _timed_as()
-    kernel_ms = max(_kernel_times(csr, min(args.steps, 10)))
+    bracketed_ms = max(_kernel_times(csr, min(args.steps, 10)))
+    kernel_ms = ms          # one kernel per step: the time per step between the timed region's two events
     ms_coo = _time_steps(coo, args.steps, 2)
     flops = 2.0 * nnz * K + nnz
     # every array once: row_ptr, col_idx, mask values, A, B, result values; the CSR-mask kernel
@@ -491,7 +505,8 @@ def run_sddmm(args):
            "path": "listed" if listed else "plain",
            "roofline": _hbm_roofline("sddmm_listed_kernel<16,4>" if listed else "sddmm_kernel<16,4,false,false>",
                                      kernel_ms, algo, traffic, provenance,
-                                     {"row_coordinate_output_bytes": 4 * nnz, "gather_model_bytes": gather,
+                                     {"kernel_ms_bracketed": round(bracketed_ms, 5),
+                                      "row_coordinate_output_bytes": 4 * nnz, "gather_model_bytes": gather,
                                       "gather_model_gbps": round(gather / kernel_ms / 1e6, 1)})}
     if args.vendor:
         mask = torch.sparse_csr_tensor(pos, crd, val, size=(M, n_cols))
@@ -518,7 +533,8 @@ def run_attention(args):
     warm = _warmup_calls(fn, args.warmup)
     ms = _time_steps(fn, args.steps, 0)
     timed = _timed_as()
-    kernel_ms = max(_kernel_times(fn, min(args.steps, 10)))
+    bracketed_ms = max(_kernel_times(fn, min(args.steps, 10)))
+    kernel_ms = ms          # one kernel per step: the time per step between the timed region's two events
     flops = 4.0 * nnz * D * Hh
     algo = 4 * Hh * S * D * 2 + 4 * (brp.numel() + bci.numel())
     achieved = flops / ms / 1e9
@@ -537,6 +553,7 @@ def run_attention(args):
                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(kernel_achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic,
                         "flops": flops, "algorithmic_bytes": algo, "kernel_ms_avg": round(kernel_ms, 5),
+                        "kernel_ms_bracketed": round(bracketed_ms, 5),
                         "hbm_gbps_algorithmic": round(algo / kernel_ms / 1e6, 1),
                         **({"traffic_measured_at": provenance} if provenance else {})}}
     # the same attention at the reference's precision: fp32 operands, probabilities and sums, one kernel

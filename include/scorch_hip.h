@@ -72,6 +72,12 @@ SCORCH_HIP_API int scorch_hip_abi_version(void);
 /* Message of the calling thread's most recent failed call ("" if none). */
 SCORCH_HIP_API const char *scorch_hip_last_error(void);
 
+/* Optional.  Loads the library's device code for the current device now.  Otherwise the HIP
+ * runtime loads it piece by piece, when the first kernel of each of the library's source files
+ * is launched: about a millisecond added to the first product of each kind.  Launches nothing;
+ * SCORCH_HIP_ERUNTIME without a usable device.  No counterpart in the reference. */
+SCORCH_HIP_API int scorch_hip_init(void);
+
 /* ------------------------------------------------------------------------
  * SpMM: C[M,N] = A_csr[M,K] * B[K,N], all of one dtype.
  *

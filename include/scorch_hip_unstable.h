@@ -346,6 +346,13 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_batched_f32(int64_t batch, int64_t M, int
                                     float *C /* [batch, M, N] */, const void *bounds, size_t bounds_bytes,
                                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* Whether a value array holds anything but `value`: *differ (device) is set to 1 if some vals[i]
+ * != value (a NaN differs from everything), else to 0.  The host layer asks it of an SDDMM mask's
+ * values once, to pass mask_vals = NULL from then on when they are all 1; an attention mask's are.
+ * No counterpart in the reference. */
+SCORCH_HIP_API int scorch_hip_values_differ_f32(int64_t n, const float *vals, float value,
+                                 int32_t *differ /* device */, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

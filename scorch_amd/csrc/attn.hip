@@ -593,3 +593,5 @@ extern "C" int scorch_hip_attn_blocksparse_split_bf16(
   return attn_entry(fn, H, S, D, block, n_active_blocks, nullptr, block_col_idx, block_mask_index, block_masks,
                     Q, K, V, scale, O, stream, &split);
 }
+
+SCORCH_DEFINE_PRELOAD(attn)

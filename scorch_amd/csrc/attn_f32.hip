@@ -403,3 +403,5 @@ extern "C" int scorch_hip_attn_blocksparse_f32(
   SCORCH_ATTN32(128);
 #undef SCORCH_ATTN32
 }
+
+SCORCH_DEFINE_PRELOAD(attn_f32)

@@ -303,3 +303,5 @@ extern "C" int scorch_hip_csr_block_fill(int64_t M, int64_t n_cols, int64_t nnz,
   SCORCH_HIP_CHECK(hipGetLastError());
   return SCORCH_HIP_OK;
 }
+
+SCORCH_DEFINE_PRELOAD(blockdesc)

@@ -498,3 +498,5 @@ extern "C" int scorch_hip_spmm_csr_blocked_f32(int64_t H, int64_t M, int64_t K, 
 #undef SCORCH_BLOCKED_SPMM
   return SCORCH_HIP_OK;
 }
+
+SCORCH_DEFINE_PRELOAD(blocked)

@@ -183,3 +183,18 @@ __device__ __forceinline__ int wave_count_below(int n, int64_t bound, KeyFn key)
 }
 
 }  // namespace scorch
+
+// ---- loading the device code ahead of the first launch ------------------------------------------
+// HIP loads a source file's device code when the first kernel of that file is launched on a
+// device, which takes about a millisecond: a product whose kernels live in a file that has not
+// been used yet pays it.  Every source file defines an empty kernel through this macro;
+// scorch_hip_init() asks the runtime for each one's attributes, which loads the file's code for
+// the current device without launching anything.
+#define SCORCH_DEFINE_PRELOAD(name)                                                                   \
+  namespace scorch {                                                                                  \
+  __global__ void preload_anchor_##name() {}                                                          \
+  hipError_t preload_##name() {                                                                       \
+    hipFuncAttributes attributes;                                                                     \
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void *>(&preload_anchor_##name)); \
+  }                                                                                                   \
+  }

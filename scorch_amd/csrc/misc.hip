@@ -557,6 +557,16 @@ __global__ __launch_bounds__(kBlockThreads) void coo_row_ptr_kernel(
   if (bad) *unsorted = 1;  // every writer stores the same value
 }
 
+// Whether some element of vals differs from `value` (a NaN differs from everything).
+__global__ void values_differ_clear_kernel(int *differ) { *differ = 0; }
+__global__ __launch_bounds__(kBlockThreads) void values_differ_kernel(int64_t n, const float *__restrict__ vals,
+                                                                       float value, int *__restrict__ differ) {
+  bool any = false;
+  const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n; i += stride) any |= !(vals[i] == value);
+  if (__ballot(any) != 0 && wave_lane() == 0) atomicOr(differ, 1);
+}
+
 }  // namespace scorch
 
 extern "C" {
@@ -719,4 +729,23 @@ int scorch_hip_coo_row_ptr(int64_t M, int64_t nnz, const int32_t *row_idx, int32
   return SCORCH_HIP_OK;
 }
 
+int scorch_hip_values_differ_f32(int64_t n, const float *vals, float value, int32_t *differ, void *stream) {
+  const char *fn = "scorch_hip_values_differ_f32";
+  if (n < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
+  SCORCH_REQUIRE(differ != nullptr, "%s: NULL output", fn);
+  SCORCH_REQUIRE(n == 0 || vals != nullptr, "%s: vals is NULL", fn);
+  SCORCH_REQUIRE(scorch::aligned_to(vals, 4) && scorch::aligned_to(differ, 4), "%s: arrays must be 4-byte aligned", fn);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  scorch::values_differ_clear_kernel<<<1, 1, 0, s>>>(differ);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  if (n == 0) return SCORCH_HIP_OK;
+  int64_t blocks = (n + scorch::kBlockThreads * 8 - 1) / (scorch::kBlockThreads * 8);
+  if (blocks > 4096) blocks = 4096;  // the kernel strides
+  scorch::values_differ_kernel<<<dim3((unsigned)blocks), scorch::kBlockThreads, 0, s>>>(n, vals, value, differ);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
 }  // extern "C"
+
+SCORCH_DEFINE_PRELOAD(misc)

@@ -11,6 +11,19 @@
 
 #include "common.hpp"
 
+namespace scorch {
+hipError_t preload_attn();
+hipError_t preload_attn_f32();
+hipError_t preload_blockdesc();
+hipError_t preload_blocked();
+hipError_t preload_misc();
+hipError_t preload_sddmm();
+hipError_t preload_spgemm();
+hipError_t preload_spmm();
+hipError_t preload_spmm_rows();
+hipError_t preload_spmm_tiled();
+}  // namespace scorch
+
 namespace {
 
 constexpr int kPlanWidths = 8;              // chunk boundaries kept for this many values of N
@@ -155,6 +168,12 @@ int prepare_softmax(scorch_hip_csr_plan *plan, hipStream_t stream) {
 }  // namespace
 
 extern "C" {
+
+int scorch_hip_init(void) {
+  hipError_t (*const loaders[])() = {scorch::preload_attn, scorch::preload_attn_f32, scorch::preload_blockdesc, scorch::preload_blocked, scorch::preload_misc, scorch::preload_sddmm, scorch::preload_spgemm, scorch::preload_spmm, scorch::preload_spmm_rows, scorch::preload_spmm_tiled};
+  for (auto load : loaders) SCORCH_HIP_CHECK(load());
+  return SCORCH_HIP_OK;
+}
 
 int scorch_hip_csr_plan_create(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
                                const int32_t *col_idx, void *stream, scorch_hip_csr_plan **out) {

@@ -622,3 +622,5 @@ int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, in
 }
 
 }  // extern "C"
+
+SCORCH_DEFINE_PRELOAD(sddmm)

@@ -1291,3 +1291,5 @@ SCORCH_DEFINE_SPGEMM(i32, int32_t)
 SCORCH_DEFINE_SPGEMM(i64, int64_t)
 
 }  // extern "C"
+
+SCORCH_DEFINE_PRELOAD(spgemm)

@@ -364,3 +364,5 @@ int scorch_hip_csr_inspect(int64_t M, int64_t K, int64_t nnz, const int32_t *row
 }
 
 }  // extern "C"
+
+SCORCH_DEFINE_PRELOAD(spmm_rows)

@@ -357,3 +357,5 @@ int scorch_hip_spmm_csr_tiled_f32(int64_t M, int64_t K, int64_t N, int64_t nnz, 
 }
 
 }  // extern "C"
+
+SCORCH_DEFINE_PRELOAD(spmm_tiled)

@@ -31,6 +31,7 @@ _SPMV = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _size, _ptr]
 SIGNATURES = {
     "scorch_hip_abi_version": (ctypes.c_int, []),
     "scorch_hip_last_error": (ctypes.c_char_p, []),
+    "scorch_hip_init": (ctypes.c_int, []),
     "scorch_hip_csr_plan_create": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, ctypes.POINTER(_ptr)]),
     "scorch_hip_csr_plan_destroy": (ctypes.c_int, [_ptr]),
     "scorch_hip_csr_plan_info": (ctypes.c_int, [_ptr, ctypes.POINTER(_i64)]),
@@ -119,6 +120,7 @@ SIGNATURES = {
                                                        _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr]),
     "scorch_hip_csr_row_indices": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr]),
     "scorch_hip_coo_row_ptr": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "scorch_hip_values_differ_f32": (ctypes.c_int, [_i64, _ptr, ctypes.c_float, _ptr, _ptr]),
     "scorch_hip_csr_block_count": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
     "scorch_hip_csr_block_fill": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr,
                                                  _ptr, _ptr]),

@@ -128,6 +128,9 @@ def _stream(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
+_code_loaded = set()     # devices on which scorch_hip_init has run
+
+
 class _on_device:
     """``with _on_device(dev):`` makes `dev` the current device like
     ``torch.cuda.device`` does, but costs next to nothing when it already is."""
@@ -142,6 +145,11 @@ class _on_device:
         if current != self.index:
             self.previous = current
             torch.cuda.set_device(self.index)
+        if self.index not in _code_loaded:
+            # the library's device code, all of it, when a device is first used: otherwise the first
+            # product of every kind pays for the part it is the first to need
+            _code_loaded.add(self.index)
+            native.check(native.lib().scorch_hip_init())
         return self
 
     def __exit__(self, *exc):
@@ -548,7 +556,11 @@ def _known_all_ones(values: torch.Tensor) -> bool:
     seen = getattr(values, "_scorch_ones", None)
     if seen is not None and seen[0] == key:
         if seen[1] is None:
-            seen = (key, bool((values == 1).all()))
+            differ = _empty(1, dtype=torch.int32, device=values.device)
+            with _on_device(values.device):
+                native.check(native.lib().scorch_hip_values_differ_f32(values.numel(), values.data_ptr(), 1.0,
+                                                                       differ.data_ptr(), _stream(values.device)))
+            seen = (key, values.dtype == torch.float32 and not differ.item())
             values._scorch_ones = seen
         return bool(seen[1])
     try:

@@ -12,6 +12,7 @@ import torch
 
 from conftest import random_csr
 from gpu_util import dev, hip_sddmm_coo, hip_sddmm_csr, host
+from scorch_amd import native
 from scorch_amd import scorch_ops_hip as H
 from scorch_amd import workloads
 
@@ -306,3 +307,29 @@ def test_a_mask_without_a_value_array_is_a_mask_of_ones(oracle, monkeypatch, pat
     expect = with_ones.clone()
     expect[11] *= 3.0
     assert torch.equal(changed, expect)
+
+
+def test_values_differ_kernel():
+    """What decides that a mask's values need not be read: 0 only when every value is the one asked about."""
+    L = native.lib()
+    flag = torch.full((2,), 7, dtype=torch.int32, device="cuda")
+
+    def differ(vals, value=1.0):
+        flag.fill_(7)
+        native.check(L.scorch_hip_values_differ_f32(vals.numel(), vals.data_ptr(), value, flag.data_ptr(),
+                                                    torch.cuda.current_stream().cuda_stream))
+        got = flag.tolist()
+        assert got[1] == 7
+        return got[0]
+
+    for n in (0, 1, 63, 64, 4097, 3_000_001):
+        ones = torch.ones(n, device="cuda")
+        assert differ(ones) == 0, n
+        assert differ(ones, 2.0) == (1 if n else 0), n
+        if n:
+            for at in {0, n // 2, n - 1}:
+                v = ones.clone()
+                v[at] = 1.0000001
+                assert differ(v) == 1, (n, at)
+                v[at] = float("nan")
+                assert differ(v) == 1, (n, at)
