@@ -449,6 +449,15 @@ def run_spmm(name, args, headline=False):
                               "values": "D^-1/2 (A+I) D^-1/2"})
         if args.window:
             rec["config"]["neighbour_window"] = args.window
+    if not headline:
+        # the same product through the C ABI's plan handles alone (what a C++ host of the reference would
+        # call: one object per operand, one call per product, no Python-side plans)
+        from scorch_amd.csr_plan import CsrPlanHandle, DensePlanHandle
+        B2d = B.reshape(K, N)
+        with CsrPlanHandle(pos, crd, K) as handle, DensePlanHandle(B2d) as dense:
+            planned = (lambda: handle.spmm_dense(val, dense)) if tiled else (lambda: handle.spmm(val, B2d))
+            rec["ms_per_step_plan_handle"] = round(_time_steps(planned, args.steps, 2), 5)
+            torch.cuda.synchronize()
     if args.graph and not headline:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())

@@ -294,8 +294,8 @@ SCORCH_HIP_API int scorch_hip_softmax_csr_f32(int64_t M, int64_t nnz, const int3
  * The first product of a kind and width allocates device memory (hipMalloc: not under graph
  * capture); scorch_hip_csr_plan_prepare does that ahead of time, after which the product calls
  * of that kind and width allocate nothing and do not synchronise.  `width` is N for
- * SCORCH_HIP_PLAN_SPMM_F32, K for SCORCH_HIP_PLAN_SDDMM_F32 and ignored for
- * SCORCH_HIP_PLAN_SOFTMAX_F32.  A plan holds boundaries for at most 8 widths of N; a ninth
+ * SCORCH_HIP_PLAN_SPMM_F32 and SCORCH_HIP_PLAN_SPMM_DENSE_F32, K for SCORCH_HIP_PLAN_SDDMM_F32
+ * and ignored for SCORCH_HIP_PLAN_SOFTMAX_F32.  A plan holds boundaries for at most 8 widths of N; a ninth
  * replaces the oldest.
  *
  * scorch_hip_csr_plan_info writes SCORCH_HIP_PLAN_INFO_INTS int64 to `info` (host): M, n_cols,
@@ -306,7 +306,8 @@ typedef struct scorch_hip_csr_plan scorch_hip_csr_plan;
 enum scorch_hip_plan_op {
   SCORCH_HIP_PLAN_SPMM_F32 = 0,
   SCORCH_HIP_PLAN_SDDMM_F32 = 1,
-  SCORCH_HIP_PLAN_SOFTMAX_F32 = 2
+  SCORCH_HIP_PLAN_SOFTMAX_F32 = 2,
+  SCORCH_HIP_PLAN_SPMM_DENSE_F32 = 3 /* products through a scorch_hip_dense_plan N wide */
 };
 #define SCORCH_HIP_PLAN_INFO_INTS 8
 SCORCH_HIP_API int scorch_hip_csr_plan_create(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
@@ -321,6 +322,31 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_plan_f32(scorch_hip_csr_plan *plan, int6
                                   void *stream);
 SCORCH_HIP_API int scorch_hip_softmax_csr_plan_f32(scorch_hip_csr_plan *plan, const float *vals, float scale,
                                     float *out, void *stream);
+
+/* The dense side of the same idea: a dense fp32 operand B[K, N] that many products use unchanged
+ * (a weight matrix: the reference's weight-sparse autoencoder multiplies every batch by the same
+ * decoder weight, bench/bench_sparse_autoencoder.py:250-276, and converts weights once outside its
+ * loop, bench/README_sparse_autoencoder.md:86).  For shapes where it pays (rows of B of 2 KiB and
+ * more, K * 128 bytes within an L2's reach) scorch_hip_dense_plan_create stores B a second time by
+ * column tiles (hipMalloc of the size of B, one read and one write of B on `stream`); for other
+ * shapes the handle only names B.  It keeps the POINTER B: the array must stay in place until the
+ * plan is destroyed, and after its VALUES have changed scorch_hip_dense_plan_update copies them
+ * again -- a product issued in between would use the old values, and nothing could notice.
+ * scorch_hip_spmm_csr_plan_dense_f32 is scorch_hip_spmm_csr_plan_f32 with B named by its plan:
+ * with the tile copy, and a sparse operand that gathers the rows of B twice or more on average,
+ * every XCD keeps one tile of the copy in its L2 while all rows of A gather from it, so B comes
+ * from memory once (the decoder shape, 4096 x 16,384 with 32 entries per row times 16,384 x 4096:
+ * 0.10 ms against 0.25 ms); otherwise it is that call.  Results agree with the other SpMM entry
+ * points to rounding and are bit-reproducible.  scorch_hip_csr_plan_prepare with
+ * SCORCH_HIP_PLAN_SPMM_DENSE_F32 and width N allocates ahead of time what these products need. */
+typedef struct scorch_hip_dense_plan scorch_hip_dense_plan;
+SCORCH_HIP_API int scorch_hip_dense_plan_create(int64_t K, int64_t N, const float *B, void *stream,
+                                 scorch_hip_dense_plan **plan /* host */);
+SCORCH_HIP_API int scorch_hip_dense_plan_update(scorch_hip_dense_plan *plan, void *stream);
+SCORCH_HIP_API int scorch_hip_dense_plan_destroy(scorch_hip_dense_plan *plan);
+SCORCH_HIP_API int scorch_hip_spmm_csr_plan_dense_f32(scorch_hip_csr_plan *plan, const float *vals,
+                                       const scorch_hip_dense_plan *dense, const float *bias, int act,
+                                       float *C, void *stream);
 
 /* ------------------------------------------------------------------------
  * Fused block-sparse attention, bf16 in / bf16 out, fp32 accumulation:

@@ -19,12 +19,53 @@ import torch
 
 from . import native
 
-PLAN_SPMM_F32, PLAN_SDDMM_F32, PLAN_SOFTMAX_F32 = 0, 1, 2
+PLAN_SPMM_F32, PLAN_SDDMM_F32, PLAN_SOFTMAX_F32, PLAN_SPMM_DENSE_F32 = 0, 1, 2, 3
 ACT_NONE, ACT_RELU = 0, 1
 
 
 def _stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class DensePlanHandle:
+    """Owns one scorch_hip_dense_plan: a dense fp32 operand (K, N) that many products use unchanged.
+    Keeps the tensor alive; after writing new values into it call update() before the next product."""
+
+    def __init__(self, B: torch.Tensor):
+        if B.dim() != 2 or B.dtype != torch.float32 or not B.is_cuda or not B.is_contiguous():
+            raise TypeError("DensePlanHandle: B must be a contiguous 2-D fp32 tensor on the GPU")
+        self.B, self.device = B, B.device
+        self.K, self.N = B.shape
+        self._handle = ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            native.check(native.lib().scorch_hip_dense_plan_create(self.K, self.N, B.data_ptr(), _stream(self.device),
+                                                                   ctypes.byref(self._handle)))
+
+    def update(self) -> None:
+        with torch.cuda.device(self.device):
+            native.check(native.lib().scorch_hip_dense_plan_update(self._live(), _stream(self.device)))
+
+    def close(self) -> None:
+        handle, self._handle = self._handle, ctypes.c_void_p()
+        if handle:
+            native.check(native.lib().scorch_hip_dense_plan_destroy(handle))
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _live(self):
+        if not self._handle:
+            raise RuntimeError("DensePlanHandle: the plan has been closed")
+        return self._handle
 
 
 class CsrPlanHandle:
@@ -104,6 +145,19 @@ class CsrPlanHandle:
             native.check(native.lib().scorch_hip_spmm_csr_plan_f32(
                 self._live(), N, self._f32(vals, self.nnz, "vals"), self._f32(B, self.n_cols * N, "B"),
                 self._f32(bias, N, "bias"), ACT_RELU if relu else ACT_NONE, out.data_ptr(), _stream(self.device)))
+        return out
+
+    def spmm_dense(self, vals: torch.Tensor, dense: DensePlanHandle, bias: Optional[torch.Tensor] = None,
+                   relu: bool = False) -> torch.Tensor:
+        """spmm() with the dense operand named by its plan (a weight matrix stored by column tiles
+        where that pays)."""
+        if relu and bias is None:
+            raise ValueError("CsrPlanHandle.spmm_dense: the activation comes with a bias")
+        out = torch.empty((self.M, dense.N), dtype=torch.float32, device=self.device)
+        with torch.cuda.device(self.device):
+            native.check(native.lib().scorch_hip_spmm_csr_plan_dense_f32(
+                self._live(), self._f32(vals, self.nnz, "vals"), dense._live(), self._f32(bias, dense.N, "bias"),
+                ACT_RELU if relu else ACT_NONE, out.data_ptr(), _stream(self.device)))
         return out
 
     def sddmm(self, mask_vals: Optional[torch.Tensor], A: torch.Tensor, B: torch.Tensor,

@@ -63,6 +63,14 @@ struct scorch_hip_csr_plan {
   }
 };
 
+struct scorch_hip_dense_plan {
+  int device = 0;
+  int64_t K = 0, N = 0;
+  const float *B = nullptr;
+  float *tiles = nullptr;  // B stored by column tiles, or null where that layout does not pay
+  size_t tiles_bytes = 0;
+};
+
 namespace {
 
 using scorch::fail;
@@ -102,10 +110,11 @@ bool spmm_by_rows(const scorch_hip_csr_plan *plan, int64_t N, bool has_bias) {
 
 // Boundaries and workspace of the merge-path kernels for dense width N (nothing for a product
 // the row-split kernel serves with and without a bias).
-int prepare_spmm(scorch_hip_csr_plan *plan, int64_t N, hipStream_t stream, Boundaries **found) {
+int prepare_spmm(scorch_hip_csr_plan *plan, int64_t N, hipStream_t stream, Boundaries **found,
+                 bool whatever_the_rows = false) {
   if (found) *found = nullptr;
   if (N < 0) return fail(SCORCH_HIP_EINVAL, "scorch_hip_csr_plan: negative N");
-  if (spmm_by_rows(plan, N, false) && spmm_by_rows(plan, N, true)) return SCORCH_HIP_OK;
+  if (!whatever_the_rows && spmm_by_rows(plan, N, false) && spmm_by_rows(plan, N, true)) return SCORCH_HIP_OK;
   if (int rc = reserve_workspace(plan, scorch_hip_spmm_csr_workspace_bytes(plan->M, plan->nnz, N, 4), stream))
     return rc;
   Boundaries *slot = nullptr;
@@ -254,6 +263,7 @@ int scorch_hip_csr_plan_prepare(scorch_hip_csr_plan *plan, int op, int64_t width
     case SCORCH_HIP_PLAN_SPMM_F32: return prepare_spmm(plan, width, s, nullptr);
     case SCORCH_HIP_PLAN_SDDMM_F32: return prepare_sddmm(plan, width, s);
     case SCORCH_HIP_PLAN_SOFTMAX_F32: return prepare_softmax(plan, s);
+    case SCORCH_HIP_PLAN_SPMM_DENSE_F32: return prepare_spmm(plan, width, s, nullptr, true);
     default: return fail(SCORCH_HIP_EINVAL, "scorch_hip_csr_plan_prepare: op %d is not a scorch_hip_plan_op", op);
   }
 }
@@ -294,6 +304,82 @@ int scorch_hip_softmax_csr_plan_f32(scorch_hip_csr_plan *plan, const float *vals
   if (int rc = prepare_softmax(plan, static_cast<hipStream_t>(stream))) return rc;
   return scorch_hip_softmax_csr_f32(plan->M, plan->nnz, plan->row_ptr, vals, scale, out, plan->workspace,
                                     plan->workspace_bytes, stream);
+}
+
+int scorch_hip_dense_plan_create(int64_t K, int64_t N, const float *B, void *stream, scorch_hip_dense_plan **out) {
+  const char *fn = "scorch_hip_dense_plan_create";
+  if (!out) return fail(SCORCH_HIP_EINVAL, "%s: plan is NULL", fn);
+  *out = nullptr;
+  if (K < 0 || N < 0) return fail(SCORCH_HIP_EINVAL, "%s: negative size (K=%lld N=%lld)", fn, (long long)K, (long long)N);
+  if (K > INT32_MAX || N > INT32_MAX) return fail(SCORCH_HIP_EUNSUPPORTED, "%s: K and N must fit int32", fn);
+  if (K > 0 && N > 0 && !B) return fail(SCORCH_HIP_EINVAL, "%s: B is NULL", fn);
+  if (!scorch::aligned_to(B, 4)) return fail(SCORCH_HIP_EINVAL, "%s: B must be 4-byte aligned", fn);
+  int device = -1;
+  SCORCH_HIP_CHECK(hipGetDevice(&device));
+  scorch_hip_dense_plan *plan = new (std::nothrow) scorch_hip_dense_plan();
+  if (!plan) return fail(SCORCH_HIP_ERUNTIME, "%s: out of host memory", fn);
+  plan->device = device;
+  plan->K = K;
+  plan->N = N;
+  plan->B = B;
+  // (whether a product gathers the rows of B more than once is known only with its sparse operand:
+  // the layout is prepared for every shape it can pay for, and each product decides)
+  if (scorch_hip_dense_tiled_recommended(K, N, INT32_MAX, 4)) {
+    plan->tiles_bytes = scorch_hip_dense_tiled_bytes(K, N, 4);
+    hipError_t err = hipMalloc(reinterpret_cast<void **>(&plan->tiles), plan->tiles_bytes);
+    int rc = err == hipSuccess ? scorch_hip_dense_to_tiled_f32(K, N, B, plan->tiles, plan->tiles_bytes, stream)
+                               : fail(SCORCH_HIP_ERUNTIME, "%s: hipMalloc of %zu bytes failed: %s", fn,
+                                      plan->tiles_bytes, hipGetErrorString(err));
+    if (rc) {
+      if (plan->tiles) (void)hipFree(plan->tiles);
+      delete plan;
+      return rc;
+    }
+  }
+  *out = plan;
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_dense_plan_update(scorch_hip_dense_plan *plan, void *stream) {
+  if (!plan) return fail(SCORCH_HIP_EINVAL, "scorch_hip_dense_plan_update: plan is NULL");
+  if (!plan->tiles) return SCORCH_HIP_OK;
+  return scorch_hip_dense_to_tiled_f32(plan->K, plan->N, plan->B, plan->tiles, plan->tiles_bytes, stream);
+}
+
+int scorch_hip_dense_plan_destroy(scorch_hip_dense_plan *plan) {
+  if (!plan) return SCORCH_HIP_OK;
+  hipError_t err = hipSuccess;
+  if (plan->tiles) {
+    int current = -1;
+    err = hipGetDevice(&current);
+    if (err == hipSuccess && current != plan->device) err = hipSetDevice(plan->device);
+    if (err == hipSuccess) err = hipDeviceSynchronize();  // products that read the tiles may be in flight
+    (void)hipFree(plan->tiles);
+    if (current >= 0 && current != plan->device) (void)hipSetDevice(current);
+  }
+  delete plan;
+  if (err != hipSuccess)
+    return fail(SCORCH_HIP_ERUNTIME, "scorch_hip_dense_plan_destroy: %s", hipGetErrorString(err));
+  return SCORCH_HIP_OK;
+}
+
+int scorch_hip_spmm_csr_plan_dense_f32(scorch_hip_csr_plan *plan, const float *vals, const scorch_hip_dense_plan *dense,
+                                       const float *bias, int act, float *C, void *stream) {
+  const char *fn = "scorch_hip_spmm_csr_plan_dense_f32";
+  if (int rc = check_plan(fn, plan)) return rc;
+  if (!dense) return fail(SCORCH_HIP_EINVAL, "%s: the dense plan is NULL", fn);
+  if (dense->device != plan->device || dense->K != plan->n_cols)
+    return fail(SCORCH_HIP_EINVAL, "%s: the dense plan is %lld x %lld on device %d, the sparse one %lld x %lld on %d",
+                fn, (long long)dense->K, (long long)dense->N, dense->device, (long long)plan->M,
+                (long long)plan->n_cols, plan->device);
+  const int64_t N = dense->N;
+  if (!dense->tiles || plan->M == 0 || !scorch_hip_dense_tiled_recommended(dense->K, N, plan->nnz, 4))
+    return scorch_hip_spmm_csr_plan_f32(plan, N, vals, dense->B, bias, act, C, stream);
+  Boundaries *bounds = nullptr;
+  if (int rc = prepare_spmm(plan, N, static_cast<hipStream_t>(stream), &bounds, true)) return rc;
+  return scorch_hip_spmm_csr_tiled_f32(plan->M, plan->n_cols, N, plan->nnz, plan->row_ptr, plan->col_idx, vals,
+                                       dense->tiles, dense->tiles_bytes, bias, act, C, bounds ? bounds->data : nullptr,
+                                       bounds ? bounds->bytes : 0, plan->workspace, plan->workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -39,6 +39,10 @@ SIGNATURES = {
     "scorch_hip_spmm_csr_plan_f32": (ctypes.c_int, [_ptr, _i64, _ptr, _ptr, _ptr, ctypes.c_int, _ptr, _ptr]),
     "scorch_hip_sddmm_csr_plan_f32": (ctypes.c_int, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "scorch_hip_softmax_csr_plan_f32": (ctypes.c_int, [_ptr, _ptr, ctypes.c_float, _ptr, _ptr]),
+    "scorch_hip_dense_plan_create": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, ctypes.POINTER(_ptr)]),
+    "scorch_hip_dense_plan_update": (ctypes.c_int, [_ptr, _ptr]),
+    "scorch_hip_dense_plan_destroy": (ctypes.c_int, [_ptr]),
+    "scorch_hip_spmm_csr_plan_dense_f32": (ctypes.c_int, [_ptr, _ptr, _ptr, _ptr, ctypes.c_int, _ptr, _ptr]),
     "scorch_hip_timing_begin": (ctypes.c_int, []),
     "scorch_hip_timing_end": (ctypes.c_int, [ctypes.POINTER(ctypes.c_float), ctypes.c_int,
                                              ctypes.POINTER(ctypes.c_int)]),

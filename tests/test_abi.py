@@ -239,6 +239,13 @@ def test_plan_handle_rejects_bad_arguments_on_the_host(L):
     assert L.scorch_hip_sddmm_csr_plan_f32(None, 8, None, at, at, at, None, None) == native.EINVAL
     assert L.scorch_hip_softmax_csr_plan_f32(None, at, 1.0, at, None) == native.EINVAL
     assert L.scorch_hip_csr_plan_destroy(None) == native.OK
+    assert L.scorch_hip_dense_plan_create(4, 4, at, None, None) == native.EINVAL
+    assert L.scorch_hip_dense_plan_create(-1, 4, at, None, ref) == native.EINVAL
+    assert L.scorch_hip_dense_plan_create(4, 4, NULL, None, ref) == native.EINVAL
+    assert handle.value is None
+    assert L.scorch_hip_dense_plan_update(None, None) == native.EINVAL
+    assert L.scorch_hip_dense_plan_destroy(None) == native.OK
+    assert L.scorch_hip_spmm_csr_plan_dense_f32(None, at, None, None, 0, at, None) == native.EINVAL
 
 
 def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):

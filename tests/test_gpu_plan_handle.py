@@ -10,7 +10,8 @@ import torch
 from conftest import random_csr
 from gpu_util import dev, hip_sddmm_csr, hip_spmm, host
 from scorch_amd import native, workloads
-from scorch_amd.csr_plan import PLAN_SDDMM_F32, PLAN_SOFTMAX_F32, PLAN_SPMM_F32, CsrPlanHandle
+from scorch_amd.csr_plan import (PLAN_SDDMM_F32, PLAN_SOFTMAX_F32, PLAN_SPMM_DENSE_F32, PLAN_SPMM_F32, CsrPlanHandle,
+                                 DensePlanHandle)
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-5
@@ -236,3 +237,50 @@ def test_prepared_products_replay_from_a_graph(oracle):
             assert oracle.rel_fro(host(out), want) <= TOL, replay
             assert np.array_equal(host(out), eager * np.float32(2.0 ** (replay + 1))), replay
         del graph
+
+
+def test_a_reused_dense_operand_through_its_plan(oracle):
+    """The decoder shape in small: B with rows of 2 KiB, gathered several times over.  Through the
+    two plans the product takes the column-tile copy; it equals the Python layer's tiled path bit
+    for bit, follows B's values only after update(), and replays from a graph."""
+    rng = np.random.default_rng(8)
+    M, K, N = 1500, 2048, 512
+    rp, ci, v = random_csr(rng, M, K, 0.02)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    bias = rng.uniform(-1, 1, N).astype(np.float32)
+    d_v, d_B, d_bias = dev(v), dev(B), dev(bias)
+    with CsrPlanHandle(dev(rp), dev(ci), K) as plan, DensePlanHandle(d_B) as dense:
+        plan.prepare(PLAN_SPMM_DENSE_F32, N)
+        assert plan.info()["device_bytes"] > 0
+        got = host(plan.spmm_dense(d_v, dense))
+        assert oracle.rel_fro(got, oracle.spmm_fp64(rp, ci, v, B)) <= TOL
+        assert np.array_equal(got, hip_spmm(rp, ci, v, B, path="tiled"))
+        with_relu = host(plan.spmm_dense(d_v, dense, d_bias, relu=True))
+        assert np.array_equal(with_relu, hip_spmm(rp, ci, v, B, bias=bias, relu=True, path="tiled"))
+        np.testing.assert_allclose(got, host(plan.spmm(d_v, d_B)), rtol=1e-4, atol=1e-5)
+        # new values in B: the plan's copy is the caller's to refresh
+        d_B.mul_(2.0)
+        assert np.array_equal(host(plan.spmm_dense(d_v, dense)), got)
+        dense.update()
+        assert np.array_equal(host(plan.spmm_dense(d_v, dense)), got * np.float32(2))
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = plan.spmm_dense(d_v, dense)
+        for replay in range(3):
+            d_v.mul_(0.5)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert np.array_equal(host(out), got * np.float32(2.0 * 0.5 ** (replay + 1))), replay
+        del graph
+    # a shape the tile layout does not pay for: the same call is the ordinary planned product
+    B2 = rng.uniform(-1, 1, (K, 48)).astype(np.float32)
+    with CsrPlanHandle(dev(rp), dev(ci), K) as plan, DensePlanHandle(dev(B2)) as dense:
+        assert np.array_equal(host(plan.spmm_dense(d_v, dense)), host(plan.spmm(d_v, dense.B)))
+    L = native.lib()
+    assert L.scorch_hip_dense_plan_destroy(None) == native.OK
+    assert L.scorch_hip_dense_plan_update(None, None) == native.EINVAL
+    with CsrPlanHandle(dev(rp), dev(ci), K) as plan, DensePlanHandle(torch.ones(K + 1, 8, device="cuda")) as dense:
+        with pytest.raises(native.ScorchHipError):
+            plan.spmm_dense(d_v, dense)                      # K does not match
