@@ -98,5 +98,30 @@ def build_library(force: bool = False, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+HOST_DEMO_SRC = os.path.join(os.path.dirname(PKG_DIR), "tests", "host_c", "plan_demo.c")
+HOST_DEMO_BIN = os.path.join(os.path.dirname(PKG_DIR), "tests", "host_c", "plan_demo")
+
+
+def build_host_demo(verbose: bool = False) -> str:
+    """Compile tests/host_c/plan_demo.c, a plain C99 host of the library (the C ABI and the HIP
+    runtime, nothing else), with gcc.  Returns the program's path.  Needs no GPU to build."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    gcc = shutil.which("gcc")
+    if not gcc:
+        raise RuntimeError("gcc not found: cannot build the C host demo")
+    cmd = [gcc, "-std=c99", "-Wall", "-Werror", "-O1", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(os.path.dirname(PKG_DIR), "include"), "-I", os.path.join(rocm, "include"),
+           HOST_DEMO_SRC, "-L", PKG_DIR, "-l:libscorch_hip.so", "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/../../scorch_amd", "-Wl,-rpath," + os.path.join(rocm, "lib"), "-o", HOST_DEMO_BIN + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("gcc failed:\n" + proc.stdout)
+    os.replace(HOST_DEMO_BIN + ".tmp", HOST_DEMO_BIN)
+    return HOST_DEMO_BIN
+
+
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv, verbose=True))
+    print(build_host_demo(verbose=True))

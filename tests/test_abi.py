@@ -276,3 +276,13 @@ def test_header_is_plain_c_and_a_c_host_can_link(tmp_path):
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert int(out[0]) == native.lib().scorch_hip_abi_version()
     assert int(out[1]) == native.lib().scorch_hip_spmm_csr_workspace_bytes(1000, 5000, 64, 4)
+
+
+def test_the_c_host_demo_builds(tmp_path):
+    """The C99 host program of tests/host_c compiles and links against the library with gcc
+    (it runs in the GPU tests)."""
+    import shutil
+    from scorch_amd import build
+    if not shutil.which("gcc") or not os.path.exists("/opt/rocm/include/hip/hip_runtime_api.h"):
+        pytest.skip("no gcc or no HIP headers")
+    assert os.path.exists(build.build_host_demo())

@@ -284,3 +284,18 @@ def test_a_reused_dense_operand_through_its_plan(oracle):
     with CsrPlanHandle(dev(rp), dev(ci), K) as plan, DensePlanHandle(torch.ones(K + 1, 8, device="cuda")) as dense:
         with pytest.raises(native.ScorchHipError):
             plan.spmm_dense(d_v, dense)                      # K does not match
+
+
+def test_a_c_host_of_the_library():
+    """tests/host_c/plan_demo.c, built by scorch_amd.build.build_host_demo: a C99 program with the
+    C ABI and the HIP runtime and nothing else does the stateless SpMM, the planned SpMM, SDDMM and
+    softmax, checks them against its own loops in double, and sees a malformed index refused."""
+    import os
+    import subprocess
+    from scorch_amd import build
+    if not os.path.exists(build.HOST_DEMO_BIN):
+        pytest.skip("tests/host_c/plan_demo is not built (python -m scorch_amd.build)")
+    proc = subprocess.run([build.HOST_DEMO_BIN], capture_output=True, text=True, timeout=100)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert proc.stdout.strip().endswith("ok"), proc.stdout
+    assert "bit-identical: 1" in proc.stdout
