@@ -205,13 +205,19 @@ SCORCH_HIP_API int scorch_hip_softmax_csr_short_rows_f32(int64_t batch, int64_t 
  * workgroup takes two items, the k-th longest and then the k-th shortest of the list, so that all
  * workgroups carry about the same work and half as many start: it pays where the items differ in
  * length (or are very short) and the launch is about one to four times what the chip holds at
- * once, and costs a few per cent elsewhere; same results bit for bit.  No counterpart in the
+ * once, and costs a few per cent elsewhere; same results bit for bit.  With priority_step > 0 a
+ * wavefront's priority on its SIMD follows the key blocks its workgroup has left to do (this item's
+ * and, before the second item of a pair, that item's), in four levels of priority_step blocks: the
+ * wavefronts that were dispatched first win a SIMD's arbitration otherwise, two of a CU's four
+ * workgroups finish a quarter of the launch ahead of the other two and the CU runs half empty from
+ * there on.  It pays where a CU holds two workgroups or more at a time; a quarter of the most any
+ * workgroup has to do is the step to give.  Same results bit for bit.  No counterpart in the
  * reference, like the two entry points above. */
 SCORCH_HIP_API size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, int64_t n_slots, int64_t D);
 SCORCH_HIP_API int scorch_hip_attn_blocksparse_split_bf16(
     int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
-    const int32_t *items, int pair_items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
-    const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
+    const int32_t *items, int pair_items, int priority_step, int64_t n_split_rows, const int32_t *split_rows,
+    int64_t n_slots, const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
     const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
     void *workspace, size_t workspace_bytes, void *stream);
 

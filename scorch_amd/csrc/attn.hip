@@ -105,7 +105,7 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     const unsigned long long *__restrict__ block_masks, const __bf16 *__restrict__ Q,
     const __bf16 *__restrict__ K, const __bf16 *__restrict__ V, float scale_log2e,
     __bf16 *__restrict__ O, int n_items, const int4 *__restrict__ items, int n_slots,
-    float *__restrict__ partials, int pairs) {
+    float *__restrict__ partials, int pairs, int prio_step) {
   using Tile = AttnTile<D>;
   constexpr int kTileBytes = Tile::kBytes;
   constexpr int kRowBytes = Tile::kRowBytes;
@@ -162,6 +162,22 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
     qb = n_blocks - 1 - item_rank;  // (masks with longer block rows further down: longest first)
     kb_begin = block_row_ptr[qb];
     kb_end = block_row_ptr[qb + 1];
+  }
+  // prio_step > 0: a wavefront's priority on its SIMD follows what its workgroup has left to do
+  // (this item's remaining key blocks and, in the first pass of a pair, the second item's), in four
+  // levels of prio_step blocks.  The wavefronts that were dispatched first win the SIMD's
+  // arbitration otherwise: of the four workgroups of a CU two then finish a quarter of the launch
+  // ahead of the other two, and the CU runs half empty from there on.
+  int later_blocks = 0;
+  if (prio_step > 0 && pairs && pass == 0 && n_items - 1 - rank > rank) {
+    const int second = uniform(n_items - 1 - rank);
+    if (items) {
+      const int *words = reinterpret_cast<const int *>(items) + 4 * (size_t)second;  // (scalar loads)
+      later_blocks = words[2] - words[1];
+    } else {
+      const int qb2 = n_blocks - 1 - second;
+      later_blocks = block_row_ptr[qb2 + 1] - block_row_ptr[qb2];
+    }
   }
   const size_t head_off = (size_t)head * (size_t)S * D;
   const __bf16 *Qh = Q + head_off;
@@ -345,6 +361,13 @@ __attribute__((amdgpu_waves_per_eu(AttnTile<D>::kWavesPerSimd))) void attn_block
   };
 
   for (int it = kb_begin; it < kb_end; it += 2) {
+    if (prio_step > 0) {
+      const int left = kb_end - it + later_blocks;  // (all of it in scalar registers)
+      if (left >= 3 * prio_step) __builtin_amdgcn_s_setprio(3);
+      else if (left >= 2 * prio_step) __builtin_amdgcn_s_setprio(2);
+      else if (left >= prio_step) __builtin_amdgcn_s_setprio(1);
+      else __builtin_amdgcn_s_setprio(0);
+    }
     key_block(Even{}, it);
     if (it + 1 < kb_end) key_block(Odd{}, it + 1);
   }
@@ -425,11 +448,12 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
                             const int32_t *block_row_ptr, const int32_t *block_col_idx,
                             const int32_t *block_mask_index, const unsigned long long *block_masks,
                             const __bf16 *q, const __bf16 *k, const __bf16 *v, float scale_log2e,
-                            __bf16 *o, int n_items, const int4 *items, int n_slots, float *partials, int pairs) {
+                            __bf16 *o, int n_items, const int4 *items, int n_slots, float *partials, int pairs,
+                            int prio_step) {
 #define SCORCH_ATTN_LAUNCH(NEG, MASKED)                                                          \
   attn_blocksparse_kernel<D, NEG, MASKED><<<grid, kBlockThreads, 0, s>>>(                        \
       S, n_blocks, H, block_row_ptr, block_col_idx, block_mask_index, block_masks, q, k, v,      \
-      scale_log2e, o, n_items, items, n_slots, partials, pairs)
+      scale_log2e, o, n_items, items, n_slots, partials, pairs, prio_step)
   const bool masked = block_mask_index != nullptr;
   if (negative) {
     if (masked) SCORCH_ATTN_LAUNCH(true, true); else SCORCH_ATTN_LAUNCH(true, false);
@@ -443,6 +467,7 @@ static void attn_launch_dim(dim3 grid, hipStream_t s, bool negative, int S, int 
 struct AttnSplit {
   int64_t n_items = 0, n_split_rows = 0, n_slots = 0;
   bool pair_items = false;              // a workgroup takes the k-th longest and then the k-th shortest item
+  int prio_step = 0;                    // > 0: wavefront priority by the blocks a workgroup has left, in levels of this many
   const int32_t *items = nullptr;       // 4 per item: block row, begin, end, slot (-1: writes O itself)
   const int32_t *split_rows = nullptr;  // 4 per split row: block row, first slot, stretches, 0
   void *workspace = nullptr;
@@ -501,6 +526,7 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
   }
   // pairs: every workgroup takes two items, see the kernel (asked for through the work-list entry)
   const int pairs = split && split->pair_items && n_items >= 2;
+  const int prio_step = split ? split->prio_step : 0;
   const dim3 grid((unsigned)((pairs ? (n_items + 1) / 2 : n_items) * H));
   const float scale_log2e = scale * 1.4426950408889634f;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -511,13 +537,13 @@ static int attn_entry(const char *fn, int64_t H, int64_t S, int64_t D, int64_t b
   mark_launch(s);
   if (D == 32)
     attn_launch_dim<32>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs, prio_step);
   else if (D == 64)
     attn_launch_dim<64>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
+                        block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs, prio_step);
   else
     attn_launch_dim<128>(grid, s, scale < 0.0f, (int)S, n_blocks, (int)H, block_row_ptr, block_col_idx,
-                         block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs);
+                         block_mask_index, masks, q, k, v, scale_log2e, o, n_items, items, n_slots, partials, pairs, prio_step);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
   if (split && split->n_split_rows > 0) {
@@ -570,13 +596,14 @@ extern "C" size_t scorch_hip_attn_blocksparse_split_workspace_bytes(int64_t H, i
 
 extern "C" int scorch_hip_attn_blocksparse_split_bf16(
     int64_t H, int64_t S, int64_t D, int64_t block, int64_t n_active_blocks, int64_t n_items,
-    const int32_t *items, int pair_items, int64_t n_split_rows, const int32_t *split_rows, int64_t n_slots,
-    const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
+    const int32_t *items, int pair_items, int priority_step, int64_t n_split_rows, const int32_t *split_rows,
+    int64_t n_slots, const int32_t *block_col_idx, const int32_t *block_mask_index, int64_t n_masks,
     const uint64_t *block_masks, const void *Q, const void *K, const void *V, float scale, void *O,
     void *workspace, size_t workspace_bytes, void *stream) {
   using namespace scorch;
   const char *fn = "scorch_hip_attn_blocksparse_split_bf16";
   if (n_masks < 0) return fail(SCORCH_HIP_EINVAL, "%s: n_masks=%lld", fn, (long long)n_masks);
+  if (priority_step < 0) return fail(SCORCH_HIP_EINVAL, "%s: priority_step=%d", fn, priority_step);
   if (block_mask_index != nullptr) {
     SCORCH_REQUIRE(n_masks == 0 || block_masks != nullptr, "%s: block_masks is NULL", fn);
     SCORCH_REQUIRE(aligned_to(block_masks, 8), "%s: block_masks must be 8-byte aligned", fn);
@@ -584,6 +611,7 @@ extern "C" int scorch_hip_attn_blocksparse_split_bf16(
   AttnSplit split;
   split.n_items = n_items;
   split.pair_items = pair_items != 0;
+  split.prio_step = priority_step;
   split.n_split_rows = n_split_rows;
   split.n_slots = n_slots;
   split.items = items;

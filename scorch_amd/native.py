@@ -110,7 +110,7 @@ SIGNATURES = {
                                                                _ptr, _ptr, _ptr, _ptr, ctypes.c_float, _ptr,
                                                                _ptr]),
     "scorch_hip_attn_blocksparse_split_workspace_bytes": (_size, [_i64, _i64, _i64]),
-    "scorch_hip_attn_blocksparse_split_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, ctypes.c_int, _i64, _ptr, _i64,
+    "scorch_hip_attn_blocksparse_split_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _i64, _ptr, ctypes.c_int, ctypes.c_int, _i64, _ptr, _i64,
                                                               _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, ctypes.c_float,
                                                               _ptr, _ptr, _size, _ptr]),
     "scorch_hip_attn_blocksparse_f32_workspace_bytes": (_size, [_i64, _i64, _i64]),

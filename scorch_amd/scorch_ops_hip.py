@@ -1317,7 +1317,7 @@ class BlockMask:
         self.n_slots = 0
         self.schedule32 = None      # the fp32 kernel's own sharing-out (see _fp32_schedule)
         self.block_row_lens = None  # active blocks per block row, on the host (numpy), once it has been read
-        self.pairing = {}           # (item list, heads, head dimension) -> whether workgroups take two items
+        self.pairing = {}           # (item list, heads, head dimension) -> (workgroups take two items?, priority step)
 
     def row_lens(self):
         """Active blocks per block row as a numpy array on the host (read from the device once)."""
@@ -1410,6 +1410,35 @@ def pair_attention_items(lens, heads: int, D: int, n_cus: int = 256) -> bool:
     mean = float(lens.mean())
     uneven = float(lens.max()) > 1.25 * mean
     return 0.6 <= rounds <= 4.0 and mean <= 64 and (uneven or mean <= 6)
+
+
+def attention_priority_step(lens, heads: int, D: int, pair: bool, n_cus: int = 256) -> int:
+    """The priority_step to hand scorch_hip_attn_blocksparse_split_bf16 for work items of `lens` key
+    blocks (0: leave the wavefronts' priorities alone).  With a step a wavefront's priority follows
+    what its workgroup has left to do, in four levels: a quarter of the most any workgroup gets.
+    It pays where a CU holds two workgroups or more at a time and the launch is short of four
+    times what the chip holds at once (measured at S = 8192, 16 heads, D = 64, on top of the
+    pairing decision: the benchmark's causal strided mask -4 to -5 %, four, twelve and twenty
+    blocks in every row -3 %, a dense mask -3 %; causal masks at S = 4096 0 to -2 %) and is left
+    out elsewhere (a causal mask with 4 heads, one workgroup per CU: +4 %; 64 heads with four
+    blocks in every row, eight rounds: +3 %; S = 16,384 with D = 128, four rounds: +1 %)."""
+    import numpy as np
+    lens = np.asarray(lens)
+    if lens.size == 0 or D not in ATTENTION_WORKGROUPS_PER_CU:
+        return 0
+    workgroups = ((lens.size + 1) // 2 if pair else lens.size) * heads
+    if workgroups < 2 * n_cus or workgroups >= 4 * n_cus * ATTENTION_WORKGROUPS_PER_CU[D]:
+        return 0            # one workgroup per CU: nothing to arbitrate; four rounds and more: nothing measurable
+    if pair:
+        ordered = np.sort(lens)[::-1]
+        half = (lens.size + 1) // 2
+        second = ordered[::-1][:half].copy()
+        if lens.size % 2:
+            second[-1] = 0                      # the middle item has no partner
+        most = int((ordered[:half] + second).max())
+    else:
+        most = int(lens.max())
+    return max(1, -(-most // 4))
 
 
 def split_long_block_rows(bm: BlockMask, longest: Optional[int] = None, list_unequal_rows: bool = False) -> BlockMask:
@@ -1554,7 +1583,7 @@ def _attn_bf16_args(q, k, v):
 
 
 def _attn_bf16_items(q, k, v, bm: BlockMask, items: torch.Tensor, split_rows: Optional[torch.Tensor], n_slots: int,
-                     scale: float, pair: bool) -> torch.Tensor:
+                     scale: float, pair: bool, priority_step: int = 0) -> torch.Tensor:
     """The fused bf16 kernel over a list of work items (scorch_hip_attn_blocksparse_split_bf16)."""
     tensors = [t for t in (bm.block_col_idx, bm.block_mask_index, bm.block_masks, items) if t is not None]
     dev = _device_of(q, k, v, *tensors)
@@ -1569,7 +1598,7 @@ def _attn_bf16_items(q, k, v, bm: BlockMask, items: torch.Tensor, split_rows: Op
         need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(H, n_slots, D)
         ws = _workspace(dev, stream, need) if need else None
         rc = L.scorch_hip_attn_blocksparse_split_bf16(
-            H, S, D, bm.block, bm.n_active_blocks, items.numel() // 4, items.data_ptr(), int(pair),
+            H, S, D, bm.block, bm.n_active_blocks, items.numel() // 4, items.data_ptr(), int(pair), int(priority_step),
             split_rows.numel() // 4 if split_rows is not None else 0, ptr(split_rows), n_slots,
             ptr(bm.block_col_idx), ptr(bm.block_mask_index) if bm.block_mask_index is not None else None,
             bm.n_masks if bm.block_masks is not None else 0, ptr(bm.block_masks), q.data_ptr(), k.data_ptr(),
@@ -1581,11 +1610,24 @@ def _attn_bf16_items(q, k, v, bm: BlockMask, items: torch.Tensor, split_rows: Op
     return out
 
 
-def _pairing(bm: BlockMask, kind: str, lens, heads: int, D: int, device) -> bool:
-    """pair_attention_items for one of the BlockMask's item lists, remembered per (list, heads, D)."""
+# For measurements: SCORCH_HIP_ATTN_PAIRING=0 / SCORCH_HIP_ATTN_PRIORITY=0 keep one work item per
+# workgroup / leave the wavefronts' priorities alone whatever the mask looks like.
+ATTENTION_PAIRING = os.environ.get("SCORCH_HIP_ATTN_PAIRING", "1") not in ("", "0")
+ATTENTION_PRIORITY = os.environ.get("SCORCH_HIP_ATTN_PRIORITY", "1") not in ("", "0")
+
+
+def _launch_plan(lens, heads: int, D: int, device):
+    """(pair the items?, priority step) for a list of work items of `lens` key blocks."""
+    n_cus = _cu_count(device)
+    pair = pair_attention_items(lens, heads, D, n_cus) if ATTENTION_PAIRING else False
+    return pair, attention_priority_step(lens, heads, D, pair, n_cus) if ATTENTION_PRIORITY else 0
+
+
+def _pairing(bm: BlockMask, kind: str, lens, heads: int, D: int, device):
+    """_launch_plan for one of the BlockMask's item lists, remembered per (list, heads, D)."""
     key = (kind, int(heads), int(D))
     if key not in bm.pairing:
-        bm.pairing[key] = pair_attention_items(lens, heads, D, _cu_count(device))
+        bm.pairing[key] = _launch_plan(lens, int(heads), int(D), device)
     return bm.pairing[key]
 
 
@@ -1600,13 +1642,13 @@ def attn_blocksparse_split_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     key = ("items", int(q.shape[0]), int(q.shape[2]))
     if key not in bm.pairing:
         if q.is_cuda and torch.cuda.is_current_stream_capturing():
-            bm_pair = False                       # (deciding needs a host read of the items)
+            plan = (False, 0)                     # (deciding needs a host read of the items)
         else:
             rows = bm.items.view(-1, 4)
-            bm_pair = _pairing(bm, "items", (rows[:, 2] - rows[:, 1]).cpu().numpy(), q.shape[0], q.shape[2], q.device)
+            plan = _pairing(bm, "items", (rows[:, 2] - rows[:, 1]).cpu().numpy(), q.shape[0], q.shape[2], q.device)
     else:
-        bm_pair = bm.pairing[key]
-    return _attn_bf16_items(q, k, v, bm, bm.items, bm.split_rows, bm.n_slots, scale, bm_pair)
+        plan = bm.pairing[key]
+    return _attn_bf16_items(q, k, v, bm, bm.items, bm.split_rows, bm.n_slots, scale, plan[0], plan[1])
 
 
 def _block_row_schedule(brp: torch.Tensor):
@@ -1639,8 +1681,9 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
     per-head SDDMM -> softmax -> SpMM pipeline of
     bench/bench_sparse_transformer.py:354-372.  With block_mask_index (int32 per active block, -1
     = fully live) and block_masks (int64, 64 words per mask) a block is restricted to the entries
-    its bit mask names.  Where it pays (pair_attention_items) the block rows go to the kernel as a
-    list of work items of which every workgroup takes two; the result is the same bit for bit."""
+    its bit mask names.  Where it pays (pair_attention_items, attention_priority_step) the block rows
+    go to the kernel as a list of work items, of which every workgroup takes two and / or whose
+    wavefronts' priorities follow the work they have left; the result is the same bit for bit."""
     q, k, v = _attn_bf16_args(q, k, v)
     brp, bci = _index(block_row_ptr, "block_row_ptr"), _index(block_col_idx, "block_col_idx")
     dev = _device_of(q, k, v, brp, bci)
@@ -1671,10 +1714,11 @@ def attn_blocksparse_bf16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, blo
         lens, items, pairing = schedule
         key = (int(H), int(D))
         if key not in pairing:
-            pairing[key] = pair_attention_items(lens, int(H), int(D), _cu_count(dev))
-        if pairing[key]:
+            pairing[key] = _launch_plan(lens, int(H), int(D), dev)
+        pair, priority_step = pairing[key]
+        if pair or priority_step:
             rows = BlockMask(int(S), block, brp, bci, bmi, block_masks if bmi is not None else None, 0)
-            return _attn_bf16_items(q, k, v, rows, items, None, 0, scale, True)
+            return _attn_bf16_items(q, k, v, rows, items, None, 0, scale, pair, priority_step)
     out = _empty_like(q)
     with _on_device(dev):
         if bmi is None:

@@ -205,8 +205,8 @@ def test_attention_rejects_unsupported_shapes(L):
     need = L.scorch_hip_attn_blocksparse_split_workspace_bytes(2, 3, 32)
     assert need == 2 * 3 * 64 * 36 * 4 and L.scorch_hip_attn_blocksparse_split_workspace_bytes(2, 0, 32) == 0
 
-    def split(D=32, n_items=5, items=FAKE, n_split=1, rows=FAKE, n_slots=3, ws=FAKE, ws_bytes=need, q=FAKE):
-        return h(2, 128, D, 64, 4, n_items, items, 0, n_split, rows, n_slots, FAKE, NULL, 0, NULL, q, FAKE, FAKE,
+    def split(D=32, n_items=5, items=FAKE, n_split=1, rows=FAKE, n_slots=3, ws=FAKE, ws_bytes=need, q=FAKE, prio=0):
+        return h(2, 128, D, 64, 4, n_items, items, 0, prio, n_split, rows, n_slots, FAKE, NULL, 0, NULL, q, FAKE, FAKE,
                  0.125, FAKE, ws, ws_bytes, NULL)
 
     assert split(D=48) == native.EUNSUPPORTED
@@ -216,6 +216,7 @@ def test_attention_rejects_unsupported_shapes(L):
     assert split(ws=NULL) == native.EWORKSPACE
     assert split(ws_bytes=need - 1) == native.EWORKSPACE
     assert split(n_items=-1) == native.EINVAL
+    assert split(prio=-1) == native.EINVAL
     assert split(q=NULL) == native.EINVAL
     assert split(n_items=0, items=NULL) == native.OK
 

@@ -352,6 +352,10 @@ def test_workgroups_that_take_two_items_change_nothing(oracle, D, kind):
         single = H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, False)
         paired = H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, True)
         assert torch.equal(single, paired)
+        # wavefront priorities by the work a workgroup has left: they order the work, not the sums
+        for step in (1, 3, 1000):
+            assert torch.equal(single, H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, False, step))
+            assert torch.equal(single, H._attn_bf16_items(q, k, v, bm, t_items, t_rows, n_slots, D ** -0.5, True, step))
         if longest is None:
             whole = single
     plain = H.attn_blocksparse_bf16(q, k, v, bm.block_row_ptr, bm.block_col_idx, D ** -0.5,
@@ -372,7 +376,8 @@ def test_the_dispatch_pairs_items_where_it_was_measured_to_pay():
     for heads, expect in ((16, True), (4, False)):
         q, k, v = (torch.randn(heads, 64 * nb, 64, device="cuda").to(torch.bfloat16) for _ in range(3))
         out = H.attn_blocksparse_bf16(q, k, v, t_brp, t_bci, 0.125)
-        assert t_brp._scorch_rows[3][(heads, 64)] is expect
+        assert t_brp._scorch_rows[3][(heads, 64)][0] is expect
+        assert (t_brp._scorch_rows[3][(heads, 64)][1] > 0) is expect     # 8 pairs per CU / one workgroup per CU
         rc_out = torch.empty_like(q)
         from scorch_amd import native
         native.check(native.lib().scorch_hip_attn_blocksparse_bf16(

@@ -560,3 +560,12 @@ def test_when_attention_workgroups_take_two_items():
     assert not pair(causal(256), 8, 128)                       # rows of 128 blocks on average
     assert not pair(np.full(nb, nb), 16, 64)                   # dense
     assert not pair(np.array([5]), 16, 64) and not pair(c4, 16, 48)
+    # the priority step: a quarter of the most a workgroup gets, where a CU holds two workgroups or more
+    step = scorch_ops_hip.attention_priority_step
+    assert step(c4, 16, 64, True) == 6 and step(c4, 16, 64, False) == 5        # pairs of 23 blocks; rows of 19
+    assert step(c4, 4, 64, False) == 5 and step(c4, 2, 64, False) == 0          # 512 and 256 workgroups on 256 CUs
+    assert step(causal(64), 16, 64, True) == 17 and step(causal(64), 4, 64, False) == 0
+    assert step(causal(63), 16, 64, True) == 16                                 # 63 + 1, ..., the middle item alone
+    assert step(np.full(nb, nb), 16, 64, False) == 32 and step(np.full(nb, 4), 64, 64, False) == 0   # eight rounds
+    assert step(causal(256), 8, 128, False) == 0                                # four rounds of two workgroups per CU
+    assert step(np.array([], np.int64), 16, 64, False) == 0 and step(c4, 16, 48, False) == 0
