@@ -62,10 +62,10 @@ MEASURED_TRAFFIC = {
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
     ("sae_decoder", "merge"): {"bytes": 1_767_900_000, "sources": _SPMM_SOURCES, "sha16": "f03cdf8f7d11457c",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
-    ("sddmm_uniform", "listed"): {"bytes": 277_100_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
-                                  "sha16": "0b80029da09f40bf", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
-    ("sddmm_uniform", "plain"): {"bytes": 848_000_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
-                                 "sha16": "0b80029da09f40bf", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("sddmm_uniform", "listed"): {"bytes": 278_000_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
+                                  "sha16": "eed3747508604c18", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
+    ("sddmm_uniform", "plain"): {"bytes": 848_200_000, "sources": (_CSRC + "sddmm.hip", _CSRC + "common.hpp"),
+                                 "sha16": "eed3747508604c18", "profile": "profiles/sddmm_kernels_uniform_65536.md"},
     ("attention_blocksparse", "fused"): {"bytes": 81_050_000, "sources": (_CSRC + "attn.hip", _CSRC + "common.hpp"),
                                          "sha16": "1c42d31b5c08e253", "profile": "profiles/attn_blocksparse_kernel_s8192_h16.md"},
 }

@@ -176,14 +176,21 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_tiled_f32(int64_t M, int64_t K, int64_t N
  * n_cols only, and a list holds its entries in the mask's order, the same on every
  * build).  scorch_hip_sddmm_csr_listed_f32 is scorch_hip_sddmm_csr_batched_f32
  * computed list by list, each list on one XCD, whose L2 then keeps that eighth of
- * B: the same products, the same results bit for bit.  K <= 256. */
+ * B: the same products, the same results bit for bit.  K <= 256.
+ * scorch_hip_sddmm_csr_list_values_f32 copies the mask's values into the lists' order
+ * (listed_vals[e] = vals[position of list entry e]); handed to the listed kernel as `listed_vals`
+ * they are read with the entries, coalesced, instead of one scattered load per entry (mask_vals is
+ * then not read).  The copy is the caller's to redo when the values change.  listed_vals may be
+ * NULL, and so may mask_vals (a mask of ones). */
 SCORCH_HIP_API size_t scorch_hip_sddmm_csr_lists_bytes(int64_t nnz);
 SCORCH_HIP_API int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
                                const int32_t *col_idx, void *lists, size_t lists_bytes, void *stream);
+SCORCH_HIP_API int scorch_hip_sddmm_csr_list_values_f32(int64_t nnz, const void *lists, size_t lists_bytes,
+                                         const float *vals, float *listed_vals /* [nnz] */, void *stream);
 SCORCH_HIP_API int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
                                     const void *lists, size_t lists_bytes, const float *mask_vals,
-                                    const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
-                                    void *stream);
+                                    const float *listed_vals, const float *A, const float *B, float *out_vals,
+                                    int32_t *out_row_idx, void *stream);
 
 /* The same for `batch` value arrays over one pattern, for a caller that knows that no row has more
  * than 4096 entries (scorch_hip_csr_inspect reports the longest row): one launch, no workspace.

@@ -291,7 +291,7 @@ int scorch_hip_sddmm_csr_plan_f32(scorch_hip_csr_plan *plan, int64_t K, const fl
   if (int rc = prepare_sddmm(plan, K, static_cast<hipStream_t>(stream))) return rc;
   if (sddmm_by_lists(plan, K))
     return scorch_hip_sddmm_csr_listed_f32(1, plan->M, plan->n_cols, K, plan->nnz, plan->lists, plan->lists_bytes,
-                                           mask_vals, A, B, out_vals, out_row_idx, stream);
+                                           mask_vals, nullptr, A, B, out_vals, out_row_idx, stream);
   return scorch_hip_sddmm_csr_f32(plan->M, plan->n_cols, K, plan->nnz, plan->row_ptr, plan->col_idx, mask_vals, A, B,
                                   out_vals, out_row_idx, stream);
 }

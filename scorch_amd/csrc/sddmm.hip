@@ -308,9 +308,9 @@ template <int GS, int VEC>
 __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
     int K, const int *__restrict__ list_ptr, const int *__restrict__ entry_pos,
     const int *__restrict__ entry_row, const int *__restrict__ entry_col,
-    const float *__restrict__ mask_vals, const float *__restrict__ A, const float *__restrict__ B,
-    float *__restrict__ out_vals, int *__restrict__ out_row_idx, int64_t nnz, int64_t batch_stride_a,
-    int64_t batch_stride_b) {
+    const float *__restrict__ mask_vals, const float *__restrict__ listed_vals, const float *__restrict__ A,
+    const float *__restrict__ B, float *__restrict__ out_vals, int *__restrict__ out_row_idx, int64_t nnz,
+    int64_t batch_stride_a, int64_t batch_stride_b) {
   using VecT = Vec<float, VEC>;
   if (blockIdx.y > 0) {  // problem blockIdx.y of a batch over one mask
     A += blockIdx.y * batch_stride_a;
@@ -341,8 +341,13 @@ __global__ __launch_bounds__(kBlockThreads) void sddmm_listed_kernel(
       cols_of[b] = valid ? entry_col[e] : 0;
     }
 #pragma unroll
-    for (int b = 0; b < kBatches; ++b)  // (no value array: every stored entry is 1)
-      scale_of[b] = pos_of[b] >= 0 ? (mask_vals ? mask_vals[pos_of[b]] : 1.0f) : 0.0f;
+    for (int b = 0; b < kBatches; ++b) {
+      // the mask's values: in list order if the caller keeps such a copy (read with the entries,
+      // coalesced), else from their places in the mask (one scattered load per entry); no value
+      // array at all: every stored entry is 1
+      const int64_t e = first + b * kWaveSize + lane;
+      scale_of[b] = pos_of[b] < 0 ? 0.0f : listed_vals ? listed_vals[e] : mask_vals ? mask_vals[pos_of[b]] : 1.0f;
+    }
 #pragma unroll
     for (int b = 0; b < kBatches; ++b) {
       if (first + b * kWaveSize >= last) break;
@@ -490,6 +495,15 @@ inline SddmmLists sddmm_lists(void *buffer, int64_t nnz) {
   return l;
 }
 
+// listed_vals[e] = vals[entry_pos[e]]: the mask's values in the order of the lists.
+__global__ __launch_bounds__(kBlockThreads) void sddmm_list_values_kernel(int64_t nnz, const int *__restrict__ entry_pos,
+                                                                           const float *__restrict__ vals,
+                                                                           float *__restrict__ listed_vals) {
+  const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+  for (int64_t e = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; e < nnz; e += stride)
+    listed_vals[e] = vals[entry_pos[e]];
+}
+
 __global__ void sddmm_lists_clear_kernel(int *list_ptr) {
   if (threadIdx.x <= kBuckets) list_ptr[threadIdx.x] = 0;
 }
@@ -567,10 +581,31 @@ int scorch_hip_sddmm_csr_lists(int64_t M, int64_t n_cols, int64_t nnz, const int
   return SCORCH_HIP_OK;
 }
 
+int scorch_hip_sddmm_csr_list_values_f32(int64_t nnz, const void *lists, size_t lists_bytes, const float *vals,
+                                         float *listed_vals, void *stream) {
+  const char *fn = "scorch_hip_sddmm_csr_list_values_f32";
+  if (nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
+  if (nnz > INT32_MAX) return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: sizes must fit int32 indices", fn);
+  if (nnz == 0) return SCORCH_HIP_OK;
+  SCORCH_REQUIRE(lists && vals && listed_vals, "%s: NULL array", fn);
+  SCORCH_REQUIRE(scorch::aligned_to(lists, 256) && scorch::aligned_to(vals, 4) && scorch::aligned_to(listed_vals, 4),
+                 "%s: lists must be 256-byte aligned, the value arrays 4-byte", fn);
+  if (lists_bytes < scorch_hip_sddmm_csr_lists_bytes(nnz))
+    return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: the lists of %lld entries take %zu bytes, %zu given", fn,
+                        (long long)nnz, scorch_hip_sddmm_csr_lists_bytes(nnz), lists_bytes);
+  const scorch::SddmmLists l = scorch::sddmm_lists(const_cast<void *>(lists), nnz);
+  int64_t blocks = (nnz + scorch::kBlockThreads * 4 - 1) / (scorch::kBlockThreads * 4);
+  if (blocks > 8192) blocks = 8192;  // the kernel strides
+  scorch::sddmm_list_values_kernel<<<dim3((unsigned)blocks), scorch::kBlockThreads, 0,
+                                     static_cast<hipStream_t>(stream)>>>(nnz, l.entry_pos, vals, listed_vals);
+  SCORCH_HIP_CHECK(hipGetLastError());
+  return SCORCH_HIP_OK;
+}
+
 int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
                                     const void *lists, size_t lists_bytes, const float *mask_vals,
-                                    const float *A, const float *B, float *out_vals, int32_t *out_row_idx,
-                                    void *stream) {
+                                    const float *listed_vals, const float *A, const float *B, float *out_vals,
+                                    int32_t *out_row_idx, void *stream) {
   const char *fn = "scorch_hip_sddmm_csr_listed_f32";
   if (batch < 0 || batch > 65535)
     return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
@@ -582,7 +617,8 @@ int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, in
   if (batch == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(lists && out_vals, "%s: NULL lists or value array", fn);
   SCORCH_REQUIRE(K == 0 || (A && B), "%s: NULL dense operand", fn);
-  SCORCH_REQUIRE(scorch::aligned_to(lists, 256) && scorch::aligned_to(mask_vals, 4) && scorch::aligned_to(out_vals, 4) &&
+  SCORCH_REQUIRE(scorch::aligned_to(lists, 256) && scorch::aligned_to(mask_vals, 4) && scorch::aligned_to(listed_vals, 4) &&
+                     scorch::aligned_to(out_vals, 4) &&
                      scorch::aligned_to(A, 4) && scorch::aligned_to(B, 4) && scorch::aligned_to(out_row_idx, 4),
                  "%s: lists must be 256-byte aligned, the other arrays 4-byte", fn);
   if (lists_bytes < scorch_hip_sddmm_csr_lists_bytes(nnz))
@@ -603,7 +639,8 @@ int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int64_t n_cols, in
   scorch::mark_launch(s);
 #define SCORCH_LISTED(GS, VEC)                                                                                   \
   scorch::sddmm_listed_kernel<GS, VEC><<<grid, scorch::kBlockThreads, 0, s>>>(                                   \
-      (int)K, l.list_ptr, l.entry_pos, l.entry_row, l.entry_col, mask_vals, A, B, out_vals, out_row_idx, nnz,   \
+      (int)K, l.list_ptr, l.entry_pos, l.entry_row, l.entry_col, mask_vals, listed_vals, A, B, out_vals,        \
+      out_row_idx, nnz,                                                                                          \
       M * K, n_cols * K)
 #define SCORCH_LISTED_PICK(VEC)                          \
   do {                                                   \

@@ -93,7 +93,8 @@ SIGNATURES = {
                                                        _ptr, _size, _ptr, _size, _ptr]),
     "scorch_hip_sddmm_csr_lists_bytes": (_size, [_i64]),
     "scorch_hip_sddmm_csr_lists": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, _ptr, _size, _ptr]),
-    "scorch_hip_sddmm_csr_listed_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _size, _ptr, _ptr, _ptr,
+    "scorch_hip_sddmm_csr_list_values_f32": (ctypes.c_int, [_i64, _ptr, _size, _ptr, _ptr, _ptr]),
+    "scorch_hip_sddmm_csr_listed_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _size, _ptr, _ptr, _ptr, _ptr,
                                                        _ptr, _ptr, _ptr]),
     "scorch_hip_spmv_csr_workspace_bytes": (_size, [_i64, _i64, _size]),
     "scorch_hip_spmv_csr_f32": (ctypes.c_int, _SPMV),

@@ -164,13 +164,14 @@ class _on_device:
 # derived data as attributes of the tensors it was derived from:
 #   from index tensors   the CsrPlan (validity, longest row, chunk boundaries, entry lists, block
 #                        description), the row pointer of a coordinate mask, an attention mask's blocks
-#   from value tensors   the column-tile copy of a wide dense operand, "this mask's values are all 1"
+#   from value tensors   the column-tile copy of a wide dense operand, "this mask's values are all 1", a
+#                        mask's values in the order of its SDDMM entry lists
 # Each is stamped with the tensor's address, its version counter and its epoch (below), and rebuilt
 # when the stamp no longer matches.  PyTorch bumps the version counter for every in-place operation
 # of its own on the tensor or on a view of it.  It does not for writes through ``t.data``, a raw
 # pointer, a numpy or DLPack alias, a kernel of another library, or the replay of a recorded graph:
 # after such a write call forget(t), or mark the tensor volatile once.
-_CACHE_ATTRIBUTES = ("_scorch_plan", "_scorch_tiled", "_scorch_seen", "_scorch_ones", "_scorch_coo_pos",
+_CACHE_ATTRIBUTES = ("_scorch_plan", "_scorch_tiled", "_scorch_seen", "_scorch_ones", "_scorch_listed", "_scorch_coo_pos",
                      "_scorch_block_mask", "_scorch_mask_checked", "_scorch_rows")
 
 
@@ -244,7 +245,7 @@ def mark_volatile(*objs, volatile: bool = True) -> None:
     index tensor (a sparsity pattern) is not affected: use forget() when a pattern is rewritten."""
     for t in _tensors_of(objs):
         if volatile:
-            for name in ("_scorch_tiled", "_scorch_seen", "_scorch_ones"):
+            for name in ("_scorch_tiled", "_scorch_seen", "_scorch_ones", "_scorch_listed"):
                 if hasattr(t, name):
                     delattr(t, name)
         try:
@@ -543,6 +544,34 @@ def _mask_values_pointer(values: Optional[torch.Tensor]):
     """What an SDDMM kernel is handed for its mask's values: nothing when they are known to be all 1
     (the kernel then reads nothing for them), else the array."""
     return None if values is None or _known_all_ones(values) else values.data_ptr()
+
+
+def _listed_mask_values(values: torch.Tensor, lists: torch.Tensor, L, stream):
+    """What the listed SDDMM kernel is handed for its mask's values: (mask_vals, listed_vals)
+    pointers.  Nothing at all when the values are known to be all 1; the values in the order of the
+    lists (read with the entries, coalesced) once the same unchanged tensor has come back and has
+    been found not to be all ones -- one gather, kept with the tensor; else the array itself (one
+    scattered load per entry).  Never a copy while a stream is capturing or for a volatile tensor:
+    a recording holds pointers, and the values may be rewritten before a replay."""
+    if _known_all_ones(values):
+        return None, None
+    if torch.cuda.is_current_stream_capturing() or is_volatile(values):
+        return values.data_ptr(), None
+    key = _stamp(values)
+    cached = getattr(values, "_scorch_listed", None)
+    if cached is not None and cached[0] == key and cached[1] is lists:
+        return values.data_ptr(), cached[2].data_ptr()
+    seen = getattr(values, "_scorch_ones", None)
+    if seen is None or seen[0] != key or seen[1] is not False:
+        return values.data_ptr(), None          # not yet seen twice unchanged
+    listed = _empty_like(values)
+    native.check(L.scorch_hip_sddmm_csr_list_values_f32(values.numel(), lists.data_ptr(), lists.numel(),
+                                                        values.data_ptr(), listed.data_ptr(), stream))
+    try:
+        values._scorch_listed = (key, lists, listed)
+    except (AttributeError, RuntimeError):
+        return values.data_ptr(), None
+    return values.data_ptr(), listed.data_ptr()
 
 
 def _known_all_ones(values: torch.Tensor) -> bool:
@@ -1053,8 +1082,9 @@ def sddmm_csr_float(result_shape, S_shape, S_mode_indices, S_values, A_shape, A_
         if bl is not None:
             rc = _blocked_sddmm(L, bl, 1, M, n_cols, K, s_val.numel(), s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
+            mask_ptr, listed_ptr = _listed_mask_values(s_val, lists, L, stream)
             rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, s_val.numel(), lists.data_ptr(), lists.numel(),
-                                                   _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(),
+                                                   mask_ptr, listed_ptr, a.data_ptr(), b.data_ptr(),
                                                    out.data_ptr(), rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, s_val.numel(), pos.data_ptr(), crd.data_ptr(),
@@ -1208,8 +1238,9 @@ def sddmm_csr_float_batched(S_shape, S_mode_indices, S_values, A: torch.Tensor, 
         if bl is not None:
             rc = _blocked_sddmm(L, bl, H, M, n_cols, K, nnz, s_val, a, b, out, rows_ptr, stream)
         elif lists is not None:
+            mask_ptr, listed_ptr = _listed_mask_values(s_val, lists, L, stream)
             rc = L.scorch_hip_sddmm_csr_listed_f32(H, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(),
-                                                   _mask_values_pointer(s_val), a.data_ptr(), b.data_ptr(),
+                                                   mask_ptr, listed_ptr, a.data_ptr(), b.data_ptr(),
                                                    out.data_ptr(), rows_ptr, stream)
         else:
             rc = L.scorch_hip_sddmm_csr_batched_f32(H, M, n_cols, K, nnz, pos.data_ptr(), crd.data_ptr(),

@@ -281,7 +281,7 @@ def test_a_mask_without_a_value_array_is_a_mask_of_ones(oracle, monkeypatch, pat
             rc = L.scorch_hip_sddmm_csr_f32(M, n_cols, K, nnz, rp.data_ptr(), ci.data_ptr(), v, A.data_ptr(),
                                             B.data_ptr(), out.data_ptr(), None, stream)
         elif path == "listed":
-            rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(), v,
+            rc = L.scorch_hip_sddmm_csr_listed_f32(1, M, n_cols, K, nnz, lists.data_ptr(), lists.numel(), v, None,
                                                    A.data_ptr(), B.data_ptr(), out.data_ptr(), None, stream)
         else:
             rc = L.scorch_hip_sddmm_coo_f32(M, n_cols, K, nnz, rows.data_ptr(), ci.data_ptr(), v, A.data_ptr(),
@@ -333,3 +333,50 @@ def test_values_differ_kernel():
                 assert differ(v) == 1, (n, at)
                 v[at] = float("nan")
                 assert differ(v) == 1, (n, at)
+
+
+def test_mask_values_in_list_order(oracle, monkeypatch):
+    """A mask whose values are not all ones: on its third product (seen, seen again unchanged,
+    found not to be ones) the listed kernel reads a copy of the values in the order of its
+    lists.  Same bits as the scattered reads; dropped when the values are written to; never made
+    for a volatile tensor."""
+    w = workloads.sddmm_uniform(M=4096, n_cols=65_536, per_row=80, K=32, seed=12, unit_mask=False)
+    M, n_cols, K = w["M"], w["n_cols"], w["K"]
+    rp, ci, vals, A, B = dev(w["row_ptr"]), dev(w["col_idx"]), dev(w["vals"]), dev(w["A"]).reshape(-1), dev(w["B"]).reshape(-1)
+    monkeypatch.setattr(H, "SDDMM_PATH", "listed")
+    call = lambda v: H.sddmm_csr_float([M, n_cols], [M, n_cols], [[], [rp, ci]], v, [M, K], [[], []], A, [n_cols, K],
+                                       [[], []], B).storage.value
+    want = oracle.sddmm_fp64(w["row_idx"], w["col_idx"], w["vals"], w["A"], w["B"])
+    first = call(vals)
+    assert getattr(vals, "_scorch_listed", None) is None
+    second = call(vals)                                   # the verdict: not all ones
+    third = call(vals)                                    # ... and the copy
+    assert vals._scorch_listed[2].numel() == vals.numel()
+    fourth = call(vals)
+    assert torch.equal(first, second) and torch.equal(first, third) and torch.equal(first, fourth)
+    assert oracle.rel_fro(host(third), want) <= 1e-5
+    # the copy holds what the lists say it holds
+    L = native.lib()
+    plan = rp._scorch_plan
+    listed = torch.empty_like(vals)
+    native.check(L.scorch_hip_sddmm_csr_list_values_f32(vals.numel(), plan.sddmm_lists.data_ptr(), plan.sddmm_lists.numel(),
+                                                        vals.data_ptr(), listed.data_ptr(),
+                                                        torch.cuda.current_stream().cuda_stream))
+    assert torch.equal(listed, vals._scorch_listed[2])
+    assert torch.equal(torch.sort(listed).values, torch.sort(vals).values)
+    # new values: the copy is dropped with the version counter, and made again two products later
+    vals.mul_(-2.0)
+    assert torch.equal(call(vals), first * -2.0)
+    assert torch.equal(call(vals), first * -2.0) and torch.equal(call(vals), first * -2.0)
+    assert vals._scorch_listed[0] == H._stamp(vals)
+    # a write PyTorch does not see: forget() drops the copy
+    vals.data.mul_(0.5)
+    H.forget(vals)
+    assert getattr(vals, "_scorch_listed", None) is None
+    assert torch.equal(call(vals), first * -1.0)
+    # volatile values never get a copy
+    other = vals.clone()
+    H.mark_volatile(other)
+    for _ in range(4):
+        assert torch.equal(call(other), first * -1.0)
+    assert getattr(other, "_scorch_listed", None) is None
