@@ -342,6 +342,11 @@ int scorch_hip_dense_plan_create(int64_t K, int64_t N, const float *B, void *str
 
 int scorch_hip_dense_plan_update(scorch_hip_dense_plan *plan, void *stream) {
   if (!plan) return fail(SCORCH_HIP_EINVAL, "scorch_hip_dense_plan_update: plan is NULL");
+  int device = -1;
+  SCORCH_HIP_CHECK(hipGetDevice(&device));
+  if (device != plan->device)
+    return fail(SCORCH_HIP_EINVAL, "scorch_hip_dense_plan_update: the plan was made on device %d, the current device is %d",
+                plan->device, device);
   if (!plan->tiles) return SCORCH_HIP_OK;
   return scorch_hip_dense_to_tiled_f32(plan->K, plan->N, plan->B, plan->tiles, plan->tiles_bytes, stream);
 }
