@@ -155,6 +155,9 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_planned_i64(int64_t M, int64_t K, int64_t
  * of A gather from it, so B comes from memory about once.  Results agree with
  * the other SpMM entry points to rounding (rows of more than 64 entries are
  * summed in another grouping) and are bit-reproducible from run to run.
+ * longest_row is the longest row of A if the caller knows it (scorch_hip_csr_inspect reports it), else
+ * 0: with no row beyond 32 to 64 entries (depending on the shape) no row is shared between wavefronts,
+ * and the launch that folds shared rows' partial sums is left out.
  * scorch_hip_dense_tiled_recommended is 1 when the layout pays: rows of B of
  * 2 KiB and more, K * 128 bytes within an L2's reach (3 MiB), and nnz >= 2 K. */
 SCORCH_HIP_API size_t scorch_hip_dense_tiled_bytes(int64_t K, int64_t N, size_t elem_size);
@@ -165,7 +168,7 @@ SCORCH_HIP_API int scorch_hip_spmm_csr_tiled_f32(int64_t M, int64_t K, int64_t N
                                   const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
                                   const float *Bt, size_t bt_bytes, const float *bias, int act, float *C,
                                   const void *bounds, size_t bounds_bytes,
-                                  void *workspace, size_t workspace_bytes, void *stream);
+                                  void *workspace, size_t workspace_bytes, int64_t longest_row, void *stream);
 
 /* SDDMM for a CSR mask whose pattern is used again and again (an attention mask
  * serves every head, layer and step), with B larger than one of the GPU's eight

@@ -384,7 +384,8 @@ int scorch_hip_spmm_csr_plan_dense_f32(scorch_hip_csr_plan *plan, const float *v
   if (int rc = prepare_spmm(plan, N, static_cast<hipStream_t>(stream), &bounds, true)) return rc;
   return scorch_hip_spmm_csr_tiled_f32(plan->M, plan->n_cols, N, plan->nnz, plan->row_ptr, plan->col_idx, vals,
                                        dense->tiles, dense->tiles_bytes, bias, act, C, bounds ? bounds->data : nullptr,
-                                       bounds ? bounds->bytes : 0, plan->workspace, plan->workspace_bytes, stream);
+                                       bounds ? bounds->bytes : 0, plan->workspace, plan->workspace_bytes,
+                                       plan->longest_row(), stream);
 }
 
 }  // extern "C"

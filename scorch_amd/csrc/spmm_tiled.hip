@@ -227,7 +227,7 @@ template <typename T, int EPI>
 int spmm_tiled_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
                      const int32_t *col_idx, const T *vals, const T *Bt, size_t bt_bytes, const T *bias, T *C,
                      const void *bounds_buffer, size_t bounds_bytes, void *workspace, size_t workspace_bytes,
-                     void *stream) {
+                     int64_t longest_row, void *stream) {
   if (int rc = check_csr_args(fn, M, K, nnz, row_ptr, col_idx, vals)) return rc;
   SCORCH_REQUIRE(N >= 0, "%s: negative N=%lld", fn, (long long)N);
   if (N > INT32_MAX - kWaveSize * 4)
@@ -287,6 +287,10 @@ int spmm_tiled_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nn
       (int)tiled_tiles(N, sizeof(T)), (int)wgs, split.spans, vector_stores, carry_row, carry_val, bounds);
   SCORCH_HIP_CHECK(hipGetLastError());
   mark_launch(s);
+  // A boundary that falls inside a row moves to the row's end when that is at most `snap` items
+  // away (chunk_boundary): with no row longer than that no chunk leaves a carry, and a caller who
+  // knows the longest row (the inspection reports it) saves the launch that would look for them.
+  if (longest_row > 0 && longest_row <= split.snap) return SCORCH_HIP_OK;
   const int64_t fix_per_block = kWavesPerBlock * kFixupChunks;
   spmm_fixup_kernel<T, 1, EPI><<<dim3((unsigned)((split.spans + fix_per_block - 1) / fix_per_block)),
                                  kBlockThreads, 0, s>>>((int)N, split.spans, carry_row, carry_val, C, bias,
@@ -338,20 +342,21 @@ int scorch_hip_dense_to_tiled_f32(int64_t K, int64_t N, const float *B, float *B
 int scorch_hip_spmm_csr_tiled_f32(int64_t M, int64_t K, int64_t N, int64_t nnz, const int32_t *row_ptr,
                                   const int32_t *col_idx, const float *vals, const float *Bt, size_t bt_bytes,
                                   const float *bias, int act, float *C, const void *bounds,
-                                  size_t bounds_bytes, void *workspace, size_t workspace_bytes, void *stream) {
+                                  size_t bounds_bytes, void *workspace, size_t workspace_bytes,
+                                  int64_t longest_row, void *stream) {
   const char *fn = "scorch_hip_spmm_csr_tiled_f32";
   if (!bias && act == SCORCH_HIP_ACT_NONE)
     return scorch::spmm_tiled_entry<float, scorch::kEpiNone>(fn, M, K, N, nnz, row_ptr, col_idx, vals, Bt,
                                                              bt_bytes, nullptr, C, bounds, bounds_bytes,
-                                                             workspace, workspace_bytes, stream);
+                                                             workspace, workspace_bytes, longest_row, stream);
   if (bias && act == SCORCH_HIP_ACT_NONE)
     return scorch::spmm_tiled_entry<float, scorch::kEpiBias>(fn, M, K, N, nnz, row_ptr, col_idx, vals, Bt,
                                                              bt_bytes, bias, C, bounds, bounds_bytes, workspace,
-                                                             workspace_bytes, stream);
+                                                             workspace_bytes, longest_row, stream);
   if (bias && act == SCORCH_HIP_ACT_RELU)
     return scorch::spmm_tiled_entry<float, scorch::kEpiBiasRelu>(fn, M, K, N, nnz, row_ptr, col_idx, vals, Bt,
                                                                  bt_bytes, bias, C, bounds, bounds_bytes,
-                                                                 workspace, workspace_bytes, stream);
+                                                                 workspace, workspace_bytes, longest_row, stream);
   return scorch::fail(SCORCH_HIP_EINVAL, "%s: activation %d (with%s bias) is not supported", fn, act,
                       bias ? "" : "out");
 }

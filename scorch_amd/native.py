@@ -67,7 +67,7 @@ SIGNATURES = {
     "scorch_hip_dense_tiled_recommended": (ctypes.c_int, [_i64, _i64, _i64, _size]),
     "scorch_hip_dense_to_tiled_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, _size, _ptr]),
     "scorch_hip_spmm_csr_tiled_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _size, _ptr,
-                                                     ctypes.c_int, _ptr, _ptr, _size, _ptr, _size, _ptr]),
+                                                     ctypes.c_int, _ptr, _ptr, _size, _ptr, _size, _i64, _ptr]),
     "scorch_hip_spmm_csr_f32_timed": (ctypes.c_int, _SPMM + [ctypes.POINTER(ctypes.c_float)]),
     "scorch_hip_spmm_csr_bias_act_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_int, _ptr, _ptr, _size, _ptr]),

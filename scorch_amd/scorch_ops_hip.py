@@ -739,7 +739,8 @@ def _spmm(dtype, result_shape, A_shape, A_mode_indices, A_values, B_shape, B_mod
         if tiled is not None:
             rc = L.scorch_hip_spmm_csr_tiled_f32(M, K, N, nnz, pos.data_ptr(), crd.data_ptr(), a_val.data_ptr(),
                                                  tiled.data_ptr(), tiled.numel() * 4, bias_ptr, act, out.data_ptr(),
-                                                 bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(), stream)
+                                                 bounds_ptr, bounds_bytes, ws.data_ptr(), ws.numel(),
+                                                 plan.max_row if plan is not None else 0, stream)
         else:
             hint = HINT_MOSTLY_EMPTY_ROWS if fill_first else 0
             rc = getattr(L, "scorch_hip_spmm_csr_planned_" + suffix)(

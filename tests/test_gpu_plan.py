@@ -308,7 +308,7 @@ def test_tiled_kernel_when_the_even_resplit_makes_chunks_longer_than_the_usual_o
 
 @pytest.mark.parametrize("longest", [1, 7, 33, 64, 200])
 @pytest.mark.parametrize("relu", [None, False, True])
-def test_tiled_kernel_over_row_lengths_and_epilogues(oracle, longest, relu):
+def test_tiled_kernel_over_row_lengths_and_epilogues(oracle, longest, relu, monkeypatch):
     """The tiled kernel against fp64 and, bit for bit where no row is shared by all lane groups
     (at most 64 entries), against the merge path: empty rows, rows cut by chunk boundaries, an
     epilogue, N not a multiple of the tile width."""
@@ -328,3 +328,9 @@ def test_tiled_kernel_over_row_lengths_and_epilogues(oracle, longest, relu):
         got = hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled")
         assert oracle.rel_fro(got, want) <= TOL
         assert np.array_equal(got, hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled"))
+        # without a plan the longest row is unknown and the launch that folds shared rows' partial sums
+        # always runs; with one it is left out when no row can be shared: the same bits either way
+        monkeypatch.setenv("SCORCH_HIP_PLAN", "0")
+        unplanned = hip_spmm(rp, ci, v, B, bias=bias, relu=bool(relu), path="tiled")
+        monkeypatch.delenv("SCORCH_HIP_PLAN")
+        assert np.array_equal(got, unplanned)
