@@ -55,6 +55,34 @@ def test_description_equals_the_construction_by_torch_operations(kind, shape):
     assert ci.size / (64 * report[5]) >= ci.size / (4096 * n_active) - 1e-12
 
 
+@pytest.mark.parametrize("n_block_cols", [257, 5000, 131_072])
+def test_description_of_a_very_wide_pattern(n_block_cols):
+    """More block columns than a workgroup has threads (the bitmap and its ranks are walked in
+    strides and stretches), up to the most the kernels take: rows of a few hundred entries spread
+    over the whole width, some clustered so that blocks hold more than one entry."""
+    rng = np.random.default_rng(n_block_cols)
+    M, n_cols = 128, 64 * n_block_cols
+    rows = []
+    for r in range(M):
+        spread = rng.choice(n_cols, int(rng.integers(0, 300)), replace=False)
+        home = 64 * int(rng.integers(0, n_block_cols))
+        cluster = home + rng.choice(64, int(rng.integers(0, 40)), replace=False)
+        rows.append(np.unique(np.concatenate([spread, cluster, [n_cols - 1] if r % 7 == 0 else []]).astype(np.int64)))
+    rp = np.concatenate([[0], np.cumsum([len(x) for x in rows])]).astype(np.int32)
+    ci = np.concatenate(rows).astype(np.int32)
+    pos, crd = dev(rp), dev(ci)
+    assert _inspect(pos, crd, n_cols)[:2] == [0, 0]
+    brp, arrays = H._describe_blocks(pos, crd, M, n_cols)
+    want = describe(pos, crd, M, n_cols)
+    assert np.array_equal(brp, host(want["block_row_ptr"]))
+    for name, expected in want.items():
+        assert torch.equal(arrays[name], expected), name
+    L = native.lib()
+    too_wide = torch.zeros(3, dtype=torch.int32, device="cuda")
+    assert L.scorch_hip_csr_block_count(64, 64 * (131_072 + 1), 0, too_wide.data_ptr(), None, too_wide.data_ptr(),
+                                        None) == native.EUNSUPPORTED
+
+
 def test_description_read_directly_from_the_mask():
     """Every stored entry is found at block_off + (stored columns below it); the work-item lists
     cover what they must; what the description is not built for is turned away."""
