@@ -134,7 +134,8 @@ def test_softmax_in_place(oracle):
     assert oracle.rel_fro(host(v), oracle.softmax_csr_fp64(rp, vals, 0.5)) <= TOL
 
 
-@pytest.mark.parametrize("lens", [[4_200_000], [3, 70_000, 0, 1_500_000, 12, 65_536, 65_537, 5000, 200_000]])
+@pytest.mark.parametrize("lens", [[4_200_000], [3, 70_000, 0, 1_500_000, 12, 65_536, 65_537, 5000, 200_000],
+                                  [17, 20_000_000]])     # (the last: more entries than 1024 stretches of 16,384 hold)
 def test_softmax_rows_shared_out_among_workgroups(oracle, lens):
     """Rows of more than 65,536 entries are served in stretches by many workgroups (a single row of
     millions would otherwise be one workgroup's): against the fp64 recomputation, the same bits on
