@@ -179,7 +179,10 @@ int prepare_softmax(scorch_hip_csr_plan *plan, hipStream_t stream) {
 extern "C" {
 
 int scorch_hip_init(void) {
-  hipError_t (*const loaders[])() = {scorch::preload_attn, scorch::preload_attn_f32, scorch::preload_blockdesc, scorch::preload_blocked, scorch::preload_misc, scorch::preload_sddmm, scorch::preload_spgemm, scorch::preload_spmm, scorch::preload_spmm_rows, scorch::preload_spmm_tiled};
+  hipError_t (*const loaders[])() = {scorch::preload_attn,      scorch::preload_attn_f32, scorch::preload_blockdesc,
+                                     scorch::preload_blocked,   scorch::preload_misc,     scorch::preload_sddmm,
+                                     scorch::preload_spgemm,    scorch::preload_spmm,     scorch::preload_spmm_rows,
+                                     scorch::preload_spmm_tiled};
   for (auto load : loaders) SCORCH_HIP_CHECK(load());
   return SCORCH_HIP_OK;
 }
