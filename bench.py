@@ -766,6 +766,15 @@ def run_extra(args):
                **base, "config": {"workload": args.workload + "_fp32", "rows": M, "nnz": nnz},
                "algorithmic_bytes": algo, "hbm_gbps_algorithmic": round(algo / ms / 1e6, 1),
                "hbm_frac_algorithmic": round(algo / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        if args.workload == "softmax_powerlaw":
+            # the same through a plan handle, which knows the pattern's longest row and leaves out the
+            # launches no row of that length needs
+            from scorch_amd.csr_plan import CsrPlanHandle
+            with CsrPlanHandle(pos, crd, M) as plan:
+                assert torch.equal(plan.softmax(val, 1.0), fn())
+                out["ms_per_step_plan_handle"] = round(_time_steps(lambda: plan.softmax(val, 1.0), args.steps,
+                                                                   args.warmup), 4)
+                out["longest_row"] = plan.info()["longest_row"]
         if args.vendor and args.workload == "spmv_powerlaw":
             A_t = torch.sparse_csr_tensor(pos, crd, val, size=(M, M))
             out["vendor_library"] = _vendor_time("torch.mv(csr, x)", lambda: torch.mv(A_t, x), args.steps, 1)

@@ -195,11 +195,14 @@ SCORCH_HIP_API int scorch_hip_sddmm_csr_listed_f32(int64_t batch, int64_t M, int
                                     const float *listed_vals, const float *A, const float *B, float *out_vals,
                                     int32_t *out_row_idx, void *stream);
 
-/* The same for `batch` value arrays over one pattern, for a caller that knows that no row has more
- * than 4096 entries (scorch_hip_csr_inspect reports the longest row): one launch, no workspace.
- * The entries of `out` that belong to a longer row would be left unwritten. */
-SCORCH_HIP_API int scorch_hip_softmax_csr_short_rows_f32(int64_t batch, int64_t M, int64_t nnz,
-                               const int32_t *row_ptr, const float *vals, float scale, float *out,
+/* The same for `batch` value arrays over one pattern, for a caller that knows the pattern's longest
+ * row (scorch_hip_csr_inspect reports it): with longest_row <= 4096 one launch and no workspace
+ * (NULL, 0); with longest_row <= 16,384 the two launches that serve longer rows in stretches are
+ * left out; the workspace is that of scorch_hip_softmax_csr_workspace_bytes otherwise.  The entries
+ * of `out` that belong to a row longer than stated may be left unwritten. */
+SCORCH_HIP_API int scorch_hip_softmax_csr_known_rows_f32(int64_t batch, int64_t M, int64_t nnz,
+                               int64_t longest_row, const int32_t *row_ptr, const float *vals,
+                               float scale, float *out, void *workspace, size_t workspace_bytes,
                                void *stream);
 
 /* The same with long block rows shared out among workgroups (a mask with a global token has a

@@ -42,6 +42,11 @@ LaunchMarks *launch_marks() {
 // serve the stretches -- softmax_split_partial_kernel a stretch's maximum and its sum of
 // exponentials relative to that, softmax_split_finish_kernel the row's maximum and sum from its
 // stretches' (in stretch order: the same bits on every run) and the stretch's results.
+// A row that holds more than one part in kSoftmaxLoneRowShare of all the giant rows' entries would set
+// the giant-row kernel's time by itself (a workgroup walks 50,000 entries in a dozen dependent round
+// trips while the others have finished), so beyond kSoftmaxLoneSplitRow entries it goes the same way, in
+// stretches of kSoftmaxLoneStretch; among many rows like itself it stays one workgroup's, whose second
+// sweep finds the row in its L2.
 // Values are loaded raw and scaled at their first use, so that a row's loads
 // are all issued before any of them is waited for.
 constexpr int kSoftmaxRegs = 4;
@@ -58,6 +63,11 @@ constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
 constexpr int kSoftmaxGiantThreads = 1024;
 constexpr int kSoftmaxSplitRow = 65536;     // rows longer than this are shared out in stretches
 constexpr int kSoftmaxStretch = 16384;      // entries of a stretch, at least
+// A row with more than 1 / kSoftmaxLoneRowShare of the entries of all giant rows is shared out from
+// kSoftmaxLoneSplitRow entries on, in shorter stretches.
+constexpr int kSoftmaxLoneRowShare = 100;
+constexpr int kSoftmaxLoneSplitRow = 16384;
+constexpr int kSoftmaxLoneStretch = 8192;
 constexpr int kSoftmaxMaxStretches = 1024;  // stretches of a row, at most (one per thread of the combining workgroup)
 constexpr int kSoftmaxSplitBlocks = 2048;   // most workgroups the two stretch kernels start
 constexpr int kSoftmaxGiantBlocks = 1024;  // most workgroups the giant-row kernel starts
@@ -195,8 +205,9 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   // [2] entries per lane, and the workgroup [3]; [4]: rows left to the giant-row kernel
   __shared__ int s_list[5][kRows];
   __shared__ int s_count[5];
-  __shared__ int s_giant_base;
+  __shared__ int s_giant_base, s_giant_entries;
   if (threadIdx.x < 5) s_count[threadIdx.x] = 0;
+  if (threadIdx.x == 5) s_giant_entries = 0;
   __syncthreads();
   const int t = threadIdx.x % G;
   int lo[kTeamRows], hi[kTeamRows];
@@ -220,6 +231,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
         s_list[tier][atomicAdd(&s_count[tier], 1)] = slot;  // order only decides which wavefront serves a row
       } else if (t == 0) {
         s_list[4][atomicAdd(&s_count[4], 1)] = (int)row;
+        atomicAdd(&s_giant_entries, len);
       }
       hi[j] = lo[j];
     }
@@ -236,7 +248,10 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   const int n_quarter = s_count[0], n_wave = s_count[1], n_long_wave = s_count[2], n_block = s_count[3],
             n_giant = s_count[4];
   if (n_giant > 0 && list_giants) {  // uniform over the workgroup; rows are independent, so the list's order is free
-    if (threadIdx.x == 0) s_giant_base = atomicAdd(giant_count, n_giant);
+    if (threadIdx.x == 0) {
+      s_giant_base = atomicAdd(giant_count, n_giant);
+      atomicAdd(giant_count + 3, s_giant_entries);  // (all entries of a matrix fit an int)
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < n_giant; i += kBlockThreads) giant_rows[s_giant_base + i] = s_list[4][i];
   }
@@ -284,9 +299,10 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   }
 }
 
-// counters[0]: giant rows listed; [1]: rows served in stretches; [2]: their stretches in all
+// counters[0]: giant rows listed; [1]: rows served in stretches; [2]: their stretches in all;
+// [3]: entries of the giant rows
 __global__ void softmax_reset_kernel(int *counters) {
-  if (threadIdx.x < 3) counters[threadIdx.x] = 0;
+  if (threadIdx.x < 4) counters[threadIdx.x] = 0;
 }
 
 // The rows that are served in stretches, in the caller's workspace: rows[j] = (row, its first
@@ -402,6 +418,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
   vals += blockIdx.y * nnz;  // problem blockIdx.y of a batch over one pattern
   out += blockIdx.y * nnz;
   const int n = *giant_count;
+  const int giant_entries = giant_count[3];
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
   const int t = (int)threadIdx.x;
@@ -415,16 +432,18 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
     for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
     return r;
   };
-  // A row of more than kSoftmaxSplitRow entries is entered in the list of rows that are served in
-  // stretches (by problem 0 of a batch: the pattern is the same for all) and skipped here.
+  // A row of more than kSoftmaxSplitRow entries (kSoftmaxLoneSplitRow for one that holds a large part
+  // of all giant rows' entries) is entered in the list of rows that are served in stretches (by problem 0 of a batch: the pattern is the same for all) and skipped here.
   // Uniform over the workgroup.
   auto leave_to_the_stretch_kernels = [&](int row, int lo, int &hi) {
     const int len = hi - lo;
-    if (len <= kSoftmaxSplitRow || split.rows == nullptr) return;
+    const bool lone = (int64_t)len * kSoftmaxLoneRowShare > giant_entries;
+    if (split.rows == nullptr || len <= (lone ? kSoftmaxLoneSplitRow : kSoftmaxSplitRow)) return;
     hi = lo;
     if (blockIdx.y != 0) return;
+    const int least = len > kSoftmaxSplitRow ? kSoftmaxStretch : kSoftmaxLoneStretch;
     int stretch = (len + kSoftmaxMaxStretches - 1) / kSoftmaxMaxStretches;
-    stretch = stretch < kSoftmaxStretch ? kSoftmaxStretch : (stretch + 1023) / 1024 * 1024;
+    stretch = stretch < least ? least : (stretch + 1023) / 1024 * 1024;
     const int n_units = (len + stretch - 1) / stretch;
     __syncthreads();  // (s_claim may still be read from the row before)
     if (threadIdx.x == 0) {
@@ -474,14 +493,18 @@ inline int64_t softmax_giant_capacity(int64_t M, int64_t nnz) {
   return by_entries < M ? by_entries : M;
 }
 
-// Rows that may have to be served in stretches, and stretches in all.
+// Rows that may have to be served in stretches (those beyond kSoftmaxSplitRow entries; of those
+// beyond kSoftmaxLoneSplitRow, the fewer than kSoftmaxLoneRowShare that can each hold more than that
+// part of the giant rows' entries), and stretches in all.
 inline int64_t softmax_split_rows(int64_t M, int64_t nnz) {
-  const int64_t by_entries = nnz / (kSoftmaxSplitRow + 1);
+  int64_t lone = nnz / (kSoftmaxLoneSplitRow + 1);
+  if (lone > kSoftmaxLoneRowShare) lone = kSoftmaxLoneRowShare;
+  const int64_t by_entries = nnz / (kSoftmaxSplitRow + 1) + lone;
   return by_entries < M ? by_entries : M;
 }
 inline int64_t softmax_split_units(int64_t M, int64_t nnz) {
   const int64_t rows = softmax_split_rows(M, nnz);
-  return rows > 0 ? nnz / kSoftmaxStretch + rows : 0;
+  return rows > 0 ? nnz / kSoftmaxLoneStretch + rows : 0;
 }
 inline size_t softmax_round_256(size_t v) { return (v + 255) / 256 * 256; }
 
@@ -607,7 +630,7 @@ size_t scorch_hip_softmax_csr_workspace_bytes(int64_t M, int64_t nnz) {
 
 static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
                              const float *vals, float scale, float *out, void *workspace,
-                             size_t workspace_bytes, void *stream, bool short_rows = false) {
+                             size_t workspace_bytes, void *stream, int64_t longest_row = -1) {
   if (batch < 0 || batch > 65535)
     return scorch::fail(SCORCH_HIP_EUNSUPPORTED, "%s: batch=%lld is outside [0, 65535]", fn, (long long)batch);
   if (M < 0 || nnz < 0) return scorch::fail(SCORCH_HIP_EINVAL, "%s: negative size", fn);
@@ -616,8 +639,10 @@ static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t n
   SCORCH_REQUIRE(row_ptr != nullptr, "%s: row_ptr is NULL", fn);
   if (batch == 0 || M == 0 || nnz == 0) return SCORCH_HIP_OK;
   SCORCH_REQUIRE(vals && out, "%s: NULL value array", fn);
-  // (short_rows: the caller vouches that no row has more than 4096 entries, so there is no list
-  // of giant rows to reset, fill or serve)
+  // longest_row >= 0: the caller vouches that no row has more entries than that.  Up to 4096 there is
+  // no list of giant rows to reset, fill or serve; up to kSoftmaxLoneSplitRow no row is served in stretches.
+  const bool short_rows = longest_row >= 0 && longest_row <= 4096;
+  const bool no_stretches = longest_row >= 0 && longest_row <= scorch::kSoftmaxLoneSplitRow;
   const size_t need = short_rows ? 0 : scorch::softmax_workspace_bytes(M, nnz);
   if (need > 0 && (!workspace || workspace_bytes < need))
     return scorch::fail(SCORCH_HIP_EWORKSPACE, "%s: workspace of %zu bytes needed, %zu given", fn, need,
@@ -653,7 +678,8 @@ static int softmax_csr_entry(const char *fn, int64_t batch, int64_t M, int64_t n
     if (most > scorch::kSoftmaxGiantBlocks) most = scorch::kSoftmaxGiantBlocks;
     if (batch > 1 && most > 128) most = 128;  // every problem brings its own workgroups
     const dim3 giant_grid((unsigned)most, (unsigned)batch);
-    const scorch::SoftmaxSplit split = scorch::softmax_split_layout(workspace, M, nnz);
+    const scorch::SoftmaxSplit split =
+        no_stretches ? scorch::SoftmaxSplit{} : scorch::softmax_split_layout(workspace, M, nnz);
     scorch::softmax_csr_giant_kernel<<<giant_grid, scorch::kSoftmaxGiantThreads, 0, s>>>(
         row_ptr, vals, scale, out, giant_count, giant_rows, nnz, split);
     SCORCH_HIP_CHECK(hipGetLastError());
@@ -688,10 +714,14 @@ int scorch_hip_softmax_csr_batched_f32(int64_t batch, int64_t M, int64_t nnz, co
                            workspace, workspace_bytes, stream);
 }
 
-int scorch_hip_softmax_csr_short_rows_f32(int64_t batch, int64_t M, int64_t nnz, const int32_t *row_ptr,
-                                          const float *vals, float scale, float *out, void *stream) {
-  return softmax_csr_entry("scorch_hip_softmax_csr_short_rows_f32", batch, M, nnz, row_ptr, vals, scale, out,
-                           nullptr, 0, stream, true);
+int scorch_hip_softmax_csr_known_rows_f32(int64_t batch, int64_t M, int64_t nnz, int64_t longest_row,
+                                          const int32_t *row_ptr, const float *vals, float scale, float *out,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  if (longest_row < 0)
+    return scorch::fail(SCORCH_HIP_EINVAL, "scorch_hip_softmax_csr_known_rows_f32: longest_row=%lld",
+                        (long long)longest_row);
+  return softmax_csr_entry("scorch_hip_softmax_csr_known_rows_f32", batch, M, nnz, row_ptr, vals, scale, out,
+                           workspace, workspace_bytes, stream, longest_row);
 }
 
 int scorch_hip_csr_row_indices(int64_t M, int64_t nnz, const int32_t *row_ptr, int32_t *row_idx,

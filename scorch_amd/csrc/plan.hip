@@ -303,10 +303,11 @@ int scorch_hip_softmax_csr_plan_f32(scorch_hip_csr_plan *plan, const float *vals
                                     void *stream) {
   if (int rc = check_plan("scorch_hip_softmax_csr_plan_f32", plan)) return rc;
   if (plan->longest_row() <= kSoftmaxShortRow)
-    return scorch_hip_softmax_csr_short_rows_f32(1, plan->M, plan->nnz, plan->row_ptr, vals, scale, out, stream);
+    return scorch_hip_softmax_csr_known_rows_f32(1, plan->M, plan->nnz, plan->longest_row(), plan->row_ptr, vals,
+                                                 scale, out, nullptr, 0, stream);
   if (int rc = prepare_softmax(plan, static_cast<hipStream_t>(stream))) return rc;
-  return scorch_hip_softmax_csr_f32(plan->M, plan->nnz, plan->row_ptr, vals, scale, out, plan->workspace,
-                                    plan->workspace_bytes, stream);
+  return scorch_hip_softmax_csr_known_rows_f32(1, plan->M, plan->nnz, plan->longest_row(), plan->row_ptr, vals,
+                                               scale, out, plan->workspace, plan->workspace_bytes, stream);
 }
 
 int scorch_hip_dense_plan_create(int64_t K, int64_t N, const float *B, void *stream, scorch_hip_dense_plan **out) {

@@ -104,7 +104,8 @@ SIGNATURES = {
     "scorch_hip_softmax_csr_workspace_bytes": (_size, [_i64, _i64]),
     "scorch_hip_softmax_csr_f32": (ctypes.c_int, [_i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr, _ptr, _size,
                                                   _ptr]),
-    "scorch_hip_softmax_csr_short_rows_f32": (ctypes.c_int, [_i64, _i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr, _ptr]),
+    "scorch_hip_softmax_csr_known_rows_f32": (ctypes.c_int, [_i64, _i64, _i64, _i64, _ptr, _ptr, ctypes.c_float, _ptr,
+                                                             _ptr, ctypes.c_size_t, _ptr]),
     "scorch_hip_attn_blocksparse_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
                                                         _ptr, ctypes.c_float, _ptr, _ptr]),
     "scorch_hip_attn_blocksparse_masked_bf16": (ctypes.c_int, [_i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _i64,

@@ -1108,6 +1108,26 @@ def _known_longest_row(pos: torch.Tensor, n_rows: int, nnz: int) -> Optional[int
     return None
 
 
+def _launch_softmax(L, dev, pos, batch: int, nnz: int, v, scale: float, out) -> None:
+    """The row softmax of `batch` value arrays over one pattern; with the pattern's longest row known,
+    the entry point that leaves out the launches no row of that length needs."""
+    M = pos.numel() - 1
+    longest = _known_longest_row(pos, M, nnz)
+    with _on_device(dev):
+        stream = _stream(dev)
+        need = 0 if longest is not None and longest <= SOFTMAX_SHORT_ROW else \
+            L.scorch_hip_softmax_csr_workspace_bytes(M, nnz)
+        ws = _workspace(dev, stream, need) if need else None
+        ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if need else (None, 0)
+        if longest is not None:
+            rc = L.scorch_hip_softmax_csr_known_rows_f32(batch, M, nnz, longest, pos.data_ptr(), v.data_ptr(),
+                                                         float(scale), out.data_ptr(), ws_ptr, ws_bytes, stream)
+        else:
+            rc = L.scorch_hip_softmax_csr_batched_f32(batch, M, nnz, pos.data_ptr(), v.data_ptr(), float(scale),
+                                                      out.data_ptr(), ws_ptr, ws_bytes, stream)
+    native.check(rc)
+
+
 def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
     """Row softmax of ``scale * values`` over a CSR pattern
     (reference: bench/bench_sparse_transformer.py:277-297)."""
@@ -1116,19 +1136,7 @@ def softmax_csr_float(row_ptr: torch.Tensor, values: torch.Tensor, scale: float 
     dev = _device_of(pos, v)
     out = _empty_like(v)
     L = native.lib()
-    longest = _known_longest_row(pos, pos.numel() - 1, v.numel())
-    with _on_device(dev):
-        stream = _stream(dev)
-        if longest is not None and longest <= SOFTMAX_SHORT_ROW:
-            rc = L.scorch_hip_softmax_csr_short_rows_f32(1, pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
-                                                         float(scale), out.data_ptr(), stream)
-        else:
-            need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, v.numel())
-            ws = _workspace(dev, stream, need) if need else None
-            rc = L.scorch_hip_softmax_csr_f32(pos.numel() - 1, v.numel(), pos.data_ptr(), v.data_ptr(),
-                                              float(scale), out.data_ptr(), ws.data_ptr() if need else None,
-                                              ws.numel() if need else 0, stream)
-    native.check(rc)
+    _launch_softmax(L, dev, pos, 1, v.numel(), v, scale, out)
     return out
 
 
@@ -1262,19 +1270,7 @@ def softmax_csr_float_batched(row_ptr: torch.Tensor, values: torch.Tensor, scale
     H, nnz = int(v.shape[0]), int(v.shape[1])
     out = _empty_like(v)
     L = native.lib()
-    longest = _known_longest_row(pos, pos.numel() - 1, nnz)
-    with _on_device(dev):
-        stream = _stream(dev)
-        if longest is not None and longest <= SOFTMAX_SHORT_ROW:
-            rc = L.scorch_hip_softmax_csr_short_rows_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(),
-                                                         float(scale), out.data_ptr(), stream)
-        else:
-            need = L.scorch_hip_softmax_csr_workspace_bytes(pos.numel() - 1, nnz)
-            ws = _workspace(dev, stream, need) if need else None
-            rc = L.scorch_hip_softmax_csr_batched_f32(H, pos.numel() - 1, nnz, pos.data_ptr(), v.data_ptr(),
-                                                      float(scale), out.data_ptr(), ws.data_ptr() if need else None,
-                                                      ws.numel() if need else 0, stream)
-    native.check(rc)
+    _launch_softmax(L, dev, pos, H, nnz, v, scale, out)
     return out
 
 

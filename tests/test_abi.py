@@ -44,7 +44,7 @@ def test_the_stable_header_holds_no_plan_step():
     lists, block descriptions, work-item lists, pinned kernels and timing aids in the other."""
     stable = declared_symbols((HEADER,))
     unstable = declared_symbols((UNSTABLE_HEADER,))
-    step = re.compile(r"inspect|bounds|planned|_rows_|tiled|lists|listed|short_rows|split|blocked|block_|batched|"
+    step = re.compile(r"inspect|bounds|planned|_rows_|tiled|lists|listed|known_rows|split|blocked|block_|batched|"
                       r"timing|timed|attn_blocksparse_f32|values_differ|list_values")
     assert [n for n in stable if step.search(n)] == []
     assert [n for n in unstable if not step.search(n)] == []
@@ -151,10 +151,12 @@ def test_spmv_softmax_rows_reject_bad_arguments(L):
     # rows longer than 4096 entries are possible from nnz = 4097 on: a workspace is needed then
     assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4096) == 0
     assert L.scorch_hip_softmax_csr_workspace_bytes(4, 4097) == 512
-    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 60_000) == 256 + 256
-    # from 65,537 entries on a row can be long enough to be served in stretches: three more arrays
-    # (259 such rows at most here, 1,037 + 259 stretches)
-    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 17_000_000) == 256 + 16640 + 4352 + 2 * 10496
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 16_384) == 256 + 256
+    # from 16,385 entries on a row can be long enough to be served in stretches (if it holds a large part
+    # of the entries of all rows beyond 4096: at most 100 rows do; from 65,537 on in any case): three more
+    # arrays (3 such rows at most, 7 + 3 stretches of 8192 or more; then 259 + 100 rows, 2,075 + 359 stretches)
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 60_000) == 256 + 256 + 256 + 2 * 256
+    assert L.scorch_hip_softmax_csr_workspace_bytes(1 << 20, 17_000_000) == 256 + 16640 + 5888 + 2 * 19712
     assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, NULL, 0, NULL) == native.EWORKSPACE
     assert L.scorch_hip_softmax_csr_f32(4, 5000, FAKE, FAKE, 1.0, FAKE, FAKE, 256, NULL) == native.EWORKSPACE
     assert L.scorch_hip_csr_row_indices(4, 4, FAKE, NULL, NULL) == native.EINVAL

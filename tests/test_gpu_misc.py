@@ -135,7 +135,9 @@ def test_softmax_in_place(oracle):
 
 
 @pytest.mark.parametrize("lens", [[4_200_000], [3, 70_000, 0, 1_500_000, 12, 65_536, 65_537, 5000, 200_000],
-                                  [17, 20_000_000]])     # (the last: more entries than 1024 stretches of 16,384 hold)
+                                  [17, 20_000_000],      # (more entries than 1024 stretches of 16,384 hold)
+                                  # more than 512 rows beyond 4096 entries: those up to 65,536 stay one workgroup's
+                                  [4100] * 600 + [20_000, 70_000, 30_000, 65_536]])
 def test_softmax_rows_shared_out_among_workgroups(oracle, lens):
     """Rows of more than 65,536 entries are served in stretches by many workgroups (a single row of
     millions would otherwise be one workgroup's): against the fp64 recomputation, the same bits on
@@ -166,6 +168,46 @@ def test_softmax_rows_shared_out_among_workgroups(oracle, lens):
     rc = L.scorch_hip_softmax_csr_f32(len(lens), v.numel(), pos.data_ptr(), inplace.data_ptr(), 0.5, inplace.data_ptr(),
                                       ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0 and torch.equal(inplace, out)
+
+
+@pytest.mark.parametrize("lens", [[3, 0, 4096, 17, 900], [3, 9000, 5000, 12, 65_536, 300, 0, 70],
+                                  [5, 65_537, 100, 300_000, 4097]])
+def test_softmax_with_the_longest_row_stated(oracle, lens):
+    """scorch_hip_softmax_csr_known_rows_f32 leaves out the launches no row of the stated length
+    needs (no list of giant rows up to 4096 entries, no stretches up to 65,536): the same bits as
+    the entry point that is told nothing, for one value array and for a batch; a negative length
+    is refused."""
+    lens = np.array(lens, np.int64)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    vals = (np.random.default_rng(int(lens.max())).standard_normal(int(rp[-1])) * 3).astype(np.float32)
+    pos = dev(rp)
+    batch = torch.stack([dev(vals), dev(vals) * -0.5 + 2.0])
+    M, nnz, longest = len(lens), int(rp[-1]), int(lens.max())
+    L = H.native.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    need = L.scorch_hip_softmax_csr_workspace_bytes(M, nnz)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+    plain, told = torch.full_like(batch, -1.0), torch.full_like(batch, -1.0)
+    assert L.scorch_hip_softmax_csr_batched_f32(2, M, nnz, pos.data_ptr(), batch.data_ptr(), 0.5, plain.data_ptr(),
+                                                ws.data_ptr(), need, stream) == 0
+    short = longest <= 4096
+    assert L.scorch_hip_softmax_csr_known_rows_f32(2, M, nnz, longest, pos.data_ptr(), batch.data_ptr(), 0.5,
+                                                   told.data_ptr(), None if short else ws.data_ptr(),
+                                                   0 if short else need, stream) == 0
+    assert torch.equal(plain, told)
+    assert oracle.rel_fro(host(told[0]), oracle.softmax_csr_fp64(rp, vals, 0.5)) <= TOL
+    if not short:      # the longer rows need the workspace
+        assert L.scorch_hip_softmax_csr_known_rows_f32(2, M, nnz, longest, pos.data_ptr(), batch.data_ptr(), 0.5,
+                                                       told.data_ptr(), None, 0, stream) == H.native.EWORKSPACE
+    assert L.scorch_hip_softmax_csr_known_rows_f32(2, M, nnz, -1, pos.data_ptr(), batch.data_ptr(), 0.5,
+                                                   told.data_ptr(), ws.data_ptr(), need, stream) == H.native.EINVAL
+    # the Python layer: a product over the pattern has inspected it, the softmax then states the longest row
+    ci = dev(np.concatenate([np.arange(n, dtype=np.int32) for n in lens]))
+    H.spmm_csr_float_v2([M, 4], [M, longest], [[], [pos, ci]], batch[0].contiguous(), [longest, 4], [[], []],
+                        torch.ones(longest, 4, device="cuda"))
+    assert H._known_longest_row(pos, M, nnz) == longest
+    assert torch.equal(H.softmax_csr_float(pos, batch[0].contiguous(), 0.5), plain[0])
+    assert torch.equal(H.softmax_csr_float_batched(pos, batch, 0.5), plain)
 
 
 def test_softmax_with_empty_rows_and_large_values(oracle):
