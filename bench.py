@@ -58,7 +58,7 @@ MEASURED_TRAFFIC = {
                                                                 _CSRC + "common.hpp"), "sha16": "36b7f160411c76eb",
                                "profile": "profiles/spmm_rows_kernel_uniform_4096.md"},
     ("sae_decoder", "tiled"): {"bytes": 344_100_000, "sources": (_CSRC + "spmm_tiled.hip", _CSRC + "spmm.hpp",
-                                                                 _CSRC + "common.hpp"), "sha16": "edf5bb2b94a7bd71",
+                                                                 _CSRC + "common.hpp"), "sha16": "ea9b5c43570e7930",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},
     ("sae_decoder", "merge"): {"bytes": 1_767_900_000, "sources": _SPMM_SOURCES, "sha16": "f03cdf8f7d11457c",
                                "profile": "profiles/spmm_tiled_kernel_sae_decoder.md"},

@@ -69,8 +69,8 @@ constexpr int kSoftmaxLoneRowShare = 100;
 constexpr int kSoftmaxLoneSplitRow = 16384;
 constexpr int kSoftmaxLoneStretch = 8192;
 constexpr int kSoftmaxMaxStretches = 1024;  // stretches of a row, at most (one per thread of the combining workgroup)
-constexpr int kSoftmaxSplitBlocks = 2048;   // most workgroups the two stretch kernels start
-constexpr int kSoftmaxGiantBlocks = 1024;  // most workgroups the giant-row kernel starts
+constexpr int kSoftmaxSplitBlocks = 512;   // most workgroups the two stretch kernels start
+constexpr int kSoftmaxGiantBlocks = 512;  // most workgroups the giant-row kernel starts
 constexpr float kSoftmaxLowest = -3.402823466e38f;
 
 // Lanes per row: the smallest power of two, between 2 and 64, whose groups hold
@@ -82,14 +82,29 @@ inline int softmax_group_width(int64_t M, int64_t nnz) {
   return g;
 }
 
+// exp(d) for d <= 0 (every exponential here is taken relative to a maximum) as one multiplication
+// and the hardware's 2^x: the library routine costs about ten instructions, and with four of
+// them and four divisions per lane and row the short-row kernel was bound by its vector
+// instructions, not by memory (31.6 M of them for the 17.8 M entries of a 1 M-row graph: 57 us of
+// issue time on 1024 SIMDs).  The product's rounding moves the result by at most |d| * 1.2e-7
+// relative: 1e-5 at the edge of the fp32 range, 1e-6 for d = -10.  -inf and the lowest float give 0.
+__device__ __forceinline__ float softmax_exp(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896341f); }
+// 1 / sum for a row's sum of exponentials (>= 1: the maximum's own term), to within one unit in
+// the last place; every entry of the row is multiplied by it where it was divided by the sum.
+__device__ __forceinline__ float softmax_reciprocal(float sum) { return __builtin_amdgcn_rcpf(sum); }
+
 // A row's entries [lo, hi) for a team of TEAM threads (this one is number t):
 // the first REGS * TEAM of them are read into registers, raw ...
+// (Every load is issued, the ones past the row's end at the array's last entry, `last`: a load under
+// a condition is a branch around it, and the loads of a row would not be in flight together.  What
+// those lanes read is replaced when the entries are scaled.)
 template <int TEAM, int REGS>
-__device__ __forceinline__ void softmax_load(int lo, int hi, int t, const float *vals, float (&v)[REGS]) {
+__device__ __forceinline__ void softmax_load(int lo, int hi, int t, const float *vals, int last,
+                                             float (&v)[REGS]) {
 #pragma unroll
   for (int u = 0; u < REGS; ++u) {
     const int p = lo + t + u * TEAM;
-    v[u] = p < hi ? vals[p] : 0.0f;
+    v[u] = vals[(unsigned)(p < hi ? p : last)];
   }
 }
 
@@ -125,7 +140,7 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
       for (int u = 0; u < kTailBatch; ++u) {
         if (p0 + u * TEAM >= hi) break;
         const float x = raw[u] * scale;
-        const float e = expf(-fabsf(x - tail_max));
+        const float e = softmax_exp(-fabsf(x - tail_max));
         const bool higher = x > tail_max;
         tail_sum = higher ? tail_sum * e + 1.0f : tail_sum + e;
         tail_max = higher ? x : tail_max;
@@ -134,17 +149,17 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
     mx = tail_max;
   }
   mx = reduce(mx, true);
-  float sum = TAIL ? tail_sum * expf(tail_max - mx) : 0.0f;
+  float sum = TAIL ? tail_sum * softmax_exp(tail_max - mx) : 0.0f;
 #pragma unroll
   for (int u = 0; u < REGS; ++u) {
-    v[u] = lo + t + u * TEAM < hi ? expf(v[u] - mx) : 0.0f;
+    v[u] = softmax_exp(v[u] - mx);  // (past the row's end: the lowest float less the maximum, which gives 0)
     sum += v[u];
   }
-  sum = reduce(sum, false);
+  const float inv_sum = softmax_reciprocal(reduce(sum, false));
 #pragma unroll
   for (int u = 0; u < REGS; ++u) {
     const int p = lo + t + u * TEAM;
-    if (p < hi) out[p] = v[u] / sum;
+    if (p < hi) out[(unsigned)p] = v[u] * inv_sum;
   }
   if (TAIL) {
     for (int p0 = rest; p0 < hi; p0 += kTailBatch * TEAM) {
@@ -157,17 +172,17 @@ __device__ __forceinline__ void softmax_finish(int lo, int hi, int t, const floa
 #pragma unroll
       for (int u = 0; u < kTailBatch; ++u) {
         const int p = p0 + u * TEAM;
-        if (p < hi) out[p] = expf(raw[u] * scale - mx) / sum;
+        if (p < hi) out[p] = softmax_exp(raw[u] * scale - mx) * inv_sum;
       }
     }
   }
 }
 
 template <int TEAM, int REGS, bool TAIL, typename Reduce>
-__device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *vals, float scale,
+__device__ __forceinline__ void softmax_row(int lo, int hi, int t, const float *vals, int last, float scale,
                                             float *out, Reduce reduce) {
   float v[REGS];
-  softmax_load<TEAM, REGS>(lo, hi, t, vals, v);
+  softmax_load<TEAM, REGS>(lo, hi, t, vals, last, v);
   softmax_finish<TEAM, REGS, TAIL>(lo, hi, t, vals, scale, out, v, reduce);
 }
 
@@ -210,16 +225,22 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   if (threadIdx.x == 5) s_giant_entries = 0;
   __syncthreads();
   const int t = threadIdx.x % G;
+  const int last = (int)nnz - 1;
+  // The row pointers of all of the group's rows are requested before any is looked at (a row past
+  // the matrix's end reads the last row's and is given no entries).
   int lo[kTeamRows], hi[kTeamRows];
+#pragma unroll
+  for (int j = 0; j < kTeamRows; ++j) {
+    const int64_t row = (int64_t)blockIdx.x * kRows + j * kGroups + threadIdx.x / G;
+    const int64_t r = row < M ? row : (int64_t)M - 1;
+    lo[j] = row_ptr[r];
+    hi[j] = row_ptr[r + 1];
+  }
 #pragma unroll
   for (int j = 0; j < kTeamRows; ++j) {
     const int slot = j * kGroups + threadIdx.x / G;
     const int64_t row = (int64_t)blockIdx.x * kRows + slot;
-    lo[j] = hi[j] = 0;
-    if (row < M) {
-      lo[j] = row_ptr[row];
-      hi[j] = row_ptr[row + 1];
-    }
+    if (row >= M) hi[j] = lo[j];
     const int len = hi[j] - lo[j];
     if (len > G * kSoftmaxRegs) {
       if (t == 0 && len <= kSoftmaxBlockRowMax) {
@@ -238,7 +259,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   }
   float v[kTeamRows][kSoftmaxRegs];
 #pragma unroll
-  for (int j = 0; j < kTeamRows; ++j) softmax_load<G, kSoftmaxRegs>(lo[j], hi[j], t, vals, v[j]);
+  for (int j = 0; j < kTeamRows; ++j) softmax_load<G, kSoftmaxRegs>(lo[j], hi[j], t, vals, last, v[j]);
 #pragma unroll
   for (int j = 0; j < kTeamRows; ++j)
     softmax_finish<G, kSoftmaxRegs, false>(lo[j], hi[j], t, vals, scale, out, v[j], softmax_shuffle_reduce<G>);
@@ -257,7 +278,8 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   }
   if (G < kSoftmaxQuarter) {
     constexpr int kTeams = kBlockThreads / kSoftmaxQuarter;
-    for (int base = 0; base < n_quarter; base += kTeams) {  // uniform over the workgroup
+    // (a wavefront none of whose four teams has a row left is done: nothing here waits for the others)
+    for (int base = 0; base + w * (kWaveSize / kSoftmaxQuarter) < n_quarter; base += kTeams) {
       const int i = base + (int)threadIdx.x / kSoftmaxQuarter;
       int l = 0, h = 0;
       if (i < n_quarter) {
@@ -265,14 +287,14 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
         l = s_lo[k];
         h = s_hi[k];
       }
-      softmax_row<kSoftmaxQuarter, kSoftmaxRegs, false>(l, h, lane % kSoftmaxQuarter, vals, scale, out,
+      softmax_row<kSoftmaxQuarter, kSoftmaxRegs, false>(l, h, lane % kSoftmaxQuarter, vals, last, scale, out,
                                                         softmax_shuffle_reduce<kSoftmaxQuarter>);
     }
   }
   if (G < kWaveSize) {
     for (int i = w; i < n_wave; i += kWavesPerBlock) {
       const int k = s_list[1][i];
-      softmax_row<kWaveSize, kSoftmaxRegs, false>(s_lo[k], s_hi[k], lane, vals, scale, out,
+      softmax_row<kWaveSize, kSoftmaxRegs, false>(s_lo[k], s_hi[k], lane, vals, last, scale, out,
                                                   softmax_shuffle_reduce<kWaveSize>);
     }
   }
@@ -280,13 +302,13 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   // wavefronts work on four such rows at once and need no barriers
   for (int i = w; i < n_long_wave; i += kWavesPerBlock) {
     const int k = s_list[2][i];
-    softmax_row<kWaveSize, kSoftmaxBlockRegs, false>(s_lo[k], s_hi[k], lane, vals, scale, out,
+    softmax_row<kWaveSize, kSoftmaxBlockRegs, false>(s_lo[k], s_hi[k], lane, vals, last, scale, out,
                                                      softmax_shuffle_reduce<kWaveSize>);
   }
   for (int i = 0; i < n_block; ++i) {  // uniform over the workgroup
     const int k = s_list[3][i];
     softmax_row<kBlockThreads, kSoftmaxBlockRegs, false>(
-        s_lo[k], s_hi[k], (int)threadIdx.x, vals, scale, out, [&](float v, bool take_max) {
+        s_lo[k], s_hi[k], (int)threadIdx.x, vals, last, scale, out, [&](float v, bool take_max) {
           v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
           __syncthreads();
           if (lane == 0) s_red[w] = v;
@@ -352,14 +374,14 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_split_partial_ke
       for (int k = 0; k < kBatch; ++k) {
         if (p0 + k * kSoftmaxGiantThreads >= end) break;
         const float x = raw[k] * scale;
-        const float e = expf(-fabsf(x - mx));
+        const float e = softmax_exp(-fabsf(x - mx));
         const bool higher = x > mx;
         sum = higher ? sum * e + 1.0f : sum + e;
         mx = higher ? x : mx;
       }
     }
     const float unit_max = reduce(mx, true);
-    const float unit_sum = reduce(sum * expf(mx - unit_max), false);  // (a thread without entries: 0 * exp(lowest - max) = 0)
+    const float unit_sum = reduce(sum * softmax_exp(mx - unit_max), false);  // (a thread without entries: 0 * exp(lowest - max) = 0)
     if (threadIdx.x == 0) split.partials[u] = make_float2(unit_max, unit_sum);
   }
 }
@@ -388,7 +410,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_split_finish_ker
     float2 part = make_float2(kSoftmaxLowest, 0.0f);  // thread t: stretch t of the row
     if ((int)threadIdx.x < row.z) part = split.partials[row.y + threadIdx.x];
     const float row_max = reduce(part.x, true);
-    const float row_sum = reduce(part.y * expf(part.x - row_max), false);
+    const float inv_sum = softmax_reciprocal(reduce(part.y * softmax_exp(part.x - row_max), false));
     const int begin = row_ptr[row.x] + unit.y * row.w;
     const int row_end = row_ptr[row.x + 1];
     const int end = row_end - begin > row.w ? begin + row.w : row_end;  // (no overflow near 2^31 entries)
@@ -403,7 +425,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_split_finish_ker
 #pragma unroll
       for (int k = 0; k < kBatch; ++k) {
         const int p = p0 + k * kSoftmaxGiantThreads;
-        if (p < end) out[p] = expf(raw[k] * scale - row_max) / row_sum;
+        if (p < end) out[p] = softmax_exp(raw[k] * scale - row_max) * inv_sum;
       }
     }
   }
@@ -422,6 +444,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
   const int lane = wave_lane();
   const int w = threadIdx.x / kWaveSize;
   const int t = (int)threadIdx.x;
+  const int last = (int)nnz - 1;
   auto reduce = [&](float v, bool take_max) {
     v = softmax_shuffle_reduce<kWaveSize>(v, take_max);  // fixed order: lanes, then wavefronts
     __syncthreads();
@@ -464,7 +487,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
   int lo = row_ptr[row], hi = row_ptr[row + 1];
   leave_to_the_stretch_kernels(row, lo, hi);
   float v[kSoftmaxGiantRegs];
-  softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo, hi, t, vals, v);
+  softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo, hi, t, vals, last, v);
   for (;;) {  // uniform over the workgroup
     const int i_next = i + gridDim.x;
     int lo_next = 0, hi_next = 0;
@@ -475,7 +498,7 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
       hi_next = row_ptr[row_next + 1];
       leave_to_the_stretch_kernels(row_next, lo_next, hi_next);
     }
-    softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo_next, hi_next, t, vals, v_next);
+    softmax_load<kSoftmaxGiantThreads, kSoftmaxGiantRegs>(lo_next, hi_next, t, vals, last, v_next);
     softmax_finish<kSoftmaxGiantThreads, kSoftmaxGiantRegs, true>(lo, hi, t, vals, scale, out, v, reduce);
     if (i_next >= n) break;
     i = i_next;

@@ -106,7 +106,11 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
   const bool has_work = first_span < spans;
 
   for (int tile = xcd; tile < n_tiles; tile += 8) {
-    const T *__restrict__ slice = Bt + (size_t)tile * (size_t)K * TC + t * VEC;
+    // A gathered row's address is the slice's (the same for the whole wavefront: scalar registers) plus
+    // a byte offset of 32 bits (the entry's, staged as such, plus the lane's 16 bytes of the tile row):
+    // one vector instruction per load where a 64-bit product and sum took four.
+    const char *__restrict__ slice = reinterpret_cast<const char *>(Bt + (size_t)tile * (size_t)K * TC);
+    const unsigned lane_bytes = (unsigned)(t * VEC * sizeof(T));
     const int col0 = tile * TC + t * VEC;
     const bool active = col0 < N;
     T bias_v[VEC];
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
         n_nz = y1 - y0;
         n_rows = x1 - x0;
         for (int k = lane; k < n_nz; k += kWaveSize) {
-          s_col[w][k] = col_idx[y0 + k];
+          s_col[w][k] = (int)((unsigned)col_idx[y0 + k] * (unsigned)kTileBytes);  // byte offset within a slice
           s_val[w][k] = vals[y0 + k];
         }
         for (int k = lane; k <= n_rows + 1; k += kWaveSize) {
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
 
       auto add_entry = [&](A (&acc)[VEC], int k) {
         const A a = (A)s_val[w][k];
-        const VecT b = *reinterpret_cast<const VecT *>(slice + (size_t)s_col[w][k] * TC);
+        const VecT b = *reinterpret_cast<const VecT *>(slice + ((unsigned)s_col[w][k] + lane_bytes));
 #pragma unroll
         for (int v = 0; v < VEC; ++v) acc[v] += a * (A)b.v[v];
       };
@@ -168,7 +172,7 @@ __global__ __launch_bounds__(kBlockThreads) void spmm_tiled_kernel(
 #pragma unroll
             for (int u = 0; u < kTiledBatch; ++u) {
               a[u] = (A)s_val[w][k + u];
-              b[u] = *reinterpret_cast<const VecT *>(slice + (size_t)s_col[w][k + u] * TC);
+              b[u] = *reinterpret_cast<const VecT *>(slice + ((unsigned)s_col[w][k + u] + lane_bytes));
             }
 #pragma unroll
             for (int u = 0; u < kTiledBatch; ++u)
@@ -233,6 +237,8 @@ int spmm_tiled_entry(const char *fn, int64_t M, int64_t K, int64_t N, int64_t nn
   if (N > INT32_MAX - kWaveSize * 4)
     return fail(SCORCH_HIP_EUNSUPPORTED, "%s: N=%lld is too large", fn, (long long)N);
   if (M == 0 || N == 0) return SCORCH_HIP_OK;  // nothing to write
+  if (K * (int64_t)kTileBytes > (int64_t)UINT32_MAX)  // (the kernel addresses a slice with 32-bit byte offsets)
+    return fail(SCORCH_HIP_EUNSUPPORTED, "%s: K=%lld rows make a slice of more than 4 GiB", fn, (long long)K);
   SCORCH_REQUIRE(C != nullptr, "%s: C is NULL", fn);
   SCORCH_REQUIRE(K == 0 || Bt != nullptr, "%s: the tiled operand is NULL", fn);
   SCORCH_REQUIRE(EPI == kEpiNone || bias != nullptr, "%s: bias is NULL", fn);
