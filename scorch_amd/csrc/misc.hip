@@ -35,18 +35,19 @@ LaunchMarks *launch_marks() {
 // read twice: a running maximum and sum first, the write second; the next
 // row's entries are requested before the current row's phases start): however such rows are placed in the matrix, few among
 // many short ones or all of them long, they are spread over the whole chip.
-// A row of more than kSoftmaxSplitRow entries is not one workgroup's either (the reference's
-// softmax is torch scatter operations over entries, bench/bench_sparse_transformer.py:277-297:
-// a single row of millions costs it what any other four million entries cost): the giant-row
-// kernel only enters it in a second list, cut into up to 1024 stretches, and two more kernels
-// serve the stretches -- softmax_split_partial_kernel a stretch's maximum and its sum of
-// exponentials relative to that, softmax_split_finish_kernel the row's maximum and sum from its
-// stretches' (in stretch order: the same bits on every run) and the stretch's results.
-// A row that holds more than one part in kSoftmaxLoneRowShare of all the giant rows' entries would set
-// the giant-row kernel's time by itself (a workgroup walks 50,000 entries in a dozen dependent round
-// trips while the others have finished), so beyond kSoftmaxLoneSplitRow entries it goes the same way, in
-// stretches of kSoftmaxLoneStretch; among many rows like itself it stays one workgroup's, whose second
-// sweep finds the row in its L2.
+// Some rows are not one workgroup's either (the reference's softmax is torch scatter operations
+// over entries, bench/bench_sparse_transformer.py:277-297: a single row of millions costs it what
+// any other four million entries cost): the giant-row kernel only enters such a row in a second
+// list, cut into up to 1024 stretches, and two more kernels serve the stretches --
+// softmax_split_partial_kernel a stretch's maximum and its sum of exponentials relative to that,
+// softmax_split_finish_kernel the row's maximum and sum from its stretches' (in stretch order: the
+// same bits on every run) and the stretch's results.  Which rows: one that holds more than one
+// part in kSoftmaxLoneRowShare of all the giant rows' entries (the short-row kernel sums them)
+// from kSoftmaxLoneSplitRow entries on -- alone, its workgroup's dozens of dependent round trips
+// would set the giant-row kernel's time while the other workgroups have finished -- and any row
+// of kSoftmaxFarRow entries or more.  A row between those that has many like itself beside it stays
+// one workgroup's: its second sweep finds the row in an L2 or the memory-side cache, where the
+// stretches' second read comes from memory (2,048 rows of 131,072 entries: 0.52 against 0.67 ms).
 // Values are loaded raw and scaled at their first use, so that a row's loads
 // are all issued before any of them is waited for.
 constexpr int kSoftmaxRegs = 4;
@@ -61,11 +62,14 @@ constexpr int kSoftmaxWaveRowMax = kSoftmaxRegs * kWaveSize;
 constexpr int kSoftmaxLongWaveRowMax = kSoftmaxBlockRegs * kWaveSize;
 constexpr int kSoftmaxBlockRowMax = kSoftmaxBlockRegs * kBlockThreads;
 constexpr int kSoftmaxGiantThreads = 1024;
-constexpr int kSoftmaxSplitRow = 65536;     // rows longer than this are shared out in stretches
+constexpr int kSoftmaxSplitRow = 65536;     // rows longer than this are shared out in stretches of kSoftmaxStretch
 constexpr int kSoftmaxStretch = 16384;      // entries of a stretch, at least
 // A row with more than 1 / kSoftmaxLoneRowShare of the entries of all giant rows is shared out from
 // kSoftmaxLoneSplitRow entries on, in shorter stretches.
 constexpr int kSoftmaxLoneRowShare = 100;
+// From this many entries on a row is shared out whatever the others are like: a workgroup's second
+// sweep over it would come from memory, not from an L2, as the stretches' second read does.
+constexpr int kSoftmaxFarRow = 1 << 19;
 constexpr int kSoftmaxLoneSplitRow = 16384;
 constexpr int kSoftmaxLoneStretch = 8192;
 constexpr int kSoftmaxMaxStretches = 1024;  // stretches of a row, at most (one per thread of the combining workgroup)
@@ -455,13 +459,13 @@ __global__ __launch_bounds__(kSoftmaxGiantThreads) void softmax_csr_giant_kernel
     for (int j = 1; j < kWaves; ++j) r = take_max ? fmaxf(r, s_red[j]) : r + s_red[j];
     return r;
   };
-  // A row of more than kSoftmaxSplitRow entries (kSoftmaxLoneSplitRow for one that holds a large part
-  // of all giant rows' entries) is entered in the list of rows that are served in stretches (by problem 0 of a batch: the pattern is the same for all) and skipped here.
-  // Uniform over the workgroup.
+  // A row that is served in stretches (see the head of this section) is entered in their list (by
+  // problem 0 of a batch: the pattern is the same for all) and skipped here.  Uniform over the workgroup.
   auto leave_to_the_stretch_kernels = [&](int row, int lo, int &hi) {
     const int len = hi - lo;
     const bool lone = (int64_t)len * kSoftmaxLoneRowShare > giant_entries;
-    if (split.rows == nullptr || len <= (lone ? kSoftmaxLoneSplitRow : kSoftmaxSplitRow)) return;
+    const int limit = lone ? kSoftmaxLoneSplitRow : len >= kSoftmaxFarRow ? kSoftmaxSplitRow : len;
+    if (split.rows == nullptr || len <= limit) return;
     hi = lo;
     if (blockIdx.y != 0) return;
     const int least = len > kSoftmaxSplitRow ? kSoftmaxStretch : kSoftmaxLoneStretch;

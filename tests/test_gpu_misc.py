@@ -137,7 +137,9 @@ def test_softmax_in_place(oracle):
 @pytest.mark.parametrize("lens", [[4_200_000], [3, 70_000, 0, 1_500_000, 12, 65_536, 65_537, 5000, 200_000],
                                   [17, 20_000_000],      # (more entries than 1024 stretches of 16,384 hold)
                                   # more than 512 rows beyond 4096 entries: those up to 65,536 stay one workgroup's
-                                  [4100] * 600 + [20_000, 70_000, 30_000, 65_536]])
+                                  [4100] * 600 + [20_000, 70_000, 30_000, 65_536],
+                                  # rows beyond 65,536 entries none of which stands out: one workgroup's each
+                                  [70_000] * 150 + [5, 600_000]])
 def test_softmax_rows_shared_out_among_workgroups(oracle, lens):
     """Rows of more than 65,536 entries are served in stretches by many workgroups (a single row of
     millions would otherwise be one workgroup's): against the fp64 recomputation, the same bits on
