@@ -210,7 +210,8 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_csr_kernel(int M,
   // further on, and only problem 0 lists the pattern's giant rows (they are the same for all)
   vals += blockIdx.y * nnz;
   out += blockIdx.y * nnz;
-  const bool list_giants = blockIdx.y == 0;
+  // (no list: the caller has vouched that no row is that long; one that is anyway is left unwritten)
+  const bool list_giants = blockIdx.y == 0 && giant_count != nullptr;
   // A lane group takes kTeamRows rows, one from each block of 256 / G consecutive rows
   // the workgroup owns, and requests the entries of all of them before it works on the
   // first: these rows are short, and with one row in flight per group the kernel waits on
