@@ -868,6 +868,9 @@ def main() -> int:
         result["configs"] = []
         for name in CONFIG_WORKLOADS:
             torch.cuda.empty_cache()
+            # the CPU leg of the configuration before leaves its OpenMP workers spinning for a moment; the
+            # first calls of the next one are host-bound and would be timed against them
+            time.sleep(0.2)
             try:
                 result["configs"].append(run_workload(name, args))
             except Exception as exc:  # one configuration failing must not lose the headline line
