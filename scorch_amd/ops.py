@@ -139,8 +139,32 @@ _direct_matmul: dict = {}
 _direct_fused: dict = {}
 
 
+_dense_requests: dict = {}
+
+
+def _requests_dense(requested, rank: int) -> bool:
+    """Whether a ``format`` argument asks for what this route returns anyway: a dense result of
+    this rank ("dd" for a matrix).  Strings are parsed once."""
+    if requested is None:
+        return True
+    key = (requested, rank) if isinstance(requested, str) else None
+    known = _dense_requests.get(key) if key is not None else None
+    if known is None:
+        try:
+            fmt = parse_format(requested)
+            known = fmt.is_dense() and fmt.get_order() == rank
+        except Exception:
+            known = False        # the general path words the error
+        if key is not None:
+            _dense_requests[key] = known
+    return known
+
+
 def _matmul_csr_dense_direct(a: STensor, b: torch.Tensor, kwargs) -> Optional[torch.Tensor]:
-    if kwargs and not (set(kwargs) <= {"time_dict", "use_cache"} and kwargs.get("use_cache", True)):
+    if kwargs and not (set(kwargs) <= {"time_dict", "use_cache", "format", "output_format"}
+                       and kwargs.get("use_cache", True)):
+        return None
+    if kwargs and not _requests_dense(kwargs.get("format", kwargs.get("output_format", None)), b.dim()):
         return None
     if b.layout != torch.strided or b.dim() not in (1, 2) or a.dim() != 2 or not b.is_cuda:
         return None
@@ -283,6 +307,11 @@ def einsum(expression: str, *tensors: Optional[Union[torch.Tensor, STensor]],
     requested = kwargs.get("format", kwargs.get("output_format", None))
     if canon == _SDDMM_EXPR and len(tensors) == 3 and requested is None:
         direct = _sddmm_direct(*tensors, time_dict)
+        if direct is not None:
+            return direct
+    if canon in (_SPMM_EXPR, "ab,b->a") and len(tensors) == 2 and isinstance(tensors[0], STensor) \
+            and isinstance(tensors[1], torch.Tensor) and tensors[1].dim() == (2 if canon == _SPMM_EXPR else 1):
+        direct = _matmul_csr_dense_direct(tensors[0], tensors[1], kwargs)   # the same product as matmul's
         if direct is not None:
             return direct
     operands = tuple(STensor.from_torch(t) if isinstance(t, torch.Tensor) else t for t in tensors)
