@@ -261,6 +261,32 @@ def test_matmul_accepts_torch_operands_and_fills_time_dict():
     assert torch.equal(scorch.matmul(scorch.from_csr(a.to_sparse_csr()), nc), out)
 
 
+def test_the_usual_spmm_calls_do_not_wrap_the_dense_operand(monkeypatch):
+    """matmul(A, B), matmul(A, B, format="dd"), einsum("ij,jk->ik", A, B) and the matrix-vector forms
+    reach the kernel without building STensors around the dense operand and the result (which
+    costs more host time than the kernel of a small product takes); a request for a sparse result
+    still goes the general way."""
+    torch.manual_seed(5)
+    a_t = torch.rand(96, 80) * (torch.rand(96, 80) < 0.1)
+    A = scorch.from_csr(a_t.to_sparse_csr()).to("cuda")
+    B, x = torch.rand(80, 24).cuda(), torch.rand(80).cuda()
+    want, want_v = scorch.matmul(A, B), scorch.matmul(A, x)
+    sparse_result = scorch.matmul(A, B, format="ds")
+    wrapped = []
+    real = STensor.from_torch
+    monkeypatch.setattr(STensor, "from_torch", staticmethod(lambda *a, **k: (wrapped.append(1), real(*a, **k))[1]))
+    for got in (scorch.matmul(A, B, format="dd"), scorch.matmul(A, B, output_format="dd"),
+                scorch.einsum("ij,jk->ik", A, B), scorch.einsum("ab,bc->ac", A, B, format="dd")):
+        assert isinstance(got, torch.Tensor) and torch.equal(got, want)
+    for got in (scorch.matmul(A, x, format="d"), scorch.einsum("ij,j->i", A, x)):
+        assert isinstance(got, torch.Tensor) and torch.equal(got, want_v)
+    assert not wrapped
+    again = scorch.matmul(A, B, format="ds")
+    assert wrapped and isinstance(again, STensor)
+    assert torch.equal(again.to_dense().to_torch(), sparse_result.to_dense().to_torch())
+    assert torch.allclose(want.cpu(), a_t @ B.cpu(), atol=1e-5)
+
+
 @pytest.mark.parametrize("dtype", [torch.float64, torch.int32, torch.int64])
 def test_matmul_other_dtypes(dtype):
     torch.manual_seed(2)
